@@ -1,0 +1,308 @@
+"""Shared machinery of the parity tests: seeded inputs, the oracle run, the GPU run through the
+C ABI, and the comparison.  The same `spec` dict drives zluda_amd.cublaslt.MatmulCall (GPU) and the
+zluda_gemm_problem handed to the CPU oracle."""
+import ctypes as C
+
+import numpy as np
+
+import oracle
+from zluda_amd import abi
+from zluda_amd.cublaslt import MatmulCall
+
+NP_OF = {abi.CUDA_R_32F: np.float32, abi.CUDA_R_32I: np.int32, abi.CUDA_R_16F: np.uint16,
+         abi.CUDA_R_16BF: np.uint16, abi.CUDA_R_8I: np.int8, abi.CUDA_R_8F_E4M3: np.uint8,
+         abi.CUDA_R_8F_E5M2: np.uint8}
+
+
+def _layout(spec, tag, rows, cols):
+    order = spec.get("order_" + tag, abi.CUBLASLT_ORDER_COL)
+    ld = spec.get("ld" + tag, rows if order == abi.CUBLASLT_ORDER_COL else cols)
+    lead = cols if order == abi.CUBLASLT_ORDER_COL else rows
+    stride = spec.get("stride_" + tag, ld * lead)
+    return order, ld, stride
+
+
+def _encode(values, typ):
+    """float32 values -> storage codes of `typ` (not FP4)."""
+    if typ == abi.CUDA_R_32F:
+        return values.astype(np.float32)
+    if typ == abi.CUDA_R_16F:
+        return oracle.encode_f16(values)
+    if typ == abi.CUDA_R_16BF:
+        return oracle.encode_bf16(values)
+    if typ == abi.CUDA_R_8F_E4M3:
+        return oracle.encode_e4m3(values)
+    if typ == abi.CUDA_R_8F_E5M2:
+        return oracle.encode_e5m2(values)
+    raise ValueError(typ)
+
+
+def decode_storage(buf, typ):
+    """storage codes -> float64 values (outputs)."""
+    if typ == abi.CUDA_R_32F:
+        return buf.astype(np.float64)
+    if typ in (abi.CUDA_R_32I, abi.CUDA_R_8I):
+        return buf.astype(np.float64)
+    if typ == abi.CUDA_R_16BF:
+        return oracle.decode_bf16(buf).astype(np.float64)
+    if typ == abi.CUDA_R_16F:
+        return buf.view(np.float16).astype(np.float64)
+    if typ == abi.CUDA_R_8F_E4M3:
+        return oracle.decode_table("e4m3")[buf].astype(np.float64)
+    if typ == abi.CUDA_R_8F_E5M2:
+        return oracle.decode_table("e5m2")[buf].astype(np.float64)
+    raise ValueError(typ)
+
+
+class Case:
+    """Host-side data of one matmul."""
+
+    def __init__(self, spec, seed, int_dist="uniform", value_scale=1.0):
+        self.spec = s = dict(spec)
+        rng = np.random.default_rng(seed)
+        m, n, k = s["m"], s["n"], s["k"]
+        batch = s.get("batch", 1)
+        ta, tb = s.get("transa", 0) != 0, s.get("transb", 0) != 0
+        s.setdefault("c_type", s["d_type"])
+        self.batch = batch
+        self.a_scale = self.b_scale = self.c_scale = self.d_scale = self.bias = None
+
+        def operand(tag, typ, rows, cols, k_is_rows, scale_mode):
+            """returns (storage array, block scale array or None)"""
+            order, ld, stride = _layout(s, tag, rows, cols)
+            total = stride * (batch - 1) + ld * (cols if order == abi.CUBLASLT_ORDER_COL else rows)
+            if typ == abi.CUDA_R_4F_E2M1:
+                # K must be the contiguous dimension
+                contig_rows = order == abi.CUBLASLT_ORDER_COL
+                assert contig_rows == k_is_rows, "FP4 operands must be K-contiguous"
+                nvec = cols if contig_rows else rows  # number of K-vectors (M or N)
+                store = rng.integers(0, 256, size=(total + 1) // 2, dtype=np.uint8)
+                scales = np.empty((batch, nvec, k // 32), np.uint8)
+                for b in range(batch):
+                    x = (rng.standard_normal((nvec, k)) * value_scale).astype(np.float32)
+                    q, sc = oracle.quantize_mxfp4(x)
+                    scales[b] = sc
+                    for v in range(nvec):
+                        off = (stride * b + v * ld) // 2
+                        store[off:off + k // 2] = q[v]
+                return store, scales
+            if typ == abi.CUDA_R_8I:
+                if int_dist == "uniform":
+                    store = rng.integers(-128, 128, size=total, dtype=np.int8)
+                else:  # round(N(0, 32)) clipped to +-127
+                    store = np.clip(np.rint(rng.standard_normal(total) * 32.0), -127, 127).astype(np.int8)
+                return store, None
+            vals = (rng.standard_normal(total) * value_scale).astype(np.float32)
+            store = _encode(vals, typ)
+            scales = None
+            if scale_mode == abi.CUBLASLT_MATMUL_MATRIX_SCALE_VEC32_UE8M0:
+                nvec = cols if k_is_rows else rows
+                scales = rng.integers(120, 135, size=(batch, nvec, k // 32), dtype=np.uint8)
+            return store, scales
+
+        self.A, a_blk = operand("a", s["a_type"], k if ta else m, m if ta else k, ta, s.get("a_scale_mode", 0))
+        self.B, b_blk = operand("b", s["b_type"], n if tb else k, k if tb else n, not tb, s.get("b_scale_mode", 0))
+        # C and D
+        _, ldc, sc = _layout(s, "c", m, n)
+        _, ldd, sd = _layout(s, "d", m, n)
+        oc = s.get("order_c", 0)
+        od = s.get("order_d", 0)
+        ctot = sc * (batch - 1) + ldc * (n if oc == 0 else m)
+        dtot = sd * (batch - 1) + ldd * (n if od == 0 else m)
+        self.has_c = s.get("with_c", False)
+        if self.has_c:
+            if s["c_type"] == abi.CUDA_R_32I:
+                self.Cm = rng.integers(-1000, 1000, size=ctot, dtype=np.int32)
+            elif s["c_type"] == abi.CUDA_R_8I:
+                self.Cm = rng.integers(-128, 128, size=ctot, dtype=np.int8)
+            else:
+                self.Cm = _encode(rng.standard_normal(ctot).astype(np.float32), s["c_type"])
+        else:
+            self.Cm = None
+        self.dtot = dtot
+        self.d_np = NP_OF[s["d_type"]]
+
+        # alpha / beta
+        pm = s.get("pointer_mode", abi.CUBLASLT_POINTER_MODE_HOST)
+        int_scale = s["scale_type"] == abi.CUDA_R_32I
+        sdt = np.int32 if int_scale else np.float32
+        avs = s.get("alpha_vector_batch_stride", 0)
+        alpha_vec = pm in (abi.CUBLASLT_POINTER_MODE_DEVICE_VECTOR,
+                           abi.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO,
+                           abi.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_HOST)
+        nalpha = (m + avs * (batch - 1)) if alpha_vec else 1
+        if "alpha" in s:
+            self.alpha = np.full(nalpha, s["alpha"], dtype=sdt)
+        elif int_scale:
+            self.alpha = rng.integers(-3, 4, size=nalpha).astype(np.int32)
+            self.alpha[self.alpha == 0] = 1
+        else:
+            lo, hi = s.get("alpha_range", (0.5, 1.5))
+            self.alpha = rng.uniform(lo, hi, size=nalpha).astype(np.float32)
+        nbeta = m if pm == abi.CUBLASLT_POINTER_MODE_DEVICE_VECTOR else 1
+        if not self.has_c:
+            self.beta = np.zeros(nbeta, dtype=sdt)
+        elif int_scale:
+            self.beta = rng.integers(1, 3, size=nbeta).astype(np.int32)
+        else:
+            self.beta = rng.uniform(0.5, 1.5, size=nbeta).astype(np.float32)
+        self.alpha_on_device = pm != abi.CUBLASLT_POINTER_MODE_HOST
+        self.beta_on_device = pm in (abi.CUBLASLT_POINTER_MODE_DEVICE, abi.CUBLASLT_POINTER_MODE_DEVICE_VECTOR)
+
+        # scales
+        def scale(mode, blk, n_outer, rng_range):
+            if mode == abi.CUBLASLT_MATMUL_MATRIX_SCALE_VEC32_UE8M0:
+                return blk
+            if mode == abi.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F:
+                return rng.uniform(*rng_range, size=n_outer).astype(np.float32)
+            if s.get("with_scalar_scales", False):
+                return rng.uniform(*rng_range, size=1).astype(np.float32)
+            return None
+        sr = s.get("scale_range", (0.5, 2.0))
+        self.a_scale = scale(s.get("a_scale_mode", 0), a_blk, m, sr)
+        self.b_scale = scale(s.get("b_scale_mode", 0), b_blk, n, sr)
+        if s.get("with_cd_scales", False):
+            self.c_scale = rng.uniform(0.5, 2.0, size=1).astype(np.float32)
+            self.d_scale = rng.uniform(0.5, 2.0, size=1).astype(np.float32)
+
+        # bias
+        epi = s.get("epilogue", abi.CUBLASLT_EPILOGUE_DEFAULT)
+        if epi in (abi.CUBLASLT_EPILOGUE_BIAS, abi.CUBLASLT_EPILOGUE_RELU_BIAS, abi.CUBLASLT_EPILOGUE_GELU_BIAS):
+            bt = s.get("bias_type", -1)
+            if bt < 0:
+                bt = abi.CUDA_R_32F if s["d_type"] in (abi.CUDA_R_8I, abi.CUDA_R_32I, abi.CUDA_R_8F_E4M3,
+                                                       abi.CUDA_R_8F_E5M2) else s["d_type"]
+            nb = m + s.get("bias_batch_stride", 0) * (batch - 1)
+            bvals = (rng.standard_normal(nb) * s.get("bias_std", 0.5)).astype(np.float32)
+            self.bias = _encode(bvals, bt)
+
+    def new_d(self):
+        """output storage pre-filled with a canary pattern"""
+        return np.frombuffer(bytes([0xCD]) * (self.dtot * np.dtype(self.d_np).itemsize), dtype=self.d_np).copy()
+
+    # ---- CPU oracle ---------------------------------------------------------------------------
+    def problem(self, ptrs):
+        """zluda_gemm_problem with the given pointer dict (host or device addresses)."""
+        s = self.spec
+        m, n, k = s["m"], s["n"], s["k"]
+        ta, tb = s.get("transa", 0) != 0, s.get("transb", 0) != 0
+        p = abi.zluda_gemm_problem()
+
+        def lay(dst, tag, typ, rows, cols):
+            order, ld, stride = _layout(s, tag, rows, cols)
+            dst.type, dst.order, dst.rows, dst.cols, dst.ld = typ, order, rows, cols, ld
+            dst.batch_count, dst.batch_stride = self.batch, stride
+        lay(p.a, "a", s["a_type"], k if ta else m, m if ta else k)
+        lay(p.b, "b", s["b_type"], n if tb else k, k if tb else n)
+        lay(p.c, "c", s["c_type"], m, n)
+        lay(p.d, "d", s["d_type"], m, n)
+        o = p.op
+        o.compute_type, o.scale_type = s["compute_type"], s["scale_type"]
+        o.pointer_mode = s.get("pointer_mode", 0)
+        o.transa, o.transb = s.get("transa", 0), s.get("transb", 0)
+        o.epilogue = s.get("epilogue", abi.CUBLASLT_EPILOGUE_DEFAULT)
+        o.bias_type = s.get("bias_type", -1)
+        o.bias_batch_stride = s.get("bias_batch_stride", 0)
+        o.alpha_vector_batch_stride = s.get("alpha_vector_batch_stride", 0)
+        o.a_scale_mode, o.b_scale_mode = s.get("a_scale_mode", 0), s.get("b_scale_mode", 0)
+        o.bias, o.a_scale, o.b_scale = ptrs.get("bias"), ptrs.get("a_scale"), ptrs.get("b_scale")
+        o.c_scale, o.d_scale = ptrs.get("c_scale"), ptrs.get("d_scale")
+        p.alpha, p.beta = ptrs["alpha"], ptrs["beta"]
+        p.A, p.B, p.C, p.D = ptrs["A"], ptrs["B"], ptrs.get("C"), ptrs["D"]
+        return p
+
+    def run_oracle(self):
+        d = self.new_d()
+        hp = lambda x: x.ctypes.data if x is not None else None
+        ptrs = {"A": hp(self.A), "B": hp(self.B), "C": hp(self.Cm), "D": hp(d), "alpha": hp(self.alpha),
+                "beta": hp(self.beta), "bias": hp(self.bias), "a_scale": hp(self.a_scale),
+                "b_scale": hp(self.b_scale), "c_scale": hp(self.c_scale), "d_scale": hp(self.d_scale)}
+        p = self.problem(ptrs)
+        st = oracle.gemm(p)
+        assert st == 0, "oracle status %d" % st
+        return d
+
+    # ---- GPU through the C ABI ------------------------------------------------------------------
+    def run_gpu(self, api, forced_kernel=None, forced_variant=-1, offset_bytes=0):
+        """Returns (status, D storage, kernel family, variant).  offset_bytes misaligns A and B."""
+        import torch
+        dev = torch.device("cuda:0")
+
+        def up(x, off=0):
+            if x is None:
+                return None, None
+            raw = np.frombuffer(x.tobytes(), dtype=np.uint8)
+            t = torch.empty(raw.size + off + 16, dtype=torch.uint8, device=dev)
+            t[off:off + raw.size] = torch.from_numpy(raw.copy()).to(dev)
+            return t, t.data_ptr() + off
+        keep = []
+        ptr = {}
+        for name, arr, off in (("A", self.A, offset_bytes), ("B", self.B, offset_bytes), ("C", self.Cm, 0),
+                               ("bias", self.bias, 0), ("a_scale", self.a_scale, 0),
+                               ("b_scale", self.b_scale, 0), ("c_scale", self.c_scale, 0),
+                               ("d_scale", self.d_scale, 0)):
+            t, p = up(arr, off)
+            keep.append(t)
+            ptr[name] = p
+        d0 = self.new_d()
+        dt, ptr["D"] = up(d0)
+        call = MatmulCall(api, self.spec, forced_kernel=forced_kernel, forced_variant=forced_variant)
+        try:
+            call.set_pointers(bias=ptr["bias"], a_scale=ptr["a_scale"], b_scale=ptr["b_scale"],
+                              c_scale=ptr["c_scale"], d_scale=ptr["d_scale"])
+            if self.alpha_on_device:
+                at, alpha = up(self.alpha)
+                keep.append(at)
+            else:
+                alpha = (C.c_int32 if self.alpha.dtype == np.int32 else C.c_float)(self.alpha[0].item())
+            if self.beta_on_device:
+                btens, beta = up(self.beta)
+                keep.append(btens)
+            else:
+                beta = (C.c_int32 if self.beta.dtype == np.int32 else C.c_float)(self.beta[0].item())
+            stream = torch.cuda.current_stream().cuda_stream
+            st = call.run(alpha, ptr["A"], ptr["B"], beta, ptr["C"], ptr["D"], None, 0, stream)
+            torch.cuda.synchronize()
+            nbytes = d0.size * d0.itemsize
+            out = dt[:nbytes].cpu().numpy().view(self.d_np).copy()
+            return st, out, call.kernel, call.variant
+        finally:
+            call.close()
+
+    # ---- comparison -------------------------------------------------------------------------------
+    def logical_index(self):
+        """flat storage indices of D(i, j, batch) as an int64 array [batch, m, n]"""
+        s = self.spec
+        m, n = s["m"], s["n"]
+        order, ld, stride = _layout(s, "d", m, n)
+        i = np.arange(m)[:, None]
+        j = np.arange(n)[None, :]
+        base = (i + j * ld) if order == abi.CUBLASLT_ORDER_COL else (i * ld + j)
+        return np.stack([base + b * stride for b in range(self.batch)])
+
+    def compare(self, got, ref, tol=None):
+        """bit-exact for integer outputs (whole storage incl. padding); otherwise padding must be
+        untouched and max |got-ref| / max(|ref|, floor) <= tol with floor = 1e-2 * rms(ref)."""
+        s = self.spec
+        if s["d_type"] in (abi.CUDA_R_32I, abi.CUDA_R_8I) and s["scale_type"] == abi.CUDA_R_32I:
+            bad = np.nonzero(got != ref)[0]
+            assert bad.size == 0, "%d mismatching int32 elements, first at %d: %d vs %d" % (
+                bad.size, bad[0], got[bad[0]], ref[bad[0]])
+            return 0.0
+        idx = self.logical_index().ravel()
+        mask = np.ones(got.size, bool)
+        mask[idx] = False
+        assert np.array_equal(got[mask], ref[mask]), "padding between ld and rows was overwritten"
+        g = decode_storage(got[idx], s["d_type"])
+        r = decode_storage(ref[idx], s["d_type"])
+        assert np.isfinite(g).all() and np.isfinite(r).all()
+        rms = float(np.sqrt(np.mean(r * r)))
+        floor = 1e-2 * rms if rms > 0 else 1.0
+        err = float(np.max(np.abs(g - r) / np.maximum(np.abs(r), floor)))
+        if tol is None:
+            tol = 1e-2
+        if s["d_type"] == abi.CUDA_R_8I:
+            assert np.max(np.abs(g - r)) <= 1, "int8 outputs differ by more than one step"
+            return err
+        assert err <= tol, "max relative error %.3e > %.1e" % (err, tol)
+        return err

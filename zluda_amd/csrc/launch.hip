@@ -1,0 +1,113 @@
+// The extern "C" launch layer: lowers a problem, picks the template instantiation the plan names
+// and enqueues it on the caller's stream.  Only the HIP runtime is used (hipLaunchKernelGGL).
+#include <hip/hip_runtime.h>
+
+#include "kernels/decode_w8a8.hpp"
+#include "kernels/gemm_generic.hpp"
+#include "mfma_launch.hpp"
+#include "planner.hpp"
+
+using namespace zluda_amd;
+
+namespace {
+
+inline int f8_fmt(uint32_t t) { return t == CUDA_R_8F_E5M2 ? 1 : 0; }
+
+uint32_t launch_mfma(const Lowered &l, const zluda_gemm_plan &plan, hipStream_t s) {
+  MfmaParams prm;
+  prm.g = l.g;
+  prm.swapped = plan.swapped;
+  if (plan.variant >= 2 * kNumMfmaVariants) return CUBLAS_STATUS_INVALID_VALUE;
+  const MfmaVariant &v = kMfmaVariants[plan.variant % kNumMfmaVariants];
+  const int np = plan.swapped ? l.g.N : l.g.M, nq = plan.swapped ? l.g.M : l.g.N;
+  prm.tiles_p = (np + v.bp - 1) / v.bp;
+  prm.tiles_q = (nq + v.bq - 1) / v.bq;
+  prm.group_p = 8;
+  if ((uint32_t)(prm.tiles_p * prm.tiles_q) != plan.grid_x) return CUBLAS_STATUS_INVALID_VALUE;
+  switch (plan.kernel) {
+  case ZLUDA_KERNEL_MFMA_I8: return launch_mfma_i8(prm, plan, s);
+  case ZLUDA_KERNEL_MFMA_MXF4: return launch_mfma_mxf4(prm, plan, s);
+  case ZLUDA_KERNEL_MFMA_F8: {
+    // MFMA operand "A" is Q, operand "B" is P (see gemm_mfma.hpp)
+    const int fa = f8_fmt(l.g.a_type), fb = f8_fmt(l.g.b_type);
+    return launch_mfma_f8(prm, plan, plan.swapped ? fa : fb, plan.swapped ? fb : fa, s);
+  }
+  default: return CUBLAS_STATUS_INTERNAL_ERROR;
+  }
+}
+
+template <int NW, int STEPS>
+void launch_decode_variant(const DecodeParams &prm, const zluda_gemm_plan &plan, int nb, bool full, hipStream_t s) {
+  dim3 grid(plan.grid_x, plan.grid_y, 1), block(NW * 64);
+  if (nb == 1) {
+    if (full) hipLaunchKernelGGL((decode_w8a8_kernel<NW, STEPS, 1, true>), grid, block, 0, s, prm);
+    else hipLaunchKernelGGL((decode_w8a8_kernel<NW, STEPS, 1, false>), grid, block, 0, s, prm);
+  } else if constexpr (STEPS <= 8) {  // two token blocks double the fragment registers
+    if (full) hipLaunchKernelGGL((decode_w8a8_kernel<NW, STEPS, 2, true>), grid, block, 0, s, prm);
+    else hipLaunchKernelGGL((decode_w8a8_kernel<NW, STEPS, 2, false>), grid, block, 0, s, prm);
+  }
+}
+
+uint32_t launch_decode(const Lowered &l, const zluda_gemm_plan &plan, hipStream_t s) {
+  const DecodeVariant &v = kDecodeVariants[plan.variant];
+  DecodeParams prm;
+  prm.g = l.g;
+  prm.swapped = plan.swapped;
+  const int T = plan.swapped ? l.g.M : l.g.N;
+  const int ksteps = (l.g.K + 63) / 64;
+  prm.spw = (ksteps + v.nw - 1) / v.nw;
+  prm.nchunks = (prm.spw + v.steps - 1) / v.steps;
+  const bool full = l.g.K == v.nw * v.steps * 64;
+  const int nb = T <= 16 ? 1 : 2;
+  if (nb == 2 && v.steps > 8) return CUBLAS_STATUS_NOT_SUPPORTED;
+  switch (plan.variant) {
+  case 0: launch_decode_variant<8, 8>(prm, plan, nb, full, s); break;
+  case 1: launch_decode_variant<8, 16>(prm, plan, nb, full, s); break;
+  case 2: launch_decode_variant<4, 16>(prm, plan, nb, full, s); break;
+  case 3: launch_decode_variant<4, 8>(prm, plan, nb, full, s); break;
+  default: return CUBLAS_STATUS_INVALID_VALUE;
+  }
+  return CUBLAS_STATUS_SUCCESS;
+}
+
+} // namespace
+
+extern "C" uint32_t zluda_gemm_device_cu_count(void) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 0;
+  static int cached[64];
+  if (dev >= 0 && dev < 64 && cached[dev]) return (uint32_t)cached[dev];
+  int cus = 0;
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+  if (dev >= 0 && dev < 64) cached[dev] = cus;
+  return (uint32_t)cus;
+}
+
+extern "C" uint32_t zluda_gemm_launch(const zluda_gemm_problem *p, const zluda_gemm_plan *plan,
+                                      void *stream) {
+  if (!p || !plan) return CUBLAS_STATUS_INVALID_VALUE;
+  Lowered l;
+  uint32_t st = lower_problem(p, false, &l);
+  if (st) return st;
+  if (!family_supports(plan->kernel, l)) return CUBLAS_STATUS_INVALID_VALUE;
+  if (p->workspace_size < plan->workspace) return CUBLAS_STATUS_INVALID_VALUE;
+  if (zluda_gemm_device_cu_count() == 0) return CUBLAS_STATUS_NOT_INITIALIZED;
+  hipStream_t s = (hipStream_t)stream;
+  switch (plan->kernel) {
+  case ZLUDA_KERNEL_GENERIC: {
+    dim3 grid(plan->grid_x, plan->grid_y, plan->grid_z);
+    const bool int_acc = l.g.a_type == CUDA_R_8I;
+    if (int_acc) hipLaunchKernelGGL(gemm_generic_kernel<true>, grid, dim3(256), 0, s, l.g);
+    else hipLaunchKernelGGL(gemm_generic_kernel<false>, grid, dim3(256), 0, s, l.g);
+    break;
+  }
+  case ZLUDA_KERNEL_MFMA_I8: case ZLUDA_KERNEL_MFMA_F8: case ZLUDA_KERNEL_MFMA_MXF4:
+    if ((st = launch_mfma(l, *plan, s))) return st;
+    break;
+  case ZLUDA_KERNEL_DECODE_W8A8:
+    if ((st = launch_decode(l, *plan, s))) return st;
+    break;
+  default: return CUBLAS_STATUS_NOT_SUPPORTED;
+  }
+  return hipGetLastError() == hipSuccess ? CUBLAS_STATUS_SUCCESS : CUBLAS_STATUS_EXECUTION_FAILED;
+}

@@ -1,0 +1,336 @@
+// Problem validation, lowering to strides, and kernel selection.  Host code only.
+//
+// The accepted surface follows the reference's (zluda_blaslt/src/impl.rs:257-305 for the
+// attributes, zluda_common/src/lib.rs:575-630 for the type maps) extended by what the quantized
+// path needs: scale pointers/modes, pointer modes, FP4/UE8M0 types.
+#include "planner.hpp"
+
+#include <algorithm>
+#include <cstdlib>
+#include <cstring>
+
+namespace zluda_amd {
+
+static int type_bits(uint32_t t) {
+  switch (t) {
+  case CUDA_R_32F: case CUDA_R_32I: return 32;
+  case CUDA_R_16F: case CUDA_R_16BF: return 16;
+  case CUDA_R_8I: case CUDA_R_8F_E4M3: case CUDA_R_8F_E5M2: return 8;
+  case CUDA_R_4F_E2M1: return 4;
+  default: return 0;
+  }
+}
+
+static bool is_float_in(uint32_t t) {
+  return t == CUDA_R_32F || t == CUDA_R_16F || t == CUDA_R_16BF || t == CUDA_R_8F_E4M3 ||
+         t == CUDA_R_8F_E5M2 || t == CUDA_R_4F_E2M1;
+}
+
+static uint32_t layout_ok(const zluda_matrix_layout &l) {
+  if (l.order != CUBLASLT_ORDER_COL && l.order != CUBLASLT_ORDER_ROW) return CUBLAS_STATUS_NOT_SUPPORTED;
+  if (!type_bits(l.type)) return CUBLAS_STATUS_NOT_SUPPORTED;
+  if (l.rows == 0 || l.cols == 0) return CUBLAS_STATUS_INVALID_VALUE;
+  if (l.rows > 0x7fffffffull || l.cols > 0x7fffffffull) return CUBLAS_STATUS_NOT_SUPPORTED;
+  const int64_t lead = l.order == CUBLASLT_ORDER_COL ? (int64_t)l.rows : (int64_t)l.cols;
+  if (l.ld < lead) return CUBLAS_STATUS_INVALID_VALUE;
+  if (l.batch_count < 1) return CUBLAS_STATUS_INVALID_VALUE;
+  return CUBLAS_STATUS_SUCCESS;
+}
+
+static int convert_scale_mode(int32_t cuda_mode, const void *ptr, bool dry, int32_t *out) {
+  switch (cuda_mode) {
+  case CUBLASLT_MATMUL_MATRIX_SCALE_SCALAR_32F: *out = ptr ? SCALE_SCALAR : SCALE_NONE; return 0;
+  case CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F: *out = SCALE_OUTER_VEC; return (ptr || dry) ? 0 : 1;
+  case CUBLASLT_MATMUL_MATRIX_SCALE_VEC32_UE8M0: *out = SCALE_BLOCK32_UE8M0; return (ptr || dry) ? 0 : 1;
+  default: return 2;
+  }
+}
+
+uint32_t lower_problem(const zluda_gemm_problem *p, bool dry, Lowered *out) {
+  if (!p || !out) return CUBLAS_STATUS_INVALID_VALUE;
+  const zluda_matmul_desc &op = p->op;
+  const zluda_matrix_layout &a = p->a, &b = p->b, &d = p->d;
+  const zluda_matrix_layout &c = p->c;
+  uint32_t st;
+  if ((st = layout_ok(a)) || (st = layout_ok(b)) || (st = layout_ok(c)) || (st = layout_ok(d))) return st;
+  if (op.transa > CUBLAS_OP_C || op.transb > CUBLAS_OP_C) return CUBLAS_STATUS_INVALID_VALUE;
+  const bool ta = op.transa != CUBLAS_OP_N, tb = op.transb != CUBLAS_OP_N;
+
+  GemmArgs g;
+  memset(&g, 0, sizeof(g));
+  const uint64_t M = d.rows, N = d.cols, K = ta ? a.rows : a.cols;
+  if ((ta ? a.cols : a.rows) != M) return CUBLAS_STATUS_INVALID_VALUE;
+  if ((tb ? b.cols : b.rows) != K) return CUBLAS_STATUS_INVALID_VALUE;
+  if ((tb ? b.rows : b.cols) != N) return CUBLAS_STATUS_INVALID_VALUE;
+  if (c.rows != M || c.cols != N) return CUBLAS_STATUS_INVALID_VALUE;
+  g.M = (int32_t)M; g.N = (int32_t)N; g.K = (int32_t)K;
+
+  const bool a_col = a.order == CUBLASLT_ORDER_COL, b_col = b.order == CUBLASLT_ORDER_COL;
+  // op(A)(i,k): stored (r,c) = ta ? (k,i) : (i,k)
+  if (!ta) { g.a_si = a_col ? 1 : a.ld; g.a_sk = a_col ? a.ld : 1; }
+  else     { g.a_sk = a_col ? 1 : a.ld; g.a_si = a_col ? a.ld : 1; }
+  // op(B)(k,j): stored (r,c) = tb ? (j,k) : (k,j)
+  if (!tb) { g.b_sk = b_col ? 1 : b.ld; g.b_sj = b_col ? b.ld : 1; }
+  else     { g.b_sj = b_col ? 1 : b.ld; g.b_sk = b_col ? b.ld : 1; }
+  g.c_si = c.order == CUBLASLT_ORDER_COL ? 1 : c.ld; g.c_sj = c.order == CUBLASLT_ORDER_COL ? c.ld : 1;
+  g.d_si = d.order == CUBLASLT_ORDER_COL ? 1 : d.ld; g.d_sj = d.order == CUBLASLT_ORDER_COL ? d.ld : 1;
+
+  g.batch = d.batch_count;
+  if (a.batch_count != g.batch || b.batch_count != g.batch || c.batch_count != g.batch)
+    return CUBLAS_STATUS_INVALID_VALUE;
+  g.a_sb = a.batch_stride; g.b_sb = b.batch_stride; g.c_sb = c.batch_stride; g.d_sb = d.batch_stride;
+  if (g.batch > 65535) return CUBLAS_STATUS_NOT_SUPPORTED;
+
+  g.a_type = a.type; g.b_type = b.type; g.c_type = c.type; g.d_type = d.type;
+
+  // ---- compute / scale type ------------------------------------------------------------------
+  const uint32_t ct = op.compute_type;
+  const bool int_path = ct == CUBLAS_COMPUTE_32I || ct == CUBLAS_COMPUTE_32I_PEDANTIC;
+  const bool f32_path = ct == CUBLAS_COMPUTE_32F || ct == CUBLAS_COMPUTE_32F_PEDANTIC ||
+                        ct == CUBLAS_COMPUTE_32F_FAST_16F || ct == CUBLAS_COMPUTE_32F_FAST_16BF ||
+                        ct == CUBLAS_COMPUTE_32F_FAST_TF32;
+  if (!int_path && !f32_path) return CUBLAS_STATUS_NOT_SUPPORTED;
+  if (int_path) {
+    if (a.type != CUDA_R_8I || b.type != CUDA_R_8I) return CUBLAS_STATUS_NOT_SUPPORTED;
+    if (op.scale_type == CUDA_R_32I) {
+      if (d.type != CUDA_R_32I || c.type != CUDA_R_32I) return CUBLAS_STATUS_NOT_SUPPORTED;
+      if (op.epilogue != CUBLASLT_EPILOGUE_DEFAULT) return CUBLAS_STATUS_NOT_SUPPORTED;
+      g.int_scale = 1;
+    } else if (op.scale_type == CUDA_R_32F) {
+      if (!(d.type == CUDA_R_8I || d.type == CUDA_R_32I || d.type == CUDA_R_16BF ||
+            d.type == CUDA_R_16F || d.type == CUDA_R_32F))
+        return CUBLAS_STATUS_NOT_SUPPORTED;
+    } else return CUBLAS_STATUS_NOT_SUPPORTED;
+  } else {
+    if (!is_float_in(a.type) || !is_float_in(b.type)) return CUBLAS_STATUS_NOT_SUPPORTED;
+    if (op.scale_type != CUDA_R_32F) return CUBLAS_STATUS_NOT_SUPPORTED;
+    if (!(d.type == CUDA_R_32F || d.type == CUDA_R_16F || d.type == CUDA_R_16BF ||
+          d.type == CUDA_R_8F_E4M3 || d.type == CUDA_R_8F_E5M2))
+      return CUBLAS_STATUS_NOT_SUPPORTED;
+    // 16/32-bit inputs: both operands of one type (as in cuBLASLt); 8/4-bit floats may mix
+    if (type_bits(a.type) >= 16 && a.type != b.type) return CUBLAS_STATUS_NOT_SUPPORTED;
+    if (type_bits(a.type) != type_bits(b.type)) return CUBLAS_STATUS_NOT_SUPPORTED;
+  }
+  if (!g.int_scale && (c.type == CUDA_R_4F_E2M1 || d.type == CUDA_R_4F_E2M1)) return CUBLAS_STATUS_NOT_SUPPORTED;
+
+  // FP4 is packed two per byte along K
+  if (a.type == CUDA_R_4F_E2M1 && (g.a_sk != 1 || (a.ld & 1) || (a.batch_stride & 1))) return CUBLAS_STATUS_NOT_SUPPORTED;
+  if (b.type == CUDA_R_4F_E2M1 && (g.b_sk != 1 || (b.ld & 1) || (b.batch_stride & 1))) return CUBLAS_STATUS_NOT_SUPPORTED;
+  if ((a.type == CUDA_R_4F_E2M1 || b.type == CUDA_R_4F_E2M1) && (K & 1)) return CUBLAS_STATUS_INVALID_VALUE;
+
+  // ---- alpha / beta ------------------------------------------------------------------------
+  switch (op.pointer_mode) {
+  case CUBLASLT_POINTER_MODE_HOST: g.alpha_mode = SCALAR_VALUE; g.beta_mode = SCALAR_VALUE; break;
+  case CUBLASLT_POINTER_MODE_DEVICE: g.alpha_mode = SCALAR_DEV; g.beta_mode = SCALAR_DEV; break;
+  case CUBLASLT_POINTER_MODE_DEVICE_VECTOR: g.alpha_mode = VECTOR_DEV; g.beta_mode = VECTOR_DEV; break;
+  case CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO: g.alpha_mode = VECTOR_DEV; g.beta_mode = SCALAR_VALUE; break;
+  case CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_HOST: g.alpha_mode = VECTOR_DEV; g.beta_mode = SCALAR_VALUE; break;
+  default: return CUBLAS_STATUS_INVALID_VALUE;
+  }
+  g.alpha_sb = op.alpha_vector_batch_stride;
+  if (op.pointer_mode == CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO && g.alpha_sb != 0)
+    return CUBLAS_STATUS_INVALID_VALUE;  // cuda_types/src/cublaslt.rs:4240-4247
+  bool beta_maybe_nonzero = true;
+  if (!dry) {
+    if (!p->alpha) return CUBLAS_STATUS_INVALID_VALUE;
+    if (g.alpha_mode == SCALAR_VALUE) memcpy(&g.alpha_val, p->alpha, 4);
+    else g.alpha_ptr = p->alpha;
+    if (op.pointer_mode == CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO) {
+      g.beta_val.i = 0;
+    } else {
+      if (!p->beta) return CUBLAS_STATUS_INVALID_VALUE;
+      if (g.beta_mode == SCALAR_VALUE) memcpy(&g.beta_val, p->beta, 4);
+      else g.beta_ptr = p->beta;
+    }
+    if (g.beta_mode == SCALAR_VALUE) beta_maybe_nonzero = g.int_scale ? g.beta_val.i != 0 : g.beta_val.f != 0.0f;
+    if (beta_maybe_nonzero && !p->C) return CUBLAS_STATUS_INVALID_VALUE;
+    if (!p->A || !p->B || !p->D) return CUBLAS_STATUS_INVALID_VALUE;
+  }
+  g.A = p->A; g.B = p->B; g.C = p->C; g.D = p->D;
+
+  // ---- scales --------------------------------------------------------------------------------
+  int r;
+  if ((r = convert_scale_mode(op.a_scale_mode, op.a_scale, dry, &g.a_scale_mode)))
+    return r == 1 ? CUBLAS_STATUS_INVALID_VALUE : CUBLAS_STATUS_NOT_SUPPORTED;
+  if ((r = convert_scale_mode(op.b_scale_mode, op.b_scale, dry, &g.b_scale_mode)))
+    return r == 1 ? CUBLAS_STATUS_INVALID_VALUE : CUBLAS_STATUS_NOT_SUPPORTED;
+  if (op.c_scale_mode != CUBLASLT_MATMUL_MATRIX_SCALE_SCALAR_32F ||
+      op.d_scale_mode != CUBLASLT_MATMUL_MATRIX_SCALE_SCALAR_32F)
+    return CUBLAS_STATUS_NOT_SUPPORTED;
+  g.a_scale = op.a_scale; g.b_scale = op.b_scale; g.c_scale = op.c_scale; g.d_scale = op.d_scale;
+  if (g.int_scale && (g.a_scale_mode || g.b_scale_mode || g.c_scale || g.d_scale))
+    return CUBLAS_STATUS_INVALID_VALUE;  // cuda_types/src/cublaslt.rs:4266-4267
+  if (g.a_scale_mode == SCALE_BLOCK32_UE8M0 && (int_path || g.a_sk != 1 || (K % 32))) return CUBLAS_STATUS_NOT_SUPPORTED;
+  if (g.b_scale_mode == SCALE_BLOCK32_UE8M0 && (int_path || g.b_sk != 1 || (K % 32))) return CUBLAS_STATUS_NOT_SUPPORTED;
+
+  // ---- epilogue ------------------------------------------------------------------------------
+  bool has_bias = false;
+  switch (op.epilogue) {
+  case CUBLASLT_EPILOGUE_DEFAULT: g.act = ACT_NONE; break;
+  case CUBLASLT_EPILOGUE_RELU: g.act = ACT_RELU; break;
+  case CUBLASLT_EPILOGUE_GELU: g.act = ACT_GELU; break;
+  case CUBLASLT_EPILOGUE_BIAS: g.act = ACT_NONE; has_bias = true; break;
+  case CUBLASLT_EPILOGUE_RELU_BIAS: g.act = ACT_RELU; has_bias = true; break;
+  case CUBLASLT_EPILOGUE_GELU_BIAS: g.act = ACT_GELU; has_bias = true; break;
+  default: return CUBLAS_STATUS_NOT_SUPPORTED;
+  }
+  if (has_bias) {
+    if (!dry && !op.bias) return CUBLAS_STATUS_INVALID_VALUE;
+    g.bias = op.bias;
+    g.bias_sb = op.bias_batch_stride;
+    if (op.bias_type >= 0) g.bias_type = (uint32_t)op.bias_type;
+    else  // cuda_types/src/cublaslt.rs:4395-4403
+      g.bias_type = (d.type == CUDA_R_8I || d.type == CUDA_R_32I || d.type == CUDA_R_8F_E4M3 ||
+                     d.type == CUDA_R_8F_E5M2) ? CUDA_R_32F : d.type;
+    if (!(g.bias_type == CUDA_R_32F || g.bias_type == CUDA_R_16F || g.bias_type == CUDA_R_16BF))
+      return CUBLAS_STATUS_NOT_SUPPORTED;
+  }
+
+  out->g = g;
+  out->a_kcontig = g.a_sk == 1;
+  out->b_kcontig = g.b_sk == 1;
+  auto al16 = [](const void *ptr, int64_t pitch_elems, int64_t bstride, int bits, bool batched) {
+    return (((uintptr_t)ptr) & 15) == 0 && ((pitch_elems * bits / 8) & 15) == 0 &&
+           (!batched || ((bstride * bits / 8) & 15) == 0);
+  };
+  out->aligned16 = al16(g.A, g.a_si, g.a_sb, type_bits(a.type), g.batch > 1) &&
+                   al16(g.B, g.b_sj, g.b_sb, type_bits(b.type), g.batch > 1) &&
+                   (((int64_t)K * type_bits(a.type) / 8) & 15) == 0;
+  // the MFMA kernels address each operand through a 2 GiB buffer window
+  const int64_t span_a = ((int64_t)(M - 1) * g.a_si + (int64_t)K) * type_bits(a.type) / 8;
+  const int64_t span_b = ((int64_t)(N - 1) * g.b_sj + (int64_t)K) * type_bits(b.type) / 8;
+  out->span_ok = span_a < 0x7fffffffll && span_b < 0x7fffffffll;
+  return CUBLAS_STATUS_SUCCESS;
+}
+
+static bool is_f8(uint32_t t) { return t == CUDA_R_8F_E4M3 || t == CUDA_R_8F_E5M2; }
+
+bool family_supports(uint32_t kernel, const Lowered &l) {
+  const GemmArgs &g = l.g;
+  const bool fast_layout = l.a_kcontig && l.b_kcontig && l.aligned16;
+  const bool d_fast = g.d_type == CUDA_R_32I || g.d_type == CUDA_R_32F || g.d_type == CUDA_R_16BF ||
+                      g.d_type == CUDA_R_16F || g.d_type == CUDA_R_8I;
+  switch (kernel) {
+  case ZLUDA_KERNEL_GENERIC: return true;
+  case ZLUDA_KERNEL_MFMA_I8:
+    return fast_layout && l.span_ok && g.a_type == CUDA_R_8I && g.b_type == CUDA_R_8I && d_fast;
+  case ZLUDA_KERNEL_MFMA_F8:
+    return fast_layout && l.span_ok && is_f8(g.a_type) && is_f8(g.b_type) &&
+           !(g.a_type == CUDA_R_8F_E5M2 && g.b_type == CUDA_R_8F_E5M2) &&
+           g.a_scale_mode != SCALE_BLOCK32_UE8M0 && g.b_scale_mode != SCALE_BLOCK32_UE8M0 && d_fast;
+  case ZLUDA_KERNEL_MFMA_MXF4:
+    return fast_layout && l.span_ok && g.a_type == CUDA_R_4F_E2M1 && g.b_type == CUDA_R_4F_E2M1 &&
+           g.a_scale_mode == SCALE_BLOCK32_UE8M0 && g.b_scale_mode == SCALE_BLOCK32_UE8M0 &&
+           (g.K % 256) == 0 && ((((uintptr_t)g.a_scale) | ((uintptr_t)g.b_scale)) & 3) == 0 && d_fast;
+  case ZLUDA_KERNEL_DECODE_W8A8:
+    return fast_layout && g.a_type == CUDA_R_8I && g.b_type == CUDA_R_8I &&
+           std::min(g.M, g.N) <= 32 && std::max(g.M, g.N) >= 64;
+  default: return false;
+  }
+}
+
+static uint32_t ceil_div(uint32_t a, uint32_t b) { return (a + b - 1) / b; }
+
+static void fill_mfma_plan(const Lowered &l, int variant, uint32_t cus, zluda_gemm_plan *plan) {
+  const GemmArgs &g = l.g;
+  const MfmaVariant &v = kMfmaVariants[variant % kNumMfmaVariants];
+  const bool swapped = g.d_si != 1;  // row-major D: compute D^T
+  const uint32_t np = swapped ? g.N : g.M, nq = swapped ? g.M : g.N;
+  const uint32_t tp = ceil_div(np, v.bp), tq = ceil_div(nq, v.bq);
+  plan->variant = variant;
+  plan->swapped = swapped;
+  plan->grid_x = tp * tq; plan->grid_y = g.batch; plan->grid_z = 1;
+  plan->block = v.wp * v.wq * 64;
+  const uint32_t lds = 2u * (v.bp + v.bq) * 128u;
+  const uint32_t per_cu = std::max(1u, std::min(160u * 1024u / lds, 2048u / plan->block));
+  plan->waves = (float)plan->grid_x * plan->grid_y / (float)(cus * per_cu);
+  plan->workspace = 0;
+}
+
+static int pick_mfma_variant(const Lowered &l, uint32_t cus) {
+  const GemmArgs &g = l.g;
+  const bool swapped = g.d_si != 1;
+  const uint32_t np = swapped ? g.N : g.M, nq = swapped ? g.M : g.N;
+  auto tiles = [&](int v) {
+    return (uint64_t)ceil_div(np, kMfmaVariants[v].bp) * ceil_div(nq, kMfmaVariants[v].bq) * g.batch;
+  };
+  // the biggest tile that still gives (nearly) every CU a workgroup
+  if (tiles(0) * 4 >= (uint64_t)cus * 3) return 0;
+  if (tiles(2) * 4 >= (uint64_t)cus * 3) return 2;
+  return 1;
+}
+
+static void fill_decode_plan(const Lowered &l, int variant, uint32_t cus, zluda_gemm_plan *plan) {
+  const GemmArgs &g = l.g;
+  const DecodeVariant &v = kDecodeVariants[variant];
+  const bool swapped = g.M < g.N;  // weights are the long operand
+  const uint32_t rows = swapped ? g.N : g.M;
+  const uint32_t nrb = ceil_div(rows, 16);
+  const uint32_t resident = cus * (v.nw == 8 ? 2 : 4);
+  uint32_t grid = nrb <= resident ? nrb : ceil_div(nrb, ceil_div(nrb, resident));
+  if (const char *e = getenv("ZLUDA_DECODE_GRID")) { int x = atoi(e); if (x > 0) grid = std::min<uint32_t>(x, nrb); }
+  plan->variant = variant;
+  plan->swapped = swapped;
+  plan->grid_x = grid; plan->grid_y = g.batch; plan->grid_z = 1;
+  plan->block = v.nw * 64;
+  plan->waves = (float)grid * g.batch / (float)resident;
+  plan->workspace = 0;
+}
+
+static int pick_decode_variant(const Lowered &l) {
+  const int K = l.g.K, T = std::min(l.g.M, l.g.N);
+  for (int v = 0; v < kNumDecodeVariants; v++)
+    if (K == kDecodeVariants[v].nw * kDecodeVariants[v].steps * 64 && (T <= 16 || kDecodeVariants[v].steps <= 8))
+      return v;
+  return 0;
+}
+
+} // namespace zluda_amd
+
+using namespace zluda_amd;
+
+extern "C" uint32_t zluda_gemm_plan_problem(const zluda_gemm_problem *p, uint32_t forced_kernel,
+                                            int32_t forced_variant, uint32_t cu_count,
+                                            zluda_gemm_plan *plan) {
+  if (!plan) return CUBLAS_STATUS_INVALID_VALUE;
+  Lowered l;
+  // planning never dereferences data: NULL pointers mean "aligned as the preferences promise"
+  uint32_t st = lower_problem(p, true, &l);
+  if (st) return st;
+  if (cu_count == 0) cu_count = 256;
+  memset(plan, 0, sizeof(*plan));
+  uint32_t kernel = forced_kernel;
+  if (kernel == ZLUDA_KERNEL_AUTO) {
+    static const uint32_t order[] = {ZLUDA_KERNEL_DECODE_W8A8, ZLUDA_KERNEL_MFMA_I8, ZLUDA_KERNEL_MFMA_F8,
+                                     ZLUDA_KERNEL_MFMA_MXF4, ZLUDA_KERNEL_GENERIC};
+    for (uint32_t k : order)
+      if (family_supports(k, l)) { kernel = k; break; }
+  } else if (!family_supports(kernel, l)) {
+    return CUBLAS_STATUS_NOT_SUPPORTED;
+  }
+  plan->kernel = kernel;
+  switch (kernel) {
+  case ZLUDA_KERNEL_GENERIC:
+    plan->variant = 0; plan->swapped = 0;
+    plan->grid_x = ceil_div(l.g.M, 64); plan->grid_y = ceil_div(l.g.N, 64); plan->grid_z = l.g.batch;
+    plan->block = 256;
+    plan->waves = (float)plan->grid_x * plan->grid_y * plan->grid_z / (float)(cu_count * 8);
+    if (plan->grid_y > 65535) return CUBLAS_STATUS_NOT_SUPPORTED;
+    break;
+  case ZLUDA_KERNEL_MFMA_I8: case ZLUDA_KERNEL_MFMA_F8: case ZLUDA_KERNEL_MFMA_MXF4: {
+    int v = forced_variant >= 0 ? forced_variant : pick_mfma_variant(l, cu_count);
+    if (v >= 2 * kNumMfmaVariants) return CUBLAS_STATUS_INVALID_VALUE;
+    fill_mfma_plan(l, v, cu_count, plan);
+    break;
+  }
+  case ZLUDA_KERNEL_DECODE_W8A8: {
+    int v = forced_variant >= 0 ? forced_variant : pick_decode_variant(l);
+    if (v >= kNumDecodeVariants) return CUBLAS_STATUS_INVALID_VALUE;
+    if (std::min(l.g.M, l.g.N) > 16 && kDecodeVariants[v].steps > 8) return CUBLAS_STATUS_NOT_SUPPORTED;
+    fill_decode_plan(l, v, cu_count, plan);
+    break;
+  }
+  default: return CUBLAS_STATUS_NOT_SUPPORTED;
+  }
+  return CUBLAS_STATUS_SUCCESS;
+}

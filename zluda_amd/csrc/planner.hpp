@@ -1,0 +1,43 @@
+// Host-side lowering of a cuBLASLt-level problem to kernel arguments, and kernel selection.
+#pragma once
+#include "../../include/cublaslt_abi.h"
+#include "../../include/zluda_gemm_launch.h"
+#include "gemm_args.hpp"
+
+namespace zluda_amd {
+
+// MFMA tile configurations (index = plan.variant for the MFMA families)
+struct MfmaVariant { int bp, bq, wp, wq; };
+constexpr MfmaVariant kMfmaVariants[] = {
+    {256, 256, 2, 2},  // 0: 4 waves, 128x128 per wave
+    {128, 128, 2, 2},  // 1: 4 waves, 64x64 per wave
+    {256, 128, 2, 2},  // 2: 4 waves, 128x64 per wave
+    {256, 256, 2, 4},  // 3: 8 waves, 128x64 per wave
+};
+constexpr int kNumMfmaVariants = sizeof(kMfmaVariants) / sizeof(kMfmaVariants[0]);
+
+// decode configurations (index = plan.variant for ZLUDA_KERNEL_DECODE_W8A8)
+struct DecodeVariant { int nw, steps; };
+constexpr DecodeVariant kDecodeVariants[] = {
+    {8, 8},   // 0: 8 waves x 512 B of K
+    {8, 16},  // 1: 8 waves x 1024 B
+    {4, 16},  // 2: 4 waves x 1024 B
+    {4, 8},   // 3: 4 waves x 512 B
+};
+constexpr int kNumDecodeVariants = sizeof(kDecodeVariants) / sizeof(kDecodeVariants[0]);
+
+struct Lowered {
+  GemmArgs g;
+  bool a_kcontig, b_kcontig;  // unit K stride
+  bool aligned16;             // A, B, their row pitches and batch strides are 16-byte aligned
+  bool span_ok;               // one batch of A and of B each spans < 2 GiB
+};
+
+// Validates `p` and fills `out`.  With dry=true (heuristic time) data pointers and host scalars are
+// not dereferenced and NULL data pointers are allowed.
+uint32_t lower_problem(const zluda_gemm_problem *p, bool dry, Lowered *out);
+
+// which kernel families can run the lowered problem
+bool family_supports(uint32_t kernel, const Lowered &l);
+
+} // namespace zluda_amd
