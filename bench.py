@@ -1,0 +1,286 @@
+#!/usr/bin/env python3
+"""Benchmark of the cublasLtMatmul hot path on one MI355X.
+
+A "step" is one cublasLtMatmul call (through the exported C ABI of zluda_amd/lib/libcublaslt.so) on
+synthetic inputs that are already resident in HBM.  The headline line reports BASELINE config 2
+(int8 x int8 -> int32, M=N=K=4096, A:T B:N); the other BASELINE configurations and the 8192^3 int8
+case ride along under "also", each with its own roofline figures and, when the installed hipBLASLt
+has a solution, the time of the reference's hipBLASLt-forwarded path on the same buffers.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c5|i8_8192] [--only]
+                  [--no-cpu] [--no-hipblaslt]
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+import numpy as np  # noqa: E402
+
+from zluda_amd import abi, cublaslt  # noqa: E402
+from zluda_amd.cublaslt import MatmulCall  # noqa: E402
+
+K = abi
+PEAK = {"i8": 5000.0, "f8": 5000.0, "f4": 10100.0, "hbm": 8000.0}  # TOP/s, TFLOP/s, GB/s (MI355X datasheet)
+
+I8 = dict(a_type=K.CUDA_R_8I, b_type=K.CUDA_R_8I, d_type=K.CUDA_R_32I, compute_type=K.CUBLAS_COMPUTE_32I,
+          scale_type=K.CUDA_R_32I, transa=1)
+WORKLOADS = {
+    "c2": dict(name="int8xint8->int32 M=N=K=4096 A:T B:N (BASELINE config 2)", kind="i8",
+               spec=dict(I8, m=4096, n=4096, k=4096), steps=50),
+    "i8_8192": dict(name="int8xint8->int32 M=N=K=8192 A:T B:N", kind="i8", spec=dict(I8, m=8192, n=8192, k=8192), steps=10),
+    "c3": dict(name="W8A8 decode M=14336 N=16 K=4096 alpha-vec + per-token scale + fp32 bias -> bf16 (BASELINE config 3)",
+               kind="hbm", steps=200,
+               spec=dict(I8, d_type=K.CUDA_R_16BF, scale_type=K.CUDA_R_32F, m=14336, n=16, k=4096,
+                         pointer_mode=K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO,
+                         b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F,
+                         epilogue=K.CUBLASLT_EPILOGUE_BIAS, bias_type=K.CUDA_R_32F)),
+    "c4": dict(name="fp8 e4m3 M=N=K=8192 per-tensor scales, bf16 bias + GELU -> bf16 (BASELINE config 4)", kind="f8",
+               steps=10,
+               spec=dict(a_type=K.CUDA_R_8F_E4M3, b_type=K.CUDA_R_8F_E4M3, d_type=K.CUDA_R_16BF,
+                         compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F, transa=1, m=8192, n=8192, k=8192,
+                         epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS, bias_type=K.CUDA_R_16BF)),
+    "c5": dict(name="MXFP4 (E2M1 + UE8M0/32) M=N=K=8192 batch 4 -> bf16 (BASELINE config 5)", kind="f4", steps=5,
+               spec=dict(a_type=K.CUDA_R_4F_E2M1, b_type=K.CUDA_R_4F_E2M1, d_type=K.CUDA_R_16BF,
+                         compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F, transa=1, m=8192, n=8192, k=8192,
+                         batch=4, a_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_VEC32_UE8M0,
+                         b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_VEC32_UE8M0)),
+}
+
+
+def algorithmic(spec):
+    """(ops, bytes) of one call: 2*M*N*K*batch and every operand/result byte exactly once."""
+    m, n, k, b = spec["m"], spec["n"], spec["k"], spec.get("batch", 1)
+    bits = K.TYPE_BITS
+    by = b * (m * k * bits[spec["a_type"]] + n * k * bits[spec["b_type"]] + m * n * bits[spec["d_type"]]) // 8
+    if spec.get("a_scale_mode") == K.CUBLASLT_MATMUL_MATRIX_SCALE_VEC32_UE8M0:
+        by += b * (m + n) * (k // 32)
+    if spec.get("b_scale_mode") == K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F:
+        by += n * 4
+    if spec.get("pointer_mode", 0) >= K.CUBLASLT_POINTER_MODE_DEVICE_VECTOR:
+        by += m * 4
+    if "bias_type" in spec:
+        by += m * bits[spec["bias_type"]] // 8
+    if spec.get("kind_scalar_scales"):
+        by += 8
+    return 2 * m * n * k * b, by
+
+
+class Buffers:
+    """Synthetic device-resident inputs of one workload (torch is only the allocator here)."""
+
+    def __init__(self, torch, key, spec, copies=1):
+        dev = "cuda:0"
+        g = torch.Generator(device=dev)
+        g.manual_seed({"c2": 1, "c3": 2, "c4": 3, "c5": 4}.get(key, 5))
+        m, n, k, b = spec["m"], spec["n"], spec["k"], spec.get("batch", 1)
+        self.keep = []
+        self.bias = self.a_scale = self.b_scale = self.alpha_dev = None
+        at = spec["a_type"]
+        if at == K.CUDA_R_8I:
+            if key == "c3":   # round(N(0,32)) clipped to +-127
+                mk = lambda r: torch.clamp(torch.round(torch.randn(r, k, device=dev, generator=g) * 32), -127, 127).to(torch.int8)
+            else:             # uniform [-128, 127]
+                mk = lambda r: torch.randint(-128, 128, (r, k), device=dev, generator=g, dtype=torch.int8)
+            self.A = [mk(m) for _ in range(copies)]
+            self.B = mk(n)
+        elif at == K.CUDA_R_8F_E4M3:
+            def mk(r):
+                x = torch.randn(r, k, device=dev, generator=g)
+                amax = x.abs().max()
+                return (x * (448.0 / amax)).to(torch.float8_e4m3fn), (amax / 448.0).reshape(1).float()
+            a, sa = mk(m)
+            bq, sb = mk(n)
+            self.A, self.B, self.a_scale, self.b_scale = [a], bq, sa, sb
+        else:  # MXFP4: per 32-block e = floor(log2(max)) - 2, elements RNE to E2M1, low nibble = even k
+            grid = torch.tensor([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0], device=dev)
+            mids = (grid[:-1] + grid[1:]) / 2
+
+            def mk(r):
+                qs, ss = [], []
+                for _ in range(b):
+                    x = torch.randn(r, k // 32, 32, device=dev, generator=g)
+                    e = torch.floor(torch.log2(x.abs().amax(dim=2, keepdim=True))) - 2
+                    y = (x * torch.exp2(-e)).clamp(-6, 6)
+                    idx = torch.bucketize(y.abs(), mids)   # nearest grid point (ties resolve downward: bench data only)
+                    code = (idx | ((y < 0).to(idx.dtype) << 3)).to(torch.uint8).reshape(r, k)
+                    qs.append(code[:, 0::2] | (code[:, 1::2] << 4))
+                    ss.append((e.reshape(r, k // 32) + 127).to(torch.uint8))
+                return torch.stack(qs).contiguous(), torch.stack(ss).contiguous()
+            a, sa = mk(m)
+            bq, sb = mk(n)
+            self.A, self.B, self.a_scale, self.b_scale = [a], bq, sa, sb
+        dt = {K.CUDA_R_32I: torch.int32, K.CUDA_R_16BF: torch.bfloat16}[spec["d_type"]]
+        self.D = torch.empty(b * m * n, device=dev, dtype=dt)
+        if key == "c3":
+            self.alpha_dev = torch.empty(m, device=dev).uniform_(0.001, 0.01, generator=g)
+            self.b_scale = torch.empty(n, device=dev).uniform_(0.005, 0.02, generator=g)
+            self.bias = torch.randn(m, device=dev, generator=g) * 0.02
+        if key == "c4":
+            self.bias = (torch.randn(m, device=dev, generator=g) * 0.02).to(torch.bfloat16)
+
+
+def time_calls(torch, fn, steps, warmup):
+    """returns (wall seconds for `steps` calls, seconds per call by HIP events on the launch stream)"""
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for i in range(steps):
+        fn(i)
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return wall, e0.elapsed_time(e1) * 1e-3 / steps
+
+
+def run_workload(torch, api, key, steps, warmup, with_hipblaslt):
+    w = WORKLOADS[key]
+    spec = w["spec"]
+    ops, nbytes = algorithmic(spec)
+    if key == "c4":
+        nbytes += 8
+    copies = 1
+    if key == "c3":
+        copies = 8   # 8 x 58.7 MB of weights > 256 MB Infinity Cache: every call streams from HBM
+    buf = Buffers(torch, key, spec, copies)
+    call = MatmulCall(api, spec)
+    call.set_pointers(bias=buf.bias.data_ptr() if buf.bias is not None else None,
+                      a_scale=buf.a_scale.data_ptr() if buf.a_scale is not None and key != "c3" else None,
+                      b_scale=buf.b_scale.data_ptr() if buf.b_scale is not None else None)
+    int_scale = spec["scale_type"] == K.CUDA_R_32I
+    one = C.c_int32(1) if int_scale else C.c_float(1.0)
+    zero = C.c_int32(0) if int_scale else C.c_float(0.0)
+    alpha = buf.alpha_dev.data_ptr() if buf.alpha_dev is not None else one
+    stream = torch.cuda.current_stream().cuda_stream
+    a_ptrs = [a.data_ptr() for a in buf.A]
+    bp, dp = buf.B.data_ptr(), buf.D.data_ptr()
+
+    def ours(i):
+        st = call.run(alpha, a_ptrs[i % copies], bp, zero, None, dp, None, 0, stream)
+        if st:
+            raise RuntimeError("cublasLtMatmul status %d on workload %s" % (st, key))
+    wall, per_call = time_calls(torch, ours, steps, warmup)
+    bound = "hbm" if w["kind"] == "hbm" else "mfma"
+    achieved = (nbytes / per_call / 1e9) if bound == "hbm" else (ops / per_call / 1e12)
+    peak = PEAK[w["kind"]]
+    res = {
+        "workload": w["name"], "steps": steps, "ms_per_step": wall / steps * 1e3,
+        "tops": ops / (wall / steps) / 1e12, "gbps": nbytes / (wall / steps) / 1e9,
+        "kernel": {"family": call.kernel, "variant": call.variant},
+        "roofline": {"bound": bound, "achieved": achieved, "peak": peak, "unit": "GB/s" if bound == "hbm" else "TFLOP/s",
+                     "frac": achieved / peak, "traffic": None, "kernel_ms": per_call * 1e3,
+                     "algorithmic_ops": ops, "algorithmic_bytes": nbytes},
+    }
+    if with_hipblaslt:
+        res["hipblaslt_forwarded"] = time_hipblaslt(torch, spec, buf, alpha, zero, a_ptrs, copies, steps, warmup, ops, nbytes)
+    call.close()
+    return res
+
+
+def time_hipblaslt(torch, spec, buf, alpha, zero, a_ptrs, copies, steps, warmup, ops, nbytes):
+    """the reference's hipBLASLt-forwarded path on the same buffers (oracle.hipblaslt_replay)"""
+    try:
+        from oracle.hipblaslt_replay import Replay
+        rp = Replay(spec)
+        if rp.why:
+            return {"available": False, "why": rp.why.strip()}
+        key_c3 = buf.alpha_dev is not None
+        ok = rp.set_pointers(bias=buf.bias.data_ptr() if buf.bias is not None else None,
+                             a_scale=buf.a_scale.data_ptr() if buf.a_scale is not None and not key_c3 else None,
+                             b_scale=buf.b_scale.data_ptr() if buf.b_scale is not None else None)
+        if not ok or not rp.find_algo():
+            why = rp.why.strip()
+            rp.close()
+            return {"available": False, "why": why}
+        stream = torch.cuda.current_stream().cuda_stream
+        bp, dp = buf.B.data_ptr(), buf.D.data_ptr()
+
+        def theirs(i):
+            st = rp.run(alpha, a_ptrs[i % copies], bp, zero, None, dp, stream)
+            if st:
+                raise RuntimeError("hipblasLtMatmul status %d" % st)
+        wall, per_call = time_calls(torch, theirs, steps, warmup)
+        rp.close()
+        return {"available": True, "ms_per_step": wall / steps * 1e3, "kernel_ms": per_call * 1e3,
+                "tops": ops / per_call / 1e12, "gbps": nbytes / per_call / 1e9}
+    except Exception as e:  # the comparison point is optional; the product numbers are not
+        return {"available": False, "why": "%s: %s" % (type(e).__name__, e)}
+
+
+def cpu_baseline(key):
+    """The CPU oracle (oracle/ref_gemm.c, OpenMP) timed on a bounded slab of the headline workload."""
+    import oracle
+    from oracle.cases import Case
+    spec = dict(WORKLOADS[key]["spec"])
+    full_m = spec["m"]
+    rows = {"c2": 1024, "i8_8192": 256, "c3": full_m, "c4": 32, "c5": 8}[key]
+    spec.update(m=rows, batch=1, alpha=1)
+    case = Case(spec, 1, int_dist="normal" if key == "c3" else "uniform")
+    t0 = time.perf_counter()
+    case.run_oracle()
+    dt = time.perf_counter() - t0
+    ops = 2 * rows * spec["n"] * spec["k"]
+    unit = "GB/s" if key == "c3" else "TOPS"
+    val = (algorithmic(spec)[1] / dt / 1e9) if key == "c3" else ops / dt / 1e12
+    return {"value": val, "unit": unit, "cores": int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)),
+            "kind": "port", "seconds": dt,
+            "sample": "%d of %d rows of D (full N=%d, K=%d, batch 1), oracle/ref_gemm.c with OpenMP" % (
+                rows, full_m, spec["n"], spec["k"])}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=0)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
+    ap.add_argument("--only", action="store_true", help="skip the other workloads")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-hipblaslt", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (pass --gpus 1)")
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a HIP device; there is no CPU path to benchmark")
+    api = cublaslt.load()
+    torch.cuda.init()
+    key = args.workload
+    steps = args.steps or WORKLOADS[key]["steps"]
+    head = run_workload(torch, api, key, steps, args.warmup, not args.no_hipblaslt)
+    also = {}
+    if not args.only:
+        for other in ("i8_8192", "c3", "c4", "c5", "c2"):
+            if other == key:
+                continue
+            try:
+                also[other] = run_workload(torch, api, other, WORKLOADS[other]["steps"], args.warmup, not args.no_hipblaslt)
+            except Exception as e:
+                also[other] = {"error": "%s: %s" % (type(e).__name__, e)}
+            torch.cuda.empty_cache()
+    unit = "GB/s" if WORKLOADS[key]["kind"] == "hbm" else "TOPS"
+    line = {
+        "metric": "cublasLtMatmul TOPS (int8/fp8/MXFP4, 8192^3) + decode GEMM HBM GB/s",
+        "value": head["gbps"] if unit == "GB/s" else head["tops"], "unit": unit, "n_gpus": 1, "steps": steps,
+        "warmup": args.warmup, "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": {"i8": "int8", "hbm": "int8", "f8": "fp8_e4m3", "f4": "fp4_e2m1"}[WORKLOADS[key]["kind"]],
+        "data": "synthetic", "config": {"workload": head["workload"], "kernel": head["kernel"]},
+        "roofline": head["roofline"],
+        "cpu_baseline": None if args.no_cpu else cpu_baseline(key),
+        "hipblaslt_forwarded": head.get("hipblaslt_forwarded"),
+        "device": torch.cuda.get_device_name(0), "cu_count": api.zluda_gemm_device_cu_count(),
+        "also": also,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

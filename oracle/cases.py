@@ -1,4 +1,5 @@
-"""Shared machinery of the parity tests: seeded inputs, the oracle run, the GPU run through the
+"""TEST INFRASTRUCTURE.  Shared machinery of the parity tests, the smoke test and the benchmark's
+cpu_baseline leg: seeded inputs, the oracle run, the GPU run through the
 C ABI, and the comparison.  The same `spec` dict drives zluda_amd.cublaslt.MatmulCall (GPU) and the
 zluda_gemm_problem handed to the CPU oracle."""
 import ctypes as C
@@ -223,8 +224,8 @@ class Case:
         return d
 
     # ---- GPU through the C ABI ------------------------------------------------------------------
-    def run_gpu(self, api, forced_kernel=None, forced_variant=-1, offset_bytes=0):
-        """Returns (status, D storage, kernel family, variant).  offset_bytes misaligns A and B."""
+    def upload(self, offset_bytes=0):
+        """copies every host array to cuda:0; returns (tensors to keep alive, address dict, D tensor)"""
         import torch
         dev = torch.device("cuda:0")
 
@@ -235,39 +236,72 @@ class Case:
             t = torch.empty(raw.size + off + 16, dtype=torch.uint8, device=dev)
             t[off:off + raw.size] = torch.from_numpy(raw.copy()).to(dev)
             return t, t.data_ptr() + off
-        keep = []
-        ptr = {}
+        keep, ptr = [], {}
         for name, arr, off in (("A", self.A, offset_bytes), ("B", self.B, offset_bytes), ("C", self.Cm, 0),
                                ("bias", self.bias, 0), ("a_scale", self.a_scale, 0),
                                ("b_scale", self.b_scale, 0), ("c_scale", self.c_scale, 0),
-                               ("d_scale", self.d_scale, 0)):
+                               ("d_scale", self.d_scale, 0), ("alpha_dev", self.alpha, 0),
+                               ("beta_dev", self.beta, 0)):
             t, p = up(arr, off)
             keep.append(t)
             ptr[name] = p
-        d0 = self.new_d()
-        dt, ptr["D"] = up(d0)
+        dt, ptr["D"] = up(self.new_d())
+        return keep, ptr, dt
+
+    def scalars(self, ptr):
+        """alpha / beta arguments as cublasLtMatmul wants them for this pointer mode"""
+        if self.alpha_on_device:
+            alpha = ptr["alpha_dev"]
+        else:
+            alpha = (C.c_int32 if self.alpha.dtype == np.int32 else C.c_float)(self.alpha[0].item())
+        if self.beta_on_device:
+            beta = ptr["beta_dev"]
+        else:
+            beta = (C.c_int32 if self.beta.dtype == np.int32 else C.c_float)(self.beta[0].item())
+        return alpha, beta
+
+    def download(self, dt):
+        nbytes = self.dtot * np.dtype(self.d_np).itemsize
+        return dt[:nbytes].cpu().numpy().view(self.d_np).copy()
+
+    def run_gpu(self, api, forced_kernel=None, forced_variant=-1, offset_bytes=0):
+        """Returns (status, D storage, kernel family, variant).  offset_bytes misaligns A and B."""
+        import torch
+        keep, ptr, dt = self.upload(offset_bytes)
         call = MatmulCall(api, self.spec, forced_kernel=forced_kernel, forced_variant=forced_variant)
         try:
             call.set_pointers(bias=ptr["bias"], a_scale=ptr["a_scale"], b_scale=ptr["b_scale"],
                               c_scale=ptr["c_scale"], d_scale=ptr["d_scale"])
-            if self.alpha_on_device:
-                at, alpha = up(self.alpha)
-                keep.append(at)
-            else:
-                alpha = (C.c_int32 if self.alpha.dtype == np.int32 else C.c_float)(self.alpha[0].item())
-            if self.beta_on_device:
-                btens, beta = up(self.beta)
-                keep.append(btens)
-            else:
-                beta = (C.c_int32 if self.beta.dtype == np.int32 else C.c_float)(self.beta[0].item())
+            alpha, beta = self.scalars(ptr)
             stream = torch.cuda.current_stream().cuda_stream
             st = call.run(alpha, ptr["A"], ptr["B"], beta, ptr["C"], ptr["D"], None, 0, stream)
             torch.cuda.synchronize()
-            nbytes = d0.size * d0.itemsize
-            out = dt[:nbytes].cpu().numpy().view(self.d_np).copy()
-            return st, out, call.kernel, call.variant
+            return st, self.download(dt), call.kernel, call.variant
         finally:
             call.close()
+
+    def run_hipblaslt(self):
+        """The reference's forwarded path.  Returns (D storage or None, reason)."""
+        import torch
+        from oracle.hipblaslt_replay import Replay
+        keep, ptr, dt = self.upload()
+        rp = Replay(self.spec)
+        try:
+            if rp.why:
+                return None, rp.why
+            if not rp.set_pointers(bias=ptr["bias"], a_scale=ptr["a_scale"], b_scale=ptr["b_scale"],
+                                   c_scale=ptr["c_scale"], d_scale=ptr["d_scale"]):
+                return None, rp.why
+            if not rp.find_algo():
+                return None, rp.why
+            alpha, beta = self.scalars(ptr)
+            st = rp.run(alpha, ptr["A"], ptr["B"], beta, ptr["C"], ptr["D"], torch.cuda.current_stream().cuda_stream)
+            torch.cuda.synchronize()
+            if st:
+                return None, "hipblasLtMatmul status %d" % st
+            return self.download(dt), ""
+        finally:
+            rp.close()
 
     # ---- comparison -------------------------------------------------------------------------------
     def logical_index(self):

@@ -1,0 +1,159 @@
+"""GPU parity: every kernel family and tile variant, through the exported C ABI, against the CPU
+oracle on the same seeded inputs.  Integer outputs must be bit-exact (whole D storage including the
+padding between rows and ld); float outputs within max |rel err| <= 1e-2 (bf16 output, fp32
+accumulate) with the documented floor of 1e-2 * rms(ref)."""
+import sys
+
+import numpy as np
+import pytest
+
+from oracle.cases import Case
+from zluda_amd import abi
+
+pytestmark = pytest.mark.gpu
+K = abi
+
+I8 = dict(a_type=K.CUDA_R_8I, b_type=K.CUDA_R_8I, d_type=K.CUDA_R_32I, compute_type=K.CUBLAS_COMPUTE_32I,
+          scale_type=K.CUDA_R_32I, transa=1)
+I8F = dict(I8, d_type=K.CUDA_R_16BF, scale_type=K.CUDA_R_32F)
+F8 = dict(a_type=K.CUDA_R_8F_E4M3, b_type=K.CUDA_R_8F_E4M3, d_type=K.CUDA_R_16BF, compute_type=K.CUBLAS_COMPUTE_32F,
+          scale_type=K.CUDA_R_32F, transa=1)
+MX = dict(a_type=K.CUDA_R_4F_E2M1, b_type=K.CUDA_R_4F_E2M1, d_type=K.CUDA_R_16BF, compute_type=K.CUBLAS_COMPUTE_32F,
+          scale_type=K.CUDA_R_32F, transa=1, a_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_VEC32_UE8M0,
+          b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_VEC32_UE8M0)
+DECODE = dict(I8F, pointer_mode=K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO,
+              b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F, epilogue=K.CUBLASLT_EPILOGUE_BIAS,
+              bias_type=K.CUDA_R_32F, alpha_range=(0.001, 0.01), scale_range=(0.005, 0.02), bias_std=0.02)
+
+
+def check(gpu_api, spec, seed, kernel=None, variant=-1, expect_kernel=None, tol=None, **case_kw):
+    print("case", spec, "seed", seed, "kernel", kernel, "variant", variant, flush=True)
+    case = Case(spec, seed, **case_kw)
+    ref = case.run_oracle()
+    st, got, k, v = case.run_gpu(gpu_api, forced_kernel=kernel, forced_variant=variant)
+    assert st == 0, "cublasLtMatmul status %d" % st
+    if expect_kernel is not None:
+        assert k == expect_kernel, "planner chose kernel %d" % k
+    return case.compare(got, ref, tol)
+
+
+# ---- int8 -> int32 MFMA, every tile variant and both load modes --------------------------------
+@pytest.mark.parametrize("variant", range(8))
+@pytest.mark.parametrize("m,n,k", [(256, 256, 128), (300, 200, 144), (512, 384, 1024)])
+def test_mfma_i8_variants(gpu_api, variant, m, n, k):
+    check(gpu_api, dict(I8, m=m, n=n, k=k, lda=k + 16 if k == 144 else k), 10 + variant, K.ZLUDA_KERNEL_MFMA_I8, variant)
+
+
+def test_mfma_i8_alpha_beta_batch_and_padding(gpu_api):
+    spec = dict(I8, m=200, n=136, k=272, batch=3, with_c=True, ldd=208, ldc=204, lda=288, stride_d=208 * 136 + 48)
+    for variant in (0, 1, 5):
+        check(gpu_api, spec, 3, K.ZLUDA_KERNEL_MFMA_I8, variant)
+    # device scalars
+    check(gpu_api, dict(spec, pointer_mode=K.CUBLASLT_POINTER_MODE_DEVICE), 4, K.ZLUDA_KERNEL_MFMA_I8, 1)
+
+
+def test_mfma_i8_row_major_output_swaps(gpu_api):
+    spec = dict(I8, transa=0, transb=1, order_a=1, order_b=1, order_c=1, order_d=1, m=192, n=320, k=256, with_c=True)
+    check(gpu_api, spec, 5, K.ZLUDA_KERNEL_MFMA_I8, 1)
+    check(gpu_api, spec, 5, K.ZLUDA_KERNEL_MFMA_I8, 4)
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4])
+def test_mfma_i8_float_epilogue(gpu_api, variant):
+    spec = dict(I8F, m=260, n=140, k=512, epilogue=K.CUBLASLT_EPILOGUE_RELU_BIAS, bias_type=K.CUDA_R_32F,
+                pointer_mode=K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_HOST, with_c=True,
+                a_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F,
+                b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F,
+                alpha_range=(0.001, 0.002), scale_range=(0.5, 1.5))
+    check(gpu_api, spec, 6, K.ZLUDA_KERNEL_MFMA_I8, variant)
+    # same with a row-major D (per-row vectors then run along the accumulator registers)
+    check(gpu_api, dict(spec, order_c=1, order_d=1), 7, K.ZLUDA_KERNEL_MFMA_I8, variant)
+    for dt in (K.CUDA_R_32F, K.CUDA_R_16F, K.CUDA_R_8I):
+        check(gpu_api, dict(spec, d_type=dt, c_type=dt, alpha_range=(0.0001, 0.0002)), 8, K.ZLUDA_KERNEL_MFMA_I8, variant)
+
+
+# ---- fp8 -------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("variant", range(8))
+def test_mfma_f8_variants(gpu_api, variant):
+    check(gpu_api, dict(F8, m=256, n=256, k=256), 20 + variant, K.ZLUDA_KERNEL_MFMA_F8, variant)
+    check(gpu_api, dict(F8, m=320, n=272, k=400, lda=416, ldb=400, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS,
+                        with_scalar_scales=True), 30 + variant, K.ZLUDA_KERNEL_MFMA_F8, variant)
+
+
+@pytest.mark.parametrize("at,bt", [(K.CUDA_R_8F_E5M2, K.CUDA_R_8F_E4M3), (K.CUDA_R_8F_E4M3, K.CUDA_R_8F_E5M2)])
+def test_mfma_f8_mixed_formats(gpu_api, at, bt):
+    for variant in (0, 1):
+        check(gpu_api, dict(F8, a_type=at, b_type=bt, m=256, n=128, k=512, d_type=K.CUDA_R_32F), 40, K.ZLUDA_KERNEL_MFMA_F8, variant)
+    check(gpu_api, dict(F8, a_type=at, b_type=bt, m=256, n=128, k=512, order_c=1, order_d=1), 41, K.ZLUDA_KERNEL_MFMA_F8, 1)
+
+
+# ---- MXFP4 -----------------------------------------------------------------------------------------
+@pytest.mark.parametrize("variant", range(8))
+def test_mfma_mxf4_variants(gpu_api, variant):
+    check(gpu_api, dict(MX, m=256, n=256, k=512), 50 + variant, K.ZLUDA_KERNEL_MFMA_MXF4, variant)
+    check(gpu_api, dict(MX, m=288, n=160, k=768, batch=2), 60 + variant, K.ZLUDA_KERNEL_MFMA_MXF4, variant)
+
+
+def test_mxf4_generic_agrees(gpu_api):
+    check(gpu_api, dict(MX, m=96, n=80, k=384), 70, K.ZLUDA_KERNEL_GENERIC)
+
+
+# ---- W8A8 decode -----------------------------------------------------------------------------------
+@pytest.mark.parametrize("variant", range(4))
+@pytest.mark.parametrize("tokens", [1, 7, 16])
+def test_decode_variants(gpu_api, variant, tokens):
+    nw, steps = [(8, 8), (8, 16), (4, 16), (4, 8)][variant]
+    kfull = nw * steps * 64
+    check(gpu_api, dict(DECODE, m=1000, n=tokens, k=kfull), 80 + variant, K.ZLUDA_KERNEL_DECODE_W8A8, variant, int_dist="normal")
+    check(gpu_api, dict(DECODE, m=528, n=tokens, k=1088), 90 + variant, K.ZLUDA_KERNEL_DECODE_W8A8, variant, int_dist="normal")
+
+
+@pytest.mark.parametrize("variant", [0, 3])
+def test_decode_two_token_blocks_and_long_k(gpu_api, variant):
+    check(gpu_api, dict(DECODE, m=640, n=32, k=4096 if variant == 0 else 2048), 100, K.ZLUDA_KERNEL_DECODE_W8A8, variant, int_dist="normal")
+    check(gpu_api, dict(DECODE, m=400, n=17, k=9280), 101, K.ZLUDA_KERNEL_DECODE_W8A8, variant, int_dist="normal")   # several chunks
+
+
+def test_decode_tokens_along_m_and_int32_out(gpu_api):
+    # row-major activations [tokens][K] x weights^T: tokens are rows of D
+    spec = dict(I8F, transa=0, transb=1, order_a=1, order_b=1, order_c=1, order_d=1, m=16, n=2048, k=4096,
+                epilogue=K.CUBLASLT_EPILOGUE_BIAS, bias_type=K.CUDA_R_32F, alpha_range=(0.001, 0.002))
+    check(gpu_api, spec, 110, expect_kernel=K.ZLUDA_KERNEL_DECODE_W8A8, int_dist="normal")
+    check(gpu_api, dict(I8, m=2048, n=8, k=4096, with_c=True), 111, expect_kernel=K.ZLUDA_KERNEL_DECODE_W8A8)
+
+
+# ---- generic kernel (layouts the MFMA kernels do not take) -------------------------------------------
+@pytest.mark.parametrize("ta,tb,oa,ob,od", [(0, 1, 0, 0, 0), (0, 0, 0, 0, 1), (1, 1, 1, 0, 0), (0, 1, 1, 1, 1)])
+def test_generic_layouts_int8(gpu_api, ta, tb, oa, ob, od):
+    spec = dict(I8, transa=ta, transb=tb, order_a=oa, order_b=ob, order_c=od, order_d=od, m=150, n=90, k=77,
+                batch=2, with_c=True)
+    check(gpu_api, spec, 120, K.ZLUDA_KERNEL_GENERIC)
+
+
+@pytest.mark.parametrize("t", [K.CUDA_R_32F, K.CUDA_R_16F, K.CUDA_R_16BF, K.CUDA_R_8F_E4M3])
+def test_generic_float_types(gpu_api, t):
+    spec = dict(a_type=t, b_type=t, d_type=K.CUDA_R_32F if t == K.CUDA_R_32F else K.CUDA_R_16BF,
+                compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F, m=130, n=70, k=96, transb=1,
+                epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS, with_c=True, with_cd_scales=True)
+    check(gpu_api, spec, 130, expect_kernel=K.ZLUDA_KERNEL_GENERIC, tol=2e-2 if t == K.CUDA_R_32F else None)
+
+
+def test_misaligned_pointers_fall_back(gpu_api):
+    case = Case(dict(I8, m=256, n=256, k=256), 140)
+    ref = case.run_oracle()
+    st, got, k, _ = case.run_gpu(gpu_api, offset_bytes=4)   # heuristic promised alignment; pointers are off by 4
+    assert st == 0 and k == K.ZLUDA_KERNEL_MFMA_I8            # the token says MFMA, the call ran the generic kernel
+    case.compare(got, ref)
+
+
+# ---- BASELINE configurations ---------------------------------------------------------------------------
+def test_config1_int8_256_nt(gpu_api):
+    check(gpu_api, dict(I8, transa=0, transb=1, m=256, n=256, k=256, alpha=1), 0, expect_kernel=K.ZLUDA_KERNEL_GENERIC)
+
+
+def test_config3_decode_full_size(gpu_api):
+    check(gpu_api, dict(DECODE, m=14336, n=16, k=4096), 2, expect_kernel=K.ZLUDA_KERNEL_DECODE_W8A8, int_dist="normal")
+
+
+def test_config2_int8_4096_full_size(gpu_api):
+    check(gpu_api, dict(I8, m=4096, n=4096, k=4096, alpha=1), 1, expect_kernel=K.ZLUDA_KERNEL_MFMA_I8)

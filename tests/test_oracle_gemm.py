@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 
 import oracle
-from helpers import Case, decode_storage
+from oracle.cases import Case, decode_storage
 from zluda_amd import abi
 
 GOLD = os.path.join(os.path.dirname(__file__), "golden")

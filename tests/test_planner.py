@@ -1,0 +1,104 @@
+"""Kernel selection and problem validation of the launch layer (host only)."""
+import ctypes as C
+
+import pytest
+
+from oracle.cases import Case
+from zluda_amd import abi
+
+K = abi
+I8 = dict(a_type=K.CUDA_R_8I, b_type=K.CUDA_R_8I, d_type=K.CUDA_R_32I, compute_type=K.CUBLAS_COMPUTE_32I,
+          scale_type=K.CUDA_R_32I)
+F8 = dict(a_type=K.CUDA_R_8F_E4M3, b_type=K.CUDA_R_8F_E4M3, d_type=K.CUDA_R_16BF, compute_type=K.CUBLAS_COMPUTE_32F,
+          scale_type=K.CUDA_R_32F)
+MX = dict(a_type=K.CUDA_R_4F_E2M1, b_type=K.CUDA_R_4F_E2M1, d_type=K.CUDA_R_16BF, compute_type=K.CUBLAS_COMPUTE_32F,
+          scale_type=K.CUDA_R_32F, a_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_VEC32_UE8M0,
+          b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_VEC32_UE8M0)
+
+
+def plan(api, spec, forced=0, variant=-1, cus=256, a_ptr=0, b_ptr=0):
+    case = Case.__new__(Case)
+    case.spec = dict(spec)
+    case.spec.setdefault("c_type", spec["d_type"])
+    case.batch = spec.get("batch", 1)
+    p = case.problem({"A": a_ptr, "B": b_ptr, "D": 0, "alpha": 0, "beta": 0})
+    out = abi.zluda_gemm_plan()
+    st = api.zluda_gemm_plan_problem(C.byref(p), forced, variant, cus, C.byref(out))
+    return st, out
+
+
+def test_baseline_configs_pick_the_intended_kernels(api):
+    st, p = plan(api, dict(I8, m=256, n=256, k=256, transa=0, transb=1))            # config 1: A:N B:T
+    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_GENERIC
+    st, p = plan(api, dict(I8, m=4096, n=4096, k=4096, transa=1))                   # config 2
+    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_I8 and p.variant == 0 and p.grid_x == 256 and p.block == 256
+    st, p = plan(api, dict(I8, m=14336, n=16, k=4096, transa=1, d_type=K.CUDA_R_16BF, scale_type=K.CUDA_R_32F,
+                           pointer_mode=K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO,
+                           b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F,
+                           epilogue=K.CUBLASLT_EPILOGUE_BIAS, bias_type=K.CUDA_R_32F))       # config 3
+    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.swapped == 0 and p.block == 512
+    st, p = plan(api, dict(F8, m=8192, n=8192, k=8192, transa=1, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS))  # config 4
+    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_F8 and p.grid_x == 1024
+    st, p = plan(api, dict(MX, m=8192, n=8192, k=8192, transa=1, batch=4))          # config 5
+    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_MXF4 and p.grid_x == 1024 and p.grid_y == 4
+    assert p.workspace == 0
+
+
+def test_small_problems_get_smaller_tiles(api):
+    st, p = plan(api, dict(I8, m=1024, n=1024, k=1024, transa=1))
+    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_I8 and p.variant == 1 and p.grid_x == 64
+    st, p = plan(api, dict(I8, m=4096, n=2048, k=1024, transa=1))
+    assert st == 0 and p.variant == 2 and p.grid_x == 16 * 16
+
+
+def test_row_major_output_swaps_operands(api):
+    st, p = plan(api, dict(I8, m=512, n=1024, k=512, order_a=1, order_b=1, transb=1, order_c=1, order_d=1))
+    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_I8 and p.swapped == 1
+    # tokens along M (row-major activations x weights^T): decode with the weights as operand B
+    st, p = plan(api, dict(I8, m=16, n=4096, k=4096, order_a=1, order_b=1, transb=1, order_c=1, order_d=1,
+                           d_type=K.CUDA_R_16BF, scale_type=K.CUDA_R_32F))
+    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.swapped == 1
+
+
+def test_misaligned_or_strided_operands_fall_back_to_generic(api):
+    spec = dict(I8, m=512, n=512, k=512, transa=1)
+    assert plan(api, spec, a_ptr=0x1004)[1].kernel == K.ZLUDA_KERNEL_GENERIC
+    assert plan(api, dict(spec, lda=520))[1].kernel == K.ZLUDA_KERNEL_GENERIC          # pitch not a multiple of 16
+    assert plan(api, dict(spec, k=520, lda=528, ldb=528))[1].kernel == K.ZLUDA_KERNEL_GENERIC   # K % 16 != 0
+    assert plan(api, dict(spec, k=528, lda=528, ldb=528))[1].kernel == K.ZLUDA_KERNEL_MFMA_I8   # K tail of 16 bytes
+    st, _ = plan(api, spec, forced=K.ZLUDA_KERNEL_MFMA_I8, a_ptr=0x1004)
+    assert st == K.CUBLAS_STATUS_NOT_SUPPORTED
+    # MXFP4 needs whole 256-element K stages for the MFMA kernel
+    assert plan(api, dict(MX, m=256, n=256, k=384, transa=1))[1].kernel == K.ZLUDA_KERNEL_GENERIC
+    assert plan(api, dict(MX, m=256, n=256, k=512, transa=1))[1].kernel == K.ZLUDA_KERNEL_MFMA_MXF4
+
+
+@pytest.mark.parametrize("bad,status", [
+    (dict(compute_type=K.CUBLAS_COMPUTE_64F), K.CUBLAS_STATUS_NOT_SUPPORTED),
+    (dict(a_type=K.CUDA_R_16F), K.CUBLAS_STATUS_NOT_SUPPORTED),                      # int compute wants int8 inputs
+    (dict(d_type=K.CUDA_R_16BF), K.CUBLAS_STATUS_NOT_SUPPORTED),                     # int32 scaling wants int32 D
+    (dict(epilogue=K.CUBLASLT_EPILOGUE_BIAS), K.CUBLAS_STATUS_NOT_SUPPORTED),        # no bias in pure integer mode
+    (dict(lda=100), K.CUBLAS_STATUS_INVALID_VALUE),                                  # ld < rows
+    (dict(order_a=K.CUBLASLT_ORDER_COL32), K.CUBLAS_STATUS_NOT_SUPPORTED),
+    (dict(pointer_mode=K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO, alpha_vector_batch_stride=8),
+     K.CUBLAS_STATUS_INVALID_VALUE),
+])
+def test_rejected_combinations(api, bad, status):
+    st, _ = plan(api, dict(dict(I8, m=128, n=128, k=128, transa=1), **bad))
+    assert st == status
+
+
+def test_fp4_must_be_k_contiguous(api):
+    st, _ = plan(api, dict(MX, m=256, n=256, k=512, transa=0))
+    assert st == K.CUBLAS_STATUS_NOT_SUPPORTED
+    st, _ = plan(api, dict(F8, m=256, n=256, k=512, transa=0))          # FP8 may be M-contiguous: generic kernel
+    assert st == 0
+
+
+def test_forced_variants(api):
+    spec = dict(I8, m=4096, n=4096, k=4096, transa=1)
+    for v, (grid, block) in enumerate([(256, 256), (1024, 256), (512, 256), (256, 512)] * 2):
+        st, p = plan(api, spec, forced=K.ZLUDA_KERNEL_MFMA_I8, variant=v)
+        assert st == 0 and p.variant == v and p.grid_x == grid and p.block == block
+    assert plan(api, spec, forced=K.ZLUDA_KERNEL_MFMA_I8, variant=8)[0] == K.CUBLAS_STATUS_INVALID_VALUE
+    assert plan(api, spec, forced=K.ZLUDA_KERNEL_MFMA_F8)[0] == K.CUBLAS_STATUS_NOT_SUPPORTED

@@ -39,6 +39,16 @@ __device__ __forceinline__ void static_for(F &f) {
   }
 }
 
+// 16 bytes per lane from a buffer straight into LDS (buffer_load_dwordx4 ... lds).  `lds_dst` is the
+// wave-uniform start of the 1 KiB block the instruction fills; lane l lands at byte l*16.
+// The address-space cast only exists in the device pass.
+__device__ __forceinline__ void lds_dma16(__amdgpu_buffer_rsrc_t rs, void *lds_dst, int voff, int soff) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void *)lds_dst, 16, voff,
+                                           soff, 0, 0);
+#endif
+}
+
 struct MfmaParams {
   GemmArgs g;
   int32_t swapped;           // P = op(B)^T rows, Q = op(A) rows
@@ -120,14 +130,10 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_kernel(MfmaParams prm) 
       // each wave instruction fills 1 KiB of LDS: 8 rows x 128 B, lane l -> byte l*16
 #pragma unroll
       for (int i = 0; i < LP; i++)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(
-            rsP, (__attribute__((address_space(3))) void *)&lds[buf][(wave * 8 + RP * i) * 8], 16,
-            voffP[i] | oob, kt * BKB, 0, 0);
+        lds_dma16(rsP, &lds[buf][(wave * 8 + RP * i) * 8], voffP[i] | oob, kt * BKB);
 #pragma unroll
       for (int i = 0; i < LQ; i++)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(
-            rsQ, (__attribute__((address_space(3))) void *)&lds[buf][(BP + wave * 8 + RP * i) * 8], 16,
-            voffQ[i] | oob, kt * BKB, 0, 0);
+        lds_dma16(rsQ, &lds[buf][(BP + wave * 8 + RP * i) * 8], voffQ[i] | oob, kt * BKB);
     }
   };
   auto lstore = [&](int buf) {
