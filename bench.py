@@ -20,7 +20,8 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-import numpy as np  # noqa: E402
+import numpy as np  # noqa: E402,F401
+import torch  # noqa: E402  -- before libcublaslt.so: one HIP runtime (torch's libamdhip64.so.7) per process
 
 from zluda_amd import abi, cublaslt  # noqa: E402
 from zluda_amd.cublaslt import MatmulCall  # noqa: E402
@@ -248,7 +249,6 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (pass --gpus 1)")
-    import torch
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a HIP device; there is no CPU path to benchmark")
     api = cublaslt.load()

@@ -553,15 +553,14 @@ cublasStatus_t cublasLtMatmul(cublasLtHandle_t lightHandle, cublasLtMatmulDesc_t
   if (cus == 0) return CUBLAS_STATUS_NOT_INITIALIZED;  // no usable HIP device: there is no CPU path
   zluda_gemm_plan plan;
   st = zluda_gemm_plan_problem(&p, kernel, variant, cus, &plan);
+  if (st == CUBLAS_STATUS_NOT_SUPPORTED && kernel != ZLUDA_KERNEL_AUTO && kernel != ZLUDA_KERNEL_GENERIC) {
+    // The algo was chosen from the descriptors alone (the heuristic assumes the MIN_ALIGNMENT_*
+    // preferences hold); the real pointers do not qualify for it.  Run the layout-agnostic kernel
+    // rather than failing the call.
+    st = zluda_gemm_plan_problem(&p, ZLUDA_KERNEL_GENERIC, -1, cus, &plan);
+  }
   if (st) return st;
   st = zluda_gemm_launch(&p, &plan, stream);
-  if (st == CUBLAS_STATUS_INVALID_VALUE && plan.kernel != ZLUDA_KERNEL_GENERIC) {
-    // The heuristic promised alignments (MIN_ALIGNMENT_*) that the real pointers do not have:
-    // run the layout-agnostic kernel instead of failing.
-    zluda_gemm_plan gen;
-    if (zluda_gemm_plan_problem(&p, ZLUDA_KERNEL_GENERIC, -1, cus, &gen) == CUBLAS_STATUS_SUCCESS)
-      st = zluda_gemm_launch(&p, &gen, stream);
-  }
   return st;
 }
 

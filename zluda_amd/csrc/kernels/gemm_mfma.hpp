@@ -31,6 +31,11 @@ constexpr int BKB = 128;  // bytes of K per LDS stage
 // depends on r mod 32 only, so rows 32 apart (the MFMA tiles of one wave) share a swizzle
 __device__ __forceinline__ int swz(int r) { return (r ^ ((r >> 3) & 3)) & 7; }
 
+// Accumulator element -> 32 raw bits.  Takes the element BY VALUE: __builtin_bit_cast applied
+// directly to a vector-element expression reads element 0 whatever the index.
+__device__ __forceinline__ int to_bits(int x) { return x; }
+__device__ __forceinline__ int to_bits(float x) { return (int)f2bits(x); }
+
 template <int N, int I = 0, class F>
 __device__ __forceinline__ void static_for(F &f) {
   if constexpr (I < N) {
@@ -319,7 +324,7 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_kernel(MfmaParams prm) 
 #pragma unroll
       for (int vv = 0; vv < 8; vv++) {
         const int ql = 8 * (vv >> 2) + 4 * gsel + (vv & 3);
-        stage[ql * SROW + b * 32 + lr] = __builtin_bit_cast(int, acc[a][b][h * 8 + vv]);
+        stage[ql * SROW + b * 32 + lr] = to_bits(acc[a][b][h * 8 + vv]);
       }
     __syncthreads();
 #pragma unroll 1
@@ -358,7 +363,8 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_kernel(MfmaParams prm) 
       float x[4];
 #pragma unroll
       for (int e = 0; e < 4; e++) {
-        const float accf = KIND == KIND_I8 ? (float)raw[e] : __builtin_bit_cast(float, raw[e]);
+        const int rawe = raw[e];
+        const float accf = KIND == KIND_I8 ? (float)rawe : bits2f((uint32_t)rawe);
         float y = (swp ? q_scale * p_scale[e] : p_scale[e] * q_scale) * accf;
         const float be = swp ? q_beta : p_beta[e];
         if (be != 0.0f && pi0 + e < NP) y += be * ep.sc * load_elem(g.C, g.c_type, cbase + e * c_sp);

@@ -3,6 +3,10 @@ ints, exactly what a CUDA application (or the reference's `CublasLtApi` test tra
 zluda_blas/src/tests.rs:33-84) sees.  No torch types cross this boundary: device memory is passed as
 integer addresses.
 
+A process that also uses PyTorch must import torch before loading this library: torch ships its own
+libamdhip64.so.7, and the library then binds to that already-loaded HIP runtime instead of bringing
+a second one into the process (two runtimes do not share a device context).
+
 There is no CPU path behind these calls: loading fails loudly when the library has not been built,
 and cublasLtMatmul returns CUBLAS_STATUS_NOT_INITIALIZED when no HIP device is usable.
 """
