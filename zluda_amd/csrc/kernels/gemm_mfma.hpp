@@ -61,6 +61,133 @@ struct MfmaParams {
   int32_t group_p;           // raster group height (tiles along P)
 };
 
+// Fused epilogue shared by the MFMA kernels.  The caller guarantees that every wave of the workgroup
+// has finished reading the LDS tiles (a barrier after the K loop); `lds_words` is the start of the
+// workgroup's LDS, reused here as per-wave staging.
+template <int KIND, int WP, int WQ, int WTP, int WTQ, class AccV>
+__device__ __forceinline__ void mfma_store_tile(const MfmaParams &prm, AccV (&acc)[WTQ / 32][WTP / 32],
+                                                int *lds_words, size_t lds_bytes, int p0, int q0, int NP,
+                                                int NQ, int bt) {
+  constexpr int TP = WTP / 32, TQ = WTQ / 32;
+  const GemmArgs &g = prm.g;
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int wp = wave % WP, wq = wave / WP;
+  const int lr = lane & 31, gsel = lane >> 5;
+  (void)lds_bytes;
+  // ---- epilogue --------------------------------------------------------------------------
+  // The accumulators go through LDS (free after the main loop) so that every lane ends up with
+  // four consecutive elements along the unit-stride dimension of D: stores are 8 B (bf16) or
+  // 16 B (int32/fp32) per lane and contiguous across the 16/32 lanes that share a D column.
+  // Each wave stages 16 Q-rows x WTP P-columns per pass in its own LDS region.
+  constexpr int SROW = WTP + 8;              // dwords; +8 keeps the two lane halves on distinct banks
+  constexpr int LPR = WTP / 4;               // lanes per staged row
+  constexpr int RPI = 64 / LPR;              // staged rows read per instruction
+  constexpr int ITER = 16 / RPI;
+  int *stage = lds_words + wave * (16 * SROW);
+
+  Epilogue ep(g, bt);
+  const bool swp = prm.swapped != 0;
+  const int pl = (lane % LPR) * 4, qsub = lane / LPR;
+  const int pi0 = p0 + wp * WTP + pl;
+  // quantities that depend on the P index only: fixed per lane for the whole epilogue
+  float p_scale[4], p_bias[4], p_beta[4];
+#pragma unroll
+  for (int e = 0; e < 4; e++) {
+    const int pi = min(pi0 + e, NP - 1);
+    p_scale[e] = g.int_scale ? 1.0f : (swp ? ep.col_scale(pi) : ep.row_scale(pi));
+    p_bias[e] = (g.int_scale || swp) ? 0.0f : ep.bias_at(pi);
+    p_beta[e] = (g.int_scale || swp) ? 0.0f : ep.beta_at(pi);
+  }
+  const int64_t d_sp = swp ? g.d_sj : g.d_si, d_sq = swp ? g.d_si : g.d_sj;  // d_sp == 1
+  const int64_t c_sp = swp ? g.c_sj : g.c_si, c_sq = swp ? g.c_si : g.c_sj;
+  const uint32_t dbits = g.d_type == CUDA_R_32F || g.d_type == CUDA_R_32I ? 32 : g.d_type == CUDA_R_8I ? 8 : 16;
+  const bool int_fast = g.int_scale && g.alpha_mode != VECTOR_DEV && g.beta_mode != VECTOR_DEV;
+  int32_t ialpha = 1, ibeta = 0;
+  if (int_fast) {
+    ialpha = g.alpha_mode == SCALAR_VALUE ? g.alpha_val.i : *(const int32_t *)g.alpha_ptr;
+    ibeta = g.beta_mode == SCALAR_VALUE ? g.beta_val.i : *(const int32_t *)g.beta_ptr;
+  }
+
+  // `pass` must be a compile-time constant: a rolled loop here would index the accumulator
+  // registers dynamically and push them to scratch for the whole kernel.
+  auto do_pass = [&](auto pass_c) {
+    constexpr int pass = decltype(pass_c)::value;
+    constexpr int a = pass >> 1, h = pass & 1;
+#pragma unroll
+    for (int b = 0; b < TP; b++)
+#pragma unroll
+      for (int vv = 0; vv < 8; vv++) {
+        const int ql = 8 * (vv >> 2) + 4 * gsel + (vv & 3);
+        stage[ql * SROW + b * 32 + lr] = to_bits(acc[a][b][h * 8 + vv]);
+      }
+    __syncthreads();
+#pragma unroll 1
+    for (int it = 0; it < ITER; it++) {
+      const int ql = it * RPI + qsub;
+      const int qi = q0 + wq * WTQ + a * 32 + h * 16 + ql;
+      const v4i raw = *(const v4i *)&stage[ql * SROW + pl];
+      if (qi >= NQ || pi0 >= NP) continue;
+      const int64_t dbase = g.d_sb * bt + (int64_t)pi0 * d_sp + (int64_t)qi * d_sq;
+      const int64_t cbase = g.c_sb * bt + (int64_t)pi0 * c_sp + (int64_t)qi * c_sq;
+      const bool full4 = pi0 + 3 < NP && ((dbase * dbits / 8) & (dbits / 2 - 1)) == 0 &&
+                         (((uintptr_t)g.D) & 15) == 0;
+      if (g.int_scale) {
+        if (int_fast) {
+          v4i r;
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            uint32_t x = (uint32_t)ialpha * (uint32_t)raw[e];
+            if (ibeta != 0 && pi0 + e < NP) x += (uint32_t)ibeta * (uint32_t)((const int32_t *)g.C)[cbase + e * c_sp];
+            r[e] = (int)x;
+          }
+          if (full4) *(v4i *)((int32_t *)g.D + dbase) = r;
+          else
+#pragma unroll
+            for (int e = 0; e < 4; e++) if (pi0 + e < NP) ((int32_t *)g.D)[dbase + e] = r[e];
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; e++)
+            if (pi0 + e < NP) ep.store_int(swp ? qi : pi0 + e, swp ? pi0 + e : qi, raw[e]);
+        }
+        continue;
+      }
+      const float q_scale = swp ? ep.row_scale(qi) : ep.col_scale(qi);
+      const float q_bias = swp ? ep.bias_at(qi) : 0.0f;
+      const float q_beta = swp ? ep.beta_at(qi) : 0.0f;
+      float x[4];
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        const int rawe = raw[e];
+        const float accf = KIND == KIND_I8 ? (float)rawe : bits2f((uint32_t)rawe);
+        float y = (swp ? q_scale * p_scale[e] : p_scale[e] * q_scale) * accf;
+        const float be = swp ? q_beta : p_beta[e];
+        if (be != 0.0f && pi0 + e < NP) y += be * ep.sc * load_elem(g.C, g.c_type, cbase + e * c_sp);
+        y += swp ? q_bias : p_bias[e];
+        x[e] = ep.finish(y);
+      }
+      if (full4 && dbits == 32 && g.d_type == CUDA_R_32F) {
+        *(float4 *)((float *)g.D + dbase) = make_float4(x[0], x[1], x[2], x[3]);
+      } else if (full4 && g.d_type == CUDA_R_16BF) {
+        uint2 pk;
+        pk.x = (uint32_t)enc_bf16(x[0]) | ((uint32_t)enc_bf16(x[1]) << 16);
+        pk.y = (uint32_t)enc_bf16(x[2]) | ((uint32_t)enc_bf16(x[3]) << 16);
+        *(uint2 *)((uint16_t *)g.D + dbase) = pk;
+      } else if (full4 && g.d_type == CUDA_R_16F) {
+        uint2 pk;
+        pk.x = (uint32_t)enc_f16(x[0]) | ((uint32_t)enc_f16(x[1]) << 16);
+        pk.y = (uint32_t)enc_f16(x[2]) | ((uint32_t)enc_f16(x[3]) << 16);
+        *(uint2 *)((uint16_t *)g.D + dbase) = pk;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+          if (pi0 + e < NP) store_elem(g.D, g.d_type, dbase + e, x[e]);
+      }
+    }
+    __syncthreads();
+  };
+  static_for<TQ * 2>(do_pass);
+}
+
 // LOADMODE 0: global -> VGPR -> ds_write_b128 (one stage ahead in registers)
 // LOADMODE 1: buffer_load ... lds  (global -> LDS directly, no staging registers)
 template <int KIND, int FQ, int FP, int BP, int BQ, int WP, int WQ, int LOADMODE>
@@ -279,119 +406,7 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_kernel(MfmaParams prm) 
     stage_fence();
   } while (++kt < KT);
 
-  // ---- epilogue --------------------------------------------------------------------------
-  // The accumulators go through LDS (free after the main loop) so that every lane ends up with
-  // four consecutive elements along the unit-stride dimension of D: stores are 8 B (bf16) or
-  // 16 B (int32/fp32) per lane and contiguous across the 16/32 lanes that share a D column.
-  // Each wave stages 16 Q-rows x WTP P-columns per pass in its own LDS region.
-  constexpr int SROW = WTP + 8;              // dwords; +8 keeps the two lane halves on distinct banks
-  constexpr int LPR = WTP / 4;               // lanes per staged row
-  constexpr int RPI = 64 / LPR;              // staged rows read per instruction
-  constexpr int ITER = 16 / RPI;
-  static_assert(sizeof(lds) >= (size_t)WP * WQ * 16 * SROW * 4, "epilogue staging must fit");
-  int *stage = (int *)&lds[0][0] + wave * (16 * SROW);
-
-  Epilogue ep(g, bt);
-  const bool swp = prm.swapped != 0;
-  const int pl = (lane % LPR) * 4, qsub = lane / LPR;
-  const int pi0 = p0 + wp * WTP + pl;
-  // quantities that depend on the P index only: fixed per lane for the whole epilogue
-  float p_scale[4], p_bias[4], p_beta[4];
-#pragma unroll
-  for (int e = 0; e < 4; e++) {
-    const int pi = min(pi0 + e, NP - 1);
-    p_scale[e] = g.int_scale ? 1.0f : (swp ? ep.col_scale(pi) : ep.row_scale(pi));
-    p_bias[e] = (g.int_scale || swp) ? 0.0f : ep.bias_at(pi);
-    p_beta[e] = (g.int_scale || swp) ? 0.0f : ep.beta_at(pi);
-  }
-  const int64_t d_sp = swp ? g.d_sj : g.d_si, d_sq = swp ? g.d_si : g.d_sj;  // d_sp == 1
-  const int64_t c_sp = swp ? g.c_sj : g.c_si, c_sq = swp ? g.c_si : g.c_sj;
-  const uint32_t dbits = g.d_type == CUDA_R_32F || g.d_type == CUDA_R_32I ? 32 : g.d_type == CUDA_R_8I ? 8 : 16;
-  const bool int_fast = g.int_scale && g.alpha_mode != VECTOR_DEV && g.beta_mode != VECTOR_DEV;
-  int32_t ialpha = 1, ibeta = 0;
-  if (int_fast) {
-    ialpha = g.alpha_mode == SCALAR_VALUE ? g.alpha_val.i : *(const int32_t *)g.alpha_ptr;
-    ibeta = g.beta_mode == SCALAR_VALUE ? g.beta_val.i : *(const int32_t *)g.beta_ptr;
-  }
-
-  // `pass` must be a compile-time constant: a rolled loop here would index the accumulator
-  // registers dynamically and push them to scratch for the whole kernel.
-  auto do_pass = [&](auto pass_c) {
-    constexpr int pass = decltype(pass_c)::value;
-    constexpr int a = pass >> 1, h = pass & 1;
-#pragma unroll
-    for (int b = 0; b < TP; b++)
-#pragma unroll
-      for (int vv = 0; vv < 8; vv++) {
-        const int ql = 8 * (vv >> 2) + 4 * gsel + (vv & 3);
-        stage[ql * SROW + b * 32 + lr] = to_bits(acc[a][b][h * 8 + vv]);
-      }
-    __syncthreads();
-#pragma unroll 1
-    for (int it = 0; it < ITER; it++) {
-      const int ql = it * RPI + qsub;
-      const int qi = q0 + wq * WTQ + a * 32 + h * 16 + ql;
-      const v4i raw = *(const v4i *)&stage[ql * SROW + pl];
-      if (qi >= NQ || pi0 >= NP) continue;
-      const int64_t dbase = g.d_sb * bt + (int64_t)pi0 * d_sp + (int64_t)qi * d_sq;
-      const int64_t cbase = g.c_sb * bt + (int64_t)pi0 * c_sp + (int64_t)qi * c_sq;
-      const bool full4 = pi0 + 3 < NP && ((dbase * dbits / 8) & (dbits / 2 - 1)) == 0 &&
-                         (((uintptr_t)g.D) & 15) == 0;
-      if (g.int_scale) {
-        if (int_fast) {
-          v4i r;
-#pragma unroll
-          for (int e = 0; e < 4; e++) {
-            uint32_t x = (uint32_t)ialpha * (uint32_t)raw[e];
-            if (ibeta != 0 && pi0 + e < NP) x += (uint32_t)ibeta * (uint32_t)((const int32_t *)g.C)[cbase + e * c_sp];
-            r[e] = (int)x;
-          }
-          if (full4) *(v4i *)((int32_t *)g.D + dbase) = r;
-          else
-#pragma unroll
-            for (int e = 0; e < 4; e++) if (pi0 + e < NP) ((int32_t *)g.D)[dbase + e] = r[e];
-        } else {
-#pragma unroll
-          for (int e = 0; e < 4; e++)
-            if (pi0 + e < NP) ep.store_int(swp ? qi : pi0 + e, swp ? pi0 + e : qi, raw[e]);
-        }
-        continue;
-      }
-      const float q_scale = swp ? ep.row_scale(qi) : ep.col_scale(qi);
-      const float q_bias = swp ? ep.bias_at(qi) : 0.0f;
-      const float q_beta = swp ? ep.beta_at(qi) : 0.0f;
-      float x[4];
-#pragma unroll
-      for (int e = 0; e < 4; e++) {
-        const int rawe = raw[e];
-        const float accf = KIND == KIND_I8 ? (float)rawe : bits2f((uint32_t)rawe);
-        float y = (swp ? q_scale * p_scale[e] : p_scale[e] * q_scale) * accf;
-        const float be = swp ? q_beta : p_beta[e];
-        if (be != 0.0f && pi0 + e < NP) y += be * ep.sc * load_elem(g.C, g.c_type, cbase + e * c_sp);
-        y += swp ? q_bias : p_bias[e];
-        x[e] = ep.finish(y);
-      }
-      if (full4 && dbits == 32 && g.d_type == CUDA_R_32F) {
-        *(float4 *)((float *)g.D + dbase) = make_float4(x[0], x[1], x[2], x[3]);
-      } else if (full4 && g.d_type == CUDA_R_16BF) {
-        uint2 pk;
-        pk.x = (uint32_t)enc_bf16(x[0]) | ((uint32_t)enc_bf16(x[1]) << 16);
-        pk.y = (uint32_t)enc_bf16(x[2]) | ((uint32_t)enc_bf16(x[3]) << 16);
-        *(uint2 *)((uint16_t *)g.D + dbase) = pk;
-      } else if (full4 && g.d_type == CUDA_R_16F) {
-        uint2 pk;
-        pk.x = (uint32_t)enc_f16(x[0]) | ((uint32_t)enc_f16(x[1]) << 16);
-        pk.y = (uint32_t)enc_f16(x[2]) | ((uint32_t)enc_f16(x[3]) << 16);
-        *(uint2 *)((uint16_t *)g.D + dbase) = pk;
-      } else {
-#pragma unroll
-        for (int e = 0; e < 4; e++)
-          if (pi0 + e < NP) store_elem(g.D, g.d_type, dbase + e, x[e]);
-      }
-    }
-    __syncthreads();
-  };
-  static_for<TQ * 2>(do_pass);
+  mfma_store_tile<KIND, WP, WQ, WTP, WTQ>(prm, acc, (int *)&lds[0][0], sizeof(lds), p0, q0, NP, NQ, bt);
 }
 
 } // namespace zluda_amd
