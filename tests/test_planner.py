@@ -31,7 +31,7 @@ def test_baseline_configs_pick_the_intended_kernels(api):
     st, p = plan(api, dict(I8, m=256, n=256, k=256, transa=0, transb=1))            # config 1: A:N B:T
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_GENERIC
     st, p = plan(api, dict(I8, m=4096, n=4096, k=4096, transa=1))                   # config 2
-    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_I8 and p.variant == 0 and p.grid_x == 256 and p.block == 256
+    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_I8 and p.variant == 0 and p.grid_x == 256 and p.block == 512
     st, p = plan(api, dict(I8, m=14336, n=16, k=4096, transa=1, d_type=K.CUDA_R_16BF, scale_type=K.CUDA_R_32F,
                            pointer_mode=K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO,
                            b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F,
@@ -46,7 +46,7 @@ def test_baseline_configs_pick_the_intended_kernels(api):
 
 def test_small_problems_get_smaller_tiles(api):
     st, p = plan(api, dict(I8, m=1024, n=1024, k=1024, transa=1))
-    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_I8 and p.variant == 1 and p.grid_x == 64
+    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_I8 and p.variant == 3 and p.grid_x == 64
     st, p = plan(api, dict(I8, m=4096, n=2048, k=1024, transa=1))
     assert st == 0 and p.variant == 2 and p.grid_x == 16 * 16
 
@@ -97,8 +97,8 @@ def test_fp4_must_be_k_contiguous(api):
 
 def test_forced_variants(api):
     spec = dict(I8, m=4096, n=4096, k=4096, transa=1)
-    for v, (grid, block) in enumerate([(256, 256), (1024, 256), (512, 256), (256, 512)] * 2):
+    for v, (grid, block) in enumerate([(256, 512), (256, 256), (512, 256), (1024, 256), (1024, 256)]):
         st, p = plan(api, spec, forced=K.ZLUDA_KERNEL_MFMA_I8, variant=v)
         assert st == 0 and p.variant == v and p.grid_x == grid and p.block == block
-    assert plan(api, spec, forced=K.ZLUDA_KERNEL_MFMA_I8, variant=8)[0] == K.CUBLAS_STATUS_INVALID_VALUE
+    assert plan(api, spec, forced=K.ZLUDA_KERNEL_MFMA_I8, variant=5)[0] == K.CUBLAS_STATUS_INVALID_VALUE
     assert plan(api, spec, forced=K.ZLUDA_KERNEL_MFMA_F8)[0] == K.CUBLAS_STATUS_NOT_SUPPORTED

@@ -1,4 +1,6 @@
-// LDS-double-buffered MFMA GEMM for K-contiguous operands on gfx950 (CDNA4).
+// Shared pieces of the MFMA GEMM kernels for K-contiguous operands on gfx950 (CDNA4): vector types,
+// LDS swizzle, direct global -> LDS copies, and the fused epilogues.  The K loop is in
+// gemm_mfma_pipe.hpp.
 //
 //   KIND_I8   : int8 x int8 -> int32         v_mfma_i32_32x32x32_i8
 //   KIND_F8   : e4m3/e5m2 -> fp32            v_mfma_f32_32x32x64_f8f6f4 (formats FP/FQ)
@@ -10,23 +12,22 @@
 // accumulator VGPRs).  For a column-major D, P = op(A) rows (i) and Q = op(B) columns (j); for a
 // row-major D the planner sets `swapped` and P/Q trade places.
 //
-// One stage holds BKB = 128 bytes of K for every row of the P and Q tiles.  LDS rows are 128 B,
-// split in eight 16-byte chunks whose position is XOR-swizzled with the row number so that both
-// the ds_write_b128 of the staging copy and the ds_read_b128 of the fragment loads are
-// conflict-free (16 consecutive rows reading the same logical chunk hit 16 distinct 16-byte
-// bank groups).
+// LDS rows of 128 B are split in eight 16-byte chunks whose position is XOR-swizzled with the row
+// number so that both the 1 KiB-per-instruction LDS fills and the ds_read_b128 fragment loads are
+// conflict-free (16 consecutive rows reading the same logical chunk hit 16 distinct 16-byte bank
+// groups).
 #pragma once
 #include "numeric.hpp"
 
 namespace zluda_amd {
 
+typedef int v2i __attribute__((ext_vector_type(2)));
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
 enum { KIND_I8 = 0, KIND_F8 = 1, KIND_MXF4 = 2 };
-constexpr int BKB = 128;  // bytes of K per LDS stage
 
 // depends on r mod 32 only, so rows 32 apart (the MFMA tiles of one wave) share a swizzle
 __device__ __forceinline__ int swz(int r) { return (r ^ ((r >> 3) & 3)) & 7; }
@@ -37,7 +38,7 @@ __device__ __forceinline__ int to_bits(int x) { return x; }
 __device__ __forceinline__ int to_bits(float x) { return (int)f2bits(x); }
 
 template <int N, int I = 0, class F>
-__device__ __forceinline__ void static_for(F &f) {
+__device__ __forceinline__ void static_for(F &&f) {
   if constexpr (I < N) {
     f(std::integral_constant<int, I>{});
     static_for<N, I + 1>(f);
@@ -61,11 +62,13 @@ struct MfmaParams {
   int32_t group_p;           // raster group height (tiles along P)
 };
 
-// Fused epilogue shared by the MFMA kernels.  The caller guarantees that every wave of the workgroup
-// has finished reading the LDS tiles (a barrier after the K loop); `lds_words` is the start of the
-// workgroup's LDS, reused here as per-wave staging.
+// General fused epilogue of the MFMA kernels: any D type, C read, vectors along either dimension,
+// partial tiles.  Correct for everything the planner admits, but it spends ~150 instructions per
+// four outputs; the fast paths in mfma_store_tile below take the common cases.
+// The caller guarantees that every wave of the workgroup has finished reading the LDS tiles (a
+// barrier after the K loop); `lds_words` is the start of the workgroup's LDS, reused as staging.
 template <int KIND, int WP, int WQ, int WTP, int WTQ, class AccV>
-__device__ __forceinline__ void mfma_store_tile(const MfmaParams &prm, AccV (&acc)[WTQ / 32][WTP / 32],
+__device__ __forceinline__ void mfma_store_tile_general(const MfmaParams &prm, AccV (&acc)[WTQ / 32][WTP / 32],
                                                 int *lds_words, size_t lds_bytes, int p0, int q0, int NP,
                                                 int NQ, int bt) {
   constexpr int TP = WTP / 32, TQ = WTQ / 32;
@@ -188,225 +191,179 @@ __device__ __forceinline__ void mfma_store_tile(const MfmaParams &prm, AccV (&ac
   static_for<TQ * 2>(do_pass);
 }
 
-// LOADMODE 0: global -> VGPR -> ds_write_b128 (one stage ahead in registers)
-// LOADMODE 1: buffer_load ... lds  (global -> LDS directly, no staging registers)
-template <int KIND, int FQ, int FP, int BP, int BQ, int WP, int WQ, int LOADMODE>
-__global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_kernel(MfmaParams prm) {
-  constexpr int NT = WP * WQ * 64;
-  constexpr int RP = NT / 8;          // rows copied per pass of the staging loop
-  constexpr int LP = BP / RP, LQ = BQ / RP;
-  constexpr int WTP = BP / WP, WTQ = BQ / WQ;  // wave tile
-  constexpr int TP = WTP / 32, TQ = WTQ / 32;  // MFMA tiles per wave
-  static_assert(BP % RP == 0 && BQ % RP == 0, "tile must be a multiple of the copy pass");
-  static_assert(RP % 32 == 0, "the swizzle of a thread's rows must not change between passes");
-  using acc_v = typename std::conditional<KIND == KIND_I8, v16i, v16f>::type;
-
-  __shared__ v4i lds[2][(BP + BQ) * 8];
-
+// Fast path 1: pure integer epilogue with alpha, beta scalars and beta == 0 on a full tile with
+// 16-byte aligned columns: D = alpha * acc straight from the accumulator registers.  Lanes 0..31 of
+// a store hold 32 consecutive int32 of one D column (one 128-byte line), so no LDS staging is
+// needed; two instructions per output element.
+template <int WP, int WQ, int WTP, int WTQ>
+__device__ __forceinline__ void mfma_store_tile_i32(const MfmaParams &prm, v16i (&acc)[WTQ / 32][WTP / 32],
+                                                    int p0, int q0, int bt, int ialpha) {
+  constexpr int TP = WTP / 32, TQ = WTQ / 32;
   const GemmArgs &g = prm.g;
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  // the wave index is uniform by construction; say so, or the buffer descriptor built from it is
+  // treated as divergent and every store is wrapped in a readfirstlane loop
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wp = wave % WP, wq = wave / WP;
-  const int bt = blockIdx.y;
-
-  // ---- workgroup -> tile: XCD-aware remap, then grouped raster --------------------------
-  // Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous run of tiles so
-  // that the tiles sharing P/Q panels also share an L2.
-  const int total = prm.tiles_p * prm.tiles_q;
-  int w = blockIdx.x;
-  if ((total & 7) == 0) w = (w & 7) * (total >> 3) + (w >> 3);
-  const int group = prm.group_p * prm.tiles_q;
-  const int gid = w / group, first_p = gid * prm.group_p;
-  const int gsz = min(prm.tiles_p - first_p, prm.group_p);
-  const int tile_p = first_p + (w % group) % gsz, tile_q = (w % group) / gsz;
-  const int p0 = tile_p * BP, q0 = tile_q * BQ;
-
-  // ---- operand views (bytes) --------------------------------------------------------------
-  const int NP = prm.swapped ? g.N : g.M, NQ = prm.swapped ? g.M : g.N;
-  constexpr int ebits = KIND == KIND_MXF4 ? 4 : 8;
-  const int Kbytes = (int)((int64_t)g.K * ebits / 8);
-  const uint8_t *Pg, *Qg;
-  int ldp, ldq;  // bytes between consecutive rows (the planner keeps whole operands < 2 GiB)
-  if (!prm.swapped) {
-    Pg = (const uint8_t *)g.A + g.a_sb * bt * ebits / 8; ldp = (int)(g.a_si * ebits / 8);
-    Qg = (const uint8_t *)g.B + g.b_sb * bt * ebits / 8; ldq = (int)(g.b_sj * ebits / 8);
-  } else {
-    Pg = (const uint8_t *)g.B + g.b_sb * bt * ebits / 8; ldp = (int)(g.b_sj * ebits / 8);
-    Qg = (const uint8_t *)g.A + g.a_sb * bt * ebits / 8; ldq = (int)(g.a_si * ebits / 8);
-  }
-  const int KT = (Kbytes + BKB - 1) / BKB;
-
-  // Raw buffer descriptors with a 2 GiB window: an offset with bit 31 set is out of range and
-  // reads as zero, which is how the K tail of the last stage is zero-filled without branches.
-  const __amdgpu_buffer_rsrc_t rsP = __builtin_amdgcn_make_buffer_rsrc((void *)Pg, 0, 0x80000000, 0x00020000);
-  const __amdgpu_buffer_rsrc_t rsQ = __builtin_amdgcn_make_buffer_rsrc((void *)Qg, 0, 0x80000000, 0x00020000);
-
-  // staging copy: thread -> row r0 + RP*i, LDS slot (t & 7), global chunk (t & 7) ^ swz(row)
-  const int r0 = t >> 3, slot = t & 7, cg = slot ^ swz(r0);
-  int voffP[LP], voffQ[LQ];
-#pragma unroll
-  for (int i = 0; i < LP; i++) voffP[i] = min(p0 + r0 + RP * i, NP - 1) * ldp + cg * 16;
-#pragma unroll
-  for (int i = 0; i < LQ; i++) voffQ[i] = min(q0 + r0 + RP * i, NQ - 1) * ldq + cg * 16;
-  const int tail_bytes = Kbytes - (KT - 1) * BKB;  // valid bytes of the last stage (1..128)
-  const int oob_last = cg * 16 < tail_bytes ? 0 : (int)0x80000000;
-
-  v4i preg[LOADMODE == 0 ? LP : 1], qreg[LOADMODE == 0 ? LQ : 1];
-  auto gload = [&](int kt, int buf) {
-    const int oob = kt == KT - 1 ? oob_last : 0;
-    if constexpr (LOADMODE == 0) {
-#pragma unroll
-      for (int i = 0; i < LP; i++) preg[i] = __builtin_amdgcn_raw_buffer_load_b128(rsP, voffP[i] | oob, kt * BKB, 0);
-#pragma unroll
-      for (int i = 0; i < LQ; i++) qreg[i] = __builtin_amdgcn_raw_buffer_load_b128(rsQ, voffQ[i] | oob, kt * BKB, 0);
-    } else {
-      // each wave instruction fills 1 KiB of LDS: 8 rows x 128 B, lane l -> byte l*16
-#pragma unroll
-      for (int i = 0; i < LP; i++)
-        lds_dma16(rsP, &lds[buf][(wave * 8 + RP * i) * 8], voffP[i] | oob, kt * BKB);
-#pragma unroll
-      for (int i = 0; i < LQ; i++)
-        lds_dma16(rsQ, &lds[buf][(BP + wave * 8 + RP * i) * 8], voffQ[i] | oob, kt * BKB);
-    }
-  };
-  auto lstore = [&](int buf) {
-    if constexpr (LOADMODE == 0) {
-#pragma unroll
-      for (int i = 0; i < LP; i++) lds[buf][(r0 + RP * i) * 8 + slot] = preg[i];
-#pragma unroll
-      for (int i = 0; i < LQ; i++) lds[buf][(BP + r0 + RP * i) * 8 + slot] = qreg[i];
-    }
-  };
-  auto stage_fence = [&]() {
-    if constexpr (LOADMODE == 1) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): LDS DMA landed
-    __syncthreads();
-  };
-
-  // ---- MX block scales: one dword (4 consecutive K blocks) per lane, row and stage ----------
-  // lane group gsel (= lane/32) owns chunks gsel*4 .. gsel*4+3 of the stage, i.e. K blocks
-  // kt*8 + gsel*4 + ks, whose scale bytes are one aligned dword of the [row][K/32] scale tensor.
   const int lr = lane & 31, gsel = lane >> 5;
-  const uint8_t *sp_row[TP], *sq_row[TQ];
-  int sp_cur[TP], sq_cur[TQ], sp_nxt[TP], sq_nxt[TQ];
-  if constexpr (KIND == KIND_MXF4) {
-    const int KB = g.K / 32;
-    const uint8_t *Ps = (const uint8_t *)(prm.swapped ? g.b_scale : g.a_scale) + (int64_t)bt * NP * KB;
-    const uint8_t *Qs = (const uint8_t *)(prm.swapped ? g.a_scale : g.b_scale) + (int64_t)bt * NQ * KB;
+  const int d_sq = (int)(prm.swapped ? g.d_si : g.d_sj);  // < 2^22 (checked by the dispatcher)
+  // Buffer stores: wave-uniform descriptor at the wave tile, per-lane byte offset of (row 4*gsel,
+  // column lr) in a VGPR, everything else in the scalar offset.
+  int32_t *Dw = (int32_t *)g.D + g.d_sb * bt + (int64_t)(q0 + wq * WTQ) * d_sq + (p0 + wp * WTP);
+  const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)Dw, 0, 0xFFFFFFFF, 0x00020000);
+  const int voff = (4 * gsel * d_sq + lr) * 4;
+  // alpha == 1 (the usual case) stores the accumulator registers as they are
+  if (ialpha == 1) {
 #pragma unroll
-    for (int i = 0; i < TP; i++)
-      sp_row[i] = Ps + (int64_t)min(p0 + wp * WTP + i * 32 + lr, NP - 1) * KB + gsel * 4;
+    for (int a = 0; a < TQ; a++)
 #pragma unroll
-    for (int i = 0; i < TQ; i++)
-      sq_row[i] = Qs + (int64_t)min(q0 + wq * WTQ + i * 32 + lr, NQ - 1) * KB + gsel * 4;
+      for (int v = 0; v < 16; v++) {
+        const int soff = (a * 32 + 8 * (v >> 2) + (v & 3)) * d_sq * 4;  // uniform
+#pragma unroll
+        for (int b = 0; b < TP; b++) __builtin_amdgcn_raw_buffer_store_b32(acc[a][b][v], rs, voff, soff + b * 128, 0);
+      }
+  } else {
+#pragma unroll
+    for (int a = 0; a < TQ; a++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        const int soff = (a * 32 + 8 * (v >> 2) + (v & 3)) * d_sq * 4;
+#pragma unroll
+        for (int b = 0; b < TP; b++)
+          __builtin_amdgcn_raw_buffer_store_b32(acc[a][b][v] * ialpha, rs, voff, soff + b * 128, 0);
+      }
   }
-  auto sload = [&](int kt) {
-    if constexpr (KIND == KIND_MXF4) {
-#pragma unroll
-      for (int i = 0; i < TP; i++) sp_nxt[i] = *(const int *)(sp_row[i] + kt * 8);
-#pragma unroll
-      for (int i = 0; i < TQ; i++) sq_nxt[i] = *(const int *)(sq_row[i] + kt * 8);
-    }
-  };
+}
 
-  acc_v acc[TQ][TP];
+// Fast path 2: float epilogue without a C read (beta == 0) on a full tile, D of type bf16, f16 or
+// f32 with aligned columns.  The accumulators are staged through LDS so that a lane owns four
+// consecutive elements of a D column (8- or 16-byte stores, 256/512 contiguous bytes per column and
+// instruction).  Everything that does not change inside the inner loop is hoisted; the loop body is
+// one ds_read_b128, the arithmetic and one store.
+template <int KIND, int WP, int WQ, int WTP, int WTQ, int ACT, int DT, class AccV>
+__device__ __forceinline__ void mfma_store_tile_f(const MfmaParams &prm, AccV (&acc)[WTQ / 32][WTP / 32],
+                                                  int *lds_words, int p0, int q0, int bt) {
+  constexpr int TP = WTP / 32, TQ = WTQ / 32;
+  constexpr int SROW = WTP + 8, LPR = WTP / 4, RPI = 64 / LPR, ITER = 16 / RPI;
+  constexpr int ESZ = DT == 2 ? 4 : 2;
+  const GemmArgs &g = prm.g;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wp = wave % WP, wq = wave / WP;
+  const int lr = lane & 31, gsel = lane >> 5;
+  int *stage = lds_words + wave * (16 * SROW);
+  Epilogue ep(g, bt);
+  const bool swp = prm.swapped != 0;
+  const int pl = (lane % LPR) * 4, qsub = lane / LPR;
+  const int pi0 = p0 + wp * WTP + pl;
+  float p_scale[4], p_bias[4];
 #pragma unroll
-  for (int a = 0; a < TQ; a++)
+  for (int e = 0; e < 4; e++) {
+    p_scale[e] = swp ? ep.col_scale(pi0 + e) : ep.row_scale(pi0 + e);
+    p_bias[e] = swp ? 0.0f : ep.bias_at(pi0 + e);
+  }
+  // vectors that run along Q (per-column scale, or per-row quantities of a row-major D)
+  const bool q_vec = swp ? (ep.alpha_v || ep.sa_v || g.bias) : (ep.sb_v != nullptr);
+  const float q_scale_u = swp ? ep.row_scale(0) : ep.col_scale(0);  // used when !q_vec
+  const int d_sq = (int)(swp ? g.d_si : g.d_sj);  // < 2^22 (checked by the dispatcher)
+  // buffer stores: uniform descriptor at the wave tile, per-lane byte offset (row qsub, column pl)
+  char *Dw = (char *)g.D + (g.d_sb * bt + (int64_t)(q0 + wq * WTQ) * d_sq + (p0 + wp * WTP)) * ESZ;
+  const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)Dw, 0, 0xFFFFFFFF, 0x00020000);
+  const int voff = (qsub * d_sq + pl) * ESZ;
+  const int read_off = qsub * SROW + pl;
+
+  auto do_pass = [&](auto pass_c) {
+    constexpr int pass = decltype(pass_c)::value;
+    constexpr int a = pass >> 1, h = pass & 1;
 #pragma unroll
     for (int b = 0; b < TP; b++)
 #pragma unroll
-      for (int v = 0; v < 16; v++) acc[a][b][v] = 0;
-
-  gload(0, 0);
-  sload(0);
-  lstore(0);
-  stage_fence();
-
-  int kt = 0;
-  do {  // K >= 1, so at least one stage
-    const int buf = kt & 1;
-    if constexpr (KIND == KIND_MXF4) {
+      for (int vv = 0; vv < 8; vv++) {
+        const int ql = 8 * (vv >> 2) + 4 * gsel + (vv & 3);
+        stage[ql * SROW + b * 32 + lr] = to_bits(acc[a][b][h * 8 + vv]);
+      }
+    __syncthreads();
+#pragma unroll 2
+    for (int it = 0; it < ITER; it++) {
+      const v4i raw = *(const v4i *)&stage[it * RPI * SROW + read_off];
+      float qs = q_scale_u, qb = 0.0f;
+      if (q_vec) {
+        const int qi = q0 + wq * WTQ + a * 32 + h * 16 + it * RPI + qsub;
+        qs = swp ? ep.row_scale(qi) : ep.col_scale(qi);
+        qb = swp ? ep.bias_at(qi) : 0.0f;
+      }
+      float x[4];
 #pragma unroll
-      for (int i = 0; i < TP; i++) sp_cur[i] = sp_nxt[i];
-#pragma unroll
-      for (int i = 0; i < TQ; i++) sq_cur[i] = sq_nxt[i];
+      for (int e = 0; e < 4; e++) {
+        const int rawe = raw[e];
+        const float accf = KIND == KIND_I8 ? (float)rawe : bits2f((uint32_t)rawe);
+        float y = (swp ? qs * p_scale[e] : p_scale[e] * qs) * accf + (swp ? qb : p_bias[e]);
+        if (ACT == ACT_RELU) y = y > 0.0f ? y : 0.0f;
+        else if (ACT == ACT_GELU) y = gelu_tanh(y);
+        x[e] = y * ep.sd;
+      }
+      const int soff = (a * 32 + h * 16 + it * RPI) * d_sq * ESZ;  // uniform
+      if constexpr (DT == 2) {
+        const v4i pk = {(int)f2bits(x[0]), (int)f2bits(x[1]), (int)f2bits(x[2]), (int)f2bits(x[3])};
+        __builtin_amdgcn_raw_buffer_store_b128(pk, rs, voff, soff, 0);
+      } else {
+        v2i pk;
+        if constexpr (DT == 0) {
+          pk[0] = (int)((uint32_t)enc_bf16(x[0]) | ((uint32_t)enc_bf16(x[1]) << 16));
+          pk[1] = (int)((uint32_t)enc_bf16(x[2]) | ((uint32_t)enc_bf16(x[3]) << 16));
+        } else {
+          pk[0] = (int)((uint32_t)enc_f16(x[0]) | ((uint32_t)enc_f16(x[1]) << 16));
+          pk[1] = (int)((uint32_t)enc_f16(x[2]) | ((uint32_t)enc_f16(x[3]) << 16));
+        }
+        __builtin_amdgcn_raw_buffer_store_b64(pk, rs, voff, soff, 0);
+      }
     }
-    if (kt + 1 < KT) { gload(kt + 1, buf ^ 1); sload(kt + 1); }
+    __syncthreads();
+  };
+  static_for<TQ * 2>(do_pass);
+}
 
-    const v4i *Pl = &lds[buf][(wp * WTP + lr) * 8];
-    const v4i *Ql = &lds[buf][(BP + wq * WTQ + lr) * 8];
-    const int sw = swz(lr);  // wave-tile bases are multiples of 32: swz(row) == swz(lr)
-
-    if constexpr (KIND == KIND_I8) {
-#pragma unroll
-      for (int ks = 0; ks < 4; ks++) {
-        const int ch = (ks * 2 + gsel) ^ sw;
-        v4i pf[TP], qf[TQ];
-#pragma unroll
-        for (int i = 0; i < TP; i++) pf[i] = Pl[i * 32 * 8 + ch];
-#pragma unroll
-        for (int i = 0; i < TQ; i++) qf[i] = Ql[i * 32 * 8 + ch];
-#pragma unroll
-        for (int a = 0; a < TQ; a++)
-#pragma unroll
-          for (int b = 0; b < TP; b++)
-            acc[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(qf[a], pf[b], acc[a][b], 0, 0, 0);
-      }
-    } else if constexpr (KIND == KIND_F8) {
-#pragma unroll
-      for (int ks = 0; ks < 2; ks++) {
-        const int c0 = (ks * 4 + gsel * 2) ^ sw, c1 = (ks * 4 + gsel * 2 + 1) ^ sw;
-        v8i pf[TP], qf[TQ];
-#pragma unroll
-        for (int i = 0; i < TP; i++) {
-          v4i lo = Pl[i * 32 * 8 + c0], hi = Pl[i * 32 * 8 + c1];
-          pf[i] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        }
-#pragma unroll
-        for (int i = 0; i < TQ; i++) {
-          v4i lo = Ql[i * 32 * 8 + c0], hi = Ql[i * 32 * 8 + c1];
-          qf[i] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        }
-#pragma unroll
-        for (int a = 0; a < TQ; a++)
-#pragma unroll
-          for (int b = 0; b < TP; b++)
-            acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(qf[a], pf[b], acc[a][b], FQ, FP,
-                                                                         0, 0, 0, 0);
-      }
+// Epilogue dispatch: the fast paths for full tiles of the common configurations, the general path
+// for the rest.  All conditions are workgroup-uniform.
+template <int KIND, int WP, int WQ, int WTP, int WTQ, class AccV>
+__device__ __forceinline__ void mfma_store_tile(const MfmaParams &prm, AccV (&acc)[WTQ / 32][WTP / 32],
+                                                int *lds_words, size_t lds_bytes, int p0, int q0, int NP,
+                                                int NQ, int bt) {
+  const GemmArgs &g = prm.g;
+  const bool swp = prm.swapped != 0;
+  const int64_t d_sq = swp ? g.d_si : g.d_sj;
+  const bool full = p0 + WP * WTP <= NP && q0 + WQ * WTQ <= NQ;
+  const int dbytes = (g.d_type == CUDA_R_32F || g.d_type == CUDA_R_32I) ? 4 : (g.d_type == CUDA_R_8I ? 1 : 2);
+  // columns of the tile start 16-byte aligned and the lane offsets fit 32 bits
+  const bool aligned = (((uintptr_t)g.D) & 15) == 0 && ((d_sq * dbytes) & 15) == 0 &&
+                       ((g.d_sb * dbytes) & 15) == 0 && d_sq < (1 << 22);
+  if constexpr (KIND == KIND_I8) {
+    if (g.int_scale && full && aligned && g.alpha_mode != VECTOR_DEV && g.beta_mode == SCALAR_VALUE &&
+        g.beta_val.i == 0) {
+      const int ialpha = g.alpha_mode == SCALAR_VALUE ? g.alpha_val.i : *(const int32_t *)g.alpha_ptr;
+      mfma_store_tile_i32<WP, WQ, WTP, WTQ>(prm, acc, p0, q0, bt, ialpha);
+      return;
+    }
+  }
+  if (!g.int_scale && full && aligned && g.beta_mode == SCALAR_VALUE && g.beta_val.f == 0.0f &&
+      (g.d_type == CUDA_R_16BF || g.d_type == CUDA_R_16F || g.d_type == CUDA_R_32F)) {
+    const int dt = g.d_type == CUDA_R_16BF ? 0 : (g.d_type == CUDA_R_16F ? 1 : 2);
+#define ZLUDA_EPI(ACT_, DT_) mfma_store_tile_f<KIND, WP, WQ, WTP, WTQ, ACT_, DT_>(prm, acc, lds_words, p0, q0, bt)
+    if (dt == 0) {
+      if (g.act == ACT_GELU) ZLUDA_EPI(ACT_GELU, 0);
+      else if (g.act == ACT_RELU) ZLUDA_EPI(ACT_RELU, 0);
+      else ZLUDA_EPI(ACT_NONE, 0);
+    } else if (dt == 1) {
+      if (g.act == ACT_GELU) ZLUDA_EPI(ACT_GELU, 1);
+      else if (g.act == ACT_RELU) ZLUDA_EPI(ACT_RELU, 1);
+      else ZLUDA_EPI(ACT_NONE, 1);
     } else {
-#pragma unroll
-      for (int ks = 0; ks < 4; ks++) {
-        const int ch = (gsel * 4 + ks) ^ sw;
-        v8i pf[TP], qf[TQ];
-#pragma unroll
-        for (int i = 0; i < TP; i++) {
-          v4i lo = Pl[i * 32 * 8 + ch];
-          pf[i] = v8i{lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
-        }
-#pragma unroll
-        for (int i = 0; i < TQ; i++) {
-          v4i lo = Ql[i * 32 * 8 + ch];
-          qf[i] = v8i{lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
-        }
-#pragma unroll
-        for (int a = 0; a < TQ; a++)
-#pragma unroll
-          for (int b = 0; b < TP; b++) {
-            // op_sel picks byte ks of each scale dword; the builtin wants it as a constant
-            switch (ks) {
-            case 0: acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(qf[a], pf[b], acc[a][b], 4, 4, 0, sq_cur[a], 0, sp_cur[b]); break;
-            case 1: acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(qf[a], pf[b], acc[a][b], 4, 4, 1, sq_cur[a], 1, sp_cur[b]); break;
-            case 2: acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(qf[a], pf[b], acc[a][b], 4, 4, 2, sq_cur[a], 2, sp_cur[b]); break;
-            default: acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(qf[a], pf[b], acc[a][b], 4, 4, 3, sq_cur[a], 3, sp_cur[b]); break;
-            }
-          }
-      }
+      if (g.act == ACT_GELU) ZLUDA_EPI(ACT_GELU, 2);
+      else if (g.act == ACT_RELU) ZLUDA_EPI(ACT_RELU, 2);
+      else ZLUDA_EPI(ACT_NONE, 2);
     }
-
-    if (kt + 1 < KT) lstore(buf ^ 1);
-    stage_fence();
-  } while (++kt < KT);
-
-  mfma_store_tile<KIND, WP, WQ, WTP, WTQ>(prm, acc, (int *)&lds[0][0], sizeof(lds), p0, q0, NP, NQ, bt);
+#undef ZLUDA_EPI
+    return;
+  }
+  mfma_store_tile_general<KIND, WP, WQ, WTP, WTQ>(prm, acc, lds_words, lds_bytes, p0, q0, NP, NQ, bt);
 }
 
 } // namespace zluda_amd

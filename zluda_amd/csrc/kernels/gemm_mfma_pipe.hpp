@@ -3,37 +3,36 @@
 //
 // Same tiling, operand naming (P / Q) and epilogue as gemm_mfma.hpp; what differs is the K loop:
 //
-//   * LDS holds NSTAGE = 4 stages of 64 K-bytes per tile row.  Global memory is copied straight into
-//     LDS (buffer_load_dwordx4 ... lds) three stages ahead of the one being multiplied, so every
-//     workgroup keeps ~3 x 32 KiB of loads in flight and the L2 / Infinity-Fabric latency is covered
-//     by three stage periods instead of one.
+//   * LDS is a ring of NSTAGE stages of BKB K-bytes per tile row, filled straight from global memory
+//     (buffer_load_dwordx4 ... lds).  BKB = 128 makes every row segment a whole 128-byte cache line:
+//     measured on MI355X, L2-resident panels stream into LDS at ~126 GB/s per CU with 128-byte
+//     segments and at half that with 64-byte segments.
+//   * A slot is refilled as soon as its last fragments are in registers (one MFMA sub-step before
+//     its stage ends), NSTAGE stages ahead of the stage it will hold.
 //   * The LDS -> register fragment loads run one MFMA sub-step ahead of the MFMAs that consume them
-//     (double-buffered fragment registers), so a wave never waits on the ds_read it just issued.
-//   * One s_barrier per stage, with a counted s_waitcnt vmcnt(n) in front of it that only waits for
+//     (double-buffered fragment registers, order pinned with sched_barrier), so a wave never waits
+//     on a ds_read it has just issued.
+//   * One s_barrier per stage with a counted s_waitcnt vmcnt(n) in front of it that only waits for
 //     the stage about to be read; younger stages stay in flight across the barrier.
 //
-// LDS rows are 64 B = four 16-byte chunks; chunk c of row r sits at slot c ^ ((r >> 2) & 3), which
-// makes both the 1 KiB-per-instruction LDS DMA writes and the ds_read_b128 fragment reads (32 rows,
-// same chunk) bank-conflict free.
+// LDS rows are BKB bytes = BKB/16 chunks of 16 bytes, XOR-swizzled with the row number so that the
+// 1 KiB-per-instruction DMA writes and the ds_read_b128 fragment reads are bank-conflict free.
 #pragma once
 #include "gemm_mfma.hpp"
 
 namespace zluda_amd {
 
-constexpr int PIPE_BKB = 64;    // K bytes per stage
-constexpr int PIPE_NSTAGE = 4;  // LDS ring depth
-
+// chunk swizzles: 8 chunks per 128-byte row (swz, gemm_mfma.hpp) or 4 chunks per 64-byte row
 __device__ __forceinline__ int swz4(int r) { return (r >> 2) & 3; }
 
-// s_waitcnt with only the vector-memory counter constrained (gfx9 encoding: vmcnt = [3:0] | [15:14])
-// Wait until at most N vector-memory operations of this wave are outstanding, then join the
-// workgroup barrier.  Written as inline assembly with a memory clobber: the compiler must neither
-// move LDS accesses across the barrier nor add the vmcnt(0) a fence would bring (younger stages have
-// to stay in flight).
+// Wait until at most N vector-memory operations of this wave are outstanding and every LDS read it
+// issued has returned, then join the workgroup barrier.  Inline assembly with a memory clobber: the
+// compiler must neither move LDS accesses across the barrier nor add the vmcnt(0) a fence would
+// bring (younger stages have to stay in flight).
 template <int N>
 __device__ __forceinline__ void wait_vmcnt_barrier() {
   static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
-  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N) : "memory");
+  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
 }
 
 // 4 bytes per lane from a buffer straight into LDS (buffer_load_dword ... lds): lane l lands at byte
@@ -45,31 +44,39 @@ __device__ __forceinline__ void lds_dma4(__amdgpu_buffer_rsrc_t rs, void *lds_ds
 #endif
 }
 
-template <int KIND, int FQ, int FP, int BP, int BQ, int WP, int WQ>
+template <int KIND, int FQ, int FP, int BP, int BQ, int WP, int WQ, int BKB_, int NSTAGE>
 __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams prm) {
   constexpr int NT = WP * WQ * 64;
-  constexpr int RPP = NT / 4;                  // rows filled per DMA pass (16 per wave)
-  constexpr int LP = BP / RPP, LQ = BQ / RPP;  // DMA instructions per thread, stage and operand
-  constexpr int LS = KIND == KIND_MXF4 ? (BP + BQ) / NT : 0;  // scale DMA instructions per thread and stage
+  constexpr int CPR = BKB_ / 16;               // 16-byte chunks per LDS row
+  constexpr int RPW = 64 / CPR;                // rows filled by one wave DMA instruction
+  constexpr int RPP = (NT / 64) * RPW;         // rows filled per DMA pass of the workgroup
+  constexpr int LP = BP / RPP, LQ = BQ / RPP;  // data DMA instructions per thread, stage and operand
+  constexpr int SDW = KIND == KIND_MXF4 ? BKB_ / 64 : 0;  // scale dwords per row and stage (4 blocks each)
+  constexpr int SROWS = (BP + BQ + NT - 1) / NT * NT;  // rows of a scale plane (padded to whole passes)
+  constexpr int LS = SDW * SROWS / NT;         // scale DMA instructions per thread and stage
   constexpr int NLOAD = LP + LQ + LS;          // vmcnt units per stage
   constexpr int WTP = BP / WP, WTQ = BQ / WQ;
   constexpr int TP = WTP / 32, TQ = WTQ / 32;
-  constexpr int KS = KIND == KIND_F8 ? 1 : 2;  // MFMA sub-steps per stage
-  // one stage in 16-byte units: P rows, Q rows, then (MXFP4) one scale dword per P row and Q row
-  constexpr int STAGE_V4 = (BP + BQ) * 4 + (KIND == KIND_MXF4 ? (BP + BQ) / 4 : 0);
-  static_assert(BP % RPP == 0 && BQ % RPP == 0 && RPP % 16 == 0, "tile / copy-pass mismatch");
-  static_assert((BP + BQ) % NT == 0 && BP % 64 == 0, "scale rows are copied 64 per wave instruction");
+  constexpr int KS = BKB_ / (KIND == KIND_F8 ? 64 : 32);  // MFMA sub-steps per stage
+  constexpr int SPT = (KS & 1) ? 2 : 1;        // stages per loop trip (fragment roles must realign)
+  // one stage in 16-byte units: P rows, Q rows, then (MXFP4) SDW planes of one scale dword per row
+  constexpr int STAGE_V4 = (BP + BQ) * CPR + SDW * SROWS / 4;
+  static_assert(BKB_ == 64 || BKB_ == 128, "row segments are half or whole cache lines");
+  static_assert(BP % RPP == 0 && BQ % RPP == 0 && RPP % 32 == 0, "tile / copy-pass mismatch");
+  static_assert(KIND != KIND_MXF4 || (BP % 64 == 0 && BQ % 64 == 0), "scale rows are copied 64 per wave instruction");
+  static_assert((NSTAGE - 1) * NLOAD < 64, "vmcnt range");
+  static_assert(NSTAGE * STAGE_V4 * 16 <= 160 * 1024, "LDS capacity");
   using acc_v = typename std::conditional<KIND == KIND_I8, v16i, v16f>::type;
   using frag_v = typename std::conditional<KIND == KIND_I8, v4i, v8i>::type;
-  struct Frags {
-    frag_v p[TP], q[TQ];
-    int sp[KIND == KIND_MXF4 ? TP : 1], sq[KIND == KIND_MXF4 ? TQ : 1];
-  };
+  struct Frags { frag_v p[TP], q[TQ]; };
+  struct Scales { int p[TP], q[TQ]; };  // MX scale dwords of one stage (one per MFMA tile row set)
 
-  __shared__ v4i lds[PIPE_NSTAGE * STAGE_V4];
+  __shared__ v4i lds[NSTAGE * STAGE_V4];
 
   const GemmArgs &g = prm.g;
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  // the wave index is uniform by construction; readfirstlane tells the compiler (LDS DMA bases and
+  // buffer descriptors derived from it then live in SGPRs)
+  const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
   const int wp = wave % WP, wq = wave / WP;
   const int lr = lane & 31, gsel = lane >> 5;
   const int bt = blockIdx.y;
@@ -96,27 +103,29 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
     Pg = (const uint8_t *)g.B + g.b_sb * bt * ebits / 8; ldp = (int)(g.b_sj * ebits / 8);
     Qg = (const uint8_t *)g.A + g.a_sb * bt * ebits / 8; ldq = (int)(g.a_si * ebits / 8);
   }
-  const int KT = (Kbytes + PIPE_BKB - 1) / PIPE_BKB;  // real stages
-  const int KT2 = (KT + 1) & ~1;                      // stages run: the loop body handles two
+  const int KT = (Kbytes + BKB_ - 1) / BKB_;      // real stages
+  const int KTR = (KT + SPT - 1) / SPT * SPT;     // stages run (padding stages multiply zeros)
 
   // 2 GiB raw buffer windows: an offset with bit 31 set is out of range and reads as zero
   const __amdgpu_buffer_rsrc_t rsP = __builtin_amdgcn_make_buffer_rsrc((void *)Pg, 0, 0x80000000, 0x00020000);
   const __amdgpu_buffer_rsrc_t rsQ = __builtin_amdgcn_make_buffer_rsrc((void *)Qg, 0, 0x80000000, 0x00020000);
 
-  // DMA: one wave instruction fills 16 rows x 64 B; lane l -> row l/4, slot l%4, global chunk
-  // slot ^ swz4(row)
-  const int drow = wave * 16 + (lane >> 2), dslot = lane & 3, dcg = dslot ^ swz4(lane >> 2);
+  // DMA: one wave instruction fills RPW rows x BKB bytes; lane l -> row l / CPR, slot l % CPR,
+  // global chunk slot ^ swizzle(row)
+  const int dr = lane / CPR, dslot = lane % CPR;
+  const int drow = wave * RPW + dr;  // passes advance by RPP, a multiple of 32: same swizzle
+  const int dcg = dslot ^ (CPR == 8 ? swz(drow) : swz4(drow));
   int voffP[LP], voffQ[LQ];
 #pragma unroll
   for (int i = 0; i < LP; i++) voffP[i] = min(p0 + drow + RPP * i, NP - 1) * ldp + dcg * 16;
 #pragma unroll
   for (int i = 0; i < LQ; i++) voffQ[i] = min(q0 + drow + RPP * i, NQ - 1) * ldq + dcg * 16;
-  const int tail_bytes = Kbytes - (KT - 1) * PIPE_BKB;
+  const int tail_bytes = Kbytes - (KT - 1) * BKB_;
   const int oob_last = dcg * 16 < tail_bytes ? 0 : (int)0x80000000;
 
-  // MX block scales: stage kt covers K blocks 4kt..4kt+3 of a row = one aligned dword of the
-  // [row][K/32] scale tensor.  Row r of the tile (P rows first, then Q rows) is copied by the thread
-  // with t + NT*i == r; bytes gsel*2 + ks of the dword belong to lane group gsel.
+  // MX block scales: stage kt covers BKB/16 K blocks of a row = SDW aligned dwords of the
+  // [row][K/32] scale tensor, kept as SDW planes of one dword per tile row (P rows, then Q rows).
+  // DMA instruction i of a thread copies plane i % SDW for tile row t + NT * (i / SDW).
   __amdgpu_buffer_rsrc_t rsS[LS > 0 ? LS : 1];
   int voffS[LS > 0 ? LS : 1];
   if constexpr (KIND == KIND_MXF4) {
@@ -125,71 +134,81 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
     const uint8_t *Qs = (const uint8_t *)(prm.swapped ? g.a_scale : g.b_scale) + (int64_t)bt * NQ * KB;
 #pragma unroll
     for (int i = 0; i < LS; i++) {
-      const int r = t + NT * i;  // BP is a multiple of 64, so a wave never straddles P and Q
+      // BP is a multiple of 64: a wave never straddles P and Q.  Rows past BP + BQ (padding of the
+      // last pass) copy a clamped row into the plane's padding.
+      const int r = t + NT * (i / SDW);
       const bool isq = r >= BP;
       rsS[i] = __builtin_amdgcn_make_buffer_rsrc((void *)(isq ? Qs : Ps), 0, 0x80000000, 0x00020000);
-      voffS[i] = isq ? min(q0 + r - BP, NQ - 1) * KB : min(p0 + r, NP - 1) * KB;
+      voffS[i] = (isq ? min(q0 + r - BP, NQ - 1) : min(p0 + r, NP - 1)) * KB + (i % SDW) * 4;
     }
   }
 
-  // stage kt -> LDS slot (16-byte units `so`); kt >= KT is a padding stage that is zero-filled
+  // stage kt -> LDS slot at 16-byte offset `so`; kt >= KT is a padding stage that is zero-filled
   auto issue_stage = [&](int kt, int so) {
     const int oob = kt >= KT ? (int)0x80000000 : (kt == KT - 1 ? oob_last : 0);
     v4i *base = &lds[so];
 #pragma unroll
     for (int i = 0; i < LP; i++)
-      lds_dma16(rsP, base + (wave * 16 + RPP * i) * 4, voffP[i] | oob, kt * PIPE_BKB);
+      lds_dma16(rsP, base + (wave * RPW + RPP * i) * CPR, voffP[i] | oob, kt * BKB_);
 #pragma unroll
     for (int i = 0; i < LQ; i++)
-      lds_dma16(rsQ, base + (BP + wave * 16 + RPP * i) * 4, voffQ[i] | oob, kt * PIPE_BKB);
+      lds_dma16(rsQ, base + (BP + wave * RPW + RPP * i) * CPR, voffQ[i] | oob, kt * BKB_);
     if constexpr (KIND == KIND_MXF4) {
-      int *sbase = (int *)(base + (BP + BQ) * 4);
+      int *sbase = (int *)(base + (BP + BQ) * CPR);
 #pragma unroll
       for (int i = 0; i < LS; i++)
-        lds_dma4(rsS[i], sbase + wave * 64 + NT * i, voffS[i], min(kt, KT - 1) * 4);
+        lds_dma4(rsS[i], sbase + (i % SDW) * SROWS + wave * 64 + NT * (i / SDW), voffS[i],
+                 min(kt, KT - 1) * (SDW * 4));
     }
   };
 
-  // fragment (and MX scale) loads of sub-step ks of the stage in LDS slot `so`
-  const int fsw = swz4(lr);  // wave-tile bases are multiples of 32: swz4(row) == swz4(lr)
-  auto load_frags = [&](int so, int ks, Frags &f) {
-    const v4i *Pl = &lds[so + (wp * WTP + lr) * 4];
-    const v4i *Ql = &lds[so + (BP + wq * WTQ + lr) * 4];
+  // fragment (and MX scale) loads of sub-step ks of the stage in the LDS slot at offset `so`
+  const int fsw = CPR == 8 ? swz(lr) : swz4(lr);  // wave-tile bases are multiples of 32
+  auto load_frags = [&](int so, auto ks_c, Frags &f) {
+    constexpr int ks = decltype(ks_c)::value;
+    const v4i *Pl = &lds[so + (wp * WTP + lr) * CPR];
+    const v4i *Ql = &lds[so + (BP + wq * WTQ + lr) * CPR];
     if constexpr (KIND == KIND_F8) {
-      const int c0 = (gsel * 2) ^ fsw, c1 = (gsel * 2 + 1) ^ fsw;
+      const int c0 = (ks * 4 + gsel * 2) ^ fsw, c1 = (ks * 4 + gsel * 2 + 1) ^ fsw;
 #pragma unroll
       for (int i = 0; i < TP; i++) {
-        const v4i lo = Pl[i * 32 * 4 + c0], hi = Pl[i * 32 * 4 + c1];
+        const v4i lo = Pl[i * 32 * CPR + c0], hi = Pl[i * 32 * CPR + c1];
         f.p[i] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
       }
 #pragma unroll
       for (int i = 0; i < TQ; i++) {
-        const v4i lo = Ql[i * 32 * 4 + c0], hi = Ql[i * 32 * 4 + c1];
+        const v4i lo = Ql[i * 32 * CPR + c0], hi = Ql[i * 32 * CPR + c1];
         f.q[i] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
       }
     } else {
-      // int8: chunk ks*2+gsel (natural K order); fp4: chunk gsel*2+ks, so that the two sub-steps of
-      // a lane group use consecutive scale bytes
-      const int ch = (KIND == KIND_I8 ? ks * 2 + gsel : gsel * 2 + ks) ^ fsw;
+      // int8: chunk ks*2+gsel (natural K order).  fp4: lane group gsel owns chunks gsel*KS .. +KS-1,
+      // so that its sub-steps use consecutive scale bytes
+      const int ch = (KIND == KIND_I8 ? ks * 2 + gsel : gsel * KS + ks) ^ fsw;
 #pragma unroll
       for (int i = 0; i < TP; i++) {
-        const v4i lo = Pl[i * 32 * 4 + ch];
+        const v4i lo = Pl[i * 32 * CPR + ch];
         if constexpr (KIND == KIND_I8) f.p[i] = lo;
         else f.p[i] = v8i{lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
       }
 #pragma unroll
       for (int i = 0; i < TQ; i++) {
-        const v4i lo = Ql[i * 32 * 4 + ch];
+        const v4i lo = Ql[i * 32 * CPR + ch];
         if constexpr (KIND == KIND_I8) f.q[i] = lo;
         else f.q[i] = v8i{lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
       }
-      if constexpr (KIND == KIND_MXF4) {
-        const int *Sl = (const int *)&lds[so + (BP + BQ) * 4];
+    }
+  };
+  // MX scales of the stage in the slot at `so`.  The K blocks of lane group gsel are
+  // gsel*KS .. gsel*KS+KS-1 of the stage:  KS == 2: one plane, bytes gsel*2 + ks;
+  // KS == 4: plane gsel, byte ks.  After the shift, op_sel = ks selects the byte in both cases.
+  auto load_scales = [&](int so, Scales &sc) {
+    if constexpr (KIND == KIND_MXF4) {
+      const int *Sl = (const int *)&lds[so + (BP + BQ) * CPR] + (KS == 4 ? gsel * SROWS : 0);
+      const int sh = KS == 2 ? gsel * 16 : 0;
 #pragma unroll
-        for (int i = 0; i < TP; i++) f.sp[i] = Sl[wp * WTP + i * 32 + lr] >> (gsel * 16);
+      for (int i = 0; i < TP; i++) sc.p[i] = Sl[wp * WTP + i * 32 + lr] >> sh;
 #pragma unroll
-        for (int i = 0; i < TQ; i++) f.sq[i] = Sl[BP + wq * WTQ + i * 32 + lr] >> (gsel * 16);
-      }
+      for (int i = 0; i < TQ; i++) sc.q[i] = Sl[BP + wq * WTQ + i * 32 + lr] >> sh;
     }
   };
 
@@ -201,8 +220,10 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
 #pragma unroll
       for (int v = 0; v < 16; v++) acc[a][b][v] = 0;
 
-  auto mfma_all = [&](const Frags &f, auto ks_c) {
+  // `sc` carries the MX scale dwords of the stage; op_sel picks byte ks of them
+  auto mfma_all = [&](const Frags &f, const Scales &sc, auto ks_c) {
     constexpr int ks = decltype(ks_c)::value;
+    (void)sc;
 #pragma unroll
     for (int a = 0; a < TQ; a++)
 #pragma unroll
@@ -212,59 +233,76 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
         else if constexpr (KIND == KIND_F8)
           acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.q[a], f.p[b], acc[a][b], FQ, FP, 0, 0, 0, 0);
         else
-          acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.q[a], f.p[b], acc[a][b], 4, 4, ks, f.sq[a],
-                                                                       ks, f.sp[b]);
+          acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.q[a], f.p[b], acc[a][b], 4, 4, ks, sc.q[a],
+                                                                       ks, sc.p[b]);
       }
   };
-  using c0_t = std::integral_constant<int, 0>;
-  using c1_t = std::integral_constant<int, 1>;
 
-  // ---- prologue: stages 0 .. 2 in flight, stage 0 landed ------------------------------------------
-  issue_stage(0, 0);
-  issue_stage(1, STAGE_V4);
-  issue_stage(2, 2 * STAGE_V4);
-  wait_vmcnt_barrier<2 * NLOAD>();
+  // ---- prologue: stages 0 .. NSTAGE-1 in flight, stage 0 landed -----------------------------------
+#pragma unroll
+  for (int s = 0; s < NSTAGE; s++) issue_stage(s, s * STAGE_V4);
+  wait_vmcnt_barrier<(NSTAGE - 1) * NLOAD>();
 
   Frags fa, fb;
-  load_frags(0, 0, fa);
+  Scales sc_cur, sc_nxt;
+  load_frags(0, std::integral_constant<int, 0>{}, fa);
+  load_scales(0, sc_nxt);
 
-  // One stage.  On entry the fragments of its first sub-step are in `cur`; on exit the fragments
-  // of the next stage's first sub-step are in `cur` (KS == 2) or in `oth` (KS == 1).  Before the
-  // last sub-step: wait for stage kt+1 (younger stages stay in flight), barrier (every wave is now
-  // also done reading stage kt-1), refill that slot with stage kt+3, fetch the next fragments.
+  // One stage.  On entry the fragments of its sub-step 0 are in `cur` and its MX scales in sc_nxt.
+  // Sub-step s multiplies the fragments fetched during sub-step s-1 while fetching those of
+  // sub-step s+1.  Before the last sub-step every fragment of the stage is in registers: wait for
+  // stage kt+1 (younger stages stay in flight), barrier, refill this very slot with stage
+  // kt+NSTAGE, and fetch the first fragments (and scales) of stage kt+1.
   auto do_stage = [&](int kt, int so, Frags &cur, Frags &oth) {
-    const int so_next = so == 3 * STAGE_V4 ? 0 : so + STAGE_V4;
-    const int so_issue = so == 0 ? 3 * STAGE_V4 : so - STAGE_V4;
-    // sched_barrier(0) pins the order "fetch the next fragments, then the whole MFMA cluster": left
-    // alone, the scheduler sinks each ds_read to just before its first use and the wave stalls on it.
-    if constexpr (KS == 2) {
-      load_frags(so, 1, oth);
+    const int so_next = so == (NSTAGE - 1) * STAGE_V4 ? 0 : so + STAGE_V4;
+    if constexpr (KIND == KIND_MXF4) sc_cur = sc_nxt;
+    static_for<KS>([&](auto s_c) {
+      constexpr int s = decltype(s_c)::value;
+      Frags &use = (s & 1) ? oth : cur;
+      Frags &nxt = (s & 1) ? cur : oth;
+      constexpr bool last = s + 1 == KS;
+      if constexpr (!last) {
+        load_frags(so, std::integral_constant<int, (s + 1 < KS ? s + 1 : 1)>{}, nxt);
+      } else {
+        wait_vmcnt_barrier<(NSTAGE - 2) * NLOAD>();
+        // reads first: the compiler cannot prove that the DMA (an LDS write) and these reads hit
+        // different slots, so whatever comes second in the source stays second in the schedule
+        load_frags(so_next, std::integral_constant<int, 0>{}, nxt);
+        load_scales(so_next, sc_nxt);
+        issue_stage(kt + NSTAGE, so);
+      }
+      mfma_all(use, sc_cur, s_c);
+      // Scheduling pattern of the sub-step: the MFMAs (which only need registers filled one sub-step
+      // ago) are issued back to back, with the fragment reads of the next sub-step slotted behind the
+      // first half of them and the LDS DMA of the refill behind the second half.  Without the
+      // pattern the scheduler either sinks every ds_read to its first use (the wave then stalls on
+      // it) or keeps the loads in one block in front of the MFMAs (the matrix pipe idles meanwhile).
+      constexpr int NM = TP * TQ, NDS = (TP + TQ) * (KIND == KIND_F8 ? 2 : 1) + (KIND == KIND_MXF4 && last ? TP + TQ : 0);
+      constexpr int NVM = last ? NLOAD : 0, H1 = NM / 2 > 0 ? NM / 2 : 1, H2 = NM - H1 > 0 ? NM - H1 : 1;
+      static_for<NM>([&](auto i_c) {
+        constexpr int i = decltype(i_c)::value;
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+        if constexpr (i < H1) {
+          constexpr int n = NDS * (i + 1) / H1 - NDS * i / H1;
+          if constexpr (n > 0) __builtin_amdgcn_sched_group_barrier(0x100, n, 0);  // DS reads
+        } else {
+          constexpr int j = i - H1, n = NVM * (j + 1) / H2 - NVM * j / H2;
+          if constexpr (n > 0) __builtin_amdgcn_sched_group_barrier(0x010, n, 0);  // VMEM (LDS DMA)
+        }
+      });
       __builtin_amdgcn_sched_barrier(0);
-      mfma_all(cur, c0_t{});
-      __builtin_amdgcn_sched_barrier(0);
-      wait_vmcnt_barrier<NLOAD>();
-      issue_stage(kt + 3, so_issue);
-      load_frags(so_next, 0, cur);
-      __builtin_amdgcn_sched_barrier(0);
-      mfma_all(oth, c1_t{});
-      __builtin_amdgcn_sched_barrier(0);
-    } else {
-      wait_vmcnt_barrier<NLOAD>();
-      issue_stage(kt + 3, so_issue);
-      load_frags(so_next, 0, oth);
-      __builtin_amdgcn_sched_barrier(0);
-      mfma_all(cur, c0_t{});
-      __builtin_amdgcn_sched_barrier(0);
-    }
+    });
   };
 
-  // K loop, two stages per trip, no other control flow.  Padding stages (kt >= KT) multiply zeros.
+  // K loop: SPT stages per trip, no other control flow
   int so = 0;
-  for (int kt = 0; kt < KT2; kt += 2) {
+  for (int kt = 0; kt < KTR; kt += SPT) {
     do_stage(kt, so, fa, fb);
-    if constexpr (KS == 2) do_stage(kt + 1, so + STAGE_V4, fa, fb);
-    else do_stage(kt + 1, so + STAGE_V4, fb, fa);
-    so = so == 0 ? 2 * STAGE_V4 : 0;
+    so = so == (NSTAGE - 1) * STAGE_V4 ? 0 : so + STAGE_V4;
+    if constexpr (SPT == 2) {
+      do_stage(kt + 1, so, fb, fa);
+      so = so == (NSTAGE - 1) * STAGE_V4 ? 0 : so + STAGE_V4;
+    }
   }
 
   // every wave is done with the LDS tiles (and every DMA has landed) before they become staging

@@ -17,8 +17,8 @@ uint32_t launch_mfma(const Lowered &l, const zluda_gemm_plan &plan, hipStream_t 
   MfmaParams prm;
   prm.g = l.g;
   prm.swapped = plan.swapped;
-  if (plan.variant >= 2 * kNumMfmaVariants) return CUBLAS_STATUS_INVALID_VALUE;
-  const MfmaVariant &v = kMfmaVariants[plan.variant % kNumMfmaVariants];
+  if (plan.variant >= (uint32_t)kNumMfmaVariants) return CUBLAS_STATUS_INVALID_VALUE;
+  const MfmaVariant &v = kMfmaVariants[plan.variant];
   const int np = plan.swapped ? l.g.N : l.g.M, nq = plan.swapped ? l.g.M : l.g.N;
   prm.tiles_p = (np + v.bp - 1) / v.bp;
   prm.tiles_q = (nq + v.bq - 1) / v.bq;

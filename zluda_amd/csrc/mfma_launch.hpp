@@ -3,27 +3,32 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
-#include "kernels/gemm_mfma.hpp"
+#include "kernels/gemm_mfma_pipe.hpp"
 #include "planner.hpp"
 
 namespace zluda_amd {
 
-// plan.variant: 0..3 = kMfmaVariants[v] with register staging, 4..7 = same tiles with
-// direct-to-LDS loads.
+// plan.variant indexes kMfmaVariants (planner.hpp); the template arguments below restate that table.
 template <int KIND, int FQ, int FP>
 inline uint32_t launch_mfma_variant(const MfmaParams &prm, const zluda_gemm_plan &plan, hipStream_t s) {
   dim3 grid(plan.grid_x, plan.grid_y, 1);
+#define ZLUDA_MFMA_CASE(V, BP, BQ, WP, WQ, BKB, NS)                                                        \
+  case V:                                                                                                  \
+    static_assert(kMfmaVariants[V].bp == BP && kMfmaVariants[V].bq == BQ && kMfmaVariants[V].wp == WP &&   \
+                  kMfmaVariants[V].wq == WQ && kMfmaVariants[V].bkb == BKB && kMfmaVariants[V].stages == NS, \
+                  "variant table mismatch");                                                               \
+    hipLaunchKernelGGL((gemm_mfma_pipe_kernel<KIND, FQ, FP, BP, BQ, WP, WQ, BKB, NS>), grid,               \
+                       dim3(WP * WQ * 64), 0, s, prm);                                                     \
+    break;
   switch (plan.variant) {
-  case 0: hipLaunchKernelGGL((gemm_mfma_kernel<KIND, FQ, FP, 256, 256, 2, 2, 0>), grid, dim3(256), 0, s, prm); break;
-  case 1: hipLaunchKernelGGL((gemm_mfma_kernel<KIND, FQ, FP, 128, 128, 2, 2, 0>), grid, dim3(256), 0, s, prm); break;
-  case 2: hipLaunchKernelGGL((gemm_mfma_kernel<KIND, FQ, FP, 256, 128, 2, 2, 0>), grid, dim3(256), 0, s, prm); break;
-  case 3: hipLaunchKernelGGL((gemm_mfma_kernel<KIND, FQ, FP, 256, 256, 2, 4, 0>), grid, dim3(512), 0, s, prm); break;
-  case 4: hipLaunchKernelGGL((gemm_mfma_kernel<KIND, FQ, FP, 256, 256, 2, 2, 1>), grid, dim3(256), 0, s, prm); break;
-  case 5: hipLaunchKernelGGL((gemm_mfma_kernel<KIND, FQ, FP, 128, 128, 2, 2, 1>), grid, dim3(256), 0, s, prm); break;
-  case 6: hipLaunchKernelGGL((gemm_mfma_kernel<KIND, FQ, FP, 256, 128, 2, 2, 1>), grid, dim3(256), 0, s, prm); break;
-  case 7: hipLaunchKernelGGL((gemm_mfma_kernel<KIND, FQ, FP, 256, 256, 2, 4, 1>), grid, dim3(512), 0, s, prm); break;
+    ZLUDA_MFMA_CASE(0, 256, 256, 2, 4, 128, 2)
+    ZLUDA_MFMA_CASE(1, 256, 256, 2, 2, 128, 2)
+    ZLUDA_MFMA_CASE(2, 256, 128, 2, 2, 128, 2)
+    ZLUDA_MFMA_CASE(3, 128, 128, 2, 2, 128, 2)
+    ZLUDA_MFMA_CASE(4, 128, 128, 2, 2, 64, 4)
   default: return CUBLAS_STATUS_INVALID_VALUE;
   }
+#undef ZLUDA_MFMA_CASE
   return CUBLAS_STATUS_SUCCESS;
 }
 

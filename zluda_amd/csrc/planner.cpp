@@ -233,7 +233,7 @@ static uint32_t ceil_div(uint32_t a, uint32_t b) { return (a + b - 1) / b; }
 
 static void fill_mfma_plan(const Lowered &l, int variant, uint32_t cus, zluda_gemm_plan *plan) {
   const GemmArgs &g = l.g;
-  const MfmaVariant &v = kMfmaVariants[variant % kNumMfmaVariants];
+  const MfmaVariant &v = kMfmaVariants[variant];
   const bool swapped = g.d_si != 1;  // row-major D: compute D^T
   const uint32_t np = swapped ? g.N : g.M, nq = swapped ? g.M : g.N;
   const uint32_t tp = ceil_div(np, v.bp), tq = ceil_div(nq, v.bq);
@@ -241,7 +241,7 @@ static void fill_mfma_plan(const Lowered &l, int variant, uint32_t cus, zluda_ge
   plan->swapped = swapped;
   plan->grid_x = tp * tq; plan->grid_y = g.batch; plan->grid_z = 1;
   plan->block = v.wp * v.wq * 64;
-  const uint32_t lds = 2u * (v.bp + v.bq) * 128u;
+  const uint32_t lds = (uint32_t)v.stages * (v.bp + v.bq) * (v.bkb + (l.g.a_type == CUDA_R_4F_E2M1 ? v.bkb / 16 : 0));
   const uint32_t per_cu = std::max(1u, std::min(160u * 1024u / lds, 2048u / plan->block));
   plan->waves = (float)plan->grid_x * plan->grid_y / (float)(cus * per_cu);
   plan->workspace = 0;
@@ -257,7 +257,7 @@ static int pick_mfma_variant(const Lowered &l, uint32_t cus) {
   // the biggest tile that still gives (nearly) every CU a workgroup
   if (tiles(0) * 4 >= (uint64_t)cus * 3) return 0;
   if (tiles(2) * 4 >= (uint64_t)cus * 3) return 2;
-  return 1;
+  return 3;
 }
 
 static void fill_decode_plan(const Lowered &l, int variant, uint32_t cus, zluda_gemm_plan *plan) {
@@ -319,7 +319,7 @@ extern "C" uint32_t zluda_gemm_plan_problem(const zluda_gemm_problem *p, uint32_
     break;
   case ZLUDA_KERNEL_MFMA_I8: case ZLUDA_KERNEL_MFMA_F8: case ZLUDA_KERNEL_MFMA_MXF4: {
     int v = forced_variant >= 0 ? forced_variant : pick_mfma_variant(l, cu_count);
-    if (v >= 2 * kNumMfmaVariants) return CUBLAS_STATUS_INVALID_VALUE;
+    if (v >= kNumMfmaVariants) return CUBLAS_STATUS_INVALID_VALUE;
     fill_mfma_plan(l, v, cu_count, plan);
     break;
   }

@@ -6,13 +6,15 @@
 
 namespace zluda_amd {
 
-// MFMA tile configurations (index = plan.variant for the MFMA families)
-struct MfmaVariant { int bp, bq, wp, wq; };
+// MFMA tile configurations (index = plan.variant for the MFMA families): workgroup tile bp x bq,
+// wp x wq waves, `bkb` bytes of K per LDS stage, `stages` LDS stages
+struct MfmaVariant { int bp, bq, wp, wq, bkb, stages; };
 constexpr MfmaVariant kMfmaVariants[] = {
-    {256, 256, 2, 2},  // 0: 4 waves, 128x128 per wave
-    {128, 128, 2, 2},  // 1: 4 waves, 64x64 per wave
-    {256, 128, 2, 2},  // 2: 4 waves, 128x64 per wave
-    {256, 256, 2, 4},  // 3: 8 waves, 128x64 per wave
+    {256, 256, 2, 4, 128, 2},  // 0: 8 waves, 128x64 per wave
+    {256, 256, 2, 2, 128, 2},  // 1: 4 waves, 128x128 per wave
+    {256, 128, 2, 2, 128, 2},  // 2: 4 waves, 128x64 per wave
+    {128, 128, 2, 2, 128, 2},  // 3: 4 waves, 64x64 per wave, two workgroups per CU
+    {128, 128, 2, 2, 64, 4},   // 4: same tile, half-line stages, deeper ring (short K)
 };
 constexpr int kNumMfmaVariants = sizeof(kMfmaVariants) / sizeof(kMfmaVariants[0]);
 
