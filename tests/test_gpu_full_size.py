@@ -47,7 +47,7 @@ def slab_check(gpu_api, spec, seed, slabs, rows=64, **kw):
 
 
 def test_config4_fp8_8192_gelu_bias(gpu_api):
-    spec = dict(a_type=K.CUDA_R_8F_E4M3, b_type=K.CUDA_R_8F_E4M3, d_type=K.CUDA_R_16BF,
+    spec = dict(a_type=K.CUDA_R_8F_E4M3, b_type=K.CUDA_R_8F_E4M3, d_type=K.CUDA_R_16BF, c_type=K.CUDA_R_16BF,
                 compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F, transa=1, m=8192, n=8192, k=8192,
                 epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS, bias_type=K.CUDA_R_16BF, with_scalar_scales=True,
                 alpha=1.0, scale_range=(0.1, 0.12), bias_std=0.5)
@@ -56,7 +56,7 @@ def test_config4_fp8_8192_gelu_bias(gpu_api):
 
 
 def test_config5_mxfp4_8192_batch4(gpu_api):
-    spec = dict(a_type=K.CUDA_R_4F_E2M1, b_type=K.CUDA_R_4F_E2M1, d_type=K.CUDA_R_16BF,
+    spec = dict(a_type=K.CUDA_R_4F_E2M1, b_type=K.CUDA_R_4F_E2M1, d_type=K.CUDA_R_16BF, c_type=K.CUDA_R_16BF,
                 compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F, transa=1, m=8192, n=8192, k=8192,
                 batch=4, a_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_VEC32_UE8M0,
                 b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_VEC32_UE8M0, alpha=1.0)
