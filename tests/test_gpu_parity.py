@@ -136,6 +136,29 @@ def test_decode_two_token_blocks_and_long_k(gpu_api, variant):
     check(gpu_api, dict(DECODE, m=400, n=17, k=9280), 101, K.ZLUDA_KERNEL_DECODE_W8A8, variant, int_dist="normal")   # several chunks
 
 
+STREAM = {4: (8, 8), 5: (8, 16), 6: (8, 28), 7: (4, 8), 8: (8, 12), 9: (8, 24), 10: (4, 4), 11: (8, 20), 12: (4, 28),
+          13: (4, 12), 14: (4, 20)}
+
+
+@pytest.mark.parametrize("variant", sorted(STREAM))
+def test_decode_stream_variants(gpu_api, variant, monkeypatch):
+    """weights streamed through LDS: every K the variant table serves, ragged row ranges (row count
+    neither a multiple of 16 nor of the grid), several 16-row blocks per workgroup, 1..32 tokens"""
+    nw, steps = STREAM[variant]
+    k = nw * steps * 64
+    check(gpu_api, dict(DECODE, m=1000, n=16, k=k), 120 + variant, K.ZLUDA_KERNEL_DECODE_W8A8, variant, int_dist="normal")
+    monkeypatch.setenv("ZLUDA_DECODE_GRID", "7")      # 142.86 rows per workgroup: 9 blocks, the last partial
+    check(gpu_api, dict(DECODE, m=1000, n=5, k=k, lda=k + 64), 140 + variant, K.ZLUDA_KERNEL_DECODE_W8A8, variant, int_dist="normal")
+    if steps <= 12:
+        check(gpu_api, dict(DECODE, m=333, n=29, k=k), 160 + variant, K.ZLUDA_KERNEL_DECODE_W8A8, variant, int_dist="normal")
+        check(gpu_api, dict(I8, m=333, n=32, k=k, with_c=True), 180 + variant, K.ZLUDA_KERNEL_DECODE_W8A8, variant)
+
+
+def test_decode_config3_shape_takes_the_stream_kernel(gpu_api):
+    st_spec = dict(DECODE, m=14336, n=16, k=4096)
+    check(gpu_api, st_spec, 2, expect_kernel=K.ZLUDA_KERNEL_DECODE_W8A8, int_dist="normal")
+
+
 def test_decode_tokens_along_m_and_int32_out(gpu_api):
     # row-major activations [tokens][K] x weights^T: tokens are rows of D
     spec = dict(I8F, transa=0, transb=1, order_a=1, order_b=1, order_c=1, order_d=1, m=16, n=2048, k=4096,

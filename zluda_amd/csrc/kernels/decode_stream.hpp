@@ -1,0 +1,198 @@
+// Skinny (<= 32 tokens) W8A8 decode GEMM, streaming form: the weights go from HBM straight into LDS
+// in whole cache lines and are re-read from LDS in the MFMA operand layout.
+//
+//   W : R rows x K int8, K-contiguous (read exactly once)     X : T <= 32 rows x K int8
+//   out(r, t) = sum_k W[r][k] * X[t][k]     int32, then the fused float / integer epilogue
+//
+// Why LDS: v_mfma_i32_16x16x64_i8 wants lane l to hold 16 K-bytes of row l%16, so a 128-bit global
+// load in that layout touches 16 rows x 64 bytes: half a cache line per row.  Measured on MI355X,
+// reading the 58.7 MB of a 14336 x 4096 weight matrix with that pattern takes 15 us against 10 us
+// for a flat read.  Here one buffer_load_dwordx4 ... lds instruction copies 4 rows x 256 contiguous
+// bytes, occupies no VGPRs while in flight, and the ds_read_b128 that follows is free to use any
+// layout.
+//
+// Work split: workgroup w owns the contiguous rows [w*R/G, (w+1)*R/G) (balanced to one row across
+// the grid, whatever R is) and walks them in blocks of 16.  K is split across the NW waves of the
+// workgroup: wave v streams bytes [v*SPW*64, (v+1)*SPW*64) of every row and keeps the matching
+// activation fragments in registers for the whole kernel.  A wave's data path is private: it fills
+// its own LDS ring (2 slots of 16 rows x 256 bytes) and only it reads them back, so the only
+// workgroup barrier is the one in front of the cross-wave reduction of a finished 16-row block.
+// A slot is refilled as soon as its fragments are in registers, so every wave always has 4-8 KiB in
+// flight (64-128 KiB per CU with 16 resident waves).
+//
+// LDS slot layout: row rho (0..15) x 16 chunks of 16 bytes; logical chunk c of row rho sits at
+// position c ^ rho, which makes both the linear 1 KiB LDS fill of one DMA instruction and the
+// 16-rows-same-chunk fragment reads bank-conflict free.
+#pragma once
+#include "decode_w8a8.hpp"
+
+namespace zluda_amd {
+
+// Workgroup barrier that orders LDS traffic only: __syncthreads() would also wait for every vector
+// memory operation of the wave, i.e. drain the weight stream at each block.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// 32-bit LDS address of a __shared__ object (the address-space cast only exists in the device pass)
+__device__ __forceinline__ uint32_t lds_addr(const void *p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void *)p;
+#else
+  (void)p;
+  return 0;
+#endif
+}
+
+// ds_read_b128 issued behind the compiler's back.  A C++ read of LDS that the compiler cannot prove
+// disjoint from an LDS DMA still in flight gets an s_waitcnt vmcnt(0) in front of it; in a loop that
+// is every read, which would serialise the weight stream.  The caller orders these reads itself
+// (frags_ready below).
+__device__ __forceinline__ v4i lds_read16_unordered(uint32_t addr) {
+  v4i r;
+  asm volatile("ds_read_b128 %0, %1" : "=v"(r) : "v"(addr));
+  return r;
+}
+// Waits for the unordered reads and ties the four fragments to the wait, so that nothing that uses
+// them can be scheduled in front of it.  The memory clobber keeps the refill of the slot behind it.
+__device__ __forceinline__ void frags_ready(v4i &a, v4i &b, v4i &c, v4i &d) {
+  asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d)::"memory");
+}
+
+template <int NW, int SPW, int NB>
+__global__ __launch_bounds__(NW * 64) void decode_stream_kernel(DecodeParams prm) {
+  constexpr int SEG = 256;             // bytes of one row per unit
+  constexpr int Q = SPW * 64 / SEG;    // units per 16-row block (and wave)
+  constexpr int NSLOT = 2;
+  constexpr int UNIT_V4 = 16 * SEG / 16;
+  constexpr int NDMA = 16 * SEG / 1024;  // DMA instructions per unit
+  static_assert(SPW % 4 == 0, "a wave's K slice is a whole number of 256-byte units");
+  __shared__ v4i ring[NW][NSLOT][UNIT_V4];
+  constexpr int RBUF = NB == 1 ? 2 : 1;  // two token blocks: one reduction buffer (LDS for two workgroups per CU)
+  __shared__ v4i red[RBUF][NW][NB][64];
+
+  const GemmArgs &g = prm.g;
+  const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int l16 = lane & 15, g4 = lane >> 4;
+  const int bt = blockIdx.y;
+
+  const int R = prm.swapped ? g.N : g.M, T = prm.swapped ? g.M : g.N;
+  const uint8_t *Wg = (const uint8_t *)(prm.swapped ? g.B : g.A) + (prm.swapped ? g.b_sb : g.a_sb) * bt;
+  const uint8_t *Xg = (const uint8_t *)(prm.swapped ? g.A : g.B) + (prm.swapped ? g.a_sb : g.b_sb) * bt;
+  const int ldw = (int)(prm.swapped ? g.b_sj : g.a_si);
+  const int64_t ldx = prm.swapped ? g.a_si : g.b_sj;
+
+  // rows of this workgroup
+  const int r0 = (int)((int64_t)blockIdx.x * R / gridDim.x);
+  const int r1 = (int)((int64_t)(blockIdx.x + 1) * R / gridDim.x);
+  const int nblk = (r1 - r0 + 15) >> 4;
+  const int kwave = wave * (SPW * 64);
+
+  // 2 GiB raw buffer window over W: an offset with bit 31 set is out of range, reads as zero and
+  // moves no data (rows past r1 of the last block, and the units issued past the last block)
+  const __amdgpu_buffer_rsrc_t rsW = __builtin_amdgcn_make_buffer_rsrc((void *)Wg, 0, 0x80000000, 0x00020000);
+  // DMA instruction i of a unit: lane -> row rho = 4*i + lane/16 at position lane%16, i.e. logical
+  // chunk (lane%16) ^ rho
+  int dma_off[NDMA];
+#pragma unroll
+  for (int i = 0; i < NDMA; i++) {
+    const int rho = 4 * i + g4;
+    dma_off[i] = rho * ldw + ((l16 ^ rho) << 4) + kwave;
+  }
+  auto issue_unit = [&](int blk, int q, int slot) {
+    const int rb = r0 + blk * 16;
+    v4i *dst = &ring[wave][slot][0];
+#pragma unroll
+    for (int i = 0; i < NDMA; i++) {
+      const int rho = 4 * i + g4;
+      const int oob = rb + rho < r1 ? 0 : (int)0x80000000;
+      lds_dma16(rsW, dst + i * 64, (rb * ldw + q * SEG + dma_off[i]) | oob, 0);
+    }
+  };
+
+  // activation fragments of this wave's K slice: lane -> token l16 (+16 per block), 16 bytes at
+  // K = kwave + step*64 + g4*16
+  v4i xf[NB][SPW];
+#pragma unroll
+  for (int nb = 0; nb < NB; nb++) {
+    const uint8_t *xr = Xg + (int64_t)min(nb * 16 + l16, T - 1) * ldx + kwave + g4 * 16;
+#pragma unroll
+    for (int s = 0; s < SPW; s++) xf[nb][s] = *(const v4i *)(xr + s * 64);
+  }
+
+  // prologue: the first NSLOT units
+  {
+    int blk = 0, q = 0;
+#pragma unroll
+    for (int u = 0; u < NSLOT; u++) {
+      issue_unit(blk, q, u);
+      if (++q == Q) { q = 0; blk++; }
+    }
+  }
+
+  // Pin the wait for the activation loads here, in straight-line code where the compiler can count
+  // (they are older than the NSLOT units just issued).  Left to its own devices it waits at their
+  // first use inside the loop, where all it can prove is vmcnt(0): that drains the stream per block.
+#pragma unroll
+  for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+    for (int s = 0; s < SPW; s++) asm volatile("" : "+v"(xf[nb][s]));
+
+  Epilogue ep(g, bt);
+  const uint32_t ring_base = lds_addr(&ring[wave][0][l16 * 16]);  // this lane's row in slot 0
+  int slot = 0;
+  // (block, unit) that the next refill fetches: NSLOT units ahead of the one being consumed
+  int fblk = NSLOT / Q, fq = NSLOT % Q;
+
+  for (int blk = 0; blk < nblk; blk++) {
+    v4i acc[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) acc[nb] = v4i{0, 0, 0, 0};
+#pragma unroll
+    for (int q = 0; q < Q; q++) {
+      // the oldest unit in flight has landed (the younger NSLOT-1 may still be on their way)
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NSLOT - 1) * NDMA) : "memory");
+      const uint32_t src = ring_base + slot * (UNIT_V4 * 16);
+      v4i w[4];
+#pragma unroll
+      for (int s = 0; s < 4; s++) w[s] = lds_read16_unordered(src + (((s * 4 + g4) ^ l16) << 4));
+      // the fragments are in registers before the slot is overwritten
+      frags_ready(w[0], w[1], w[2], w[3]);
+      issue_unit(fblk, fq, slot);
+      if (++fq == Q) { fq = 0; fblk++; }
+      slot ^= 1;
+#pragma unroll
+      for (int s = 0; s < 4; s++)
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++)
+          acc[nb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[s], xf[nb][q * 4 + s], acc[nb], 0, 0, 0);
+    }
+
+    // cross-wave reduction of the finished block; the reducing wave rotates
+    const int buf = RBUF == 2 ? (blk & 1) : 0;
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) red[buf][wave][nb][lane] = acc[nb];
+    lds_barrier();
+    if (wave == blk % NW) {
+#pragma unroll
+      for (int nb = 0; nb < NB; nb++) {
+        v4i s = red[buf][0][nb][lane];
+#pragma unroll
+        for (int w2 = 1; w2 < NW; w2++) s += red[buf][w2][nb][lane];
+        const int tok = nb * 16 + l16;
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+          const int row = r0 + blk * 16 + g4 * 4 + v;
+          if (row < r1 && tok < T) {
+            const int i = prm.swapped ? tok : row, j = prm.swapped ? row : tok;
+            if (g.int_scale) ep.store_int(i, j, s[v]);
+            else ep.store_f(i, j, (float)s[v]);
+          }
+        }
+      }
+    }
+    if (RBUF == 1) lds_barrier();  // the single buffer is rewritten by the next block
+  }
+  // the zero-fill units issued past the last block still target this workgroup's LDS
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
+} // namespace zluda_amd

@@ -2,6 +2,7 @@
 // and enqueues it on the caller's stream.  Only the HIP runtime is used (hipLaunchKernelGGL).
 #include <hip/hip_runtime.h>
 
+#include "kernels/decode_stream.hpp"
 #include "kernels/decode_w8a8.hpp"
 #include "kernels/gemm_generic.hpp"
 #include "mfma_launch.hpp"
@@ -48,7 +49,21 @@ void launch_decode_variant(const DecodeParams &prm, const zluda_gemm_plan &plan,
   }
 }
 
+template <int NW, int SPW>
+uint32_t launch_decode_stream(const DecodeParams &prm, const zluda_gemm_plan &plan, int nb, hipStream_t s) {
+  dim3 grid(plan.grid_x, plan.grid_y, 1), block(NW * 64);
+  if (nb == 1) {
+    hipLaunchKernelGGL((decode_stream_kernel<NW, SPW, 1>), grid, block, 0, s, prm);
+  } else if constexpr (SPW <= kDecodeStreamMaxStepsTwoBlocks) {
+    hipLaunchKernelGGL((decode_stream_kernel<NW, SPW, 2>), grid, block, 0, s, prm);
+  } else {
+    return CUBLAS_STATUS_NOT_SUPPORTED;
+  }
+  return CUBLAS_STATUS_SUCCESS;
+}
+
 uint32_t launch_decode(const Lowered &l, const zluda_gemm_plan &plan, hipStream_t s) {
+  if (plan.variant >= (uint32_t)kNumDecodeVariants) return CUBLAS_STATUS_INVALID_VALUE;
   const DecodeVariant &v = kDecodeVariants[plan.variant];
   DecodeParams prm;
   prm.g = l.g;
@@ -59,6 +74,32 @@ uint32_t launch_decode(const Lowered &l, const zluda_gemm_plan &plan, hipStream_
   prm.nchunks = (prm.spw + v.steps - 1) / v.steps;
   const bool full = l.g.K == v.nw * v.steps * 64;
   const int nb = T <= 16 ? 1 : 2;
+  if (v.stream) {
+    // the kernel addresses W through one 2 GiB buffer window and assumes K == nw * steps * 64
+    const int64_t rows = plan.swapped ? l.g.N : l.g.M, ldw = plan.swapped ? l.g.b_sj : l.g.a_si;
+    if (!full || rows * ldw >= 0x7fffffffll || plan.grid_x > (uint32_t)((rows + 15) / 16))
+      return CUBLAS_STATUS_NOT_SUPPORTED;
+    switch (plan.variant) {
+#define ZLUDA_STREAM_CASE(V, NW, SPW)                                                         \
+  case V:                                                                                     \
+    static_assert(kDecodeVariants[V].nw == NW && kDecodeVariants[V].steps == SPW && kDecodeVariants[V].stream, \
+                  "variant table mismatch");                                                  \
+    return launch_decode_stream<NW, SPW>(prm, plan, nb, s);
+      ZLUDA_STREAM_CASE(4, 8, 8)
+      ZLUDA_STREAM_CASE(5, 8, 16)
+      ZLUDA_STREAM_CASE(6, 8, 28)
+      ZLUDA_STREAM_CASE(7, 4, 8)
+      ZLUDA_STREAM_CASE(8, 8, 12)
+      ZLUDA_STREAM_CASE(9, 8, 24)
+      ZLUDA_STREAM_CASE(10, 4, 4)
+      ZLUDA_STREAM_CASE(11, 8, 20)
+      ZLUDA_STREAM_CASE(12, 4, 28)
+      ZLUDA_STREAM_CASE(13, 4, 12)
+      ZLUDA_STREAM_CASE(14, 4, 20)
+#undef ZLUDA_STREAM_CASE
+    default: return CUBLAS_STATUS_INVALID_VALUE;
+    }
+  }
   if (nb == 2 && v.steps > 8) return CUBLAS_STATUS_NOT_SUPPORTED;
   switch (plan.variant) {
   case 0: launch_decode_variant<8, 8>(prm, plan, nb, full, s); break;

@@ -260,6 +260,17 @@ static int pick_mfma_variant(const Lowered &l, uint32_t cus) {
   return 3;
 }
 
+static bool decode_variant_ok(const Lowered &l, int variant) {
+  const GemmArgs &g = l.g;
+  const DecodeVariant &v = kDecodeVariants[variant];
+  const int T = std::min(g.M, g.N);
+  if (!v.stream) return T <= 16 || v.steps <= 8;  // two token blocks double the fragment registers
+  const bool swapped = g.M < g.N;
+  const int64_t rows = swapped ? g.N : g.M, ldw = swapped ? g.b_sj : g.a_si;
+  return g.K == v.nw * v.steps * 64 && rows * ldw < 0x7fffffffll &&
+         (T <= 16 || v.steps <= kDecodeStreamMaxStepsTwoBlocks);
+}
+
 static void fill_decode_plan(const Lowered &l, int variant, uint32_t cus, zluda_gemm_plan *plan) {
   const GemmArgs &g = l.g;
   const DecodeVariant &v = kDecodeVariants[variant];
@@ -267,7 +278,9 @@ static void fill_decode_plan(const Lowered &l, int variant, uint32_t cus, zluda_
   const uint32_t rows = swapped ? g.N : g.M;
   const uint32_t nrb = ceil_div(rows, 16);
   const uint32_t resident = cus * (v.nw == 8 ? 2 : 4);
-  uint32_t grid = nrb <= resident ? nrb : ceil_div(nrb, ceil_div(nrb, resident));
+  uint32_t grid;
+  if (v.stream) grid = std::min(nrb, resident);  // contiguous, balanced row ranges
+  else grid = nrb <= resident ? nrb : ceil_div(nrb, ceil_div(nrb, resident));
   if (const char *e = getenv("ZLUDA_DECODE_GRID")) { int x = atoi(e); if (x > 0) grid = std::min<uint32_t>(x, nrb); }
   plan->variant = variant;
   plan->swapped = swapped;
@@ -278,9 +291,11 @@ static void fill_decode_plan(const Lowered &l, int variant, uint32_t cus, zluda_
 }
 
 static int pick_decode_variant(const Lowered &l) {
-  const int K = l.g.K, T = std::min(l.g.M, l.g.N);
+  const int K = l.g.K;
   for (int v = 0; v < kNumDecodeVariants; v++)
-    if (K == kDecodeVariants[v].nw * kDecodeVariants[v].steps * 64 && (T <= 16 || kDecodeVariants[v].steps <= 8))
+    if (kDecodeVariants[v].stream && decode_variant_ok(l, v)) return v;
+  for (int v = 0; v < kNumDecodeVariants; v++)
+    if (!kDecodeVariants[v].stream && K == kDecodeVariants[v].nw * kDecodeVariants[v].steps * 64 && decode_variant_ok(l, v))
       return v;
   return 0;
 }
@@ -326,7 +341,7 @@ extern "C" uint32_t zluda_gemm_plan_problem(const zluda_gemm_problem *p, uint32_
   case ZLUDA_KERNEL_DECODE_W8A8: {
     int v = forced_variant >= 0 ? forced_variant : pick_decode_variant(l);
     if (v >= kNumDecodeVariants) return CUBLAS_STATUS_INVALID_VALUE;
-    if (std::min(l.g.M, l.g.N) > 16 && kDecodeVariants[v].steps > 8) return CUBLAS_STATUS_NOT_SUPPORTED;
+    if (!decode_variant_ok(l, v)) return CUBLAS_STATUS_NOT_SUPPORTED;
     fill_decode_plan(l, v, cu_count, plan);
     break;
   }

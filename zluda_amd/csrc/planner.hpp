@@ -18,15 +18,29 @@ constexpr MfmaVariant kMfmaVariants[] = {
 };
 constexpr int kNumMfmaVariants = sizeof(kMfmaVariants) / sizeof(kMfmaVariants[0]);
 
-// decode configurations (index = plan.variant for ZLUDA_KERNEL_DECODE_W8A8)
-struct DecodeVariant { int nw, steps; };
+// decode configurations (index = plan.variant for ZLUDA_KERNEL_DECODE_W8A8).
+// stream == 0: weights loaded straight into registers, any K (grid-stride over 16-row blocks).
+// stream == 1: weights streamed through LDS in whole cache lines; K must equal nw * steps * 64.
+struct DecodeVariant { int nw, steps, stream; };
 constexpr DecodeVariant kDecodeVariants[] = {
-    {8, 8},   // 0: 8 waves x 512 B of K
-    {8, 16},  // 1: 8 waves x 1024 B
-    {4, 16},  // 2: 4 waves x 1024 B
-    {4, 8},   // 3: 4 waves x 512 B
+    {8, 8, 0},   // 0: 8 waves x 512 B of K per pass
+    {8, 16, 0},  // 1: 8 waves x 1024 B
+    {4, 16, 0},  // 2: 4 waves x 1024 B
+    {4, 8, 0},   // 3: 4 waves x 512 B
+    {8, 8, 1},   // 4: K = 4096
+    {8, 16, 1},  // 5: K = 8192
+    {8, 28, 1},  // 6: K = 14336
+    {4, 8, 1},   // 7: K = 2048
+    {8, 12, 1},  // 8: K = 6144
+    {8, 24, 1},  // 9: K = 12288
+    {4, 4, 1},   // 10: K = 1024
+    {8, 20, 1},  // 11: K = 10240
+    {4, 28, 1},  // 12: K = 7168
+    {4, 12, 1},  // 13: K = 3072
+    {4, 20, 1},  // 14: K = 5120
 };
 constexpr int kNumDecodeVariants = sizeof(kDecodeVariants) / sizeof(kDecodeVariants[0]);
+constexpr int kDecodeStreamMaxStepsTwoBlocks = 12;  // 17..32 tokens double the activation registers
 
 struct Lowered {
   GemmArgs g;
