@@ -143,6 +143,29 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(DecodeParams prm
   int fblk = NSLOT / Q, fq = NSLOT % Q;
 
   for (int blk = 0; blk < nblk; blk++) {
+    const bool reducer = wave == blk % NW;  // the reducing wave rotates
+    // The reducer fetches the epilogue factors of its outputs while the block streams: by the time
+    // the weights have gone through the MFMAs they have long arrived, and the epilogue is left
+    // without a memory round trip of its own.  Raw loads only: converting or combining them here
+    // would make the compiler wait for each load on the spot.
+    float f_al[NB][4], f_sa[NB][4], f_sb[NB][4], f_be[NB][4];
+    uint32_t f_bias[NB][4];
+    auto prefetch_factors = [&]() {
+      if (reducer && !g.int_scale) {
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+          for (int v = 0; v < 4; v++) {
+            const int row = min(r0 + blk * 16 + g4 * 4 + v, r1 - 1), tok = min(nb * 16 + l16, T - 1);
+            const int i = prm.swapped ? tok : row, j = prm.swapped ? row : tok;
+            f_al[nb][v] = ep.alpha_v ? ep.alpha_v[i] : ep.alpha_s;
+            f_sa[nb][v] = ep.sa_v ? ep.sa_v[i] : ep.sa_s;
+            f_sb[nb][v] = ep.sb_v ? ep.sb_v[j] : ep.sb_s;
+            f_be[nb][v] = ep.beta_v ? ep.beta_v[i] : ep.beta_s;
+            f_bias[nb][v] = ep.bias_raw(i);
+          }
+      }
+    };
     v4i acc[NB];
 #pragma unroll
     for (int nb = 0; nb < NB; nb++) acc[nb] = v4i{0, 0, 0, 0};
@@ -156,6 +179,10 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(DecodeParams prm
       for (int s = 0; s < 4; s++) w[s] = lds_read16_unordered(src + (((s * 4 + g4) ^ l16) << 4));
       // the fragments are in registers before the slot is overwritten
       frags_ready(w[0], w[1], w[2], w[3]);
+      // Issued between the wait for this unit and the refill: the counted wait of the next unit
+      // (everything but the NDMA youngest operations) then covers these loads without waiting for
+      // anything younger than the unit it needs.
+      if (q == 0) prefetch_factors();
       issue_unit(fblk, fq, slot);
       if (++fq == Q) { fq = 0; fblk++; }
       slot ^= 1;
@@ -166,12 +193,12 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(DecodeParams prm
           acc[nb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[s], xf[nb][q * 4 + s], acc[nb], 0, 0, 0);
     }
 
-    // cross-wave reduction of the finished block; the reducing wave rotates
+    // cross-wave reduction of the finished block
     const int buf = RBUF == 2 ? (blk & 1) : 0;
 #pragma unroll
     for (int nb = 0; nb < NB; nb++) red[buf][wave][nb][lane] = acc[nb];
     lds_barrier();
-    if (wave == blk % NW) {
+    if (reducer) {
 #pragma unroll
       for (int nb = 0; nb < NB; nb++) {
         v4i s = red[buf][0][nb][lane];
@@ -184,7 +211,7 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(DecodeParams prm
           if (row < r1 && tok < T) {
             const int i = prm.swapped ? tok : row, j = prm.swapped ? row : tok;
             if (g.int_scale) ep.store_int(i, j, s[v]);
-            else ep.store_f(i, j, (float)s[v]);
+            else ep.store_f(i, j, (float)s[v], f_al[nb][v] * f_sa[nb][v], f_sb[nb][v], f_be[nb][v], ep.bias_from_raw(f_bias[nb][v]));
           }
         }
       }

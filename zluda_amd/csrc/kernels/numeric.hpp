@@ -178,6 +178,18 @@ struct Epilogue {
     return g.bias ? load_elem(g.bias, g.bias_type, i + g.bias_sb * bt) : 0.0f;
   }
 
+  // The same bias in two steps, for callers that fetch early and convert late (the planner admits
+  // fp32, fp16 and bf16 bias vectors): the raw storage bits, then their value.
+  __device__ __forceinline__ uint32_t bias_raw(int i) const {
+    if (!g.bias) return 0;
+    const int64_t idx = i + g.bias_sb * bt;
+    return g.bias_type == CUDA_R_32F ? ((const uint32_t *)g.bias)[idx] : (uint32_t)((const uint16_t *)g.bias)[idx];
+  }
+  __device__ __forceinline__ float bias_from_raw(uint32_t raw) const {
+    if (!g.bias) return 0.0f;
+    return g.bias_type == CUDA_R_32F ? bits2f(raw) : g.bias_type == CUDA_R_16F ? dec_f16((uint16_t)raw) : dec_bf16((uint16_t)raw);
+  }
+
   __device__ __forceinline__ float finish(float x) const {
     if (g.act == ACT_RELU) x = x > 0.0f ? x : 0.0f;
     else if (g.act == ACT_GELU) x = gelu_tanh(x);
