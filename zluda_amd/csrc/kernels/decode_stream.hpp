@@ -80,9 +80,12 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(DecodeParams prm
   const int ldw = (int)(prm.swapped ? g.b_sj : g.a_si);
   const int64_t ldx = prm.swapped ? g.a_si : g.b_sj;
 
-  // rows of this workgroup
-  const int r0 = (int)((int64_t)blockIdx.x * R / gridDim.x);
-  const int r1 = (int)((int64_t)(blockIdx.x + 1) * R / gridDim.x);
+  // rows of this workgroup: R = rows_base * grid + rows_rem, the first rows_rem workgroups take one
+  // row more (the split is done on the host: a 64-bit division here would sit in front of the
+  // first load of every wave)
+  const int wg = blockIdx.x;
+  const int r0 = wg * prm.rows_base + min(wg, prm.rows_rem);
+  const int r1 = r0 + prm.rows_base + (wg < prm.rows_rem ? 1 : 0);
   const int nblk = (r1 - r0 + 15) >> 4;
   const int kwave = wave * (SPW * 64);
 
@@ -108,6 +111,16 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(DecodeParams prm
     }
   };
 
+  // prologue: the first NSLOT units, before anything else touches memory
+  {
+    int blk = 0, q = 0;
+#pragma unroll
+    for (int u = 0; u < NSLOT; u++) {
+      issue_unit(blk, q, u);
+      if (++q == Q) { q = 0; blk++; }
+    }
+  }
+
   // activation fragments of this wave's K slice: lane -> token l16 (+16 per block), 16 bytes at
   // K = kwave + step*64 + g4*16
   v4i xf[NB][SPW];
@@ -118,19 +131,10 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(DecodeParams prm
     for (int s = 0; s < SPW; s++) xf[nb][s] = *(const v4i *)(xr + s * 64);
   }
 
-  // prologue: the first NSLOT units
-  {
-    int blk = 0, q = 0;
-#pragma unroll
-    for (int u = 0; u < NSLOT; u++) {
-      issue_unit(blk, q, u);
-      if (++q == Q) { q = 0; blk++; }
-    }
-  }
-
-  // Pin the wait for the activation loads here, in straight-line code where the compiler can count
-  // (they are older than the NSLOT units just issued).  Left to its own devices it waits at their
-  // first use inside the loop, where all it can prove is vmcnt(0): that drains the stream per block.
+  // Pin the wait for the activation loads here, in straight-line code.  Left to its own devices the
+  // compiler waits at their first use inside the loop, where all it can prove is vmcnt(0): that
+  // drains the stream per block.  Here the wait costs nothing: the first units were issued at the
+  // same moment and are needed next.
 #pragma unroll
   for (int nb = 0; nb < NB; nb++)
 #pragma unroll

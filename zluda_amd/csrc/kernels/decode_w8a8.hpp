@@ -22,6 +22,7 @@ struct DecodeParams {
   int32_t swapped;  // 0: W = op(A) (rows i of D), X = op(B) (tokens j);  1: W = op(B)^T, X = op(A)
   int32_t spw;      // MFMA K-steps (64 bytes of K each) per wave
   int32_t nchunks;  // ceil(spw / STEPS)
+  int32_t rows_base, rows_rem;  // stream kernel: rows per workgroup and how many workgroups take one more
 };
 
 template <int NW, int STEPS, int NB, bool FULL>

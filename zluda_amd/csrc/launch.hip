@@ -68,6 +68,7 @@ uint32_t launch_decode(const Lowered &l, const zluda_gemm_plan &plan, hipStream_
   DecodeParams prm;
   prm.g = l.g;
   prm.swapped = plan.swapped;
+  prm.rows_base = prm.rows_rem = 0;
   const int T = plan.swapped ? l.g.M : l.g.N;
   const int ksteps = (l.g.K + 63) / 64;
   prm.spw = (ksteps + v.nw - 1) / v.nw;
@@ -79,6 +80,8 @@ uint32_t launch_decode(const Lowered &l, const zluda_gemm_plan &plan, hipStream_
     const int64_t rows = plan.swapped ? l.g.N : l.g.M, ldw = plan.swapped ? l.g.b_sj : l.g.a_si;
     if (!full || rows * ldw >= 0x7fffffffll || plan.grid_x > (uint32_t)((rows + 15) / 16))
       return CUBLAS_STATUS_NOT_SUPPORTED;
+    prm.rows_base = (int32_t)(rows / plan.grid_x);
+    prm.rows_rem = (int32_t)(rows % plan.grid_x);
     switch (plan.variant) {
 #define ZLUDA_STREAM_CASE(V, NW, SPW)                                                         \
   case V:                                                                                     \
