@@ -33,8 +33,9 @@
  *   - float GEMMs: exact rational arithmetic on tiny shapes, numpy float64 otherwise
  *   - epilogue (alpha vector, outer scales, bias, relu/gelu): scalar formulas in numpy
  * PARITY UNPINNED (no fixture in the reference, no hipBLASLt run possible without a GPU):
- *   - which GELU hipBLASLt applies: the tanh form is restated here; the GPU test suite compares
- *     against hipBLASLt itself on the GPU box
+ *   - which GELU hipBLASLt applies: the tanh form is restated here.  No CPU-side fixture pins it;
+ *     on a GPU box tests/test_gpu_vs_hipblaslt.py tells the tanh and erf forms apart against
+ *     hipBLASLt itself (it applies the tanh form)
  *   - the memory layout of the UE8M0 scale tensors (restated as plain [row][K/32] bytes)
  */
 #include <math.h>
