@@ -54,6 +54,12 @@ WORKLOADS = {
 }
 
 
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
+# script (each counter scaled by what it reads for the 256 MiB copy of --copy-probe: x2.000 and x1.000).
+# The summaries are profiles/<kernel>_<workload>.txt; re-measure after changing a kernel's tiling.
+MEASURED_TRAFFIC = {"c2": 167907166, "i8_8192": 1074794350, "c3": 60376779, "c4": 941560714, "c5": 2248533521}
+
+
 def algorithmic(spec):
     """(ops, bytes) of one call: 2*M*N*K*batch and every operand/result byte exactly once."""
     m, n, k, b = spec["m"], spec["n"], spec["k"], spec.get("batch", 1)
@@ -177,7 +183,7 @@ def run_workload(torch, api, key, steps, warmup, with_hipblaslt):
         "tops": ops / (wall / steps) / 1e12, "gbps": nbytes / (wall / steps) / 1e9,
         "kernel": {"family": call.kernel, "variant": call.variant},
         "roofline": {"bound": bound, "achieved": achieved, "peak": peak, "unit": "GB/s" if bound == "hbm" else "TFLOP/s",
-                     "frac": achieved / peak, "traffic": None, "kernel_ms": per_call * 1e3,
+                     "frac": achieved / peak, "traffic": MEASURED_TRAFFIC.get(key), "kernel_ms": per_call * 1e3,
                      "algorithmic_ops": ops, "algorithmic_bytes": nbytes},
     }
     if with_hipblaslt:
