@@ -57,7 +57,19 @@ __device__ __forceinline__ void frags_ready(v4i &a, v4i &b, v4i &c, v4i &d) {
   asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d)::"memory");
 }
 
-template <int NW, int SPW, int NB>
+// frags_ready for an array of values read with lds_read16_unordered
+template <int N>
+__device__ __forceinline__ void lds_values_ready(v4i (&x)[N]) {
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+  for (int i = 0; i < N; i++) asm volatile("" : "+v"(x[i]));
+}
+
+// FAST: the host has checked that every output leaves through the packed 8-byte store below (float
+// epilogue without C, 16-bit D contiguous along the weight rows, 8-byte aligned, row count a multiple
+// of 4); the element-wise epilogue with all its type dispatch is then not even compiled in, which
+// keeps the code the reducing wave runs between two blocks short.
+template <int NW, int SPW, int NB, bool FAST>
 __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(DecodeParams prm) {
   constexpr int SEG = 256;             // bytes of one row per unit
   constexpr int Q = SPW * 64 / SEG;    // units per 16-row block (and wave)
@@ -80,12 +92,13 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(DecodeParams prm
   const int ldw = (int)(prm.swapped ? g.b_sj : g.a_si);
   const int64_t ldx = prm.swapped ? g.a_si : g.b_sj;
 
-  // rows of this workgroup: R = rows_base * grid + rows_rem, the first rows_rem workgroups take one
-  // row more (the split is done on the host: a 64-bit division here would sit in front of the
-  // first load of every wave)
+  // rows of this workgroup, in quads of 4 rows so that every lane's 4 outputs start on a multiple
+  // of 4: ceil(R / 4) = rows_base * grid + rows_rem quads, the first rows_rem workgroups take one
+  // more (the split is done on the host: a 64-bit division here would sit in front of the first
+  // load of every wave)
   const int wg = blockIdx.x;
-  const int r0 = wg * prm.rows_base + min(wg, prm.rows_rem);
-  const int r1 = r0 + prm.rows_base + (wg < prm.rows_rem ? 1 : 0);
+  const int r0 = 4 * (wg * prm.rows_base + min(wg, prm.rows_rem));
+  const int r1 = min(R, r0 + 4 * (prm.rows_base + (wg < prm.rows_rem ? 1 : 0)));
   const int nblk = (r1 - r0 + 15) >> 4;
   const int kwave = wave * (SPW * 64);
 
@@ -141,6 +154,15 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(DecodeParams prm
     for (int s = 0; s < SPW; s++) asm volatile("" : "+v"(xf[nb][s]));
 
   Epilogue ep(g, bt);
+  // Packed output: a lane's 4 outputs are 4 consecutive weight rows of one token.  When D is 16-bit,
+  // contiguous along the weight rows and suitably aligned, and no C is read, they leave as one
+  // 8-byte store instead of four scattered 2-byte ones.
+  const int64_t d_sr = prm.swapped ? g.d_sj : g.d_si, d_st = prm.swapped ? g.d_si : g.d_sj;
+  const bool packed = FAST || !g.int_scale && (g.d_type == CUDA_R_16BF || g.d_type == CUDA_R_16F) && d_sr == 1 &&
+                      g.beta_mode == SCALAR_VALUE && g.beta_val.f == 0.0f && ((uintptr_t)g.D & 7) == 0 &&
+                      (d_st & 3) == 0 && (g.d_sb & 3) == 0;
+  uint16_t *const Dp = (uint16_t *)g.D + g.d_sb * bt;
+  const uint32_t red_base = lds_addr(&red[0][0][0][lane]);
   const uint32_t ring_base = lds_addr(&ring[wave][0][l16 * 16]);  // this lane's row in slot 0
   int slot = 0;
   // (block, unit) that the next refill fetches: NSLOT units ahead of the one being consumed
@@ -155,7 +177,7 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(DecodeParams prm
     float f_al[NB][4], f_sa[NB][4], f_sb[NB][4], f_be[NB][4];
     uint32_t f_bias[NB][4];
     auto prefetch_factors = [&]() {
-      if (reducer && !g.int_scale) {
+      if (reducer && (FAST || !g.int_scale)) {
 #pragma unroll
         for (int nb = 0; nb < NB; nb++)
 #pragma unroll
@@ -165,7 +187,7 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(DecodeParams prm
             f_al[nb][v] = ep.alpha_v ? ep.alpha_v[i] : ep.alpha_s;
             f_sa[nb][v] = ep.sa_v ? ep.sa_v[i] : ep.sa_s;
             f_sb[nb][v] = ep.sb_v ? ep.sb_v[j] : ep.sb_s;
-            f_be[nb][v] = ep.beta_v ? ep.beta_v[i] : ep.beta_s;
+            if constexpr (!FAST) f_be[nb][v] = ep.beta_v ? ep.beta_v[i] : ep.beta_s;
             f_bias[nb][v] = ep.bias_raw(i);
           }
       }
@@ -187,6 +209,18 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(DecodeParams prm
       // (everything but the NDMA youngest operations) then covers these loads without waiting for
       // anything younger than the unit it needs.
       if (q == 0) prefetch_factors();
+      // One unit later the counted wait above has covered those loads as well.  Telling the compiler
+      // here (where it can count: the loads are older than one refill) keeps it from waiting for
+      // them in the epilogue, where its only safe choice is vmcnt(0), i.e. the units in flight.
+      if (Q > 1 && q == Q - 1 && reducer && (FAST || !g.int_scale)) {
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+          for (int v = 0; v < 4; v++) {
+            asm volatile("" : "+v"(f_al[nb][v]), "+v"(f_sa[nb][v]), "+v"(f_sb[nb][v]), "+v"(f_bias[nb][v]));
+            if constexpr (!FAST) asm volatile("" : "+v"(f_be[nb][v]));
+          }
+      }
       issue_unit(fblk, fq, slot);
       if (++fq == Q) { fq = 0; fblk++; }
       slot ^= 1;
@@ -205,17 +239,43 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(DecodeParams prm
     if (reducer) {
 #pragma unroll
       for (int nb = 0; nb < NB; nb++) {
-        v4i s = red[buf][0][nb][lane];
+        // unordered reads again: a C++ read of LDS would wait for this wave's units in flight
+        v4i part[NW];
 #pragma unroll
-        for (int w2 = 1; w2 < NW; w2++) s += red[buf][w2][nb][lane];
+        for (int w2 = 0; w2 < NW; w2++) part[w2] = lds_read16_unordered(red_base + ((buf * NW + w2) * NB + nb) * 1024);
+        lds_values_ready(part);
+        v4i s = part[0];
+#pragma unroll
+        for (int w2 = 1; w2 < NW; w2++) s += part[w2];
         const int tok = nb * 16 + l16;
+        const int row0 = r0 + blk * 16 + g4 * 4;
+        if (FAST || (packed && row0 + 3 < r1)) {
+          if (tok < T && row0 < r1) {  // FAST: r1 is a multiple of 4, a quad is inside or outside
+            float y[4];
 #pragma unroll
-        for (int v = 0; v < 4; v++) {
-          const int row = r0 + blk * 16 + g4 * 4 + v;
-          if (row < r1 && tok < T) {
-            const int i = prm.swapped ? tok : row, j = prm.swapped ? row : tok;
-            if (g.int_scale) ep.store_int(i, j, s[v]);
-            else ep.store_f(i, j, (float)s[v], f_al[nb][v] * f_sa[nb][v], f_sb[nb][v], f_be[nb][v], ep.bias_from_raw(f_bias[nb][v]));
+            for (int v = 0; v < 4; v++)
+              y[v] = ep.finish(((f_al[nb][v] * f_sa[nb][v]) * f_sb[nb][v]) * (float)s[v] + ep.bias_from_raw(f_bias[nb][v]));
+            uint2 pk;
+            if (g.d_type == CUDA_R_16BF) {
+              pk.x = (uint32_t)enc_bf16(y[0]) | ((uint32_t)enc_bf16(y[1]) << 16);
+              pk.y = (uint32_t)enc_bf16(y[2]) | ((uint32_t)enc_bf16(y[3]) << 16);
+            } else {
+              pk.x = (uint32_t)enc_f16(y[0]) | ((uint32_t)enc_f16(y[1]) << 16);
+              pk.y = (uint32_t)enc_f16(y[2]) | ((uint32_t)enc_f16(y[3]) << 16);
+            }
+            *(uint2 *)(Dp + (int64_t)tok * d_st + row0) = pk;
+          }
+          continue;
+        }
+        if constexpr (!FAST) {
+#pragma unroll
+          for (int v = 0; v < 4; v++) {
+            const int row = row0 + v;
+            if (row < r1 && tok < T) {
+              const int i = prm.swapped ? tok : row, j = prm.swapped ? row : tok;
+              if (g.int_scale) ep.store_int(i, j, s[v]);
+              else ep.store_f(i, j, (float)s[v], f_al[nb][v] * f_sa[nb][v], f_sb[nb][v], f_be[nb][v], ep.bias_from_raw(f_bias[nb][v]));
+            }
           }
         }
       }

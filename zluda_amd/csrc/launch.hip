@@ -49,13 +49,25 @@ void launch_decode_variant(const DecodeParams &prm, const zluda_gemm_plan &plan,
   }
 }
 
+// every output of the problem can leave through the packed 8-byte store of decode_stream_kernel
+bool decode_packed_output(const GemmArgs &g, bool swapped) {
+  const int64_t d_sr = swapped ? g.d_sj : g.d_si, d_st = swapped ? g.d_si : g.d_sj;
+  const int rows = swapped ? g.N : g.M;
+  return !g.int_scale && (g.d_type == CUDA_R_16BF || g.d_type == CUDA_R_16F) && d_sr == 1 &&
+         g.beta_mode == SCALAR_VALUE && g.beta_val.f == 0.0f && ((uintptr_t)g.D & 7) == 0 && (d_st & 3) == 0 &&
+         (g.d_sb & 3) == 0 && (rows & 3) == 0;
+}
+
 template <int NW, int SPW>
 uint32_t launch_decode_stream(const DecodeParams &prm, const zluda_gemm_plan &plan, int nb, hipStream_t s) {
   dim3 grid(plan.grid_x, plan.grid_y, 1), block(NW * 64);
+  const bool fast = decode_packed_output(prm.g, prm.swapped != 0);
   if (nb == 1) {
-    hipLaunchKernelGGL((decode_stream_kernel<NW, SPW, 1>), grid, block, 0, s, prm);
+    if (fast) hipLaunchKernelGGL((decode_stream_kernel<NW, SPW, 1, true>), grid, block, 0, s, prm);
+    else hipLaunchKernelGGL((decode_stream_kernel<NW, SPW, 1, false>), grid, block, 0, s, prm);
   } else if constexpr (SPW <= kDecodeStreamMaxStepsTwoBlocks) {
-    hipLaunchKernelGGL((decode_stream_kernel<NW, SPW, 2>), grid, block, 0, s, prm);
+    if (fast) hipLaunchKernelGGL((decode_stream_kernel<NW, SPW, 2, true>), grid, block, 0, s, prm);
+    else hipLaunchKernelGGL((decode_stream_kernel<NW, SPW, 2, false>), grid, block, 0, s, prm);
   } else {
     return CUBLAS_STATUS_NOT_SUPPORTED;
   }
@@ -80,8 +92,9 @@ uint32_t launch_decode(const Lowered &l, const zluda_gemm_plan &plan, hipStream_
     const int64_t rows = plan.swapped ? l.g.N : l.g.M, ldw = plan.swapped ? l.g.b_sj : l.g.a_si;
     if (!full || rows * ldw >= 0x7fffffffll || plan.grid_x > (uint32_t)((rows + 15) / 16))
       return CUBLAS_STATUS_NOT_SUPPORTED;
-    prm.rows_base = (int32_t)(rows / plan.grid_x);
-    prm.rows_rem = (int32_t)(rows % plan.grid_x);
+    const int64_t quads = (rows + 3) / 4;  // the kernel splits the rows in quads of 4
+    prm.rows_base = (int32_t)(quads / plan.grid_x);
+    prm.rows_rem = (int32_t)(quads % plan.grid_x);
     switch (plan.variant) {
 #define ZLUDA_STREAM_CASE(V, NW, SPW)                                                         \
   case V:                                                                                     \
