@@ -280,7 +280,8 @@ __device__ __forceinline__ void mfma_store_tile_f(const MfmaParams &prm, AccV (&
         const int ql = 8 * (vv >> 2) + 4 * gsel + (vv & 3);
         stage[ql * SROW + b * 32 + lr] = to_bits(acc[a][b][h * 8 + vv]);
       }
-    __syncthreads();
+    // no workgroup barrier: the staging rows belong to this wave alone, and LDS executes the
+    // writes and reads of one wave in program order
 #pragma unroll 2
     for (int it = 0; it < ITER; it++) {
       const v4i raw = *(const v4i *)&stage[it * RPI * SROW + read_off];
@@ -316,7 +317,6 @@ __device__ __forceinline__ void mfma_store_tile_f(const MfmaParams &prm, AccV (&
         __builtin_amdgcn_raw_buffer_store_b64(pk, rs, voff, soff, 0);
       }
     }
-    __syncthreads();
   };
   static_for<TQ * 2>(do_pass);
 }

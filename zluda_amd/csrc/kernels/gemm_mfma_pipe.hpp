@@ -35,15 +35,6 @@ __device__ __forceinline__ void wait_vmcnt_barrier() {
   asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
 }
 
-// 4 bytes per lane from a buffer straight into LDS (buffer_load_dword ... lds): lane l lands at byte
-// l*4 of the 256-byte block starting at the wave-uniform `lds_dst`.
-__device__ __forceinline__ void lds_dma4(__amdgpu_buffer_rsrc_t rs, void *lds_dst, int voff, int soff) {
-#if defined(__HIP_DEVICE_COMPILE__)
-  __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void *)lds_dst, 4, voff,
-                                           soff, 0, 0);
-#endif
-}
-
 template <int KIND, int FQ, int FP, int BP, int BQ, int WP, int WQ, int BKB_, int NSTAGE>
 __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams prm) {
   constexpr int NT = WP * WQ * 64;
@@ -51,27 +42,35 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
   constexpr int RPW = 64 / CPR;                // rows filled by one wave DMA instruction
   constexpr int RPP = (NT / 64) * RPW;         // rows filled per DMA pass of the workgroup
   constexpr int LP = BP / RPP, LQ = BQ / RPP;  // data DMA instructions per thread, stage and operand
-  constexpr int SDW = KIND == KIND_MXF4 ? BKB_ / 64 : 0;  // scale dwords per row and stage (4 blocks each)
-  constexpr int SROWS = (BP + BQ + NT - 1) / NT * NT;  // rows of a scale plane (padded to whole passes)
-  constexpr int LS = SDW * SROWS / NT;         // scale DMA instructions per thread and stage
+  // MX block scales travel in chunks of 32 scale bytes per tile row (1024 K elements = CH stages),
+  // double buffered behind the data stages.  One DMA instruction copies 32 rows x 32 bytes; every
+  // wave issues LS of them per stage (the instructions a chunk does not need go out of range and
+  // move nothing, so that the vmcnt bookkeeping is the same in every stage).
+  constexpr bool MX = KIND == KIND_MXF4;
+  constexpr int SB = BKB_ / 16;                // scale bytes per row and stage
+  constexpr int CH = 32 / SB;                  // stages per scale chunk
+  constexpr int SPARTS = (BP + BQ) / 32;       // DMA instructions per chunk
+  constexpr int NWV = NT / 64;
+  constexpr int LS = MX ? (SPARTS + NWV * (CH - NSTAGE) - 1) / (NWV * (CH - NSTAGE)) : 0;
+  constexpr int PRO_S = MX ? (SPARTS + NWV - 1) / NWV : 0;  // per wave, for the first chunk
+  constexpr int CHUNK_V4 = MX ? (BP + BQ) * 2 : 0;
   constexpr int NLOAD = LP + LQ + LS;          // vmcnt units per stage
   constexpr int WTP = BP / WP, WTQ = BQ / WQ;
   constexpr int TP = WTP / 32, TQ = WTQ / 32;
   constexpr int KS = BKB_ / (KIND == KIND_F8 ? 64 : 32);  // MFMA sub-steps per stage
   constexpr int SPT = (KS & 1) ? 2 : 1;        // stages per loop trip (fragment roles must realign)
-  // one stage in 16-byte units: P rows, Q rows, then (MXFP4) SDW planes of one scale dword per row
-  constexpr int STAGE_V4 = (BP + BQ) * CPR + SDW * SROWS / 4;
+  constexpr int STAGE_V4 = (BP + BQ) * CPR;    // one stage in 16-byte units: P rows, then Q rows
   static_assert(BKB_ == 64 || BKB_ == 128, "row segments are half or whole cache lines");
   static_assert(BP % RPP == 0 && BQ % RPP == 0 && RPP % 32 == 0, "tile / copy-pass mismatch");
-  static_assert(KIND != KIND_MXF4 || (BP % 64 == 0 && BQ % 64 == 0), "scale rows are copied 64 per wave instruction");
+  static_assert(!MX || (BP % 32 == 0 && BQ % 32 == 0 && CH > NSTAGE), "scale chunks: 32 rows per instruction, fetched NSTAGE stages early");
   static_assert((NSTAGE - 1) * NLOAD < 64, "vmcnt range");
-  static_assert(NSTAGE * STAGE_V4 * 16 <= 160 * 1024, "LDS capacity");
+  static_assert((NSTAGE * STAGE_V4 + 2 * CHUNK_V4) * 16 <= 160 * 1024, "LDS capacity");
   using acc_v = typename std::conditional<KIND == KIND_I8, v16i, v16f>::type;
   using frag_v = typename std::conditional<KIND == KIND_I8, v4i, v8i>::type;
   struct Frags { frag_v p[TP], q[TQ]; };
   struct Scales { int p[TP], q[TQ]; };  // MX scale dwords of one stage (one per MFMA tile row set)
 
-  __shared__ v4i lds[NSTAGE * STAGE_V4];
+  __shared__ v4i lds[NSTAGE * STAGE_V4 + 2 * CHUNK_V4];
 
   const GemmArgs &g = prm.g;
   // the wave index is uniform by construction; readfirstlane tells the compiler (LDS DMA bases and
@@ -123,25 +122,40 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
   const int tail_bytes = Kbytes - (KT - 1) * BKB_;
   const int oob_last = dcg * 16 < tail_bytes ? 0 : (int)0x80000000;
 
-  // MX block scales: stage kt covers BKB/16 K blocks of a row = SDW aligned dwords of the
-  // [row][K/32] scale tensor, kept as SDW planes of one dword per tile row (P rows, then Q rows).
-  // DMA instruction i of a thread copies plane i % SDW for tile row t + NT * (i / SDW).
-  __amdgpu_buffer_rsrc_t rsS[LS > 0 ? LS : 1];
-  int voffS[LS > 0 ? LS : 1];
-  if constexpr (KIND == KIND_MXF4) {
-    const int KB = g.K / 32;
+  // MX block scales: the [row][K/32] byte tensors of both operands, through buffer windows of
+  // their exact size (a chunk that runs past the end of a row reads the next row, past the end of
+  // the tensor zeros; neither is ever used).  Chunk c, instruction `part`: lane l -> tile row
+  // 32*part + l/2, 16-byte half l%2 of that row's bytes [32c, 32c+32).
+  const int KB = g.K / 32;
+  __amdgpu_buffer_rsrc_t rsSP = rsP, rsSQ = rsQ;
+  int srowP = 0, srowQ = 0;
+  if constexpr (MX) {
     const uint8_t *Ps = (const uint8_t *)(prm.swapped ? g.b_scale : g.a_scale) + (int64_t)bt * NP * KB;
     const uint8_t *Qs = (const uint8_t *)(prm.swapped ? g.a_scale : g.b_scale) + (int64_t)bt * NQ * KB;
-#pragma unroll
-    for (int i = 0; i < LS; i++) {
-      // BP is a multiple of 64: a wave never straddles P and Q.  Rows past BP + BQ (padding of the
-      // last pass) copy a clamped row into the plane's padding.
-      const int r = t + NT * (i / SDW);
-      const bool isq = r >= BP;
-      rsS[i] = __builtin_amdgcn_make_buffer_rsrc((void *)(isq ? Qs : Ps), 0, 0x80000000, 0x00020000);
-      voffS[i] = (isq ? min(q0 + r - BP, NQ - 1) : min(p0 + r, NP - 1)) * KB + (i % SDW) * 4;
-    }
+    rsSP = __builtin_amdgcn_make_buffer_rsrc((void *)Ps, 0, NP * KB, 0x00020000);
+    rsSQ = __builtin_amdgcn_make_buffer_rsrc((void *)Qs, 0, NQ * KB, 0x00020000);
+    srowP = p0 + (lane >> 1);
+    srowQ = q0 - BP + (lane >> 1);
   }
+  // An out-of-range instruction still writes (zeros) to LDS.  The spare ones (part >= SPARTS) are
+  // pointed at the 1 KiB of data slot `so` that this same wave fills with its very next data
+  // instruction: loads of one wave complete in order, so the zeros never survive.
+  auto issue_scale_part = [&](int c, int part, int so) {
+    if constexpr (MX) {
+      const bool spare = part >= SPARTS;
+      const bool isq = part >= BP / 32;  // wave-uniform: a part never straddles P and Q
+      const int row = isq ? min(srowQ + 32 * part, NQ - 1) : min(srowP + 32 * part, NP - 1);
+      const int oob = (!spare && c * 32 < KB) ? 0 : (int)0x80000000;
+      v4i *dst = spare ? &lds[so + wave * RPW * CPR] : &lds[NSTAGE * STAGE_V4 + (c & 1) * CHUNK_V4 + part * 64];
+      lds_dma16(isq ? rsSQ : rsSP, dst, (row * KB + c * 32 + (lane & 1) * 16) | oob, 0);
+    }
+  };
+  // the LS scale instructions a wave issues in front of the data that refills slot `so` during
+  // (consumer) stage kt: its share of chunk kt/CH + 1
+  auto issue_scales_for = [&](int kt, int so) {
+#pragma unroll
+    for (int i = 0; i < LS; i++) issue_scale_part(kt / CH + 1, ((kt % CH) * LS + i) * NWV + wave, so);
+  };
 
   // stage kt -> LDS slot at 16-byte offset `so`; kt >= KT is a padding stage that is zero-filled
   auto issue_stage = [&](int kt, int so) {
@@ -153,13 +167,6 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
 #pragma unroll
     for (int i = 0; i < LQ; i++)
       lds_dma16(rsQ, base + (BP + wave * RPW + RPP * i) * CPR, voffQ[i] | oob, kt * BKB_);
-    if constexpr (KIND == KIND_MXF4) {
-      int *sbase = (int *)(base + (BP + BQ) * CPR);
-#pragma unroll
-      for (int i = 0; i < LS; i++)
-        lds_dma4(rsS[i], sbase + (i % SDW) * SROWS + wave * 64 + NT * (i / SDW), voffS[i],
-                 min(kt, KT - 1) * (SDW * 4));
-    }
   };
 
   // fragment (and MX scale) loads of sub-step ks of the stage in the LDS slot at offset `so`
@@ -198,17 +205,18 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
       }
     }
   };
-  // MX scales of the stage in the slot at `so`.  The K blocks of lane group gsel are
-  // gsel*KS .. gsel*KS+KS-1 of the stage:  KS == 2: one plane, bytes gsel*2 + ks;
-  // KS == 4: plane gsel, byte ks.  After the shift, op_sel = ks selects the byte in both cases.
-  auto load_scales = [&](int so, Scales &sc) {
-    if constexpr (KIND == KIND_MXF4) {
-      const int *Sl = (const int *)&lds[so + (BP + BQ) * CPR] + (KS == 4 ? gsel * SROWS : 0);
+  // MX scales of stage kt.  The K blocks of lane group gsel are gsel*KS .. gsel*KS+KS-1 of the
+  // stage:  KS == 2: bytes gsel*2 + ks of the stage's one dword;  KS == 4: dword gsel, byte ks.
+  // After the shift, op_sel = ks selects the byte in both cases.
+  auto load_scales = [&](int kt, Scales &sc) {
+    if constexpr (MX) {
+      const int j = kt % CH;
+      const int *Sl = (const int *)&lds[NSTAGE * STAGE_V4 + ((kt / CH) & 1) * CHUNK_V4] + (KS == 4 ? 2 * j + gsel : j);
       const int sh = KS == 2 ? gsel * 16 : 0;
 #pragma unroll
-      for (int i = 0; i < TP; i++) sc.p[i] = Sl[wp * WTP + i * 32 + lr] >> sh;
+      for (int i = 0; i < TP; i++) sc.p[i] = Sl[(wp * WTP + i * 32 + lr) * 8] >> sh;
 #pragma unroll
-      for (int i = 0; i < TQ; i++) sc.q[i] = Sl[BP + wq * WTQ + i * 32 + lr] >> sh;
+      for (int i = 0; i < TQ; i++) sc.q[i] = Sl[(BP + wq * WTQ + i * 32 + lr) * 8] >> sh;
     }
   };
 
@@ -239,8 +247,16 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
   };
 
   // ---- prologue: stages 0 .. NSTAGE-1 in flight, stage 0 landed -----------------------------------
+  // (the first scale chunk goes first: the counted wait for stage 0 then covers it; every data stage
+  // is preceded by its LS scale instructions, here as in the loop, so that the counts are uniform)
 #pragma unroll
-  for (int s = 0; s < NSTAGE; s++) issue_stage(s, s * STAGE_V4);
+  for (int i = 0; i < PRO_S; i++) issue_scale_part(0, i * NWV + wave, 0);
+#pragma unroll
+  for (int s = 0; s < NSTAGE; s++) {
+#pragma unroll
+    for (int i = 0; i < LS; i++) issue_scale_part(0, SPARTS, s * STAGE_V4);  // spare: moves nothing
+    issue_stage(s, s * STAGE_V4);
+  }
   wait_vmcnt_barrier<(NSTAGE - 1) * NLOAD>();
 
   Frags fa, fb;
@@ -268,7 +284,8 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
         // reads first: the compiler cannot prove that the DMA (an LDS write) and these reads hit
         // different slots, so whatever comes second in the source stays second in the schedule
         load_frags(so_next, std::integral_constant<int, 0>{}, nxt);
-        load_scales(so_next, sc_nxt);
+        load_scales(kt + 1, sc_nxt);
+        issue_scales_for(kt, so);
         issue_stage(kt + NSTAGE, so);
       }
       mfma_all(use, sc_cur, s_c);

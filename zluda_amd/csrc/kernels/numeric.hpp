@@ -82,7 +82,8 @@ __device__ __forceinline__ float gelu_tanh(float x) {
   // 0.5 x (1 + tanh(u)) == x * sigmoid(2u) ; u = sqrt(2/pi) (x + 0.044715 x^3)
   const float k0 = 0.7978845608028654f, k1 = 0.044715f;
   float u = k0 * (x + k1 * x * x * x);
-  return x / (1.0f + __expf(-2.0f * u));
+  // rcp instead of a full-precision division: 1 ulp, far inside the 16-bit outputs this feeds
+  return x * __builtin_amdgcn_rcpf(1.0f + __expf(-2.0f * u));
 }
 
 // element loads for C / bias / generic operands

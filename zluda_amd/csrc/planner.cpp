@@ -241,7 +241,8 @@ static void fill_mfma_plan(const Lowered &l, int variant, uint32_t cus, zluda_ge
   plan->swapped = swapped;
   plan->grid_x = tp * tq; plan->grid_y = g.batch; plan->grid_z = 1;
   plan->block = v.wp * v.wq * 64;
-  const uint32_t lds = (uint32_t)v.stages * (v.bp + v.bq) * (v.bkb + (l.g.a_type == CUDA_R_4F_E2M1 ? v.bkb / 16 : 0));
+  // data stages, plus two chunks of 32 scale bytes per tile row for MXFP4
+  const uint32_t lds = (uint32_t)v.stages * (v.bp + v.bq) * v.bkb + (l.g.a_type == CUDA_R_4F_E2M1 ? 64u * (v.bp + v.bq) : 0u);
   const uint32_t per_cu = std::max(1u, std::min(160u * 1024u / lds, 2048u / plan->block));
   plan->waves = (float)plan->grid_x * plan->grid_y / (float)(cus * per_cu);
   plan->workspace = 0;
