@@ -308,17 +308,73 @@ __device__ __forceinline__ void mfma_store_tile_f(const MfmaParams &prm, AccV (&
       } else {
         v2i pk;
         if constexpr (DT == 0) {
-          pk[0] = (int)((uint32_t)enc_bf16(x[0]) | ((uint32_t)enc_bf16(x[1]) << 16));
-          pk[1] = (int)((uint32_t)enc_bf16(x[2]) | ((uint32_t)enc_bf16(x[3]) << 16));
+          pk[0] = (int)pack_bf16x2(x[0], x[1]);
+          pk[1] = (int)pack_bf16x2(x[2], x[3]);
         } else {
-          pk[0] = (int)((uint32_t)enc_f16(x[0]) | ((uint32_t)enc_f16(x[1]) << 16));
-          pk[1] = (int)((uint32_t)enc_f16(x[2]) | ((uint32_t)enc_f16(x[3]) << 16));
+          pk[0] = (int)pack_f16x2(x[0], x[1]);
+          pk[1] = (int)pack_f16x2(x[2], x[3]);
         }
         __builtin_amdgcn_raw_buffer_store_b64(pk, rs, voff, soff, 0);
       }
     }
   };
   static_for<TQ * 2>(do_pass);
+}
+
+// Fast path 3: the same float epilogue when nothing varies along Q (no per-column scale vector for a
+// column-major D, no per-row vectors for a row-major one), D bf16 or f16: straight from the
+// accumulator registers, no LDS.  Lane (lr, gsel) holds element (column lr, row 8*(v/4)+4*gsel+v%4)
+// of each 32x32 tile; rows 2k and 2k+1 are paired: after one DPP swap with the neighbouring lane the
+// even lane owns columns (lr, lr+1) of row 2k and the odd lane columns (lr-1, lr) of row 2k+1, so
+// every lane stores one dword of two 16-bit results and a store instruction writes four 64-byte row
+// segments.
+template <int KIND, int WP, int WQ, int WTP, int WTQ, int ACT, int DT, class AccV>
+__device__ __forceinline__ void mfma_store_tile_f16_direct(const MfmaParams &prm, AccV (&acc)[WTQ / 32][WTP / 32],
+                                                           int p0, int q0, int bt) {
+  static_assert(DT == 0 || DT == 1, "16-bit outputs");
+  constexpr int TP = WTP / 32, TQ = WTQ / 32;
+  const GemmArgs &g = prm.g;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wp = wave % WP, wq = wave / WP;
+  const int lr = lane & 31, gsel = lane >> 5, odd = lane & 1;
+  Epilogue ep(g, bt);
+  const bool swp = prm.swapped != 0;
+  const float q_scale = swp ? ep.row_scale(0) : ep.col_scale(0);
+  float p_scale[TP], p_bias[TP];
+#pragma unroll
+  for (int b = 0; b < TP; b++) {
+    const int pi = p0 + wp * WTP + b * 32 + lr;
+    p_scale[b] = swp ? ep.col_scale(pi) : ep.row_scale(pi);
+    p_bias[b] = swp ? 0.0f : ep.bias_at(pi);
+  }
+  const int d_sq = (int)(swp ? g.d_si : g.d_sj);  // < 2^22 (checked by the dispatcher)
+  char *Dw = (char *)g.D + (g.d_sb * bt + (int64_t)(q0 + wq * WTQ) * d_sq + (p0 + wp * WTP)) * 2;
+  const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)Dw, 0, 0xFFFFFFFF, 0x00020000);
+  const int voff = ((4 * gsel + odd) * d_sq + (lr & ~1)) * 2;
+  auto value = [&](float accf, int b) {
+    float y = (swp ? q_scale * p_scale[b] : p_scale[b] * q_scale) * accf + p_bias[b];
+    if (ACT == ACT_RELU) y = y > 0.0f ? y : 0.0f;
+    else if (ACT == ACT_GELU) y = gelu_tanh(y);
+    return y * ep.sd;
+  };
+#pragma unroll
+  for (int a = 0; a < TQ; a++)
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+      const int soff = (a * 32 + 8 * (k >> 1) + 2 * (k & 1)) * d_sq * 2;  // uniform: row 2k of tile a
+#pragma unroll
+      for (int b = 0; b < TP; b++) {
+        const float fa = KIND == KIND_I8 ? (float)to_bits(acc[a][b][2 * k]) : bits2f((uint32_t)to_bits(acc[a][b][2 * k]));
+        const float fb = KIND == KIND_I8 ? (float)to_bits(acc[a][b][2 * k + 1]) : bits2f((uint32_t)to_bits(acc[a][b][2 * k + 1]));
+        const float ya = value(fa, b), yb = value(fb, b);
+        // even lanes keep row 2k and need the neighbour's row-2k value; odd lanes the other way round
+        const float mine = odd ? yb : ya, give = odd ? ya : yb;
+        const float got = bits2f((uint32_t)__builtin_amdgcn_mov_dpp((int)f2bits(give), 0xB1 /* quad_perm [1,0,3,2] */, 0xF, 0xF, true));
+        const float lo = odd ? got : mine, hi = odd ? mine : got;
+        const uint32_t pk = DT == 0 ? pack_bf16x2(lo, hi) : pack_f16x2(lo, hi);
+        __builtin_amdgcn_raw_buffer_store_b32((int)pk, rs, voff, soff + b * 64, 0);
+      }
+    }
 }
 
 // Epilogue dispatch: the fast paths for full tiles of the common configurations, the general path
@@ -346,6 +402,23 @@ __device__ __forceinline__ void mfma_store_tile(const MfmaParams &prm, AccV (&ac
   if (!g.int_scale && full && aligned && g.beta_mode == SCALAR_VALUE && g.beta_val.f == 0.0f &&
       (g.d_type == CUDA_R_16BF || g.d_type == CUDA_R_16F || g.d_type == CUDA_R_32F)) {
     const int dt = g.d_type == CUDA_R_16BF ? 0 : (g.d_type == CUDA_R_16F ? 1 : 2);
+    // vectors that run along Q need the LDS-staged form
+    const bool q_vec = swp ? (g.alpha_mode == VECTOR_DEV || g.a_scale_mode == SCALE_OUTER_VEC || g.bias != nullptr)
+                           : (g.b_scale_mode == SCALE_OUTER_VEC);
+    if (!q_vec && dt != 2) {
+#define ZLUDA_EPI_D(ACT_, DT_) mfma_store_tile_f16_direct<KIND, WP, WQ, WTP, WTQ, ACT_, DT_>(prm, acc, p0, q0, bt)
+      if (dt == 0) {
+        if (g.act == ACT_GELU) ZLUDA_EPI_D(ACT_GELU, 0);
+        else if (g.act == ACT_RELU) ZLUDA_EPI_D(ACT_RELU, 0);
+        else ZLUDA_EPI_D(ACT_NONE, 0);
+      } else {
+        if (g.act == ACT_GELU) ZLUDA_EPI_D(ACT_GELU, 1);
+        else if (g.act == ACT_RELU) ZLUDA_EPI_D(ACT_RELU, 1);
+        else ZLUDA_EPI_D(ACT_NONE, 1);
+      }
+#undef ZLUDA_EPI_D
+      return;
+    }
 #define ZLUDA_EPI(ACT_, DT_) mfma_store_tile_f<KIND, WP, WQ, WTP, WTQ, ACT_, DT_>(prm, acc, lds_words, p0, q0, bt)
     if (dt == 0) {
       if (g.act == ACT_GELU) ZLUDA_EPI(ACT_GELU, 0);

@@ -15,11 +15,17 @@ __device__ __forceinline__ float bits2f(uint32_t u) { return __builtin_bit_cast(
 __device__ __forceinline__ uint32_t f2bits(float f) { return __builtin_bit_cast(uint32_t, f); }
 
 __device__ __forceinline__ float dec_bf16(uint16_t v) { return bits2f((uint32_t)v << 16); }
-__device__ __forceinline__ uint16_t enc_bf16(float f) {
-  uint32_t u = f2bits(f);
-  if (f != f) return (uint16_t)((u >> 16) | 0x40);
-  u += 0x7FFFu + ((u >> 16) & 1u);
-  return (uint16_t)(u >> 16);
+// fp32 -> bf16, round to nearest even: gfx950 has the conversion in hardware (v_cvt_pk_bf16_f32)
+__device__ __forceinline__ uint16_t enc_bf16(float f) { return __builtin_bit_cast(uint16_t, (__bf16)f); }
+// two at once: `lo` in bits 0..15
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  const f32x2 v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+}
+__device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi) {
+  return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)lo) | ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)hi) << 16);
 }
 __device__ __forceinline__ float dec_f16(uint16_t v) {
   return (float)__builtin_bit_cast(_Float16, v);
@@ -80,10 +86,12 @@ __device__ __forceinline__ uint8_t enc_e5m2(float f) { return enc_small<5, 2, 15
 
 __device__ __forceinline__ float gelu_tanh(float x) {
   // 0.5 x (1 + tanh(u)) == x * sigmoid(2u) ; u = sqrt(2/pi) (x + 0.044715 x^3)
-  const float k0 = 0.7978845608028654f, k1 = 0.044715f;
-  float u = k0 * (x + k1 * x * x * x);
-  // rcp instead of a full-precision division: 1 ulp, far inside the 16-bit outputs this feeds
-  return x * __builtin_amdgcn_rcpf(1.0f + __expf(-2.0f * u));
+  // exp(-2u) = exp2(x * (c0 + c1 x^2)) with c0 = -2 sqrt(2/pi) log2(e), c1 = 0.044715 c0: two FMAs, one
+  // v_exp_f32, one v_rcp_f32 (1 ulp each, far inside the 16-bit outputs this feeds).  x -> -inf gives
+  // exp2 = +inf, rcp = 0, result -0; x -> +inf gives exp2 = 0, result x.
+  const float c0 = -2.0f * 0.7978845608028654f * 1.4426950408889634f, c1 = 0.044715f * c0;
+  const float z = x * __builtin_fmaf(x * x, c1, c0);
+  return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(z));
 }
 
 // element loads for C / bias / generic operands
