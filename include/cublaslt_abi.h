@@ -315,7 +315,8 @@ cublasStatus_t cublasLtMatmulAlgoGetHeuristic(
     cublasLtMatmulPreference_t preference, int requestedAlgoCount,
     cublasLtMatmulHeuristicResult_t *heuristicResultsArray, int *returnAlgoCount);
 
-/* [n/s] */
+/* [ext] algorithm enumeration (cuda_macros/src/cublaslt.rs:397-421): an algorithm id is one of the
+ * kernel families of zluda_gemm_launch.h that can run the type combination */
 cublasStatus_t cublasLtMatmulAlgoGetIds(cublasLtHandle_t lightHandle,
                                         cublasComputeType_t computeType, cudaDataType_t scaleType,
                                         cudaDataType_t Atype, cudaDataType_t Btype,
@@ -334,7 +335,8 @@ cublasStatus_t cublasLtMatmulAlgoCheck(cublasLtHandle_t lightHandle,
                                        cublasLtMatrixLayout_t Cdesc, cublasLtMatrixLayout_t Ddesc,
                                        const cublasLtMatmulAlgo_t *algo,
                                        cublasLtMatmulHeuristicResult_t *result);
-/* [n/s] */
+/* [ext] capabilities and configuration of an algo token (cuda_macros/src/cublaslt.rs:470-518).  The
+ * tile variant is CUBLASLT_ALGO_CONFIG_CUSTOM_OPTION: 0 = planner's choice, v + 1 = variant v. */
 cublasStatus_t cublasLtMatmulAlgoCapGetAttribute(const cublasLtMatmulAlgo_t *algo,
                                                  cublasLtMatmulAlgoCapAttributes_t attr, void *buf,
                                                  size_t sizeInBytes, size_t *sizeWritten);

@@ -94,6 +94,10 @@ uint32_t zluda_gemm_plan_problem(const zluda_gemm_problem *p, uint32_t forced_ke
 uint32_t zluda_gemm_launch(const zluda_gemm_problem *p, const zluda_gemm_plan *plan,
                            void *stream);
 
+/* Number of tile configurations (plan.variant values) of a kernel family; 1 for the generic kernel,
+ * 0 for an unknown family. */
+uint32_t zluda_gemm_variant_count(uint32_t kernel);
+
 /* Number of compute units of the current HIP device (0 when no device is usable). */
 uint32_t zluda_gemm_device_cu_count(void);
 

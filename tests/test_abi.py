@@ -163,7 +163,6 @@ def test_unimplemented_exports_return_not_supported(api):
     assert api.cublasLtLoggerOpenFile(b"/dev/null") == NS
     assert api.cublasLtHeuristicsCacheSetCapacity(8) == NS
     assert api.cublasLtMatrixTransformDescCreate(C.byref(C.c_void_p()), abi.CUDA_R_32F) == NS
-    assert api.cublasLtMatmulAlgoInit(None, 0, 0, 0, 0, 0, 0, 0, None) == NS
     assert api.cublasLtMatmulPreferenceInit_internal(None, 64) == NS
     assert api.cublasLtDisableCpuInstructionsSetMask(1) == 0
     assert api.cublasLtDisableCpuInstructionsSetMask(0) == 1
@@ -221,3 +220,67 @@ def test_matmul_without_device_fails_loudly(api):
     st = call.run(one, C.addressof(buf), C.addressof(buf), zero, None, C.addressof(buf))
     assert st == abi.CUBLAS_STATUS_NOT_INITIALIZED
     call.close()
+
+
+def test_algorithm_enumeration_and_configuration(api):
+    """cublasLtMatmulAlgoGetIds / AlgoInit / AlgoCapGetAttribute / AlgoConfig{Set,Get}Attribute
+    (cuda_macros/src/cublaslt.rs:397-518): ids are kernel families, the tile variant is CUSTOM_OPTION"""
+    h = C.c_void_p()
+    assert api.cublasLtCreate(C.byref(h)) == 0
+    ids = (C.c_int * 8)()
+    n = C.c_int(0)
+    i8 = (abi.CUBLAS_COMPUTE_32I, abi.CUDA_R_32I, abi.CUDA_R_8I, abi.CUDA_R_8I, abi.CUDA_R_32I, abi.CUDA_R_32I)
+    assert api.cublasLtMatmulAlgoGetIds(h, *i8, 8, ids, C.byref(n)) == 0
+    assert sorted(ids[:n.value]) == [abi.ZLUDA_KERNEL_GENERIC, abi.ZLUDA_KERNEL_MFMA_I8, abi.ZLUDA_KERNEL_DECODE_W8A8]
+    assert api.cublasLtMatmulAlgoGetIds(h, *i8, 1, ids, C.byref(n)) == 0 and n.value == 1
+    f8 = (abi.CUBLAS_COMPUTE_32F, abi.CUDA_R_32F, abi.CUDA_R_8F_E4M3, abi.CUDA_R_8F_E4M3, abi.CUDA_R_16BF, abi.CUDA_R_16BF)
+    assert api.cublasLtMatmulAlgoGetIds(h, *f8, 8, ids, C.byref(n)) == 0
+    assert sorted(ids[:n.value]) == [abi.ZLUDA_KERNEL_GENERIC, abi.ZLUDA_KERNEL_MFMA_F8]
+    f4 = (abi.CUBLAS_COMPUTE_32F, abi.CUDA_R_32F, abi.CUDA_R_4F_E2M1, abi.CUDA_R_4F_E2M1, abi.CUDA_R_16BF, abi.CUDA_R_16BF)
+    assert api.cublasLtMatmulAlgoGetIds(h, *f4, 8, ids, C.byref(n)) == 0
+    assert sorted(ids[:n.value]) == [abi.ZLUDA_KERNEL_GENERIC, abi.ZLUDA_KERNEL_MFMA_MXF4]
+    # a combination nothing runs
+    bad = (abi.CUBLAS_COMPUTE_32I, abi.CUDA_R_32I, abi.CUDA_R_32F, abi.CUDA_R_32F, abi.CUDA_R_32I, abi.CUDA_R_32I)
+    assert api.cublasLtMatmulAlgoGetIds(h, *bad, 8, ids, C.byref(n)) == 0 and n.value == 0
+
+    algo = abi.cublasLtMatmulAlgo_t()
+    assert api.cublasLtMatmulAlgoInit(h, *i8, abi.ZLUDA_KERNEL_MFMA_F8, C.byref(algo)) == IV
+    assert api.cublasLtMatmulAlgoInit(h, *i8, abi.ZLUDA_KERNEL_MFMA_I8, C.byref(algo)) == 0
+    assert api.cublasLtMatmulAlgoInit(None, *i8, abi.ZLUDA_KERNEL_MFMA_I8, C.byref(algo)) == IV
+
+    def get(fn, attr, ctype):
+        v, w = ctype(), C.c_size_t()
+        assert fn(C.byref(algo), attr, C.addressof(v), C.sizeof(v), C.byref(w)) == 0 and w.value == C.sizeof(v)
+        return v.value
+    assert get(api.cublasLtMatmulAlgoConfigGetAttribute, 0, C.c_int32) == abi.ZLUDA_KERNEL_MFMA_I8      # ID
+    assert get(api.cublasLtMatmulAlgoConfigGetAttribute, 5, C.c_uint32) == 0                            # CUSTOM_OPTION
+    assert get(api.cublasLtMatmulAlgoConfigGetAttribute, 2, C.c_int32) == 1                             # SPLITK_NUM
+    nvar = get(api.cublasLtMatmulAlgoCapGetAttribute, 7, C.c_int32)                                     # CUSTOM_OPTION_MAX
+    assert nvar == api.zluda_gemm_variant_count(abi.ZLUDA_KERNEL_MFMA_I8) >= 4
+    assert get(api.cublasLtMatmulAlgoCapGetAttribute, 3, C.c_int32) == 1                                # STRIDED_BATCH
+    assert get(api.cublasLtMatmulAlgoCapGetAttribute, 16, C.c_uint32) == 16                             # MIN_ALIGNMENT_A
+    w = C.c_size_t()
+    assert api.cublasLtMatmulAlgoCapGetAttribute(C.byref(algo), 15, None, 0, C.byref(w)) == 0 and w.value == 8
+    assert api.cublasLtMatmulAlgoCapGetAttribute(C.byref(algo), 99, None, 0, C.byref(w)) == IV
+
+    def put(attr, ctype, value):
+        v = ctype(value)
+        return api.cublasLtMatmulAlgoConfigSetAttribute(C.byref(algo), attr, C.addressof(v), C.sizeof(v))
+    assert put(5, C.c_uint32, 3) == 0 and get(api.cublasLtMatmulAlgoConfigGetAttribute, 5, C.c_uint32) == 3
+    assert put(5, C.c_uint32, nvar + 1) == IV
+    assert put(0, C.c_int32, 3) == IV            # the id is read-only
+    assert put(2, C.c_int32, 4) == NS            # no split-K
+    assert put(1, C.c_uint32, 0) == 0 and put(1, C.c_uint32, 7) == NS
+
+    # the configured token runs through AlgoCheck like a heuristic result: variant 2 of the int8 family
+    spec = dict(m=4096, n=4096, k=4096, a_type=abi.CUDA_R_8I, b_type=abi.CUDA_R_8I, d_type=abi.CUDA_R_32I,
+                compute_type=abi.CUBLAS_COMPUTE_32I, scale_type=abi.CUDA_R_32I, transa=abi.CUBLAS_OP_T)
+    call = MatmulCall(api, spec)
+    res = abi.cublasLtMatmulHeuristicResult_t()
+    assert api.cublasLtMatmulAlgoCheck(call.handle, call.desc, call.a_desc, call.b_desc, call.c_desc, call.d_desc, C.byref(algo), C.byref(res)) == 0
+    assert res.algo.data[1] == 2 and res.state == 0
+    call.close()
+    # garbage tokens are rejected
+    junk = abi.cublasLtMatmulAlgo_t()
+    assert api.cublasLtMatmulAlgoConfigGetAttribute(C.byref(junk), 0, None, 0, C.byref(w)) == IV
+    assert api.cublasLtDestroy(h) == 0

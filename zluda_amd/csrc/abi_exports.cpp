@@ -590,30 +590,158 @@ cublasStatus_t cublasLtMatrixTransformDescGetAttribute(cublasLtMatrixTransformDe
                                                        size_t, size_t *) {
   return CUBLAS_STATUS_NOT_SUPPORTED;
 }
-cublasStatus_t cublasLtMatmulAlgoGetIds(cublasLtHandle_t, cublasComputeType_t, cudaDataType_t,
-                                        cudaDataType_t, cudaDataType_t, cudaDataType_t, cudaDataType_t,
-                                        int, int *, int *) {
-  return CUBLAS_STATUS_NOT_SUPPORTED;
+// ---- algorithm enumeration (cuda_macros/src/cublaslt.rs:397-518; `unimplemented` in the reference) ----
+// An algorithm id is a kernel family (ZLUDA_KERNEL_*); its one tunable, the tile variant, is exposed
+// as CUBLASLT_ALGO_CONFIG_CUSTOM_OPTION (0 = let the planner choose, v + 1 = variant v).
+
+// the families that can run a type combination at all (layouts decide the rest at AlgoCheck time)
+static int families_for_types(uint32_t computeType, uint32_t scaleType, uint32_t A, uint32_t B, uint32_t C,
+                              uint32_t D, int *ids) {
+  zluda_gemm_problem p;
+  memset(&p, 0, sizeof(p));
+  p.op.compute_type = computeType; p.op.scale_type = scaleType; p.op.bias_type = -1;
+  p.op.transa = CUBLAS_OP_T; p.op.transb = CUBLAS_OP_N; p.op.epilogue = CUBLASLT_EPILOGUE_DEFAULT;
+  const uint64_t n = 1024;
+  p.a = {A, CUBLASLT_ORDER_COL, n, n, (int64_t)n, 1, (int64_t)(n * n)};
+  p.b = {B, CUBLASLT_ORDER_COL, n, n, (int64_t)n, 1, (int64_t)(n * n)};
+  p.c = {C, CUBLASLT_ORDER_COL, n, n, (int64_t)n, 1, (int64_t)(n * n)};
+  p.d = {D, CUBLASLT_ORDER_COL, n, n, (int64_t)n, 1, (int64_t)(n * n)};
+  if (A == CUDA_R_4F_E2M1) p.op.a_scale_mode = p.op.b_scale_mode = CUBLASLT_MATMUL_MATRIX_SCALE_VEC32_UE8M0;
+  int count = 0;
+  zluda_gemm_plan plan;
+  // 1024^3 A:T B:N admits every square-GEMM family; the decode family wants a skinny shape
+  for (uint32_t k = ZLUDA_KERNEL_GENERIC; k <= ZLUDA_KERNEL_MFMA_MXF4; k++)
+    if (zluda_gemm_plan_problem(&p, k, -1, 256, &plan) == CUBLAS_STATUS_SUCCESS) ids[count++] = (int)k;
+  p.b.cols = p.c.cols = p.d.cols = 16;
+  if (zluda_gemm_plan_problem(&p, ZLUDA_KERNEL_DECODE_W8A8, -1, 256, &plan) == CUBLAS_STATUS_SUCCESS)
+    ids[count++] = ZLUDA_KERNEL_DECODE_W8A8;
+  return count;
 }
-cublasStatus_t cublasLtMatmulAlgoInit(cublasLtHandle_t, cublasComputeType_t, cudaDataType_t,
-                                      cudaDataType_t, cudaDataType_t, cudaDataType_t, cudaDataType_t,
-                                      int, cublasLtMatmulAlgo_t *) {
-  return CUBLAS_STATUS_NOT_SUPPORTED;
+
+cublasStatus_t cublasLtMatmulAlgoGetIds(cublasLtHandle_t lightHandle, cublasComputeType_t computeType,
+                                        cudaDataType_t scaleType, cudaDataType_t Atype, cudaDataType_t Btype,
+                                        cudaDataType_t Ctype, cudaDataType_t Dtype, int requestedAlgoCount,
+                                        int *algoIdsArray, int *returnAlgoCount) {
+  if (!resolve_handle(lightHandle) || !algoIdsArray || !returnAlgoCount || requestedAlgoCount < 0)
+    return CUBLAS_STATUS_INVALID_VALUE;
+  int ids[8];
+  const int n = families_for_types(computeType, scaleType, Atype, Btype, Ctype, Dtype, ids);
+  *returnAlgoCount = n < requestedAlgoCount ? n : requestedAlgoCount;
+  for (int i = 0; i < *returnAlgoCount; i++) algoIdsArray[i] = ids[i];
+  return CUBLAS_STATUS_SUCCESS;
 }
-cublasStatus_t cublasLtMatmulAlgoCapGetAttribute(const cublasLtMatmulAlgo_t *,
-                                                 cublasLtMatmulAlgoCapAttributes_t, void *, size_t,
-                                                 size_t *) {
-  return CUBLAS_STATUS_NOT_SUPPORTED;
+
+cublasStatus_t cublasLtMatmulAlgoInit(cublasLtHandle_t lightHandle, cublasComputeType_t computeType,
+                                      cudaDataType_t scaleType, cudaDataType_t Atype, cudaDataType_t Btype,
+                                      cudaDataType_t Ctype, cudaDataType_t Dtype, int algoId,
+                                      cublasLtMatmulAlgo_t *algo) {
+  if (!resolve_handle(lightHandle) || !algo) return CUBLAS_STATUS_INVALID_VALUE;
+  int ids[8];
+  const int n = families_for_types(computeType, scaleType, Atype, Btype, Ctype, Dtype, ids);
+  for (int i = 0; i < n; i++)
+    if (ids[i] == algoId) {
+      zluda_gemm_plan plan;
+      memset(&plan, 0, sizeof(plan));
+      plan.kernel = (uint32_t)algoId;
+      plan.variant = (uint32_t)-1;  // planner's choice until CUSTOM_OPTION says otherwise
+      pack_algo(plan, algo);
+      return CUBLAS_STATUS_SUCCESS;
+    }
+  return CUBLAS_STATUS_INVALID_VALUE;  // "algoId is not a valid id for these types" in cuBLASLt's terms
 }
-cublasStatus_t cublasLtMatmulAlgoConfigSetAttribute(cublasLtMatmulAlgo_t *,
-                                                    cublasLtMatmulAlgoConfigAttributes_t, const void *,
-                                                    size_t) {
-  return CUBLAS_STATUS_NOT_SUPPORTED;
+
+static int variants_of(uint32_t kernel) { return (int)zluda_gemm_variant_count(kernel); }
+
+cublasStatus_t cublasLtMatmulAlgoCapGetAttribute(const cublasLtMatmulAlgo_t *algo,
+                                                 cublasLtMatmulAlgoCapAttributes_t attr, void *buf,
+                                                 size_t sizeInBytes, size_t *sizeWritten) {
+  uint32_t kernel;
+  int32_t variant;
+  if (!algo || !unpack_algo(algo, &kernel, &variant)) return CUBLAS_STATUS_INVALID_VALUE;
+  int32_t i32 = 0;
+  uint32_t u32 = 0;
+  uint64_t u64 = 0;
+  switch (attr) {
+  case 0 /* SPLITK_SUPPORT */: i32 = 0; return access(false, i32, nullptr, buf, sizeInBytes, sizeWritten);
+  case 1 /* REDUCTION_SCHEME_MASK */: u32 = 0; return access(false, u32, nullptr, buf, sizeInBytes, sizeWritten);
+  case 2 /* CTA_SWIZZLING_SUPPORT */: u32 = 0; return access(false, u32, nullptr, buf, sizeInBytes, sizeWritten);
+  case 3 /* STRIDED_BATCH_SUPPORT */: i32 = 1; return access(false, i32, nullptr, buf, sizeInBytes, sizeWritten);
+  case 4 /* OUT_OF_PLACE_RESULT_SUPPORT */: i32 = 1; return access(false, i32, nullptr, buf, sizeInBytes, sizeWritten);
+  case 5 /* UPLO_SUPPORT */: i32 = 0; return access(false, i32, nullptr, buf, sizeInBytes, sizeWritten);
+  case 6 /* TILE_IDS */: case 13 /* STAGES_IDS */:
+    u32 = 0;  // one entry, CUBLASLT_MATMUL_TILE_UNDEFINED / STAGES_UNDEFINED: tiles are chosen through CUSTOM_OPTION
+    return access(false, u32, nullptr, buf, sizeInBytes, sizeWritten);
+  case 7 /* CUSTOM_OPTION_MAX */: i32 = variants_of(kernel); return access(false, i32, nullptr, buf, sizeInBytes, sizeWritten);
+  case 10 /* CUSTOM_MEMORY_ORDER */: i32 = 0; return access(false, i32, nullptr, buf, sizeInBytes, sizeWritten);
+  case 11 /* POINTER_MODE_MASK */: u32 = 0x1f; return access(false, u32, nullptr, buf, sizeInBytes, sizeWritten);
+  case 12 /* EPILOGUE_MASK */:
+    u32 = CUBLASLT_EPILOGUE_DEFAULT | CUBLASLT_EPILOGUE_RELU | CUBLASLT_EPILOGUE_BIAS | CUBLASLT_EPILOGUE_GELU;
+    return access(false, u32, nullptr, buf, sizeInBytes, sizeWritten);
+  case 14 /* LD_NEGATIVE */: i32 = 0; return access(false, i32, nullptr, buf, sizeInBytes, sizeWritten);
+  case 15 /* NUMERICAL_IMPL_FLAGS */: u64 = ~0ull; return access(false, u64, nullptr, buf, sizeInBytes, sizeWritten);
+  case 16: case 17: /* MIN_ALIGNMENT_A/B_BYTES */
+    u32 = kernel == ZLUDA_KERNEL_GENERIC ? 1 : 16;
+    return access(false, u32, nullptr, buf, sizeInBytes, sizeWritten);
+  case 18: case 19: /* MIN_ALIGNMENT_C/D_BYTES */ u32 = 1; return access(false, u32, nullptr, buf, sizeInBytes, sizeWritten);
+  case 21 /* POINTER_ARRAY_BATCH_SUPPORT */: case 22 /* FLOATING_POINT_EMULATION_SUPPORT */:
+    i32 = 0;
+    return access(false, i32, nullptr, buf, sizeInBytes, sizeWritten);
+  default: return CUBLAS_STATUS_INVALID_VALUE;
+  }
 }
-cublasStatus_t cublasLtMatmulAlgoConfigGetAttribute(const cublasLtMatmulAlgo_t *,
-                                                    cublasLtMatmulAlgoConfigAttributes_t, void *, size_t,
-                                                    size_t *) {
-  return CUBLAS_STATUS_NOT_SUPPORTED;
+
+// CONFIG attributes: ID (read-only) and CUSTOM_OPTION carry information; the others only accept /
+// report the one value this implementation has (no split-K, no swizzle option, undefined tile and
+// stage ids, automatic inner and cluster shapes).
+static cublasStatus_t algo_config(cublasLtMatmulAlgo_t *algo, uint32_t attr, bool set, const void *in, void *out,
+                                  size_t size, size_t *written) {
+  uint32_t kernel;
+  int32_t variant;
+  if (!algo || !unpack_algo(algo, &kernel, &variant)) return CUBLAS_STATUS_INVALID_VALUE;
+  switch (attr) {
+  case 0 /* ID */: {
+    int32_t id = (int32_t)kernel;
+    if (set) return CUBLAS_STATUS_INVALID_VALUE;
+    return access(false, id, nullptr, out, size, written);
+  }
+  case 5 /* CUSTOM_OPTION */: {
+    uint32_t opt = variant < 0 ? 0u : (uint32_t)variant + 1;
+    cublasStatus_t st = access(set, opt, in, out, size, written);
+    if (set && !st) {
+      if ((int)opt > variants_of(kernel)) return CUBLAS_STATUS_INVALID_VALUE;
+      algo->data[1] = opt == 0 ? (uint64_t)(uint32_t)-1 : opt - 1;
+    }
+    return st;
+  }
+  case 2 /* SPLITK_NUM */: {
+    int32_t v = 1;
+    cublasStatus_t st = access(set, v, in, out, size, written);
+    return (set && !st && v != 1 && v != 0) ? CUBLAS_STATUS_NOT_SUPPORTED : st;
+  }
+  case 1 /* TILE_ID */: case 3 /* REDUCTION_SCHEME */: case 4 /* CTA_SWIZZLING */: case 6 /* STAGES_ID */: {
+    uint32_t v = 0;
+    cublasStatus_t st = access(set, v, in, out, size, written);
+    return (set && !st && v != 0) ? CUBLAS_STATUS_NOT_SUPPORTED : st;
+  }
+  case 7 /* INNER_SHAPE_ID */: case 8 /* CLUSTER_SHAPE_ID */: {
+    uint16_t v = 0;
+    cublasStatus_t st = access(set, v, in, out, size, written);
+    return (set && !st && v != 0) ? CUBLAS_STATUS_NOT_SUPPORTED : st;
+  }
+  default: return CUBLAS_STATUS_INVALID_VALUE;
+  }
+}
+
+cublasStatus_t cublasLtMatmulAlgoConfigSetAttribute(cublasLtMatmulAlgo_t *algo,
+                                                    cublasLtMatmulAlgoConfigAttributes_t attr, const void *buf,
+                                                    size_t sizeInBytes) {
+  if (!buf) return CUBLAS_STATUS_INVALID_VALUE;
+  return algo_config(algo, attr, true, buf, nullptr, sizeInBytes, nullptr);
+}
+cublasStatus_t cublasLtMatmulAlgoConfigGetAttribute(const cublasLtMatmulAlgo_t *algo,
+                                                    cublasLtMatmulAlgoConfigAttributes_t attr, void *buf,
+                                                    size_t sizeInBytes, size_t *sizeWritten) {
+  return algo_config(const_cast<cublasLtMatmulAlgo_t *>(algo), attr, false, nullptr, buf, sizeInBytes, sizeWritten);
 }
 cublasStatus_t cublasLtLoggerSetCallback(cublasLtLoggerCallback_t) { return CUBLAS_STATUS_NOT_SUPPORTED; }
 cublasStatus_t cublasLtLoggerSetFile(FILE *) { return CUBLAS_STATUS_NOT_SUPPORTED; }

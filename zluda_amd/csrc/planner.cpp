@@ -305,6 +305,15 @@ static int pick_decode_variant(const Lowered &l) {
 
 using namespace zluda_amd;
 
+extern "C" uint32_t zluda_gemm_variant_count(uint32_t kernel) {
+  switch (kernel) {
+  case ZLUDA_KERNEL_GENERIC: return 1;
+  case ZLUDA_KERNEL_MFMA_I8: case ZLUDA_KERNEL_MFMA_F8: case ZLUDA_KERNEL_MFMA_MXF4: return kNumMfmaVariants;
+  case ZLUDA_KERNEL_DECODE_W8A8: return kNumDecodeVariants;
+  default: return 0;
+  }
+}
+
 extern "C" uint32_t zluda_gemm_plan_problem(const zluda_gemm_problem *p, uint32_t forced_kernel,
                                             int32_t forced_variant, uint32_t cu_count,
                                             zluda_gemm_plan *plan) {
