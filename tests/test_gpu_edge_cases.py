@@ -1,0 +1,112 @@
+"""Edge cases of cublasLtMatmul through the planner's own choice (no forced kernel): degenerate and
+ragged shapes, long K, many batches, in-place C == D, device-side scalars, error returns on a live
+device.  Same bars as tests/test_gpu_parity.py."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from oracle.cases import Case
+from zluda_amd import abi
+from zluda_amd.cublaslt import MatmulCall
+
+pytestmark = pytest.mark.gpu
+K = abi
+
+I8 = dict(a_type=K.CUDA_R_8I, b_type=K.CUDA_R_8I, c_type=K.CUDA_R_32I, d_type=K.CUDA_R_32I,
+          compute_type=K.CUBLAS_COMPUTE_32I, scale_type=K.CUDA_R_32I, transa=1)
+F8 = dict(a_type=K.CUDA_R_8F_E4M3, b_type=K.CUDA_R_8F_E4M3, c_type=K.CUDA_R_16BF, d_type=K.CUDA_R_16BF,
+          compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F, transa=1)
+MX = dict(a_type=K.CUDA_R_4F_E2M1, b_type=K.CUDA_R_4F_E2M1, c_type=K.CUDA_R_16BF, d_type=K.CUDA_R_16BF,
+          compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F, transa=1,
+          a_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_VEC32_UE8M0, b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_VEC32_UE8M0)
+
+
+def run(gpu_api, spec, seed, **kw):
+    print("edge case", spec, flush=True)
+    case = Case(spec, seed, **kw)
+    ref = case.run_oracle()
+    st, got, kern, variant = case.run_gpu(gpu_api)
+    assert st == 0, "cublasLtMatmul status %d" % st
+    case.compare(got, ref)
+    return kern
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 1, 1), (1, 1, 16), (1, 37, 5), (37, 1, 48), (3, 5, 7), (17, 33, 129), (255, 257, 16)])
+def test_tiny_and_odd_int8_shapes(gpu_api, m, n, k):
+    run(gpu_api, dict(I8, m=m, n=n, k=k), 300 + m)
+
+
+@pytest.mark.parametrize("m,n,k", [(257, 255, 4112), (512, 256, 32768), (256, 512, 16)])
+def test_int8_ragged_tiles_long_and_short_k(gpu_api, m, n, k):
+    """partial tiles on both edges; K = 32768 (256 stages; |sum| <= 2^29, no overflow); K = one chunk"""
+    assert run(gpu_api, dict(I8, m=m, n=n, k=k), 310) == K.ZLUDA_KERNEL_MFMA_I8
+
+
+def test_int8_many_small_batches(gpu_api):
+    run(gpu_api, dict(I8, m=64, n=48, k=80, batch=33, with_c=True), 320)
+
+
+def test_fp8_and_mxfp4_ragged(gpu_api):
+    assert run(gpu_api, dict(F8, m=300, n=130, k=464, epilogue=K.CUBLASLT_EPILOGUE_RELU_BIAS, with_c=True), 330) == K.ZLUDA_KERNEL_MFMA_F8
+    # K = 256 * odd: scale rows of 8 * odd bytes (chunks run across row boundaries)
+    assert run(gpu_api, dict(MX, m=130, n=300, k=1280, batch=3), 331) == K.ZLUDA_KERNEL_MFMA_MXF4
+    assert run(gpu_api, dict(MX, m=256, n=256, k=256), 332) == K.ZLUDA_KERNEL_MFMA_MXF4
+    # K not a multiple of 256: outside the MFMA family's contract, served by the generic kernel
+    assert run(gpu_api, dict(MX, m=64, n=64, k=96), 333) == K.ZLUDA_KERNEL_GENERIC
+
+
+def test_decode_shapes_around_the_limits(gpu_api):
+    dec = dict(I8, c_type=K.CUDA_R_16BF, d_type=K.CUDA_R_16BF, scale_type=K.CUDA_R_32F, alpha_range=(0.001, 0.01))
+    assert run(gpu_api, dict(dec, m=64, n=1, k=4096), 340, int_dist="normal") == K.ZLUDA_KERNEL_DECODE_W8A8
+    assert run(gpu_api, dict(dec, m=4099, n=32, k=4096), 341, int_dist="normal") == K.ZLUDA_KERNEL_DECODE_W8A8   # rows % 4 != 0
+    assert run(gpu_api, dict(dec, m=2048, n=3, k=11008), 342, int_dist="normal") == K.ZLUDA_KERNEL_DECODE_W8A8  # K outside the stream table
+    assert run(gpu_api, dict(dec, m=512, n=16, k=4096, batch=3), 343, int_dist="normal") == K.ZLUDA_KERNEL_DECODE_W8A8
+    # 33 tokens: no longer a decode shape
+    assert run(gpu_api, dict(dec, m=2048, n=33, k=4096), 344, int_dist="normal") == K.ZLUDA_KERNEL_MFMA_I8
+    # f16 output, ld > rows (the packed store needs ld % 4 == 0: 2052 qualifies, 2051 does not)
+    for ld in (2052, 2051):
+        run(gpu_api, dict(dec, c_type=K.CUDA_R_16F, d_type=K.CUDA_R_16F, m=2048, n=8, k=4096, ldd=ld, ldc=ld), 345, int_dist="normal")
+
+
+def test_in_place_c_equals_d_and_device_scalars(gpu_api):
+    """C == D with beta != 0 (allowed: ext/hipblaslt-sys/src/lib.rs:1166-1177), alpha/beta read from device memory"""
+    import torch
+    spec = dict(I8, m=384, n=256, k=512, with_c=True, pointer_mode=K.CUBLASLT_POINTER_MODE_DEVICE)
+    case = Case(spec, 350)
+    ref = case.run_oracle()
+    keep, ptr, dt = case.upload()
+    # start D as a copy of C and pass the same pointer for both
+    nbytes = case.Cm.nbytes
+    d_t = torch.frombuffer(bytearray(case.Cm.tobytes()), dtype=torch.uint8).cuda()
+    call = MatmulCall(gpu_api, spec)
+    alpha, beta = case.scalars(ptr)
+    st = call.run(alpha, ptr["A"], ptr["B"], beta, d_t.data_ptr(), d_t.data_ptr(), None, 0, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    call.close()
+    assert st == 0
+    got = np.frombuffer(d_t.cpu().numpy().tobytes(), dtype=np.int32)
+    assert nbytes == got.nbytes
+    assert np.array_equal(got, ref)
+
+
+def test_error_returns_with_a_live_device(gpu_api):
+    import torch
+    spec = dict(I8, m=256, n=256, k=256)
+    call = MatmulCall(gpu_api, spec)
+    a = torch.zeros(256 * 256, dtype=torch.int8, device="cuda:0")
+    d = torch.zeros(256 * 256, dtype=torch.int32, device="cuda:0")
+    one, zero = C.c_int32(1), C.c_int32(0)
+    stream = torch.cuda.current_stream().cuda_stream
+    assert call.run(one, a.data_ptr(), a.data_ptr(), zero, None, d.data_ptr(), None, 0, stream) == 0
+    assert call.run(one, None, a.data_ptr(), zero, None, d.data_ptr(), None, 0, stream) == K.CUBLAS_STATUS_INVALID_VALUE
+    assert call.run(None, a.data_ptr(), a.data_ptr(), zero, None, d.data_ptr(), None, 0, stream) == K.CUBLAS_STATUS_INVALID_VALUE
+    two = C.c_int32(2)   # beta != 0 without C
+    assert call.run(one, a.data_ptr(), a.data_ptr(), two, None, None, None, 0, stream) == K.CUBLAS_STATUS_INVALID_VALUE
+    # a foreign algo token
+    junk = abi.cublasLtMatmulAlgo_t()
+    junk.data[0] = 0x1234
+    call.algo = junk
+    assert call.run(one, a.data_ptr(), a.data_ptr(), zero, None, d.data_ptr(), None, 0, stream) == K.CUBLAS_STATUS_INVALID_VALUE
+    call.close()
+    torch.cuda.synchronize()
