@@ -94,6 +94,23 @@ uint32_t zluda_gemm_plan_problem(const zluda_gemm_problem *p, uint32_t forced_ke
 uint32_t zluda_gemm_launch(const zluda_gemm_problem *p, const zluda_gemm_plan *plan,
                            void *stream);
 
+/* cublasGemmEx / cublasGemmStridedBatchedEx on the same kernels: column-major operands, C is read
+ * (when beta != 0) and overwritten, alpha and beta are host scalars of the type the compute type
+ * implies (int32 for CUBLAS_COMPUTE_32I*, float for CUBLAS_COMPUTE_32F*).  This is what
+ * zluda_blas::gemm_ex / gemm_strided_batched_ex (zluda_blas/src/impl.rs:242-289, 376-432) would call
+ * for the integer and 8-bit float cases their rocBLAS mapping rejects today
+ * (zluda_common/src/lib.rs:553-564).  batch_count == 1 ignores the strides. */
+uint32_t zluda_gemm_strided_batched_ex(uint32_t transa, uint32_t transb, int32_t m, int32_t n, int32_t k,
+                                       const void *alpha, const void *A, uint32_t a_type, int64_t lda,
+                                       int64_t stride_a, const void *B, uint32_t b_type, int64_t ldb,
+                                       int64_t stride_b, const void *beta, void *C, uint32_t c_type,
+                                       int64_t ldc, int64_t stride_c, int32_t batch_count,
+                                       uint32_t compute_type, void *stream);
+uint32_t zluda_gemm_ex(uint32_t transa, uint32_t transb, int32_t m, int32_t n, int32_t k, const void *alpha,
+                       const void *A, uint32_t a_type, int64_t lda, const void *B, uint32_t b_type,
+                       int64_t ldb, const void *beta, void *C, uint32_t c_type, int64_t ldc,
+                       uint32_t compute_type, void *stream);
+
 /* Number of tile configurations (plan.variant values) of a kernel family; 1 for the generic kernel,
  * 0 for an unknown family. */
 uint32_t zluda_gemm_variant_count(uint32_t kernel);

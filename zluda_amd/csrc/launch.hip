@@ -2,6 +2,8 @@
 // and enqueues it on the caller's stream.  Only the HIP runtime is used (hipLaunchKernelGGL).
 #include <hip/hip_runtime.h>
 
+#include <cstring>
+
 #include "kernels/decode_stream.hpp"
 #include "kernels/decode_w8a8.hpp"
 #include "kernels/gemm_generic.hpp"
@@ -167,4 +169,49 @@ extern "C" uint32_t zluda_gemm_launch(const zluda_gemm_problem *p, const zluda_g
   default: return CUBLAS_STATUS_NOT_SUPPORTED;
   }
   return hipGetLastError() == hipSuccess ? CUBLAS_STATUS_SUCCESS : CUBLAS_STATUS_EXECUTION_FAILED;
+}
+
+// ---- cublasGemmEx-shaped entry points --------------------------------------------------------
+extern "C" uint32_t zluda_gemm_strided_batched_ex(uint32_t transa, uint32_t transb, int32_t m, int32_t n,
+                                                  int32_t k, const void *alpha, const void *A, uint32_t a_type,
+                                                  int64_t lda, int64_t stride_a, const void *B, uint32_t b_type,
+                                                  int64_t ldb, int64_t stride_b, const void *beta, void *C,
+                                                  uint32_t c_type, int64_t ldc, int64_t stride_c,
+                                                  int32_t batch_count, uint32_t compute_type, void *stream) {
+  if (m < 0 || n < 0 || k < 0 || batch_count < 0) return CUBLAS_STATUS_INVALID_VALUE;
+  if (m == 0 || n == 0 || batch_count == 0) return CUBLAS_STATUS_SUCCESS;  // nothing to write
+  if (k == 0) return CUBLAS_STATUS_NOT_SUPPORTED;  // C = beta * C only: not a matmul problem of this layer
+  const bool int_path = compute_type == CUBLAS_COMPUTE_32I || compute_type == CUBLAS_COMPUTE_32I_PEDANTIC;
+  zluda_gemm_problem p;
+  memset(&p, 0, sizeof(p));
+  p.op.compute_type = compute_type;
+  p.op.scale_type = int_path ? CUDA_R_32I : CUDA_R_32F;
+  p.op.pointer_mode = CUBLASLT_POINTER_MODE_HOST;
+  p.op.transa = transa; p.op.transb = transb;
+  p.op.epilogue = CUBLASLT_EPILOGUE_DEFAULT;
+  p.op.bias_type = -1;
+  const bool ta = transa != CUBLAS_OP_N, tb = transb != CUBLAS_OP_N;
+  p.a = {a_type, CUBLASLT_ORDER_COL, (uint64_t)(ta ? k : m), (uint64_t)(ta ? m : k), lda, batch_count, stride_a};
+  p.b = {b_type, CUBLASLT_ORDER_COL, (uint64_t)(tb ? n : k), (uint64_t)(tb ? k : n), ldb, batch_count, stride_b};
+  p.c = {c_type, CUBLASLT_ORDER_COL, (uint64_t)m, (uint64_t)n, ldc, batch_count, stride_c};
+  p.d = p.c;
+  p.alpha = alpha; p.beta = beta;
+  p.A = A; p.B = B; p.C = C; p.D = C;
+  zluda_gemm_plan plan;
+  uint32_t st = zluda_gemm_plan_problem(&p, ZLUDA_KERNEL_AUTO, -1, zluda_gemm_device_cu_count(), &plan);
+  if (st == CUBLAS_STATUS_SUCCESS) st = zluda_gemm_launch(&p, &plan, stream);
+  if (st == CUBLAS_STATUS_NOT_SUPPORTED || st == CUBLAS_STATUS_INVALID_VALUE) {
+    // the chosen family may refuse the actual pointers (alignment): the generic kernel takes anything valid
+    if (zluda_gemm_plan_problem(&p, ZLUDA_KERNEL_GENERIC, -1, zluda_gemm_device_cu_count(), &plan) == CUBLAS_STATUS_SUCCESS)
+      st = zluda_gemm_launch(&p, &plan, stream);
+  }
+  return st;
+}
+
+extern "C" uint32_t zluda_gemm_ex(uint32_t transa, uint32_t transb, int32_t m, int32_t n, int32_t k,
+                                  const void *alpha, const void *A, uint32_t a_type, int64_t lda, const void *B,
+                                  uint32_t b_type, int64_t ldb, const void *beta, void *C, uint32_t c_type,
+                                  int64_t ldc, uint32_t compute_type, void *stream) {
+  return zluda_gemm_strided_batched_ex(transa, transb, m, n, k, alpha, A, a_type, lda, 0, B, b_type, ldb, 0, beta, C,
+                                       c_type, ldc, 0, 1, compute_type, stream);
 }
