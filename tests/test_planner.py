@@ -37,7 +37,7 @@ def test_baseline_configs_pick_the_intended_kernels(api):
                            b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F,
                            epilogue=K.CUBLASLT_EPILOGUE_BIAS, bias_type=K.CUDA_R_32F))       # config 3
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.swapped == 0 and p.block == 512
-    assert p.variant == 4 and p.grid_x == 512      # streamed through LDS, two workgroups per CU
+    assert p.variant == 4 and p.grid_x == 256      # streamed through LDS, one 8-wave workgroup per CU
     st, p = plan(api, dict(F8, m=8192, n=8192, k=8192, transa=1, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS))  # config 4
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_F8 and p.grid_x == 1024
     st, p = plan(api, dict(MX, m=8192, n=8192, k=8192, transa=1, batch=4))          # config 5

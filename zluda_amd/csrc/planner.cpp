@@ -278,7 +278,10 @@ static void fill_decode_plan(const Lowered &l, int variant, uint32_t cus, zluda_
   const bool swapped = g.M < g.N;  // weights are the long operand
   const uint32_t rows = swapped ? g.N : g.M;
   const uint32_t nrb = ceil_div(rows, 16);
-  const uint32_t resident = cus * (v.nw == 8 ? 2 : 4);
+  // Stream kernel: 8 waves x 2 slots x 4 KiB = 64 KiB in flight per CU is the measured optimum on
+  // MI355X (14.8 us for 58.7 MB; 128 KiB in flight: 15.8-16.8 us, 32 KiB: 15.9 us), so one 8-wave
+  // workgroup per CU, two 4-wave ones.
+  const uint32_t resident = v.stream ? cus * (v.nw == 8 ? 1 : 2) : cus * (v.nw == 8 ? 2 : 4);
   uint32_t grid;
   if (v.stream) grid = std::min(nrb, resident);  // contiguous, balanced row ranges
   else grid = nrb <= resident ? nrb : ceil_div(nrb, ceil_div(nrb, resident));
