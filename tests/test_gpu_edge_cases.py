@@ -62,8 +62,11 @@ def test_decode_shapes_around_the_limits(gpu_api):
     assert run(gpu_api, dict(dec, m=4099, n=32, k=4096), 341, int_dist="normal") == K.ZLUDA_KERNEL_DECODE_W8A8   # rows % 4 != 0
     assert run(gpu_api, dict(dec, m=2048, n=3, k=11008), 342, int_dist="normal") == K.ZLUDA_KERNEL_DECODE_W8A8  # K outside the stream table
     assert run(gpu_api, dict(dec, m=512, n=16, k=4096, batch=3), 343, int_dist="normal") == K.ZLUDA_KERNEL_DECODE_W8A8
-    # 33 tokens: no longer a decode shape
-    assert run(gpu_api, dict(dec, m=2048, n=33, k=4096), 344, int_dist="normal") == K.ZLUDA_KERNEL_MFMA_I8
+    # up to 64 tokens stream (K = 4096: 4 token blocks x 8 steps of activation fragments); 65 do not
+    assert run(gpu_api, dict(dec, m=2048, n=33, k=4096), 344, int_dist="normal") == K.ZLUDA_KERNEL_DECODE_W8A8
+    assert run(gpu_api, dict(dec, m=2048, n=64, k=4096), 346, int_dist="normal") == K.ZLUDA_KERNEL_DECODE_W8A8
+    assert run(gpu_api, dict(dec, m=2048, n=65, k=4096), 347, int_dist="normal") == K.ZLUDA_KERNEL_MFMA_I8
+    assert run(gpu_api, dict(dec, m=2048, n=48, k=8192), 348, int_dist="normal") == K.ZLUDA_KERNEL_MFMA_I8   # 3 x 16 fragments
     # f16 output, ld > rows (the packed store needs ld % 4 == 0: 2052 qualifies, 2051 does not)
     for ld in (2052, 2051):
         run(gpu_api, dict(dec, c_type=K.CUDA_R_16F, d_type=K.CUDA_R_16F, m=2048, n=8, k=4096, ldd=ld, ldc=ld), 345, int_dist="normal")

@@ -149,9 +149,11 @@ def test_decode_stream_variants(gpu_api, variant, monkeypatch):
     check(gpu_api, dict(DECODE, m=1000, n=16, k=k), 120 + variant, K.ZLUDA_KERNEL_DECODE_W8A8, variant, int_dist="normal")
     monkeypatch.setenv("ZLUDA_DECODE_GRID", "7")      # 142.86 rows per workgroup: 9 blocks, the last partial
     check(gpu_api, dict(DECODE, m=1000, n=5, k=k, lda=k + 64), 140 + variant, K.ZLUDA_KERNEL_DECODE_W8A8, variant, int_dist="normal")
-    if steps <= 12:
-        check(gpu_api, dict(DECODE, m=333, n=29, k=k), 160 + variant, K.ZLUDA_KERNEL_DECODE_W8A8, variant, int_dist="normal")
-        check(gpu_api, dict(I8, m=333, n=32, k=k, with_c=True), 180 + variant, K.ZLUDA_KERNEL_DECODE_W8A8, variant)
+    # more tokens: blocks of 16, as many as the activation registers allow (blocks x steps <= 32)
+    for blocks, tokens in ((2, 29), (3, 41), (4, 64)):
+        if blocks * steps <= 32:
+            check(gpu_api, dict(DECODE, m=332, n=tokens, k=k), 160 + variant, K.ZLUDA_KERNEL_DECODE_W8A8, variant, int_dist="normal")
+            check(gpu_api, dict(I8, m=333, n=tokens - 1, k=k, with_c=True), 180 + variant, K.ZLUDA_KERNEL_DECODE_W8A8, variant)
 
 
 def test_decode_config3_shape_takes_the_stream_kernel(gpu_api):

@@ -47,7 +47,7 @@ def test_baseline_configs_pick_the_intended_kernels(api):
 
 def test_small_problems_get_smaller_tiles(api):
     st, p = plan(api, dict(I8, m=1024, n=1024, k=1024, transa=1))
-    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_I8 and p.variant == 3 and p.grid_x == 64
+    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_I8 and p.variant == 4 and p.grid_x == 64
     st, p = plan(api, dict(I8, m=4096, n=2048, k=1024, transa=1))
     assert st == 0 and p.variant == 2 and p.grid_x == 16 * 16
 

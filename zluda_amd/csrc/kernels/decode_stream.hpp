@@ -17,6 +17,9 @@
 // activation fragments in registers for the whole kernel.  A wave's data path is private: it fills
 // its own LDS ring (2 slots of 16 rows x 256 bytes) and only it reads them back, so the only
 // workgroup barrier is the one in front of the cross-wave reduction of a finished 16-row block.
+// A block has 64 x NB (token, quad of rows) pairs; whoever owns a pair sums its NW partial values,
+// applies the epilogue and writes the quad with one store: one rotating wave for up to 32 tokens,
+// all waves (one pair per lane) beyond that.
 // A slot is refilled as soon as its fragments are in registers, so every wave always has 4-8 KiB in
 // flight (64-128 KiB per CU with 16 resident waves).
 //
@@ -78,8 +81,7 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(DecodeParams prm
   constexpr int NDMA = 16 * SEG / 1024;  // DMA instructions per unit
   static_assert(SPW % 4 == 0, "a wave's K slice is a whole number of 256-byte units");
   __shared__ v4i ring[NW][NSLOT][UNIT_V4];
-  constexpr int RBUF = NB == 1 ? 2 : 1;  // two token blocks: one reduction buffer (LDS for two workgroups per CU)
-  __shared__ v4i red[RBUF][NW][NB][64];
+  __shared__ v4i red[2][NW][NB][64];
 
   const GemmArgs &g = prm.g;
   const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
@@ -162,33 +164,51 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(DecodeParams prm
                       g.beta_mode == SCALAR_VALUE && g.beta_val.f == 0.0f && ((uintptr_t)g.D & 7) == 0 &&
                       (d_st & 3) == 0 && (g.d_sb & 3) == 0;
   uint16_t *const Dp = (uint16_t *)g.D + g.d_sb * bt;
-  const uint32_t red_base = lds_addr(&red[0][0][0][lane]);
+  const uint32_t red_base0 = lds_addr(&red[0][0][0][0]);
   const uint32_t ring_base = lds_addr(&ring[wave][0][l16 * 16]);  // this lane's row in slot 0
   int slot = 0;
   // (block, unit) that the next refill fetches: NSLOT units ahead of the one being consumed
   int fblk = NSLOT / Q, fq = NSLOT % Q;
 
   for (int blk = 0; blk < nblk; blk++) {
-    const bool reducer = wave == blk % NW;  // the reducing wave rotates
-    // The reducer fetches the epilogue factors of its outputs while the block streams: by the time
-    // the weights have gone through the MFMAs they have long arrived, and the epilogue is left
-    // without a memory round trip of its own.  Raw loads only: converting or combining them here
-    // would make the compiler wait for each load on the spot.
-    float f_al[NB][4], f_sa[NB][4], f_sb[NB][4], f_be[NB][4];
-    uint32_t f_bias[NB][4];
-    auto prefetch_factors = [&]() {
-      if (reducer && (FAST || !g.int_scale)) {
+    // Who runs the epilogue of the block's 64 * NB (token, quad of rows) pairs.
+    //   NB <= 2: one wave (rotating) takes them all, NB per lane.  Its epilogue costs ~1 us per block,
+    //            but the other waves are left alone, which measures faster for few tokens.
+    //   NB >= 3: every wave takes 64 * NB / NW pairs, one per lane; one wave alone would hold up the
+    //            others for several microseconds per block and need 20 * NB registers for the factors.
+    // Pair p lives in accumulator lane p % 64 of token block p / 64 of every wave.
+    constexpr bool SHARED = NB >= 3;
+    constexpr int PPL = SHARED ? 1 : NB;  // pairs per participating lane
+    static_assert(!SHARED || (64 * NB % NW == 0 && 64 * NB / NW <= 64), "pairs are dealt out evenly, at most one per lane");
+    constexpr int PAIRS_W = 64 * NB / NW;
+    const bool has_pair = SHARED ? lane < PAIRS_W : wave == blk % NW;
+    int my_nb[PPL], src_lane[PPL], my_tok[PPL], my_row0[PPL];
 #pragma unroll
-        for (int nb = 0; nb < NB; nb++)
+    for (int pp = 0; pp < PPL; pp++) {
+      const int pair = SHARED ? wave * PAIRS_W + (lane < PAIRS_W ? lane : 0) : pp * 64 + lane;
+      my_nb[pp] = pair >> 6; src_lane[pp] = pair & 63;
+      my_tok[pp] = my_nb[pp] * 16 + (src_lane[pp] & 15);
+      my_row0[pp] = r0 + blk * 16 + (src_lane[pp] >> 4) * 4;
+    }
+    // The epilogue factors of those pairs are fetched while the block streams: by the time the
+    // weights have gone through the MFMAs they have long arrived, and the epilogue is left without
+    // a memory round trip of its own.  Raw loads only: converting or combining them here would make
+    // the compiler wait for each load on the spot.
+    float f_al[PPL][4], f_sa[PPL][4], f_sb[PPL][4], f_be[PPL][4];
+    uint32_t f_bias[PPL][4];
+    auto prefetch_factors = [&]() {
+      if (has_pair && (FAST || !g.int_scale)) {
+#pragma unroll
+        for (int pp = 0; pp < PPL; pp++)
 #pragma unroll
           for (int v = 0; v < 4; v++) {
-            const int row = min(r0 + blk * 16 + g4 * 4 + v, r1 - 1), tok = min(nb * 16 + l16, T - 1);
+            const int row = min(my_row0[pp] + v, r1 - 1), tok = min(my_tok[pp], T - 1);
             const int i = prm.swapped ? tok : row, j = prm.swapped ? row : tok;
-            f_al[nb][v] = ep.alpha_v ? ep.alpha_v[i] : ep.alpha_s;
-            f_sa[nb][v] = ep.sa_v ? ep.sa_v[i] : ep.sa_s;
-            f_sb[nb][v] = ep.sb_v ? ep.sb_v[j] : ep.sb_s;
-            if constexpr (!FAST) f_be[nb][v] = ep.beta_v ? ep.beta_v[i] : ep.beta_s;
-            f_bias[nb][v] = ep.bias_raw(i);
+            f_al[pp][v] = ep.alpha_v ? ep.alpha_v[i] : ep.alpha_s;
+            f_sa[pp][v] = ep.sa_v ? ep.sa_v[i] : ep.sa_s;
+            f_sb[pp][v] = ep.sb_v ? ep.sb_v[j] : ep.sb_s;
+            if constexpr (!FAST) f_be[pp][v] = ep.beta_v ? ep.beta_v[i] : ep.beta_s;
+            f_bias[pp][v] = ep.bias_raw(i);
           }
       }
     };
@@ -212,13 +232,13 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(DecodeParams prm
       // One unit later the counted wait above has covered those loads as well.  Telling the compiler
       // here (where it can count: the loads are older than one refill) keeps it from waiting for
       // them in the epilogue, where its only safe choice is vmcnt(0), i.e. the units in flight.
-      if (Q > 1 && q == Q - 1 && reducer && (FAST || !g.int_scale)) {
+      if (Q > 1 && q == Q - 1 && has_pair && (FAST || !g.int_scale)) {
 #pragma unroll
-        for (int nb = 0; nb < NB; nb++)
+        for (int pp = 0; pp < PPL; pp++)
 #pragma unroll
           for (int v = 0; v < 4; v++) {
-            asm volatile("" : "+v"(f_al[nb][v]), "+v"(f_sa[nb][v]), "+v"(f_sb[nb][v]), "+v"(f_bias[nb][v]));
-            if constexpr (!FAST) asm volatile("" : "+v"(f_be[nb][v]));
+            asm volatile("" : "+v"(f_al[pp][v]), "+v"(f_sa[pp][v]), "+v"(f_sb[pp][v]), "+v"(f_bias[pp][v]));
+            if constexpr (!FAST) asm volatile("" : "+v"(f_be[pp][v]));
           }
       }
       issue_unit(fblk, fq, slot);
@@ -231,56 +251,55 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(DecodeParams prm
           acc[nb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[s], xf[nb][q * 4 + s], acc[nb], 0, 0, 0);
     }
 
-    // cross-wave reduction of the finished block
-    const int buf = RBUF == 2 ? (blk & 1) : 0;
+    // cross-wave reduction of the finished block (double-buffered: a wave writes its partial sums
+    // of block b + 2 only after the barrier of block b + 1, which every wave reaches after its reads
+    // of block b)
+    const int buf = blk & 1;
 #pragma unroll
     for (int nb = 0; nb < NB; nb++) red[buf][wave][nb][lane] = acc[nb];
     lds_barrier();
-    if (reducer) {
+    if (has_pair) {
 #pragma unroll
-      for (int nb = 0; nb < NB; nb++) {
+      for (int pp = 0; pp < PPL; pp++) {
         // unordered reads again: a C++ read of LDS would wait for this wave's units in flight
         v4i part[NW];
 #pragma unroll
-        for (int w2 = 0; w2 < NW; w2++) part[w2] = lds_read16_unordered(red_base + ((buf * NW + w2) * NB + nb) * 1024);
+        for (int w2 = 0; w2 < NW; w2++)
+          part[w2] = lds_read16_unordered(red_base0 + (((buf * NW + w2) * NB + my_nb[pp]) * 64 + src_lane[pp]) * 16);
         lds_values_ready(part);
         v4i s = part[0];
 #pragma unroll
         for (int w2 = 1; w2 < NW; w2++) s += part[w2];
-        const int tok = nb * 16 + l16;
-        const int row0 = r0 + blk * 16 + g4 * 4;
+        const int tok = my_tok[pp], row0 = my_row0[pp];
         if (FAST || (packed && row0 + 3 < r1)) {
           if (tok < T && row0 < r1) {  // FAST: r1 is a multiple of 4, a quad is inside or outside
             float y[4];
 #pragma unroll
             for (int v = 0; v < 4; v++)
-              y[v] = ep.finish(((f_al[nb][v] * f_sa[nb][v]) * f_sb[nb][v]) * (float)s[v] + ep.bias_from_raw(f_bias[nb][v]));
+              y[v] = ep.finish(((f_al[pp][v] * f_sa[pp][v]) * f_sb[pp][v]) * (float)s[v] + ep.bias_from_raw(f_bias[pp][v]));
             uint2 pk;
             if (g.d_type == CUDA_R_16BF) {
-              pk.x = (uint32_t)enc_bf16(y[0]) | ((uint32_t)enc_bf16(y[1]) << 16);
-              pk.y = (uint32_t)enc_bf16(y[2]) | ((uint32_t)enc_bf16(y[3]) << 16);
+              pk.x = pack_bf16x2(y[0], y[1]);
+              pk.y = pack_bf16x2(y[2], y[3]);
             } else {
-              pk.x = (uint32_t)enc_f16(y[0]) | ((uint32_t)enc_f16(y[1]) << 16);
-              pk.y = (uint32_t)enc_f16(y[2]) | ((uint32_t)enc_f16(y[3]) << 16);
+              pk.x = pack_f16x2(y[0], y[1]);
+              pk.y = pack_f16x2(y[2], y[3]);
             }
             *(uint2 *)(Dp + (int64_t)tok * d_st + row0) = pk;
           }
-          continue;
-        }
-        if constexpr (!FAST) {
+        } else if constexpr (!FAST) {
 #pragma unroll
           for (int v = 0; v < 4; v++) {
             const int row = row0 + v;
             if (row < r1 && tok < T) {
               const int i = prm.swapped ? tok : row, j = prm.swapped ? row : tok;
               if (g.int_scale) ep.store_int(i, j, s[v]);
-              else ep.store_f(i, j, (float)s[v], f_al[nb][v] * f_sa[nb][v], f_sb[nb][v], f_be[nb][v], ep.bias_from_raw(f_bias[nb][v]));
+              else ep.store_f(i, j, (float)s[v], f_al[pp][v] * f_sa[pp][v], f_sb[pp][v], f_be[pp][v], ep.bias_from_raw(f_bias[pp][v]));
             }
           }
         }
       }
     }
-    if (RBUF == 1) lds_barrier();  // the single buffer is rewritten by the next block
   }
   // the zero-fill units issued past the last block still target this workgroup's LDS
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");

@@ -51,6 +51,14 @@ void launch_decode_variant(const DecodeParams &prm, const zluda_gemm_plan &plan,
   }
 }
 
+template <int N, int I = 0, class F>
+void static_for_host(F &&f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for_host<N, I + 1>(f);
+  }
+}
+
 // every output of the problem can leave through the packed 8-byte store of decode_stream_kernel
 bool decode_packed_output(const GemmArgs &g, bool swapped) {
   const int64_t d_sr = swapped ? g.d_sj : g.d_si, d_st = swapped ? g.d_si : g.d_sj;
@@ -64,16 +72,18 @@ template <int NW, int SPW>
 uint32_t launch_decode_stream(const DecodeParams &prm, const zluda_gemm_plan &plan, int nb, hipStream_t s) {
   dim3 grid(plan.grid_x, plan.grid_y, 1), block(NW * 64);
   const bool fast = decode_packed_output(prm.g, prm.swapped != 0);
-  if (nb == 1) {
-    if (fast) hipLaunchKernelGGL((decode_stream_kernel<NW, SPW, 1, true>), grid, block, 0, s, prm);
-    else hipLaunchKernelGGL((decode_stream_kernel<NW, SPW, 1, false>), grid, block, 0, s, prm);
-  } else if constexpr (SPW <= kDecodeStreamMaxStepsTwoBlocks) {
-    if (fast) hipLaunchKernelGGL((decode_stream_kernel<NW, SPW, 2, true>), grid, block, 0, s, prm);
-    else hipLaunchKernelGGL((decode_stream_kernel<NW, SPW, 2, false>), grid, block, 0, s, prm);
-  } else {
-    return CUBLAS_STATUS_NOT_SUPPORTED;
-  }
-  return CUBLAS_STATUS_SUCCESS;
+  bool done = false;
+  static_for_host<4>([&](auto nb_c) {
+    constexpr int NB = decltype(nb_c)::value + 1;
+    if constexpr (NB * SPW <= kDecodeStreamMaxFragments) {
+      if (nb == NB) {
+        if (fast) hipLaunchKernelGGL((decode_stream_kernel<NW, SPW, NB, true>), grid, block, 0, s, prm);
+        else hipLaunchKernelGGL((decode_stream_kernel<NW, SPW, NB, false>), grid, block, 0, s, prm);
+        done = true;
+      }
+    }
+  });
+  return done ? CUBLAS_STATUS_SUCCESS : CUBLAS_STATUS_NOT_SUPPORTED;
 }
 
 uint32_t launch_decode(const Lowered &l, const zluda_gemm_plan &plan, hipStream_t s) {
@@ -88,7 +98,7 @@ uint32_t launch_decode(const Lowered &l, const zluda_gemm_plan &plan, hipStream_
   prm.spw = (ksteps + v.nw - 1) / v.nw;
   prm.nchunks = (prm.spw + v.steps - 1) / v.steps;
   const bool full = l.g.K == v.nw * v.steps * 64;
-  const int nb = T <= 16 ? 1 : 2;
+  const int nb = (T + 15) / 16;
   if (v.stream) {
     // the kernel addresses W through one 2 GiB buffer window and assumes K == nw * steps * 64
     const int64_t rows = plan.swapped ? l.g.N : l.g.M, ldw = plan.swapped ? l.g.b_sj : l.g.a_si;
@@ -118,7 +128,7 @@ uint32_t launch_decode(const Lowered &l, const zluda_gemm_plan &plan, hipStream_
     default: return CUBLAS_STATUS_INVALID_VALUE;
     }
   }
-  if (nb == 2 && v.steps > 8) return CUBLAS_STATUS_NOT_SUPPORTED;
+  if (nb > 2 || (nb == 2 && v.steps > 8)) return CUBLAS_STATUS_NOT_SUPPORTED;
   switch (plan.variant) {
   case 0: launch_decode_variant<8, 8>(prm, plan, nb, full, s); break;
   case 1: launch_decode_variant<8, 16>(prm, plan, nb, full, s); break;

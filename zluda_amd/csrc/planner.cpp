@@ -205,6 +205,22 @@ uint32_t lower_problem(const zluda_gemm_problem *p, bool dry, Lowered *out) {
 
 static bool is_f8(uint32_t t) { return t == CUDA_R_8F_E4M3 || t == CUDA_R_8F_E5M2; }
 
+static bool decode_variant_ok(const Lowered &l, int variant) {
+  const GemmArgs &g = l.g;
+  const DecodeVariant &v = kDecodeVariants[variant];
+  const int T = std::min(g.M, g.N), nb = (T + 15) / 16;
+  if (!v.stream) return nb == 1 || (nb == 2 && v.steps <= 8);  // token blocks multiply the fragment registers
+  const bool swapped = g.M < g.N;
+  const int64_t rows = swapped ? g.N : g.M, ldw = swapped ? g.b_sj : g.a_si;
+  return g.K == v.nw * v.steps * 64 && rows * ldw < 0x7fffffffll && nb * v.steps <= kDecodeStreamMaxFragments;
+}
+
+static bool any_decode_variant_ok(const Lowered &l) {
+  for (int v = 0; v < kNumDecodeVariants; v++)
+    if (decode_variant_ok(l, v)) return true;
+  return false;
+}
+
 bool family_supports(uint32_t kernel, const Lowered &l) {
   const GemmArgs &g = l.g;
   const bool fast_layout = l.a_kcontig && l.b_kcontig && l.aligned16;
@@ -224,7 +240,7 @@ bool family_supports(uint32_t kernel, const Lowered &l) {
            (g.K % 256) == 0 && ((((uintptr_t)g.a_scale) | ((uintptr_t)g.b_scale)) & 3) == 0 && d_fast;
   case ZLUDA_KERNEL_DECODE_W8A8:
     return fast_layout && g.a_type == CUDA_R_8I && g.b_type == CUDA_R_8I &&
-           std::min(g.M, g.N) <= 32 && std::max(g.M, g.N) >= 64;
+           std::min(g.M, g.N) <= kDecodeMaxTokens && std::max(g.M, g.N) >= 64 && any_decode_variant_ok(l);
   default: return false;
   }
 }
@@ -248,28 +264,26 @@ static void fill_mfma_plan(const Lowered &l, int variant, uint32_t cus, zluda_ge
   plan->workspace = 0;
 }
 
+// Relative throughput of one CU running tiles of each variant (measured on MI355X, int8 and fp8, K >= 1024;
+// variant 0 = 1).  Smaller tiles read more LDS and L2 bytes per MFMA.
+static const float kMfmaVariantEfficiency[kNumMfmaVariants] = {1.00f, 0.95f, 0.80f, 0.70f, 0.72f};
+
 static int pick_mfma_variant(const Lowered &l, uint32_t cus) {
   const GemmArgs &g = l.g;
   const bool swapped = g.d_si != 1;
   const uint32_t np = swapped ? g.N : g.M, nq = swapped ? g.M : g.N;
-  auto tiles = [&](int v) {
-    return (uint64_t)ceil_div(np, kMfmaVariants[v].bp) * ceil_div(nq, kMfmaVariants[v].bq) * g.batch;
-  };
-  // the biggest tile that still gives (nearly) every CU a workgroup
-  if (tiles(0) * 4 >= (uint64_t)cus * 3) return 0;
-  if (tiles(2) * 4 >= (uint64_t)cus * 3) return 2;
-  return 3;
-}
-
-static bool decode_variant_ok(const Lowered &l, int variant) {
-  const GemmArgs &g = l.g;
-  const DecodeVariant &v = kDecodeVariants[variant];
-  const int T = std::min(g.M, g.N);
-  if (!v.stream) return T <= 16 || v.steps <= 8;  // two token blocks double the fragment registers
-  const bool swapped = g.M < g.N;
-  const int64_t rows = swapped ? g.N : g.M, ldw = swapped ? g.b_sj : g.a_si;
-  return g.K == v.nw * v.steps * 64 && rows * ldw < 0x7fffffffll &&
-         (T <= 16 || v.steps <= kDecodeStreamMaxStepsTwoBlocks);
+  // cost = rounds of workgroups over the CUs x time of one tile; the tile shapes trade efficiency
+  // per CU against how evenly the problem fills the chip
+  int best = 0;
+  double best_cost = 0;
+  for (int v = 0; v < kNumMfmaVariants; v++) {
+    const MfmaVariant &t = kMfmaVariants[v];
+    const uint64_t tiles = (uint64_t)ceil_div(np, t.bp) * ceil_div(nq, t.bq) * g.batch;
+    const uint64_t rounds = (tiles + cus - 1) / cus;
+    const double cost = (double)rounds * t.bp * t.bq / kMfmaVariantEfficiency[v];
+    if (v == 0 || cost < best_cost) { best = v; best_cost = cost; }
+  }
+  return best;
 }
 
 static void fill_decode_plan(const Lowered &l, int variant, uint32_t cus, zluda_gemm_plan *plan) {

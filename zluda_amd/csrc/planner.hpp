@@ -40,7 +40,10 @@ constexpr DecodeVariant kDecodeVariants[] = {
     {4, 20, 1},  // 14: K = 5120
 };
 constexpr int kNumDecodeVariants = sizeof(kDecodeVariants) / sizeof(kDecodeVariants[0]);
-constexpr int kDecodeStreamMaxStepsTwoBlocks = 12;  // 17..32 tokens double the activation registers
+// Tokens come in blocks of 16; a wave keeps blocks x steps activation fragments (4 VGPRs each) in
+// registers for the whole kernel.
+constexpr int kDecodeStreamMaxFragments = 32;  // stream kernel: up to 64 tokens at K = 4096
+constexpr int kDecodeMaxTokens = 64;
 
 struct Lowered {
   GemmArgs g;
