@@ -264,17 +264,23 @@ class Case:
         nbytes = self.dtot * np.dtype(self.d_np).itemsize
         return dt[:nbytes].cpu().numpy().view(self.d_np).copy()
 
-    def run_gpu(self, api, forced_kernel=None, forced_variant=-1, offset_bytes=0):
-        """Returns (status, D storage, kernel family, variant).  offset_bytes misaligns A and B."""
+    def run_gpu(self, api, forced_kernel=None, forced_variant=-1, offset_bytes=0, workspace_bytes=0):
+        """Returns (status, D storage, kernel family, variant).  offset_bytes misaligns A and B;
+        workspace_bytes > 0 offers that much workspace (preference and call), which is what lets the
+        planner split K.  self.last_workspace_needed = what the heuristic asked for."""
         import torch
         keep, ptr, dt = self.upload(offset_bytes)
-        call = MatmulCall(api, self.spec, forced_kernel=forced_kernel, forced_variant=forced_variant)
+        call = MatmulCall(api, self.spec, forced_kernel=forced_kernel, forced_variant=forced_variant,
+                          max_workspace=workspace_bytes)
+        ws = torch.empty(max(workspace_bytes, 16), dtype=torch.uint8, device="cuda:0") if workspace_bytes else None
+        self.last_workspace_needed = call.heuristic[0].workspaceSize if call.heuristic else None
         try:
             call.set_pointers(bias=ptr["bias"], a_scale=ptr["a_scale"], b_scale=ptr["b_scale"],
                               c_scale=ptr["c_scale"], d_scale=ptr["d_scale"])
             alpha, beta = self.scalars(ptr)
             stream = torch.cuda.current_stream().cuda_stream
-            st = call.run(alpha, ptr["A"], ptr["B"], beta, ptr["C"], ptr["D"], None, 0, stream)
+            st = call.run(alpha, ptr["A"], ptr["B"], beta, ptr["C"], ptr["D"],
+                          ws.data_ptr() if ws is not None else None, workspace_bytes, stream)
             torch.cuda.synchronize()
             return st, self.download(dt), call.kernel, call.variant
         finally:

@@ -62,11 +62,10 @@ def test_decode_shapes_around_the_limits(gpu_api):
     assert run(gpu_api, dict(dec, m=4099, n=32, k=4096), 341, int_dist="normal") == K.ZLUDA_KERNEL_DECODE_W8A8   # rows % 4 != 0
     assert run(gpu_api, dict(dec, m=2048, n=3, k=11008), 342, int_dist="normal") == K.ZLUDA_KERNEL_DECODE_W8A8  # K outside the stream table
     assert run(gpu_api, dict(dec, m=512, n=16, k=4096, batch=3), 343, int_dist="normal") == K.ZLUDA_KERNEL_DECODE_W8A8
-    # up to 64 tokens stream (K = 4096: 4 token blocks x 8 steps of activation fragments); 65 do not
-    assert run(gpu_api, dict(dec, m=2048, n=33, k=4096), 344, int_dist="normal") == K.ZLUDA_KERNEL_DECODE_W8A8
-    assert run(gpu_api, dict(dec, m=2048, n=64, k=4096), 346, int_dist="normal") == K.ZLUDA_KERNEL_DECODE_W8A8
-    assert run(gpu_api, dict(dec, m=2048, n=65, k=4096), 347, int_dist="normal") == K.ZLUDA_KERNEL_MFMA_I8
-    assert run(gpu_api, dict(dec, m=2048, n=48, k=8192), 348, int_dist="normal") == K.ZLUDA_KERNEL_MFMA_I8   # 3 x 16 fragments
+    # beyond 32 tokens the planner prefers small MFMA tiles (the decode family itself runs up to 64)
+    assert run(gpu_api, dict(dec, m=2048, n=32, k=4096), 344, int_dist="normal") == K.ZLUDA_KERNEL_DECODE_W8A8
+    assert run(gpu_api, dict(dec, m=2048, n=33, k=4096), 346, int_dist="normal") == K.ZLUDA_KERNEL_MFMA_I8
+    assert run(gpu_api, dict(dec, m=2048, n=64, k=4096), 347, int_dist="normal") == K.ZLUDA_KERNEL_MFMA_I8
     # f16 output, ld > rows (the packed store needs ld % 4 == 0: 2052 qualifies, 2051 does not)
     for ld in (2052, 2051):
         run(gpu_api, dict(dec, c_type=K.CUDA_R_16F, d_type=K.CUDA_R_16F, m=2048, n=8, k=4096, ldd=ld, ldc=ld), 345, int_dist="normal")
@@ -162,3 +161,32 @@ def test_gemm_ex_entry_points(gpu_api, ta, tb):
                                  C.addressof(one), None, K.CUDA_R_32I, 1, K.CUBLAS_COMPUTE_32I, stream) == 0
     assert gpu_api.zluda_gemm_ex(0, 0, -1, 4, 4, C.addressof(one), None, K.CUDA_R_8I, 1, None, K.CUDA_R_8I, 4,
                                  C.addressof(one), None, K.CUDA_R_32I, 1, K.CUBLAS_COMPUTE_32I, stream) == K.CUBLAS_STATUS_INVALID_VALUE
+
+
+def test_split_k_through_the_workspace(gpu_api):
+    """few tiles, long K: with a workspace the planner splits K (partial tiles + reduce kernel);
+    int8 stays bit-exact, the float epilogues keep their tolerance, every layout/epilogue feature
+    goes through the second kernel"""
+    ws = 64 << 20
+    for spec, seed in ((dict(I8, m=1024, n=256, k=8192), 370),
+                       (dict(I8, m=300, n=200, k=8208, with_c=True, batch=2, ldd=304, ldc=320), 371),
+                       (dict(I8, transa=0, transb=1, order_a=1, order_b=1, order_c=1, order_d=1, m=192, n=320, k=8192, with_c=True), 372),
+                       (dict(I8, c_type=K.CUDA_R_16BF, d_type=K.CUDA_R_16BF, scale_type=K.CUDA_R_32F, m=512, n=128, k=6144,
+                             epilogue=K.CUBLASLT_EPILOGUE_RELU_BIAS, bias_type=K.CUDA_R_32F,
+                             pointer_mode=K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO,
+                             b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F, alpha_range=(0.001, 0.002)), 373),
+                       (dict(F8, m=640, n=256, k=8192, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS, with_scalar_scales=True,
+                             scale_range=(0.02, 0.03)), 374)):
+        print("split-K case", spec, flush=True)
+        case = Case(spec, seed)
+        ref = case.run_oracle()
+        st, got, kern, variant = case.run_gpu(gpu_api, workspace_bytes=ws)
+        assert st == 0 and kern in (K.ZLUDA_KERNEL_MFMA_I8, K.ZLUDA_KERNEL_MFMA_F8)
+        assert case.last_workspace_needed and case.last_workspace_needed <= ws, "the planner did not split K"
+        case.compare(got, ref)
+    # the same token with too little workspace at call time: the call must not use it
+    case = Case(dict(I8, m=1024, n=256, k=8192), 375)
+    ref = case.run_oracle()
+    st, got, kern, variant = case.run_gpu(gpu_api, workspace_bytes=0)
+    assert st == 0 and case.last_workspace_needed == 0
+    case.compare(got, ref)

@@ -16,12 +16,13 @@ MX = dict(a_type=K.CUDA_R_4F_E2M1, b_type=K.CUDA_R_4F_E2M1, d_type=K.CUDA_R_16BF
           b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_VEC32_UE8M0)
 
 
-def plan(api, spec, forced=0, variant=-1, cus=256, a_ptr=0, b_ptr=0):
+def plan(api, spec, forced=0, variant=-1, cus=256, a_ptr=0, b_ptr=0, workspace=0):
     case = Case.__new__(Case)
     case.spec = dict(spec)
     case.spec.setdefault("c_type", spec["d_type"])
     case.batch = spec.get("batch", 1)
     p = case.problem({"A": a_ptr, "B": b_ptr, "D": 0, "alpha": 0, "beta": 0})
+    p.workspace_size = workspace
     out = abi.zluda_gemm_plan()
     st = api.zluda_gemm_plan_problem(C.byref(p), forced, variant, cus, C.byref(out))
     return st, out
@@ -47,7 +48,7 @@ def test_baseline_configs_pick_the_intended_kernels(api):
 
 def test_small_problems_get_smaller_tiles(api):
     st, p = plan(api, dict(I8, m=1024, n=1024, k=1024, transa=1))
-    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_I8 and p.variant == 4 and p.grid_x == 64
+    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_I8 and p.variant == 6 and p.grid_x == 256
     st, p = plan(api, dict(I8, m=4096, n=2048, k=1024, transa=1))
     assert st == 0 and p.variant == 2 and p.grid_x == 16 * 16
 
@@ -98,8 +99,29 @@ def test_fp4_must_be_k_contiguous(api):
 
 def test_forced_variants(api):
     spec = dict(I8, m=4096, n=4096, k=4096, transa=1)
-    for v, (grid, block) in enumerate([(256, 512), (256, 256), (512, 256), (1024, 256), (1024, 256)]):
+    for v, (grid, block) in enumerate([(256, 512), (256, 256), (512, 256), (1024, 256), (1024, 256), (2048, 256), (4096, 256)]):
         st, p = plan(api, spec, forced=K.ZLUDA_KERNEL_MFMA_I8, variant=v)
         assert st == 0 and p.variant == v and p.grid_x == grid and p.block == block
-    assert plan(api, spec, forced=K.ZLUDA_KERNEL_MFMA_I8, variant=5)[0] == K.CUBLAS_STATUS_INVALID_VALUE
+    assert plan(api, spec, forced=K.ZLUDA_KERNEL_MFMA_I8, variant=7)[0] == K.CUBLAS_STATUS_INVALID_VALUE
     assert plan(api, spec, forced=K.ZLUDA_KERNEL_MFMA_F8)[0] == K.CUBLAS_STATUS_NOT_SUPPORTED
+
+
+def test_split_k_needs_workspace_and_few_tiles(api):
+    """few tiles and a long K: grid_z workgroups share a tile's K range when the workspace holds the
+    padded partial tiles (4 bytes x splits x batch x padded M x padded N); never otherwise"""
+    spec = dict(I8, m=1024, n=256, k=8192, transa=1)
+
+    def plan_ws(spec, ws):
+        return plan(api, spec, workspace=ws)
+    st, p = plan_ws(spec, 0)
+    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_I8 and p.grid_z == 1 and p.workspace == 0
+    st, p = plan_ws(spec, 64 << 20)
+    assert st == 0 and p.grid_z > 1 and p.grid_x * p.grid_z <= 256
+    assert p.workspace == p.grid_z * 1024 * 256 * 4 <= 64 << 20
+    # a workspace that holds only 3 partial matrices limits the split
+    st, p3 = plan_ws(spec, 3 * 1024 * 256 * 4)
+    assert st == 0 and p3.grid_z == 3 and p3.workspace == 3 * 1024 * 256 * 4
+    # enough tiles already, short K, or MXFP4: no split
+    assert plan_ws(dict(I8, m=4096, n=4096, k=8192, transa=1), 1 << 30)[1].grid_z == 1
+    assert plan_ws(dict(I8, m=1024, n=256, k=256, transa=1), 1 << 30)[1].grid_z == 1
+    assert plan_ws(dict(MX, m=1024, n=256, k=8192, transa=1), 1 << 30)[1].grid_z == 1

@@ -478,6 +478,7 @@ cublasStatus_t cublasLtMatmulAlgoGetHeuristic(
   cublasStatus_t st = build_problem(operationDesc, Adesc, Bdesc, Cdesc, Ddesc, &p);
   if (st) return st;
   *returnAlgoCount = 0;
+  p.workspace_size = pref->max_workspace;  // what split-K may count on
   const uint32_t cus = zluda_gemm_device_cu_count();
   // candidates, best first: the planner's own choice, then the generic kernel
   uint32_t forced = ZLUDA_KERNEL_AUTO;

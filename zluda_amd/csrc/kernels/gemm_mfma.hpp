@@ -60,6 +60,10 @@ struct MfmaParams {
   int32_t swapped;           // P = op(B)^T rows, Q = op(A) rows
   int32_t tiles_p, tiles_q;  // tile counts along P and Q
   int32_t group_p;           // raster group height (tiles along P)
+  // split-K (splits > 1): workgroup z of gridDim.z handles stages [z * split_stages, ...) of K and
+  // writes its raw partial tile to ws[(z * batch + bt)][tiles_q * BQ][tiles_p * BP] (int32 / fp32)
+  int32_t splits, split_stages;
+  void *ws;
 };
 
 // General fused epilogue of the MFMA kernels: any D type, C read, vectors along either dimension,
@@ -232,6 +236,27 @@ __device__ __forceinline__ void mfma_store_tile_i32(const MfmaParams &prm, v16i 
           __builtin_amdgcn_raw_buffer_store_b32(acc[a][b][v] * ialpha, rs, voff, soff + b * 128, 0);
       }
   }
+}
+
+// Split-K partial tile: the raw accumulators (int32, or fp32 bit patterns) of a whole tile into the
+// padded workspace matrix of pitch `ws_pitch` dwords; same store pattern as mfma_store_tile_i32.
+template <int WP, int WQ, int WTP, int WTQ, class AccV>
+__device__ __forceinline__ void mfma_store_tile_raw(int32_t *ws_tile, int ws_pitch, AccV (&acc)[WTQ / 32][WTP / 32]) {
+  constexpr int TP = WTP / 32, TQ = WTQ / 32;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wp = wave % WP, wq = wave / WP;
+  const int lr = lane & 31, gsel = lane >> 5;
+  int32_t *Dw = ws_tile + (int64_t)(wq * WTQ) * ws_pitch + wp * WTP;
+  const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)Dw, 0, 0xFFFFFFFF, 0x00020000);
+  const int voff = (4 * gsel * ws_pitch + lr) * 4;
+#pragma unroll
+  for (int a = 0; a < TQ; a++)
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+      const int soff = (a * 32 + 8 * (v >> 2) + (v & 3)) * ws_pitch * 4;  // uniform
+#pragma unroll
+      for (int b = 0; b < TP; b++) __builtin_amdgcn_raw_buffer_store_b32(to_bits(acc[a][b][v]), rs, voff, soff + b * 128, 0);
+    }
 }
 
 // Fast path 2: float epilogue without a C read (beta == 0) on a full tile, D of type bf16, f16 or

@@ -102,7 +102,15 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
     Pg = (const uint8_t *)g.B + g.b_sb * bt * ebits / 8; ldp = (int)(g.b_sj * ebits / 8);
     Qg = (const uint8_t *)g.A + g.a_sb * bt * ebits / 8; ldq = (int)(g.a_si * ebits / 8);
   }
-  const int KT = (Kbytes + BKB_ - 1) / BKB_;      // real stages
+  // split-K: this workgroup's share of the stages; the pointers move, the rest of the kernel sees a
+  // shorter K
+  int Kbytes_local = Kbytes;
+  if (prm.splits > 1) {
+    const int k0 = (int)blockIdx.z * prm.split_stages * BKB_;
+    Pg += k0; Qg += k0;
+    Kbytes_local = max(0, min(Kbytes - k0, prm.split_stages * BKB_));
+  }
+  const int KT = (Kbytes_local + BKB_ - 1) / BKB_;  // real stages
   const int KTR = (KT + SPT - 1) / SPT * SPT;     // stages run (padding stages multiply zeros)
 
   // 2 GiB raw buffer windows: an offset with bit 31 set is out of range and reads as zero
@@ -119,7 +127,7 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
   for (int i = 0; i < LP; i++) voffP[i] = min(p0 + drow + RPP * i, NP - 1) * ldp + dcg * 16;
 #pragma unroll
   for (int i = 0; i < LQ; i++) voffQ[i] = min(q0 + drow + RPP * i, NQ - 1) * ldq + dcg * 16;
-  const int tail_bytes = Kbytes - (KT - 1) * BKB_;
+  const int tail_bytes = Kbytes_local - (KT - 1) * BKB_;
   const int oob_last = dcg * 16 < tail_bytes ? 0 : (int)0x80000000;
 
   // MX block scales: the [row][K/32] byte tensors of both operands, through buffer windows of
@@ -325,6 +333,12 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
   // every wave is done with the LDS tiles (and every DMA has landed) before they become staging
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
+  if (prm.splits > 1) {
+    const int ws_np = prm.tiles_p * BP, ws_nq = prm.tiles_q * BQ;
+    int32_t *ws_tile = (int32_t *)prm.ws + ((int64_t)blockIdx.z * g.batch + bt) * ws_np * ws_nq + (int64_t)q0 * ws_np + p0;
+    mfma_store_tile_raw<WP, WQ, WTP, WTQ>(ws_tile, ws_np, acc);
+    return;
+  }
   mfma_store_tile<KIND, WP, WQ, WTP, WTQ>(prm, acc, (int *)&lds[0], sizeof(lds), p0, q0, NP, NQ, bt);
 }
 

@@ -7,6 +7,7 @@
 #include "kernels/decode_stream.hpp"
 #include "kernels/decode_w8a8.hpp"
 #include "kernels/gemm_generic.hpp"
+#include "kernels/splitk_reduce.hpp"
 #include "mfma_launch.hpp"
 #include "planner.hpp"
 
@@ -16,7 +17,7 @@ namespace {
 
 inline int f8_fmt(uint32_t t) { return t == CUDA_R_8F_E5M2 ? 1 : 0; }
 
-uint32_t launch_mfma(const Lowered &l, const zluda_gemm_plan &plan, hipStream_t s) {
+uint32_t launch_mfma(const Lowered &l, const zluda_gemm_plan &plan, const zluda_gemm_problem *p, hipStream_t s) {
   MfmaParams prm;
   prm.g = l.g;
   prm.swapped = plan.swapped;
@@ -26,17 +27,43 @@ uint32_t launch_mfma(const Lowered &l, const zluda_gemm_plan &plan, hipStream_t 
   prm.tiles_p = (np + v.bp - 1) / v.bp;
   prm.tiles_q = (nq + v.bq - 1) / v.bq;
   prm.group_p = 8;
+  prm.splits = 1; prm.split_stages = 0; prm.ws = nullptr;
   if ((uint32_t)(prm.tiles_p * prm.tiles_q) != plan.grid_x) return CUBLAS_STATUS_INVALID_VALUE;
+  if (plan.grid_z > 1) {
+    // split-K: partial tiles go through the caller's workspace
+    if (plan.kernel == ZLUDA_KERNEL_MFMA_MXF4) return CUBLAS_STATUS_INVALID_VALUE;
+    const uint64_t need = (uint64_t)plan.grid_z * l.g.batch * prm.tiles_p * v.bp * prm.tiles_q * v.bq * 4;
+    if (!p->workspace || (((uintptr_t)p->workspace) & 15) || p->workspace_size < need || plan.workspace != need)
+      return CUBLAS_STATUS_INVALID_VALUE;
+    const int kbytes = l.g.K;  // 8-bit operands
+    const int stages = (kbytes + v.bkb - 1) / v.bkb;
+    prm.splits = (int32_t)plan.grid_z;
+    prm.split_stages = (stages + prm.splits - 1) / prm.splits;
+    prm.ws = p->workspace;
+  }
+  uint32_t st;
   switch (plan.kernel) {
-  case ZLUDA_KERNEL_MFMA_I8: return launch_mfma_i8(prm, plan, s);
-  case ZLUDA_KERNEL_MFMA_MXF4: return launch_mfma_mxf4(prm, plan, s);
+  case ZLUDA_KERNEL_MFMA_I8: st = launch_mfma_i8(prm, plan, s); break;
+  case ZLUDA_KERNEL_MFMA_MXF4: st = launch_mfma_mxf4(prm, plan, s); break;
   case ZLUDA_KERNEL_MFMA_F8: {
     // MFMA operand "A" is Q, operand "B" is P (see gemm_mfma.hpp)
     const int fa = f8_fmt(l.g.a_type), fb = f8_fmt(l.g.b_type);
-    return launch_mfma_f8(prm, plan, plan.swapped ? fa : fb, plan.swapped ? fb : fa, s);
+    st = launch_mfma_f8(prm, plan, plan.swapped ? fa : fb, plan.swapped ? fb : fa, s);
+    break;
   }
   default: return CUBLAS_STATUS_INTERNAL_ERROR;
   }
+  if (st || prm.splits == 1) return st;
+  SplitKReduceParams rp;
+  rp.g = l.g;
+  rp.swapped = plan.swapped;
+  rp.splits = prm.splits;
+  rp.acc_is_int = plan.kernel == ZLUDA_KERNEL_MFMA_I8;
+  rp.ws_np = prm.tiles_p * v.bp;
+  rp.ws_nq = prm.tiles_q * v.bq;
+  rp.ws = (const int32_t *)p->workspace;
+  hipLaunchKernelGGL(splitk_reduce_kernel, dim3((np + 1023) / 1024, nq, l.g.batch), dim3(256), 0, s, rp);
+  return CUBLAS_STATUS_SUCCESS;
 }
 
 template <int NW, int STEPS>
@@ -171,7 +198,7 @@ extern "C" uint32_t zluda_gemm_launch(const zluda_gemm_problem *p, const zluda_g
     break;
   }
   case ZLUDA_KERNEL_MFMA_I8: case ZLUDA_KERNEL_MFMA_F8: case ZLUDA_KERNEL_MFMA_MXF4:
-    if ((st = launch_mfma(l, *plan, s))) return st;
+    if ((st = launch_mfma(l, *plan, p, s))) return st;
     break;
   case ZLUDA_KERNEL_DECODE_W8A8:
     if ((st = launch_decode(l, *plan, s))) return st;

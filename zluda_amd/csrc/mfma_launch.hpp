@@ -11,7 +11,7 @@ namespace zluda_amd {
 // plan.variant indexes kMfmaVariants (planner.hpp); the template arguments below restate that table.
 template <int KIND, int FQ, int FP>
 inline uint32_t launch_mfma_variant(const MfmaParams &prm, const zluda_gemm_plan &plan, hipStream_t s) {
-  dim3 grid(plan.grid_x, plan.grid_y, 1);
+  dim3 grid(plan.grid_x, plan.grid_y, plan.grid_z > 1 ? plan.grid_z : 1);  // z: split-K shares
 #define ZLUDA_MFMA_CASE(V, BP, BQ, WP, WQ, BKB, NS)                                                        \
   case V:                                                                                                  \
     static_assert(kMfmaVariants[V].bp == BP && kMfmaVariants[V].bq == BQ && kMfmaVariants[V].wp == WP &&   \
@@ -26,6 +26,8 @@ inline uint32_t launch_mfma_variant(const MfmaParams &prm, const zluda_gemm_plan
     ZLUDA_MFMA_CASE(2, 256, 128, 2, 2, 128, 2)
     ZLUDA_MFMA_CASE(3, 128, 128, 2, 2, 128, 2)
     ZLUDA_MFMA_CASE(4, 128, 128, 2, 2, 64, 4)
+    ZLUDA_MFMA_CASE(5, 128, 64, 2, 2, 128, 3)
+    ZLUDA_MFMA_CASE(6, 64, 64, 2, 2, 128, 3)
   default: return CUBLAS_STATUS_INVALID_VALUE;
   }
 #undef ZLUDA_MFMA_CASE

@@ -247,7 +247,8 @@ bool family_supports(uint32_t kernel, const Lowered &l) {
 
 static uint32_t ceil_div(uint32_t a, uint32_t b) { return (a + b - 1) / b; }
 
-static void fill_mfma_plan(const Lowered &l, int variant, uint32_t cus, zluda_gemm_plan *plan) {
+static void fill_mfma_plan(const Lowered &l, int variant, uint32_t cus, uint64_t workspace_size,
+                           zluda_gemm_plan *plan) {
   const GemmArgs &g = l.g;
   const MfmaVariant &v = kMfmaVariants[variant];
   const bool swapped = g.d_si != 1;  // row-major D: compute D^T
@@ -262,11 +263,29 @@ static void fill_mfma_plan(const Lowered &l, int variant, uint32_t cus, zluda_ge
   const uint32_t per_cu = std::max(1u, std::min(160u * 1024u / lds, 2048u / plan->block));
   plan->waves = (float)plan->grid_x * plan->grid_y / (float)(cus * per_cu);
   plan->workspace = 0;
+  // Split-K: when even the chosen tiles leave half of the CUs idle and K is long, grid_z workgroups
+  // share a tile's K range, write their fp32 / int32 partial tiles to the workspace and a second
+  // kernel sums them and applies the epilogue.  Only if the caller's workspace holds the partial
+  // tiles (padded to whole tiles); never for MXFP4 (its scale chunks are tied to absolute K).
+  const uint64_t tiles = (uint64_t)plan->grid_x * plan->grid_y;
+  const uint32_t kt = ceil_div((uint32_t)((int64_t)g.K * (g.a_type == CUDA_R_4F_E2M1 ? 4 : 8) / 8), v.bkb);
+  // (below ~6 KiB of K per row the second kernel and the workspace traffic cost more than the idle CUs)
+  const uint32_t kbytes = kt * v.bkb;
+  if (g.a_type != CUDA_R_4F_E2M1 && tiles * 2 <= cus && kbytes >= 6144 && (uint64_t)tp * v.bp <= (1u << 20)) {
+    uint32_t s = (uint32_t)std::min<uint64_t>({8, cus / tiles, kbytes / 2048});
+    const uint64_t per_split = (uint64_t)g.batch * tp * v.bp * tq * v.bq * 4;
+    while (s > 1 && s * per_split > workspace_size) s--;
+    if (s > 1) {
+      plan->grid_z = s;
+      plan->workspace = s * per_split;
+      plan->waves = (float)tiles * s / (float)(cus * per_cu);
+    }
+  }
 }
 
 // Relative throughput of one CU running tiles of each variant (measured on MI355X, int8 and fp8, K >= 1024;
 // variant 0 = 1).  Smaller tiles read more LDS and L2 bytes per MFMA.
-static const float kMfmaVariantEfficiency[kNumMfmaVariants] = {1.00f, 0.95f, 0.80f, 0.70f, 0.72f};
+static const float kMfmaVariantEfficiency[kNumMfmaVariants] = {1.00f, 0.95f, 0.80f, 0.70f, 0.72f, 0.55f, 0.40f};
 
 static int pick_mfma_variant(const Lowered &l, uint32_t cus) {
   const GemmArgs &g = l.g;
@@ -345,8 +364,10 @@ extern "C" uint32_t zluda_gemm_plan_problem(const zluda_gemm_problem *p, uint32_
   if (kernel == ZLUDA_KERNEL_AUTO) {
     static const uint32_t order[] = {ZLUDA_KERNEL_DECODE_W8A8, ZLUDA_KERNEL_MFMA_I8, ZLUDA_KERNEL_MFMA_F8,
                                      ZLUDA_KERNEL_MFMA_MXF4, ZLUDA_KERNEL_GENERIC};
-    for (uint32_t k : order)
+    for (uint32_t k : order) {
+      if (k == ZLUDA_KERNEL_DECODE_W8A8 && std::min(l.g.M, l.g.N) > kDecodeAutoMaxTokens) continue;
       if (family_supports(k, l)) { kernel = k; break; }
+    }
   } else if (!family_supports(kernel, l)) {
     return CUBLAS_STATUS_NOT_SUPPORTED;
   }
@@ -362,7 +383,7 @@ extern "C" uint32_t zluda_gemm_plan_problem(const zluda_gemm_problem *p, uint32_
   case ZLUDA_KERNEL_MFMA_I8: case ZLUDA_KERNEL_MFMA_F8: case ZLUDA_KERNEL_MFMA_MXF4: {
     int v = forced_variant >= 0 ? forced_variant : pick_mfma_variant(l, cu_count);
     if (v >= kNumMfmaVariants) return CUBLAS_STATUS_INVALID_VALUE;
-    fill_mfma_plan(l, v, cu_count, plan);
+    fill_mfma_plan(l, v, cu_count, p->workspace_size, plan);
     break;
   }
   case ZLUDA_KERNEL_DECODE_W8A8: {

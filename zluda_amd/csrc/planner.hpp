@@ -15,6 +15,8 @@ constexpr MfmaVariant kMfmaVariants[] = {
     {256, 128, 2, 2, 128, 2},  // 2: 4 waves, 128x64 per wave
     {128, 128, 2, 2, 128, 2},  // 3: 4 waves, 64x64 per wave, two workgroups per CU
     {128, 128, 2, 2, 64, 4},   // 4: same tile, half-line stages, deeper ring (short K)
+    {128, 64, 2, 2, 128, 3},   // 5: 4 waves, 64x32 per wave: skinny problems
+    {64, 64, 2, 2, 128, 3},    // 6: 4 waves, 32x32 per wave: problems of a few hundred tiles at most
 };
 constexpr int kNumMfmaVariants = sizeof(kMfmaVariants) / sizeof(kMfmaVariants[0]);
 
@@ -43,7 +45,8 @@ constexpr int kNumDecodeVariants = sizeof(kDecodeVariants) / sizeof(kDecodeVaria
 // Tokens come in blocks of 16; a wave keeps blocks x steps activation fragments (4 VGPRs each) in
 // registers for the whole kernel.
 constexpr int kDecodeStreamMaxFragments = 32;  // stream kernel: up to 64 tokens at K = 4096
-constexpr int kDecodeMaxTokens = 64;
+constexpr int kDecodeMaxTokens = 64;      // what the family can run
+constexpr int kDecodeAutoMaxTokens = 32;  // what the planner gives it: beyond, 64x64 MFMA tiles measure faster
 
 struct Lowered {
   GemmArgs g;
