@@ -57,7 +57,7 @@ WORKLOADS = {
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # script (each counter scaled by what it reads for the 256 MiB copy of --copy-probe: x2.000 and x1.000).
 # The summaries are profiles/<kernel>_<workload>.txt; re-measure after changing a kernel's tiling.
-MEASURED_TRAFFIC = {"c2": 167907551, "i8_8192": 1074766608, "c3": 60248442, "c4": 941143436, "c5": 2250512335}
+MEASURED_TRAFFIC = {"c2": 167932106, "i8_8192": 1074777202, "c3": 60076820, "c4": 941640909, "c5": 2250162262}
 
 
 def algorithmic(spec):
