@@ -248,7 +248,9 @@ cublasStatus_t cublasLtMatrixTransform(cublasLtHandle_t lightHandle,
                                        const void *B, cublasLtMatrixLayout_t Bdesc, void *C,
                                        cublasLtMatrixLayout_t Cdesc, cudaStream_t stream);
 
-/* [n/s] */
+/* [ext] initialises caller-provided storage (256 bytes for a matmul descriptor, 64 for a layout or a
+ * preference: cuda_types/src/cublaslt.rs:43-83) the way the matching Create call does; such an object
+ * is never passed to Destroy.  Unimplemented in the reference (zluda_blaslt/src/lib.rs:44-70). */
 cublasStatus_t cublasLtMatrixLayoutInit_internal(cublasLtMatrixLayout_t matLayout, size_t size,
                                                  cudaDataType_t type, uint64_t rows,
                                                  uint64_t cols, int64_t ld);
@@ -264,7 +266,7 @@ cublasStatus_t cublasLtMatrixLayoutGetAttribute(cublasLtMatrixLayout_t matLayout
                                                 cublasLtMatrixLayoutAttribute_t attr, void *buf,
                                                 size_t sizeInBytes, size_t *sizeWritten);
 
-/* [n/s] */
+/* [ext] as cublasLtMatrixLayoutInit_internal */
 cublasStatus_t cublasLtMatmulDescInit_internal(cublasLtMatmulDesc_t matmulDesc, size_t size,
                                                cublasComputeType_t computeType,
                                                cudaDataType_t scaleType);
@@ -294,7 +296,7 @@ cublasStatus_t cublasLtMatrixTransformDescGetAttribute(
     cublasLtMatrixTransformDesc_t transformDesc, cublasLtMatrixTransformDescAttributes_t attr,
     void *buf, size_t sizeInBytes, size_t *sizeWritten);
 
-/* [n/s] */
+/* [ext] as cublasLtMatrixLayoutInit_internal */
 cublasStatus_t cublasLtMatmulPreferenceInit_internal(cublasLtMatmulPreference_t pref, size_t size);
 /* [live] zluda_blaslt/src/impl.rs:330-358 */
 cublasStatus_t cublasLtMatmulPreferenceCreate(cublasLtMatmulPreference_t *pref);

@@ -163,9 +163,43 @@ def test_unimplemented_exports_return_not_supported(api):
     assert api.cublasLtLoggerOpenFile(b"/dev/null") == NS
     assert api.cublasLtHeuristicsCacheSetCapacity(8) == NS
     assert api.cublasLtMatrixTransformDescCreate(C.byref(C.c_void_p()), abi.CUDA_R_32F) == NS
-    assert api.cublasLtMatmulPreferenceInit_internal(None, 64) == NS
+    assert api.cublasLtMatrixTransformDescInit_internal(C.create_string_buffer(64), 64, abi.CUDA_R_32F) == NS
     assert api.cublasLtDisableCpuInstructionsSetMask(1) == 0
     assert api.cublasLtDisableCpuInstructionsSetMask(0) == 1
+
+
+def test_init_internal_builds_descriptors_in_caller_storage(api):
+    """the cublasLt*Init() inlines of the CUDA header pass their own opaque structs: 256 bytes for a matmul
+    descriptor, 64 for a layout or a preference (cuda_types/src/cublaslt.rs:43-83)"""
+    IV = abi.CUBLAS_STATUS_INVALID_VALUE
+    desc, pref = C.create_string_buffer(256), C.create_string_buffer(64)
+    lay = [C.create_string_buffer(64) for _ in range(3)]
+    assert api.cublasLtMatmulDescInit_internal(desc, 256, abi.CUBLAS_COMPUTE_32I, abi.CUDA_R_32I) == 0
+    assert api.cublasLtMatmulDescInit_internal(desc, 16, abi.CUBLAS_COMPUTE_32I, abi.CUDA_R_32I) == IV
+    assert api.cublasLtMatmulDescInit_internal(None, 256, abi.CUBLAS_COMPUTE_32I, abi.CUDA_R_32I) == IV
+    assert api.cublasLtMatmulPreferenceInit_internal(pref, 64) == 0
+    assert api.cublasLtMatmulPreferenceInit_internal(None, 64) == IV
+    assert api.cublasLtMatmulPreferenceInit_internal(pref, 8) == IV
+    for buf, typ in zip(lay, (abi.CUDA_R_8I, abi.CUDA_R_8I, abi.CUDA_R_32I)):
+        assert api.cublasLtMatrixLayoutInit_internal(buf, 64, typ, 512, 512, 512) == 0
+    assert api.cublasLtMatrixLayoutInit_internal(lay[0], 32, abi.CUDA_R_8I, 512, 512, 512) == IV
+    # they behave like created ones: attributes, heuristic
+    op = C.c_int32(abi.CUBLAS_OP_T)
+    assert api.cublasLtMatmulDescSetAttribute(desc, abi.CUBLASLT_MATMUL_DESC_TRANSA, C.byref(op), 4) == 0
+    back, wrote = C.c_int32(-1), C.c_size_t()
+    assert api.cublasLtMatmulDescGetAttribute(desc, abi.CUBLASLT_MATMUL_DESC_TRANSA, C.byref(back), 4, C.byref(wrote)) == 0
+    assert back.value == abi.CUBLAS_OP_T and wrote.value == 4
+    rows = C.c_uint64()
+    assert api.cublasLtMatrixLayoutGetAttribute(lay[2], abi.CUBLASLT_MATRIX_LAYOUT_ROWS, C.byref(rows), 8, None) == 0
+    assert rows.value == 512
+    h = C.c_void_p()
+    assert api.cublasLtCreate(C.byref(h)) == 0
+    res = (abi.cublasLtMatmulHeuristicResult_t * 2)()
+    n = C.c_int()
+    assert api.cublasLtMatmulAlgoGetHeuristic(h, desc, lay[0], lay[1], lay[2], lay[2], pref, 2, res, C.byref(n)) == 0
+    assert n.value == 2 and res[0].state == 0
+    assert (res[0].algo.data[0] & 0xffffffff) == abi.ZLUDA_KERNEL_MFMA_I8
+    assert api.cublasLtDestroy(h) == 0
 
 
 def test_heuristic_tokens_and_algo_check(api):

@@ -249,6 +249,32 @@ cublasStatus_t pref_attr(PrefObj *o, uint32_t attr, bool set, const void *in, vo
   }
 }
 
+// Initial contents of the three descriptor kinds.  They hold no pointers of their own, so they may
+// live on the heap (Create) or in the caller's opaque storage (Init_internal: 256 bytes for a matmul
+// descriptor, 64 for a layout or a preference, cuda_types/src/cublaslt.rs:43-83).
+void init_layout(LayoutObj *o, cudaDataType_t type, uint64_t rows, uint64_t cols, int64_t ld) {
+  o->magic = LAYOUT_MAGIC;
+  o->l = zluda_matrix_layout{type, CUBLASLT_ORDER_COL, rows, cols, ld, 1, 0};
+}
+void init_desc(MatmulDescObj *o, cublasComputeType_t computeType, cudaDataType_t scaleType) {
+  memset(o, 0, sizeof(*o));
+  o->magic = DESC_MAGIC;
+  o->d.compute_type = computeType;
+  o->d.scale_type = scaleType;
+  o->d.pointer_mode = CUBLASLT_POINTER_MODE_HOST;
+  o->d.transa = o->d.transb = CUBLAS_OP_N;
+  o->d.epilogue = CUBLASLT_EPILOGUE_DEFAULT;
+  o->d.bias_type = -1;
+}
+void init_pref(PrefObj *o) {
+  memset(o, 0, sizeof(*o));
+  o->magic = PREF_MAGIC;
+  for (uint32_t &a : o->min_align) a = 256;
+}
+static_assert(sizeof(MatmulDescObj) <= 256 && alignof(MatmulDescObj) <= 8, "fits cublasLtMatmulDescOpaque_t");
+static_assert(sizeof(LayoutObj) <= 64 && alignof(LayoutObj) <= 8, "fits cublasLtMatrixLayoutOpaque_t");
+static_assert(sizeof(PrefObj) <= 64 && alignof(PrefObj) <= 8, "fits cublasLtMatmulPreferenceOpaque_t");
+
 // descriptors -> problem.  Cdesc may be NULL (= Ddesc).
 cublasStatus_t build_problem(cublasLtMatmulDesc_t op, cublasLtMatrixLayout_t A, cublasLtMatrixLayout_t B,
                              cublasLtMatrixLayout_t C, cublasLtMatrixLayout_t D, zluda_gemm_problem *p) {
@@ -354,8 +380,7 @@ cublasStatus_t cublasLtMatrixLayoutCreate(cublasLtMatrixLayout_t *matLayout, cud
   if (!matLayout) return CUBLAS_STATUS_INVALID_VALUE;
   LayoutObj *o = new (std::nothrow) LayoutObj();
   if (!o) return CUBLAS_STATUS_ALLOC_FAILED;
-  o->magic = LAYOUT_MAGIC;
-  o->l = zluda_matrix_layout{type, CUBLASLT_ORDER_COL, rows, cols, ld, 1, 0};
+  init_layout(o, type, rows, cols, ld);
   *matLayout = reinterpret_cast<cublasLtMatrixLayout_t>(o);
   return CUBLAS_STATUS_SUCCESS;
 }
@@ -380,9 +405,13 @@ cublasStatus_t cublasLtMatrixLayoutGetAttribute(cublasLtMatrixLayout_t matLayout
   if (!o) return CUBLAS_STATUS_INVALID_VALUE;
   return layout_attr(o, attr, false, nullptr, buf, sizeInBytes, sizeWritten);
 }
-cublasStatus_t cublasLtMatrixLayoutInit_internal(cublasLtMatrixLayout_t, size_t, cudaDataType_t,
-                                                 uint64_t, uint64_t, int64_t) {
-  return CUBLAS_STATUS_NOT_SUPPORTED;
+// what the cublasLtMatrixLayoutInit() inline of the CUDA header calls with the caller's own storage
+cublasStatus_t cublasLtMatrixLayoutInit_internal(cublasLtMatrixLayout_t matLayout, size_t size,
+                                                 cudaDataType_t type, uint64_t rows, uint64_t cols,
+                                                 int64_t ld) {
+  if (!matLayout || size < sizeof(LayoutObj)) return CUBLAS_STATUS_INVALID_VALUE;
+  init_layout(reinterpret_cast<LayoutObj *>(matLayout), type, rows, cols, ld);
+  return CUBLAS_STATUS_SUCCESS;
 }
 
 // ---- matmul descriptor -----------------------------------------------------------------------
@@ -391,14 +420,7 @@ cublasStatus_t cublasLtMatmulDescCreate(cublasLtMatmulDesc_t *matmulDesc,
   if (!matmulDesc) return CUBLAS_STATUS_INVALID_VALUE;
   MatmulDescObj *o = new (std::nothrow) MatmulDescObj();
   if (!o) return CUBLAS_STATUS_ALLOC_FAILED;
-  memset(o, 0, sizeof(*o));
-  o->magic = DESC_MAGIC;
-  o->d.compute_type = computeType;
-  o->d.scale_type = scaleType;
-  o->d.pointer_mode = CUBLASLT_POINTER_MODE_HOST;
-  o->d.transa = o->d.transb = CUBLAS_OP_N;
-  o->d.epilogue = CUBLASLT_EPILOGUE_DEFAULT;
-  o->d.bias_type = -1;
+  init_desc(o, computeType, scaleType);
   *matmulDesc = reinterpret_cast<cublasLtMatmulDesc_t>(o);
   return CUBLAS_STATUS_SUCCESS;
 }
@@ -423,9 +445,11 @@ cublasStatus_t cublasLtMatmulDescGetAttribute(cublasLtMatmulDesc_t matmulDesc,
   if (!o) return CUBLAS_STATUS_INVALID_VALUE;
   return desc_attr(o, attr, false, nullptr, buf, sizeInBytes, sizeWritten);
 }
-cublasStatus_t cublasLtMatmulDescInit_internal(cublasLtMatmulDesc_t, size_t, cublasComputeType_t,
-                                               cudaDataType_t) {
-  return CUBLAS_STATUS_NOT_SUPPORTED;
+cublasStatus_t cublasLtMatmulDescInit_internal(cublasLtMatmulDesc_t matmulDesc, size_t size,
+                                               cublasComputeType_t computeType, cudaDataType_t scaleType) {
+  if (!matmulDesc || size < sizeof(MatmulDescObj)) return CUBLAS_STATUS_INVALID_VALUE;
+  init_desc(reinterpret_cast<MatmulDescObj *>(matmulDesc), computeType, scaleType);
+  return CUBLAS_STATUS_SUCCESS;
 }
 
 // ---- preference ----------------------------------------------------------------------------------
@@ -433,9 +457,7 @@ cublasStatus_t cublasLtMatmulPreferenceCreate(cublasLtMatmulPreference_t *pref) 
   if (!pref) return CUBLAS_STATUS_INVALID_VALUE;
   PrefObj *o = new (std::nothrow) PrefObj();
   if (!o) return CUBLAS_STATUS_ALLOC_FAILED;
-  memset(o, 0, sizeof(*o));
-  o->magic = PREF_MAGIC;
-  for (uint32_t &a : o->min_align) a = 256;
+  init_pref(o);
   *pref = reinterpret_cast<cublasLtMatmulPreference_t>(o);
   return CUBLAS_STATUS_SUCCESS;
 }
@@ -460,8 +482,10 @@ cublasStatus_t cublasLtMatmulPreferenceGetAttribute(cublasLtMatmulPreference_t p
   if (!o) return CUBLAS_STATUS_INVALID_VALUE;
   return pref_attr(o, attr, false, nullptr, buf, sizeInBytes, sizeWritten);
 }
-cublasStatus_t cublasLtMatmulPreferenceInit_internal(cublasLtMatmulPreference_t, size_t) {
-  return CUBLAS_STATUS_NOT_SUPPORTED;
+cublasStatus_t cublasLtMatmulPreferenceInit_internal(cublasLtMatmulPreference_t pref, size_t size) {
+  if (!pref || size < sizeof(PrefObj)) return CUBLAS_STATUS_INVALID_VALUE;
+  init_pref(reinterpret_cast<PrefObj *>(pref));
+  return CUBLAS_STATUS_SUCCESS;
 }
 
 // ---- heuristic and matmul ----------------------------------------------------------------------
