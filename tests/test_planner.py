@@ -30,7 +30,7 @@ def plan(api, spec, forced=0, variant=-1, cus=256, a_ptr=0, b_ptr=0, workspace=0
 
 def test_baseline_configs_pick_the_intended_kernels(api):
     st, p = plan(api, dict(I8, m=256, n=256, k=256, transa=0, transb=1))            # config 1: A:N B:T
-    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_GENERIC
+    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_TR8 and p.variant == 1 and p.grid_x == 16 and p.block == 256
     st, p = plan(api, dict(I8, m=4096, n=4096, k=4096, transa=1))                   # config 2
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_I8 and p.variant == 0 and p.grid_x == 256 and p.block == 512
     st, p = plan(api, dict(I8, m=14336, n=16, k=4096, transa=1, d_type=K.CUDA_R_16BF, scale_type=K.CUDA_R_32F,
@@ -62,16 +62,28 @@ def test_row_major_output_swaps_operands(api):
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.swapped == 1
 
 
-def test_misaligned_or_strided_operands_fall_back_to_generic(api):
+def test_misaligned_or_strided_operands_leave_the_dma_kernels(api):
     spec = dict(I8, m=512, n=512, k=512, transa=1)
-    assert plan(api, spec, a_ptr=0x1004)[1].kernel == K.ZLUDA_KERNEL_GENERIC
-    assert plan(api, dict(spec, lda=520))[1].kernel == K.ZLUDA_KERNEL_GENERIC          # pitch not a multiple of 16
-    assert plan(api, dict(spec, k=520, lda=528, ldb=528))[1].kernel == K.ZLUDA_KERNEL_GENERIC   # K % 16 != 0
+    TR8, GEN = K.ZLUDA_KERNEL_MFMA_TR8, K.ZLUDA_KERNEL_GENERIC
+    # 4-byte alignment is enough for the register-staged kernel, 16 for the LDS DMA ones
+    assert plan(api, spec, a_ptr=0x1004)[1].kernel == TR8
+    assert plan(api, spec, a_ptr=0x1002)[1].kernel == GEN
+    assert plan(api, dict(spec, lda=520))[1].kernel == TR8                             # pitch not a multiple of 16
+    assert plan(api, dict(spec, lda=514))[1].kernel == GEN                             # ... nor of 4
+    assert plan(api, dict(spec, k=520, lda=528, ldb=528))[1].kernel == GEN             # K-contiguous, K % 16 != 0
     assert plan(api, dict(spec, k=528, lda=528, ldb=528))[1].kernel == K.ZLUDA_KERNEL_MFMA_I8   # K tail of 16 bytes
     st, _ = plan(api, spec, forced=K.ZLUDA_KERNEL_MFMA_I8, a_ptr=0x1004)
     assert st == K.CUBLAS_STATUS_NOT_SUPPORTED
+    # operands that are not K-contiguous: any K
+    assert plan(api, dict(spec, transa=0, transb=1, k=100))[1].kernel == TR8
+    assert plan(api, dict(spec, transa=0, transb=0, k=100, ldb=100))[1].kernel == GEN  # B K-contiguous: K % 16
+    assert plan(api, dict(spec, transa=0, transb=0, k=112, ldb=112))[1].kernel == TR8
+    assert plan(api, dict(spec, transa=0, lda=518))[1].kernel == GEN                   # stride of a K row % 4
+    # large problems get the larger tile
+    st, p = plan(api, dict(spec, transa=0, transb=1, m=4096, n=4096))
+    assert st == 0 and p.kernel == TR8 and p.variant == 0 and p.grid_x == 1024
     # MXFP4 needs whole 256-element K stages for the MFMA kernel
-    assert plan(api, dict(MX, m=256, n=256, k=384, transa=1))[1].kernel == K.ZLUDA_KERNEL_GENERIC
+    assert plan(api, dict(MX, m=256, n=256, k=384, transa=1))[1].kernel == GEN
     assert plan(api, dict(MX, m=256, n=256, k=512, transa=1))[1].kernel == K.ZLUDA_KERNEL_MFMA_MXF4
 
 

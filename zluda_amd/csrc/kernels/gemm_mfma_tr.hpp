@@ -1,0 +1,238 @@
+// MFMA GEMM for 8-bit operands (int8, OCP fp8) of which at least one is NOT K-contiguous: a
+// column-major A without transpose (unit stride along M), a B with transpose (unit stride along N),
+// and their row-major counterparts.  v_mfma_i32_32x32x32_i8 / v_mfma_f32_32x32x64_f8f6f4 want 16 / 32
+// consecutive K bytes of one matrix row per lane, so such an operand is transposed on its way into
+// LDS; from there on the kernel is the K-contiguous one (same fragment layout, same epilogues:
+// gemm_mfma.hpp).
+//
+//   * 4 waves (2 x 2), workgroup tile BP x BQ (128 x 128 or 64 x 64), 64 K bytes per stage, two LDS
+//     stages, one barrier per stage.  Global loads of stage kt+1 are issued into registers right after
+//     the barrier of stage kt and written to LDS at the top of the next trip (register prefetch: the
+//     data cannot go straight to LDS because it has to be transposed).  Several workgroups share a
+//     CU (40 KiB of LDS, ~130 VGPRs), which is what hides the barrier.
+//   * Operand with unit stride along its row index ("MC"): a lane loads a block of 4 K rows x IW row
+//     indices (IW = rows/16 bytes: dword, dwordx2), lanes of a wave run along the row index first so
+//     that an instruction reads whole 64..128-byte pieces of 4 K rows; 8 v_perm_b32 per 4 x 4 bytes
+//     turn the block into one dword of 4 consecutive K bytes per row, written with ds_write_b32.
+//   * Operand with unit stride along K ("KC"): 16 bytes per lane, ds_write_b128.
+//   * LDS rows have a pitch of 80 bytes and are stored in permuted order, rho(i) = 16 r + ((g + s r) mod 16)
+//     for i = IW g + r, s = 16 / IW.  With that every ds_write_b32 instruction of the transposing path
+//     hits 64 distinct banks (row pitch 20 dwords: 20 x 16 consecutive rows are 16 distinct multiples
+//     of 4 mod 64) and every ds_read_b128 of 16 consecutive matrix rows hits 16 distinct 16-byte
+//     groups (pitch 5 groups, 5 coprime to 16, rho of 16 consecutive rows distinct mod 16).
+#pragma once
+#include "gemm_mfma.hpp"
+
+namespace zluda_amd {
+
+// LDS row of matrix row i (0 <= i < ROWS) of a tile operand
+template <int ROWS>
+__device__ __forceinline__ constexpr int tr_rho(int g, int r) {
+  constexpr int IW = ROWS / 16, STEP = 16 / IW;
+  (void)IW;
+  return 16 * r + ((g + STEP * r) & 15);
+}
+template <int ROWS>
+__device__ __forceinline__ int tr_rho_of(int i) {
+  constexpr int IW = ROWS / 16;
+  return tr_rho<ROWS>(i / IW, i % IW);
+}
+
+// 4 x 4 byte transpose: x[j] holds bytes (row 0..3) of K index j; out[r] = K bytes 0..3 of row r
+__device__ __forceinline__ void transpose4x4(int x0, int x1, int x2, int x3, int (&out)[4]) {
+  // v_perm_b32(s0, s1, sel): result byte n = byte sel[n] of the 8 bytes {s0 (4..7), s1 (0..3)}
+  const int t01l = __builtin_amdgcn_perm(x1, x0, 0x05010400);  // x0.b0 x1.b0 x0.b1 x1.b1
+  const int t01h = __builtin_amdgcn_perm(x1, x0, 0x07030602);  // x0.b2 x1.b2 x0.b3 x1.b3
+  const int t23l = __builtin_amdgcn_perm(x3, x2, 0x05010400);
+  const int t23h = __builtin_amdgcn_perm(x3, x2, 0x07030602);
+  out[0] = __builtin_amdgcn_perm(t23l, t01l, 0x05040100);
+  out[1] = __builtin_amdgcn_perm(t23l, t01l, 0x07060302);
+  out[2] = __builtin_amdgcn_perm(t23h, t01h, 0x05040100);
+  out[3] = __builtin_amdgcn_perm(t23h, t01h, 0x07060302);
+}
+
+// Global -> register -> LDS path of one tile operand with ROWS rows; KC: unit stride along K.
+template <int ROWS, bool KC>
+struct TrOperand {
+  static constexpr int IW = ROWS / 16;        // MC: row indices per lane (bytes per load)
+  static constexpr int NW = IW / 4;           // MC: dwords per load
+  static constexpr int NCH = ROWS / 64;       // KC: 16-byte chunks per lane and stage
+  static constexpr int NREG = KC ? NCH * 4 : NW * 4;
+  static_assert(ROWS == 64 || ROWS == 128, "tile operands of 64 or 128 rows");
+
+  __amdgpu_buffer_rsrc_t rs;
+  int voff[KC ? NCH : 1];
+  int kstep;     // byte offset of one stage
+  int kbytes;    // K
+  int ld;        // MC: stride of one K row
+  int regs[NREG];
+
+  // base: first byte of the operand (this batch); row0: first tile row; nrows: rows of the whole
+  // operand; ld_row / ld_k: byte strides (one of them is 1)
+  __device__ __forceinline__ void init(const uint8_t *base, int row0, int nrows, int ld_row, int ld_k, int K) {
+    const int t = threadIdx.x;
+    kbytes = K;
+    if constexpr (KC) {
+      rs = __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, 0x80000000, 0x00020000);
+#pragma unroll
+      for (int n = 0; n < NCH; n++) voff[n] = min(row0 + (t >> 2) + 64 * n, nrows - 1) * ld_row + (t & 3) * 16;
+      kstep = 64;
+      ld = 0;
+    } else {
+      // the operand's extent, up to the end of its last dword (the range check is per dword; base
+      // and ld_k are multiples of 4, so that dword lies in the same allocation granule): K rows past
+      // the end read as zero
+      rs = __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, ((K - 1) * ld_k + nrows + 3) & ~3, 0x00020000);
+      voff[0] = ((t >> 4) * 4) * ld_k + row0 + (t & 15) * IW;
+      kstep = 64 * ld_k;
+      ld = ld_k;
+    }
+  }
+
+  __device__ __forceinline__ void load(int kt) {
+    if constexpr (KC) {
+#pragma unroll
+      for (int n = 0; n < NCH; n++) {
+        const int oob = kt * 64 + (int)(threadIdx.x & 3) * 16 < kbytes ? 0 : (int)0x80000000;
+        const v4i v = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rs, voff[n] | oob, kt * kstep, 0));
+        regs[n * 4 + 0] = v[0]; regs[n * 4 + 1] = v[1]; regs[n * 4 + 2] = v[2]; regs[n * 4 + 3] = v[3];
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        if constexpr (NW == 1) {
+          regs[j] = __builtin_amdgcn_raw_buffer_load_b32(rs, voff[0] + j * ld, kt * kstep, 0);
+        } else {
+          const v2i v = __builtin_bit_cast(v2i, __builtin_amdgcn_raw_buffer_load_b64(rs, voff[0] + j * ld, kt * kstep, 0));
+          regs[j * 2] = v[0]; regs[j * 2 + 1] = v[1];
+        }
+      }
+    }
+  }
+
+  // `dst`: the operand's rows of one LDS stage (80-byte pitch = 5 v4i)
+  __device__ __forceinline__ void store(v4i *dst) const {
+    const int t = threadIdx.x;
+    if constexpr (KC) {
+#pragma unroll
+      for (int n = 0; n < NCH; n++)
+        dst[tr_rho_of<ROWS>((t >> 2) + 64 * n) * 5 + (t & 3)] = v4i{regs[n * 4], regs[n * 4 + 1], regs[n * 4 + 2], regs[n * 4 + 3]};
+    } else {
+      int *d32 = (int *)dst;
+      const int g = t & 15, kb = t >> 4;
+#pragma unroll
+      for (int c = 0; c < NW; c++) {
+        int out[4];
+        transpose4x4(regs[0 * NW + c], regs[1 * NW + c], regs[2 * NW + c], regs[3 * NW + c], out);
+#pragma unroll
+        for (int r = 0; r < 4; r++) d32[tr_rho<ROWS>(g, 4 * c + r) * 20 + kb] = out[r];
+      }
+    }
+  }
+};
+
+template <int KIND, int FQ, int FP, int BP, int BQ, bool PKC, bool QKC>
+__global__ __launch_bounds__(256) void gemm_mfma_tr_kernel(MfmaParams prm) {
+  static_assert(KIND == KIND_I8 || KIND == KIND_F8, "8-bit operands");
+  constexpr int WP = 2, WQ = 2;
+  constexpr int WTP = BP / WP, WTQ = BQ / WQ, TP = WTP / 32, TQ = WTQ / 32;
+  constexpr int KS = KIND == KIND_F8 ? 1 : 2;  // MFMA sub-steps per 64-byte stage
+  constexpr int STAGE_V4 = (BP + BQ) * 5;
+  using acc_v = typename std::conditional<KIND == KIND_I8, v16i, v16f>::type;
+  using frag_v = typename std::conditional<KIND == KIND_I8, v4i, v8i>::type;
+
+  __shared__ v4i lds[2 * STAGE_V4];
+
+  const GemmArgs &g = prm.g;
+  const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int wp = wave % WP, wq = wave / WP;
+  const int lr = lane & 31, gsel = lane >> 5;
+  const int bt = blockIdx.y;
+
+  // workgroup -> tile: as in gemm_mfma_pipe_kernel
+  const int total = prm.tiles_p * prm.tiles_q;
+  int w = blockIdx.x;
+  if ((total & 7) == 0) w = (w & 7) * (total >> 3) + (w >> 3);
+  const int group = prm.group_p * prm.tiles_q;
+  const int gid = w / group, first_p = gid * prm.group_p;
+  const int gsz = min(prm.tiles_p - first_p, prm.group_p);
+  const int tile_p = first_p + (w % group) % gsz, tile_q = (w % group) / gsz;
+  const int p0 = tile_p * BP, q0 = tile_q * BQ;
+  const int NP = prm.swapped ? g.N : g.M, NQ = prm.swapped ? g.M : g.N;
+
+  TrOperand<BP, PKC> P;
+  TrOperand<BQ, QKC> Q;
+  if (!prm.swapped) {
+    P.init((const uint8_t *)g.A + g.a_sb * bt, p0, NP, (int)g.a_si, (int)g.a_sk, g.K);
+    Q.init((const uint8_t *)g.B + g.b_sb * bt, q0, NQ, (int)g.b_sj, (int)g.b_sk, g.K);
+  } else {
+    P.init((const uint8_t *)g.B + g.b_sb * bt, p0, NP, (int)g.b_sj, (int)g.b_sk, g.K);
+    Q.init((const uint8_t *)g.A + g.a_sb * bt, q0, NQ, (int)g.a_si, (int)g.a_sk, g.K);
+  }
+  const int KT = (g.K + 63) / 64;
+
+  // LDS rows (in v4i units) of this lane's fragment rows
+  int prow[TP], qrow[TQ];
+#pragma unroll
+  for (int b = 0; b < TP; b++) prow[b] = tr_rho_of<BP>(wp * WTP + b * 32 + lr) * 5;
+#pragma unroll
+  for (int a = 0; a < TQ; a++) qrow[a] = (BP + tr_rho_of<BQ>(wq * WTQ + a * 32 + lr)) * 5;
+
+  acc_v acc[TQ][TP];
+#pragma unroll
+  for (int a = 0; a < TQ; a++)
+#pragma unroll
+    for (int b = 0; b < TP; b++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[a][b][v] = 0;
+
+  P.load(0);
+  Q.load(0);
+  for (int kt = 0; kt < KT; kt++) {
+    v4i *stage = &lds[(kt & 1) * STAGE_V4];
+    P.store(stage);
+    Q.store(stage + BP * 5);
+    // the other stage is free again: every wave passed this barrier one trip ago, after it had read it
+    __syncthreads();
+    P.load(kt + 1);  // one past the end reads zeros, which nothing consumes
+    Q.load(kt + 1);
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      frag_v fp[TP], fq[TQ];
+      if constexpr (KIND == KIND_I8) {
+        const int ch = ks * 2 + gsel;
+#pragma unroll
+        for (int b = 0; b < TP; b++) fp[b] = stage[prow[b] + ch];
+#pragma unroll
+        for (int a = 0; a < TQ; a++) fq[a] = stage[qrow[a] + ch];
+      } else {
+        const int c0 = gsel * 2;
+#pragma unroll
+        for (int b = 0; b < TP; b++) {
+          const v4i lo = stage[prow[b] + c0], hi = stage[prow[b] + c0 + 1];
+          fp[b] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        }
+#pragma unroll
+        for (int a = 0; a < TQ; a++) {
+          const v4i lo = stage[qrow[a] + c0], hi = stage[qrow[a] + c0 + 1];
+          fq[a] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        }
+      }
+#pragma unroll
+      for (int a = 0; a < TQ; a++)
+#pragma unroll
+        for (int b = 0; b < TP; b++) {
+          if constexpr (KIND == KIND_I8)
+            acc[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fq[a], fp[b], acc[a][b], 0, 0, 0);
+          else
+            acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fq[a], fp[b], acc[a][b], FQ, FP, 0, 0, 0, 0);
+        }
+    }
+  }
+
+  // every wave is done with the LDS stages before they become epilogue staging
+  __syncthreads();
+  mfma_store_tile<KIND, WP, WQ, WTP, WTQ>(prm, acc, (int *)&lds[0], sizeof(lds), p0, q0, NP, NQ, bt);
+}
+
+} // namespace zluda_amd

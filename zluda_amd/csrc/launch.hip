@@ -9,6 +9,7 @@
 #include "kernels/gemm_generic.hpp"
 #include "kernels/splitk_reduce.hpp"
 #include "mfma_launch.hpp"
+#include "mfma_tr_launch.hpp"
 #include "planner.hpp"
 
 using namespace zluda_amd;
@@ -64,6 +65,25 @@ uint32_t launch_mfma(const Lowered &l, const zluda_gemm_plan &plan, const zluda_
   rp.ws = (const int32_t *)p->workspace;
   hipLaunchKernelGGL(splitk_reduce_kernel, dim3((np + 1023) / 1024, nq, l.g.batch), dim3(256), 0, s, rp);
   return CUBLAS_STATUS_SUCCESS;
+}
+
+uint32_t launch_tr(const Lowered &l, const zluda_gemm_plan &plan, hipStream_t s) {
+  if (plan.variant >= (uint32_t)kNumTrVariants) return CUBLAS_STATUS_INVALID_VALUE;
+  const TrVariant &v = kTrVariants[plan.variant];
+  MfmaParams prm;
+  prm.g = l.g;
+  prm.swapped = plan.swapped;
+  const int np = plan.swapped ? l.g.N : l.g.M, nq = plan.swapped ? l.g.M : l.g.N;
+  prm.tiles_p = (np + v.bp - 1) / v.bp;
+  prm.tiles_q = (nq + v.bq - 1) / v.bq;
+  prm.group_p = 8;
+  prm.splits = 1; prm.split_stages = 0; prm.ws = nullptr;
+  if ((uint32_t)(prm.tiles_p * prm.tiles_q) != plan.grid_x) return CUBLAS_STATUS_INVALID_VALUE;
+  // P is op(A) for a column-major D, op(B)^T otherwise
+  const bool pkc = plan.swapped ? l.b_kcontig : l.a_kcontig, qkc = plan.swapped ? l.a_kcontig : l.b_kcontig;
+  if (l.g.a_type == CUDA_R_8I) return launch_tr_i8(prm, plan, pkc, qkc, s);
+  const int fa = f8_fmt(l.g.a_type), fb = f8_fmt(l.g.b_type);
+  return launch_tr_f8(prm, plan, plan.swapped ? fa : fb, plan.swapped ? fb : fa, pkc, qkc, s);
 }
 
 template <int NW, int STEPS>
@@ -202,6 +222,9 @@ extern "C" uint32_t zluda_gemm_launch(const zluda_gemm_problem *p, const zluda_g
     break;
   case ZLUDA_KERNEL_DECODE_W8A8:
     if ((st = launch_decode(l, *plan, s))) return st;
+    break;
+  case ZLUDA_KERNEL_MFMA_TR8:
+    if ((st = launch_tr(l, *plan, s))) return st;
     break;
   default: return CUBLAS_STATUS_NOT_SUPPORTED;
   }

@@ -1,0 +1,7 @@
+// int8 instantiations of the transposing MFMA kernel (v_mfma_i32_32x32x32_i8).
+#include "mfma_tr_launch.hpp"
+namespace zluda_amd {
+uint32_t launch_tr_i8(const MfmaParams &prm, const zluda_gemm_plan &plan, bool pkc, bool qkc, hipStream_t s) {
+  return launch_tr_variant<KIND_I8, 0, 0>(prm, plan, pkc, qkc, s);
+}
+} // namespace zluda_amd

@@ -238,6 +238,20 @@ bool family_supports(uint32_t kernel, const Lowered &l) {
     return fast_layout && l.span_ok && g.a_type == CUDA_R_4F_E2M1 && g.b_type == CUDA_R_4F_E2M1 &&
            g.a_scale_mode == SCALE_BLOCK32_UE8M0 && g.b_scale_mode == SCALE_BLOCK32_UE8M0 &&
            (g.K % 256) == 0 && ((((uintptr_t)g.a_scale) | ((uintptr_t)g.b_scale)) & 3) == 0 && d_fast;
+  case ZLUDA_KERNEL_MFMA_TR8: {
+    // 8-bit operands, each with unit stride along K or along its row index; dword-aligned loads
+    const bool types = (g.a_type == CUDA_R_8I && g.b_type == CUDA_R_8I) ||
+                       (is_f8(g.a_type) && is_f8(g.b_type) && !(g.a_type == CUDA_R_8F_E5M2 && g.b_type == CUDA_R_8F_E5M2));
+    auto operand_ok = [&](const void *ptr, int64_t s_row, int64_t s_k, int64_t s_b, int rows) {
+      if ((((uintptr_t)ptr) & 3) || (g.batch > 1 && (s_b & 3))) return false;
+      const int64_t span = (int64_t)(rows - 1) * s_row + (int64_t)(g.K - 1) * s_k + 1;
+      if (span >= 0x7fffffffll) return false;
+      if (s_k == 1) return (s_row & 3) == 0 && (g.K & 15) == 0;  // 16-byte pieces along K
+      return s_row == 1 && (s_k & 3) == 0;
+    };
+    return types && d_fast && g.a_scale_mode != SCALE_BLOCK32_UE8M0 && g.b_scale_mode != SCALE_BLOCK32_UE8M0 &&
+           operand_ok(g.A, g.a_si, g.a_sk, g.a_sb, g.M) && operand_ok(g.B, g.b_sj, g.b_sk, g.b_sb, g.N);
+  }
   case ZLUDA_KERNEL_DECODE_W8A8:
     return fast_layout && g.a_type == CUDA_R_8I && g.b_type == CUDA_R_8I &&
            std::min(g.M, g.N) <= kDecodeMaxTokens && std::max(g.M, g.N) >= 64 && any_decode_variant_ok(l);
@@ -305,6 +319,27 @@ static int pick_mfma_variant(const Lowered &l, uint32_t cus) {
   return best;
 }
 
+static void fill_tr_plan(const Lowered &l, int variant, uint32_t cus, zluda_gemm_plan *plan) {
+  const GemmArgs &g = l.g;
+  const TrVariant &v = kTrVariants[variant];
+  const bool swapped = g.d_si != 1;
+  const uint32_t np = swapped ? g.N : g.M, nq = swapped ? g.M : g.N;
+  plan->variant = variant;
+  plan->swapped = swapped;
+  plan->grid_x = ceil_div(np, v.bp) * ceil_div(nq, v.bq); plan->grid_y = g.batch; plan->grid_z = 1;
+  plan->block = 256;
+  const uint32_t per_cu = 160u * 1024u / (2u * (v.bp + v.bq) * 80u);  // LDS: two stages of 80-byte rows
+  plan->waves = (float)plan->grid_x * plan->grid_y / (float)(cus * std::min(per_cu, 8u));
+  plan->workspace = 0;
+}
+
+// the larger tile unless it leaves CUs without a workgroup
+static int pick_tr_variant(const Lowered &l, uint32_t cus) {
+  const GemmArgs &g = l.g;
+  const uint64_t tiles = (uint64_t)ceil_div(g.M, kTrVariants[0].bp) * ceil_div(g.N, kTrVariants[0].bq) * g.batch;
+  return tiles >= cus ? 0 : 1;
+}
+
 static void fill_decode_plan(const Lowered &l, int variant, uint32_t cus, zluda_gemm_plan *plan) {
   const GemmArgs &g = l.g;
   const DecodeVariant &v = kDecodeVariants[variant];
@@ -346,6 +381,7 @@ extern "C" uint32_t zluda_gemm_variant_count(uint32_t kernel) {
   case ZLUDA_KERNEL_GENERIC: return 1;
   case ZLUDA_KERNEL_MFMA_I8: case ZLUDA_KERNEL_MFMA_F8: case ZLUDA_KERNEL_MFMA_MXF4: return kNumMfmaVariants;
   case ZLUDA_KERNEL_DECODE_W8A8: return kNumDecodeVariants;
+  case ZLUDA_KERNEL_MFMA_TR8: return kNumTrVariants;
   default: return 0;
   }
 }
@@ -363,7 +399,7 @@ extern "C" uint32_t zluda_gemm_plan_problem(const zluda_gemm_problem *p, uint32_
   uint32_t kernel = forced_kernel;
   if (kernel == ZLUDA_KERNEL_AUTO) {
     static const uint32_t order[] = {ZLUDA_KERNEL_DECODE_W8A8, ZLUDA_KERNEL_MFMA_I8, ZLUDA_KERNEL_MFMA_F8,
-                                     ZLUDA_KERNEL_MFMA_MXF4, ZLUDA_KERNEL_GENERIC};
+                                     ZLUDA_KERNEL_MFMA_MXF4, ZLUDA_KERNEL_MFMA_TR8, ZLUDA_KERNEL_GENERIC};
     for (uint32_t k : order) {
       if (k == ZLUDA_KERNEL_DECODE_W8A8 && std::min(l.g.M, l.g.N) > kDecodeAutoMaxTokens) continue;
       if (family_supports(k, l)) { kernel = k; break; }
@@ -384,6 +420,12 @@ extern "C" uint32_t zluda_gemm_plan_problem(const zluda_gemm_problem *p, uint32_
     int v = forced_variant >= 0 ? forced_variant : pick_mfma_variant(l, cu_count);
     if (v >= kNumMfmaVariants) return CUBLAS_STATUS_INVALID_VALUE;
     fill_mfma_plan(l, v, cu_count, p->workspace_size, plan);
+    break;
+  }
+  case ZLUDA_KERNEL_MFMA_TR8: {
+    int v = forced_variant >= 0 ? forced_variant : pick_tr_variant(l, cu_count);
+    if (v >= kNumTrVariants) return CUBLAS_STATUS_INVALID_VALUE;
+    fill_tr_plan(l, v, cu_count, plan);
     break;
   }
   case ZLUDA_KERNEL_DECODE_W8A8: {

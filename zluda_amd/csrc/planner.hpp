@@ -20,6 +20,15 @@ constexpr MfmaVariant kMfmaVariants[] = {
 };
 constexpr int kNumMfmaVariants = sizeof(kMfmaVariants) / sizeof(kMfmaVariants[0]);
 
+// tile configurations of the transposing 8-bit MFMA kernel (index = plan.variant for
+// ZLUDA_KERNEL_MFMA_TR8): workgroup tile bp x bq, always 2 x 2 waves and 64 K bytes per stage
+struct TrVariant { int bp, bq; };
+constexpr TrVariant kTrVariants[] = {
+    {128, 128},  // 0
+    {64, 64},    // 1: problems that leave CUs idle with the larger tile
+};
+constexpr int kNumTrVariants = sizeof(kTrVariants) / sizeof(kTrVariants[0]);
+
 // decode configurations (index = plan.variant for ZLUDA_KERNEL_DECODE_W8A8).
 // stream == 0: weights loaded straight into registers, any K (grid-stride over 16-row blocks).
 // stream == 1: weights streamed through LDS in whole cache lines; K must equal nw * steps * 64.
