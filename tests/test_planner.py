@@ -30,7 +30,7 @@ def plan(api, spec, forced=0, variant=-1, cus=256, a_ptr=0, b_ptr=0, workspace=0
 
 def test_baseline_configs_pick_the_intended_kernels(api):
     st, p = plan(api, dict(I8, m=256, n=256, k=256, transa=0, transb=1))            # config 1: A:N B:T
-    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_TR8 and p.variant == 1 and p.grid_x == 16 and p.block == 256
+    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_TR8 and p.variant == 2 and p.grid_x == 16 and p.block == 256
     st, p = plan(api, dict(I8, m=4096, n=4096, k=4096, transa=1))                   # config 2
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_I8 and p.variant == 0 and p.grid_x == 256 and p.block == 512
     st, p = plan(api, dict(I8, m=14336, n=16, k=4096, transa=1, d_type=K.CUDA_R_16BF, scale_type=K.CUDA_R_32F,
@@ -79,9 +79,16 @@ def test_misaligned_or_strided_operands_leave_the_dma_kernels(api):
     assert plan(api, dict(spec, transa=0, transb=0, k=100, ldb=100))[1].kernel == GEN  # B K-contiguous: K % 16
     assert plan(api, dict(spec, transa=0, transb=0, k=112, ldb=112))[1].kernel == TR8
     assert plan(api, dict(spec, transa=0, lda=518))[1].kernel == GEN                   # stride of a K row % 4
-    # large problems get the larger tile
+    # tile choice: 256x256 once every CU gets one, 64x64 for what would leave CUs idle
     st, p = plan(api, dict(spec, transa=0, transb=1, m=4096, n=4096))
-    assert st == 0 and p.kernel == TR8 and p.variant == 0 and p.grid_x == 1024
+    assert st == 0 and p.kernel == TR8 and p.variant == 0 and p.grid_x == 256 and p.block == 512
+    st, p = plan(api, dict(spec, transa=0, transb=1, m=4096, n=1024, k=4096))
+    assert st == 0 and p.variant == 2 and p.grid_x == 1024 and p.block == 256
+    st, p = plan(api, dict(spec, transa=0, transb=1, m=8192, n=4096, k=1024))
+    assert st == 0 and p.variant == 0 and p.grid_x == 512
+    assert api.zluda_gemm_variant_count(TR8) == 3
+    assert plan(api, dict(spec, transa=0, transb=1), forced=TR8, variant=3)[0] == K.CUBLAS_STATUS_INVALID_VALUE
+    assert plan(api, dict(MX, m=256, n=256, k=512, transa=1), forced=TR8)[0] == K.CUBLAS_STATUS_NOT_SUPPORTED
     # MXFP4 needs whole 256-element K stages for the MFMA kernel
     assert plan(api, dict(MX, m=256, n=256, k=384, transa=1))[1].kernel == GEN
     assert plan(api, dict(MX, m=256, n=256, k=512, transa=1))[1].kernel == K.ZLUDA_KERNEL_MFMA_MXF4

@@ -5,13 +5,14 @@
 // LDS; from there on the kernel is the K-contiguous one (same fragment layout, same epilogues:
 // gemm_mfma.hpp).
 //
-//   * 4 waves (2 x 2), workgroup tile BP x BQ (128 x 128 or 64 x 64), 64 K bytes per stage, two LDS
-//     stages, one barrier per stage.  Global loads of stage kt+1 are issued into registers right after
+//   * WP x WQ waves (2 x 2, or 2 x 4 for the 256 x 256 tile), workgroup tile BP x BQ, 64 K bytes per
+//     stage, two LDS stages, one barrier per stage.  An operand is loaded by 256 threads: with four
+//     waves every thread serves both operands, with eight the first four waves serve P, the others Q.  Global loads of stage kt+1 are issued into registers right after
 //     the barrier of stage kt and written to LDS at the top of the next trip (register prefetch: the
 //     data cannot go straight to LDS because it has to be transposed).  Several workgroups share a
 //     CU (40 KiB of LDS, ~130 VGPRs), which is what hides the barrier.
 //   * Operand with unit stride along its row index ("MC"): a lane loads a block of 4 K rows x IW row
-//     indices (IW = rows/16 bytes: dword, dwordx2), lanes of a wave run along the row index first so
+//     indices (IW = rows/16 bytes: dword, dwordx2, dwordx4), lanes of a wave run along the row index first so
 //     that an instruction reads whole 64..128-byte pieces of 4 K rows; 8 v_perm_b32 per 4 x 4 bytes
 //     turn the block into one dword of 4 consecutive K bytes per row, written with ds_write_b32.
 //   * Operand with unit stride along K ("KC"): 16 bytes per lane, ds_write_b128.
@@ -58,20 +59,22 @@ struct TrOperand {
   static constexpr int NW = IW / 4;           // MC: dwords per load
   static constexpr int NCH = ROWS / 64;       // KC: 16-byte chunks per lane and stage
   static constexpr int NREG = KC ? NCH * 4 : NW * 4;
-  static_assert(ROWS == 64 || ROWS == 128, "tile operands of 64 or 128 rows");
+  static_assert(ROWS == 64 || ROWS == 128 || ROWS == 256, "tile operands of 64, 128 or 256 rows");
 
   __amdgpu_buffer_rsrc_t rs;
   int voff[KC ? NCH : 1];
   int kstep;     // byte offset of one stage
   int kbytes;    // K
   int ld;        // MC: stride of one K row
+  int tc;        // KC: byte offset of this lane's chunk in a stage
   int regs[NREG];
 
   // base: first byte of the operand (this batch); row0: first tile row; nrows: rows of the whole
   // operand; ld_row / ld_k: byte strides (one of them is 1)
-  __device__ __forceinline__ void init(const uint8_t *base, int row0, int nrows, int ld_row, int ld_k, int K) {
-    const int t = threadIdx.x;
+  // t: index of the thread among the 256 that load this operand
+  __device__ __forceinline__ void init(int t, const uint8_t *base, int row0, int nrows, int ld_row, int ld_k, int K) {
     kbytes = K;
+    tc = (t & 3) * 16;
     if constexpr (KC) {
       rs = __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, 0x80000000, 0x00020000);
 #pragma unroll
@@ -93,7 +96,7 @@ struct TrOperand {
     if constexpr (KC) {
 #pragma unroll
       for (int n = 0; n < NCH; n++) {
-        const int oob = kt * 64 + (int)(threadIdx.x & 3) * 16 < kbytes ? 0 : (int)0x80000000;
+        const int oob = kt * 64 + tc < kbytes ? 0 : (int)0x80000000;
         const v4i v = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rs, voff[n] | oob, kt * kstep, 0));
         regs[n * 4 + 0] = v[0]; regs[n * 4 + 1] = v[1]; regs[n * 4 + 2] = v[2]; regs[n * 4 + 3] = v[3];
       }
@@ -102,17 +105,19 @@ struct TrOperand {
       for (int j = 0; j < 4; j++) {
         if constexpr (NW == 1) {
           regs[j] = __builtin_amdgcn_raw_buffer_load_b32(rs, voff[0] + j * ld, kt * kstep, 0);
-        } else {
+        } else if constexpr (NW == 2) {
           const v2i v = __builtin_bit_cast(v2i, __builtin_amdgcn_raw_buffer_load_b64(rs, voff[0] + j * ld, kt * kstep, 0));
           regs[j * 2] = v[0]; regs[j * 2 + 1] = v[1];
+        } else {
+          const v4i v = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rs, voff[0] + j * ld, kt * kstep, 0));
+          regs[j * 4] = v[0]; regs[j * 4 + 1] = v[1]; regs[j * 4 + 2] = v[2]; regs[j * 4 + 3] = v[3];
         }
       }
     }
   }
 
   // `dst`: the operand's rows of one LDS stage (80-byte pitch = 5 v4i)
-  __device__ __forceinline__ void store(v4i *dst) const {
-    const int t = threadIdx.x;
+  __device__ __forceinline__ void store(int t, v4i *dst) const {
     if constexpr (KC) {
 #pragma unroll
       for (int n = 0; n < NCH; n++)
@@ -131,10 +136,12 @@ struct TrOperand {
   }
 };
 
-template <int KIND, int FQ, int FP, int BP, int BQ, bool PKC, bool QKC>
-__global__ __launch_bounds__(256) void gemm_mfma_tr_kernel(MfmaParams prm) {
+template <int KIND, int FQ, int FP, int BP, int BQ, int WP, int WQ, bool PKC, bool QKC>
+__global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_tr_kernel(MfmaParams prm) {
   static_assert(KIND == KIND_I8 || KIND == KIND_F8, "8-bit operands");
-  constexpr int WP = 2, WQ = 2;
+  constexpr int NT = WP * WQ * 64;
+  constexpr bool SPLIT = NT == 512;  // waves 0-3 load P, waves 4-7 load Q
+  static_assert(NT == 256 || NT == 512, "an operand is loaded by 256 threads");
   constexpr int WTP = BP / WP, WTQ = BQ / WQ, TP = WTP / 32, TQ = WTQ / 32;
   constexpr int KS = KIND == KIND_F8 ? 1 : 2;  // MFMA sub-steps per 64-byte stage
   constexpr int STAGE_V4 = (BP + BQ) * 5;
@@ -162,12 +169,14 @@ __global__ __launch_bounds__(256) void gemm_mfma_tr_kernel(MfmaParams prm) {
 
   TrOperand<BP, PKC> P;
   TrOperand<BQ, QKC> Q;
+  const int tl = t & 255;
+  const bool do_p = !SPLIT || wave < 4, do_q = !SPLIT || wave >= 4;  // wave-uniform
   if (!prm.swapped) {
-    P.init((const uint8_t *)g.A + g.a_sb * bt, p0, NP, (int)g.a_si, (int)g.a_sk, g.K);
-    Q.init((const uint8_t *)g.B + g.b_sb * bt, q0, NQ, (int)g.b_sj, (int)g.b_sk, g.K);
+    if (do_p) P.init(tl, (const uint8_t *)g.A + g.a_sb * bt, p0, NP, (int)g.a_si, (int)g.a_sk, g.K);
+    if (do_q) Q.init(tl, (const uint8_t *)g.B + g.b_sb * bt, q0, NQ, (int)g.b_sj, (int)g.b_sk, g.K);
   } else {
-    P.init((const uint8_t *)g.B + g.b_sb * bt, p0, NP, (int)g.b_sj, (int)g.b_sk, g.K);
-    Q.init((const uint8_t *)g.A + g.a_sb * bt, q0, NQ, (int)g.a_si, (int)g.a_sk, g.K);
+    if (do_p) P.init(tl, (const uint8_t *)g.B + g.b_sb * bt, p0, NP, (int)g.b_sj, (int)g.b_sk, g.K);
+    if (do_q) Q.init(tl, (const uint8_t *)g.A + g.a_sb * bt, q0, NQ, (int)g.a_si, (int)g.a_sk, g.K);
   }
   const int KT = (g.K + 63) / 64;
 
@@ -186,16 +195,16 @@ __global__ __launch_bounds__(256) void gemm_mfma_tr_kernel(MfmaParams prm) {
 #pragma unroll
       for (int v = 0; v < 16; v++) acc[a][b][v] = 0;
 
-  P.load(0);
-  Q.load(0);
+  if (do_p) P.load(0);
+  if (do_q) Q.load(0);
   for (int kt = 0; kt < KT; kt++) {
     v4i *stage = &lds[(kt & 1) * STAGE_V4];
-    P.store(stage);
-    Q.store(stage + BP * 5);
+    if (do_p) P.store(tl, stage);
+    if (do_q) Q.store(tl, stage + BP * 5);
     // the other stage is free again: every wave passed this barrier one trip ago, after it had read it
     __syncthreads();
-    P.load(kt + 1);  // one past the end reads zeros, which nothing consumes
-    Q.load(kt + 1);
+    if (do_p) P.load(kt + 1);  // one past the end reads zeros, which nothing consumes
+    if (do_q) Q.load(kt + 1);
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
       frag_v fp[TP], fq[TQ];

@@ -11,24 +11,33 @@ namespace zluda_amd {
 // plan.variant indexes kTrVariants (planner.hpp); pkc / qkc: operand P / Q has unit stride along K
 template <int KIND, int FQ, int FP>
 inline uint32_t launch_tr_variant(const MfmaParams &prm, const zluda_gemm_plan &plan, bool pkc, bool qkc, hipStream_t s) {
-  const dim3 grid(plan.grid_x, plan.grid_y, 1), block(256);
-  static_assert(kNumTrVariants == 2 && kTrVariants[0].bp == 128 && kTrVariants[0].bq == 128 &&
-                kTrVariants[1].bp == 64 && kTrVariants[1].bq == 64, "variant table mismatch");
-#define ZLUDA_TR_CASE(B, PK, QK)                                                                                \
+  const dim3 grid(plan.grid_x, plan.grid_y, 1);
+#define ZLUDA_TR_MODE(BP, BQ, WP, WQ, PK, QK)                                                                   \
   if (pkc == PK && qkc == QK) {                                                                                 \
-    hipLaunchKernelGGL((gemm_mfma_tr_kernel<KIND, FQ, FP, B, B, PK, QK>), grid, block, 0, s, prm);              \
+    hipLaunchKernelGGL((gemm_mfma_tr_kernel<KIND, FQ, FP, BP, BQ, WP, WQ, PK, QK>), grid, dim3(WP * WQ * 64), 0, s, prm); \
     return CUBLAS_STATUS_SUCCESS;                                                                               \
   }
-  if (plan.variant == 0) {
-    ZLUDA_TR_CASE(128, false, false) ZLUDA_TR_CASE(128, false, true) ZLUDA_TR_CASE(128, true, false) ZLUDA_TR_CASE(128, true, true)
-  } else if (plan.variant == 1) {
-    ZLUDA_TR_CASE(64, false, false) ZLUDA_TR_CASE(64, false, true) ZLUDA_TR_CASE(64, true, false) ZLUDA_TR_CASE(64, true, true)
+#define ZLUDA_TR_CASE(V, BP, BQ, WP, WQ)                                                                        \
+  case V:                                                                                                       \
+    static_assert(kTrVariants[V].bp == BP && kTrVariants[V].bq == BQ && kTrVariants[V].wp == WP &&              \
+                  kTrVariants[V].wq == WQ, "variant table mismatch");                                           \
+    ZLUDA_TR_MODE(BP, BQ, WP, WQ, false, false) ZLUDA_TR_MODE(BP, BQ, WP, WQ, false, true)                      \
+    ZLUDA_TR_MODE(BP, BQ, WP, WQ, true, false) ZLUDA_TR_MODE(BP, BQ, WP, WQ, true, true)                        \
+    break;
+  switch (plan.variant) {
+    ZLUDA_TR_CASE(0, 256, 256, 2, 4)
+    ZLUDA_TR_CASE(1, 128, 128, 2, 2)
+    ZLUDA_TR_CASE(2, 64, 64, 2, 2)
+  default: break;
   }
 #undef ZLUDA_TR_CASE
+#undef ZLUDA_TR_MODE
   return CUBLAS_STATUS_INVALID_VALUE;
 }
 
 uint32_t launch_tr_i8(const MfmaParams &prm, const zluda_gemm_plan &plan, bool pkc, bool qkc, hipStream_t s);
 uint32_t launch_tr_f8(const MfmaParams &prm, const zluda_gemm_plan &plan, int fq, int fp, bool pkc, bool qkc, hipStream_t s);
+uint32_t launch_tr_f8_e5m2q(const MfmaParams &prm, const zluda_gemm_plan &plan, bool pkc, bool qkc, hipStream_t s);
+uint32_t launch_tr_f8_e5m2p(const MfmaParams &prm, const zluda_gemm_plan &plan, bool pkc, bool qkc, hipStream_t s);
 
 } // namespace zluda_amd

@@ -327,17 +327,34 @@ static void fill_tr_plan(const Lowered &l, int variant, uint32_t cus, zluda_gemm
   plan->variant = variant;
   plan->swapped = swapped;
   plan->grid_x = ceil_div(np, v.bp) * ceil_div(nq, v.bq); plan->grid_y = g.batch; plan->grid_z = 1;
-  plan->block = 256;
+  plan->block = v.wp * v.wq * 64;
   const uint32_t per_cu = 160u * 1024u / (2u * (v.bp + v.bq) * 80u);  // LDS: two stages of 80-byte rows
   plan->waves = (float)plan->grid_x * plan->grid_y / (float)(cus * std::min(per_cu, 8u));
   plan->workspace = 0;
 }
 
-// the larger tile unless it leaves CUs without a workgroup
+// Tile choice of the transposing kernel.  Cost of a variant = rounds over the workgroup slots of the
+// chip x workgroups that share a CU x tile area / relative throughput of a CU running that tile
+// (measured on MI355X, int8: 8192^3 takes 636 / 1050 / 1300 us with the three tiles; one 128x128
+// workgroup alone on a CU runs at two thirds of that rate, hence the slots).
+static const float kTrVariantEfficiency[kNumTrVariants] = {1.00f, 0.60f, 0.48f};
+static const uint32_t kTrVariantPerCu[kNumTrVariants] = {1, 2, 4};
+
 static int pick_tr_variant(const Lowered &l, uint32_t cus) {
   const GemmArgs &g = l.g;
-  const uint64_t tiles = (uint64_t)ceil_div(g.M, kTrVariants[0].bp) * ceil_div(g.N, kTrVariants[0].bq) * g.batch;
-  return tiles >= cus ? 0 : 1;
+  const bool swapped = g.d_si != 1;
+  const uint32_t np = swapped ? g.N : g.M, nq = swapped ? g.M : g.N;
+  int best = 0;
+  double best_cost = 0;
+  for (int v = 0; v < kNumTrVariants; v++) {
+    const TrVariant &t = kTrVariants[v];
+    const uint64_t tiles = (uint64_t)ceil_div(np, t.bp) * ceil_div(nq, t.bq) * g.batch;
+    const uint64_t slots = (uint64_t)cus * kTrVariantPerCu[v];
+    const uint64_t rounds = (tiles + slots - 1) / slots;
+    const double cost = (double)rounds * kTrVariantPerCu[v] * t.bp * t.bq / kTrVariantEfficiency[v];
+    if (v == 0 || cost < best_cost) { best = v; best_cost = cost; }
+  }
+  return best;
 }
 
 static void fill_decode_plan(const Lowered &l, int variant, uint32_t cus, zluda_gemm_plan *plan) {

@@ -21,11 +21,12 @@ constexpr MfmaVariant kMfmaVariants[] = {
 constexpr int kNumMfmaVariants = sizeof(kMfmaVariants) / sizeof(kMfmaVariants[0]);
 
 // tile configurations of the transposing 8-bit MFMA kernel (index = plan.variant for
-// ZLUDA_KERNEL_MFMA_TR8): workgroup tile bp x bq, always 2 x 2 waves and 64 K bytes per stage
-struct TrVariant { int bp, bq; };
+// ZLUDA_KERNEL_MFMA_TR8): workgroup tile bp x bq, wp x wq waves, always 64 K bytes per stage
+struct TrVariant { int bp, bq, wp, wq; };
 constexpr TrVariant kTrVariants[] = {
-    {128, 128},  // 0
-    {64, 64},    // 1: problems that leave CUs idle with the larger tile
+    {256, 256, 2, 4},  // 0: 8 waves, 128x64 per wave, one workgroup per CU
+    {128, 128, 2, 2},  // 1: 4 waves, 64x64 per wave, two workgroups per CU
+    {64, 64, 2, 2},    // 2: 4 waves, 32x32 per wave, four or more per CU: small and skinny problems
 };
 constexpr int kNumTrVariants = sizeof(kTrVariants) / sizeof(kTrVariants[0]);
 
