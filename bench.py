@@ -7,7 +7,7 @@ synthetic inputs that are already resident in HBM.  The headline line reports BA
 case ride along under "also", each with its own roofline figures and, when the installed hipBLASLt
 has a solution, the time of the reference's hipBLASLt-forwarded path on the same buffers.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c5|i8_8192] [--only]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c2|c3|c4|c5|i8_8192] [--only]
                   [--no-cpu] [--no-hipblaslt] [--copy-probe]
 """
 import argparse
@@ -32,6 +32,8 @@ PEAK = {"i8": 5000.0, "f8": 5000.0, "f4": 10100.0, "hbm": 8000.0}  # TOP/s, TFLO
 I8 = dict(a_type=K.CUDA_R_8I, b_type=K.CUDA_R_8I, d_type=K.CUDA_R_32I, compute_type=K.CUBLAS_COMPUTE_32I,
           scale_type=K.CUDA_R_32I, transa=1)
 WORKLOADS = {
+    "c1": dict(name="int8xint8->int32 M=N=K=256 A:N B:T (BASELINE config 1)", kind="i8",
+               spec=dict(I8, m=256, n=256, k=256, transa=0, transb=1), steps=200),
     "c2": dict(name="int8xint8->int32 M=N=K=4096 A:T B:N (BASELINE config 2)", kind="i8",
                spec=dict(I8, m=4096, n=4096, k=4096), steps=50),
     "i8_8192": dict(name="int8xint8->int32 M=N=K=8192 A:T B:N", kind="i8", spec=dict(I8, m=8192, n=8192, k=8192), steps=10),
@@ -230,7 +232,7 @@ def cpu_baseline(key, budget_s=12.0):
     from oracle.cases import Case
     spec = dict(WORKLOADS[key]["spec"])
     full_m = spec["m"]
-    rows = {"c2": full_m, "i8_8192": 2048, "c3": full_m, "c4": 256, "c5": 64}[key]
+    rows = {"c1": full_m, "c2": full_m, "i8_8192": 2048, "c3": full_m, "c4": 256, "c5": 64}[key]
     spec.update(m=rows, batch=1, alpha=1)
     case = Case(spec, 1, int_dist="normal" if key == "c3" else "uniform")
     case.run_oracle()   # page in, spin up the OpenMP team
@@ -279,7 +281,7 @@ def main():
     head = run_workload(torch, api, key, steps, args.warmup, not args.no_hipblaslt)
     also = {}
     if not args.only:
-        for other in ("i8_8192", "c3", "c4", "c5", "c2"):
+        for other in ("i8_8192", "c3", "c4", "c5", "c2", "c1"):
             if other == key:
                 continue
             try:

@@ -83,7 +83,9 @@ def test_misaligned_or_strided_operands_leave_the_dma_kernels(api):
     st, p = plan(api, dict(spec, transa=0, transb=1, m=4096, n=4096))
     assert st == 0 and p.kernel == TR8 and p.variant == 0 and p.grid_x == 256 and p.block == 512
     st, p = plan(api, dict(spec, transa=0, transb=1, m=4096, n=1024, k=4096))
-    assert st == 0 and p.variant == 2 and p.grid_x == 1024 and p.block == 256
+    assert st == 0 and p.variant == 1 and p.grid_x == 256 and p.block == 256
+    st, p = plan(api, dict(spec, transa=0, transb=1, m=1024, n=1024, k=1024))
+    assert st == 0 and p.variant == 2 and p.grid_x == 256 and p.block == 256
     st, p = plan(api, dict(spec, transa=0, transb=1, m=8192, n=4096, k=1024))
     assert st == 0 and p.variant == 0 and p.grid_x == 512
     assert api.zluda_gemm_variant_count(TR8) == 3

@@ -6,14 +6,17 @@
 // gemm_mfma.hpp).
 //
 //   * WP x WQ waves (2 x 2, or 2 x 4 for the 256 x 256 tile), workgroup tile BP x BQ, 64 K bytes per
-//     stage, two LDS stages, one barrier per stage.  An operand is loaded by 256 threads: with four
-//     waves every thread serves both operands, with eight the first four waves serve P, the others Q.  Global loads of stage kt+1 are issued into registers right after
-//     the barrier of stage kt and written to LDS at the top of the next trip (register prefetch: the
-//     data cannot go straight to LDS because it has to be transposed).  Several workgroups share a
-//     CU (40 KiB of LDS, ~130 VGPRs), which is what hides the barrier.
+//     stage, two LDS stages, one barrier per stage.  Every thread serves both operands, in groups of
+//     256 threads: with eight waves the second group takes the upper 128 rows of P and of Q (no
+//     control flow depends on the wave, so the loop body stays one block the scheduler can mix).
+//     The data cannot go straight to LDS because it has to be transposed, so it is prefetched
+//     into registers (two register sets per operand): while the first half of stage kt is
+//     multiplied, the registers of stage kt+1 are transposed into the other LDS stage; the barrier
+//     sits in the middle of the stage, so that the second half of the MFMAs covers the fragment reads
+//     of stage kt+1 and the issue of the loads of stage kt+3.
 //   * Operand with unit stride along its row index ("MC"): a lane loads a block of 4 K rows x IW row
-//     indices (IW = rows/16 bytes: dword, dwordx2, dwordx4), lanes of a wave run along the row index first so
-//     that an instruction reads whole 64..128-byte pieces of 4 K rows; 8 v_perm_b32 per 4 x 4 bytes
+//     indices (IW = rows/16 bytes: dword, dwordx2, dwordx4), lanes of a wave run along the row index
+//     first so that an instruction reads whole 64..256-byte pieces of 4 K rows; 8 v_perm_b32 per 4 x 4 bytes
 //     turn the block into one dword of 4 consecutive K bytes per row, written with ds_write_b32.
 //   * Operand with unit stride along K ("KC"): 16 bytes per lane, ds_write_b128.
 //   * LDS rows have a pitch of 80 bytes and are stored in permuted order, rho(i) = 16 r + ((g + s r) mod 16)
@@ -52,14 +55,15 @@ __device__ __forceinline__ void transpose4x4(int x0, int x1, int x2, int x3, int
   out[3] = __builtin_amdgcn_perm(t23h, t01h, 0x07060302);
 }
 
-// Global -> register -> LDS path of one tile operand with ROWS rows; KC: unit stride along K.
+// Global -> register -> LDS path of ROWS rows of a tile operand, served by 256 threads; KC: unit
+// stride along K.
 template <int ROWS, bool KC>
 struct TrOperand {
   static constexpr int IW = ROWS / 16;        // MC: row indices per lane (bytes per load)
   static constexpr int NW = IW / 4;           // MC: dwords per load
   static constexpr int NCH = ROWS / 64;       // KC: 16-byte chunks per lane and stage
   static constexpr int NREG = KC ? NCH * 4 : NW * 4;
-  static_assert(ROWS == 64 || ROWS == 128 || ROWS == 256, "tile operands of 64, 128 or 256 rows");
+  static_assert(ROWS == 64 || ROWS == 128 || ROWS == 256, "64, 128 or 256 rows per group of 256 threads");
 
   __amdgpu_buffer_rsrc_t rs;
   int voff[KC ? NCH : 1];
@@ -67,7 +71,6 @@ struct TrOperand {
   int kbytes;    // K
   int ld;        // MC: stride of one K row
   int tc;        // KC: byte offset of this lane's chunk in a stage
-  int regs[NREG];
 
   // base: first byte of the operand (this batch); row0: first tile row; nrows: rows of the whole
   // operand; ld_row / ld_k: byte strides (one of them is 1)
@@ -92,7 +95,7 @@ struct TrOperand {
     }
   }
 
-  __device__ __forceinline__ void load(int kt) {
+  __device__ __forceinline__ void load(int kt, int (&regs)[NREG]) const {
     if constexpr (KC) {
 #pragma unroll
       for (int n = 0; n < NCH; n++) {
@@ -117,7 +120,7 @@ struct TrOperand {
   }
 
   // `dst`: the operand's rows of one LDS stage (80-byte pitch = 5 v4i)
-  __device__ __forceinline__ void store(int t, v4i *dst) const {
+  __device__ __forceinline__ void store(int t, v4i *dst, const int (&regs)[NREG]) const {
     if constexpr (KC) {
 #pragma unroll
       for (int n = 0; n < NCH; n++)
@@ -140,8 +143,8 @@ template <int KIND, int FQ, int FP, int BP, int BQ, int WP, int WQ, bool PKC, bo
 __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_tr_kernel(MfmaParams prm) {
   static_assert(KIND == KIND_I8 || KIND == KIND_F8, "8-bit operands");
   constexpr int NT = WP * WQ * 64;
-  constexpr bool SPLIT = NT == 512;  // waves 0-3 load P, waves 4-7 load Q
-  static_assert(NT == 256 || NT == 512, "an operand is loaded by 256 threads");
+  static_assert(NT == 256 || NT == 512, "operand rows are dealt to groups of 256 threads");
+  constexpr int LP = BP * 256 / NT, LQ = BQ * 256 / NT;  // rows of P / Q one group loads
   constexpr int WTP = BP / WP, WTQ = BQ / WQ, TP = WTP / 32, TQ = WTQ / 32;
   constexpr int KS = KIND == KIND_F8 ? 1 : 2;  // MFMA sub-steps per 64-byte stage
   constexpr int STAGE_V4 = (BP + BQ) * 5;
@@ -167,25 +170,31 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_tr_kernel(MfmaParams pr
   const int p0 = tile_p * BP, q0 = tile_q * BQ;
   const int NP = prm.swapped ? g.N : g.M, NQ = prm.swapped ? g.M : g.N;
 
-  TrOperand<BP, PKC> P;
-  TrOperand<BQ, QKC> Q;
-  const int tl = t & 255;
-  const bool do_p = !SPLIT || wave < 4, do_q = !SPLIT || wave >= 4;  // wave-uniform
+  TrOperand<LP, PKC> P;
+  TrOperand<LQ, QKC> Q;
+  const int tl = t & 255, grp = wave >> 2;
+  const int lds_p = grp * LP * 5, lds_q = (BP + grp * LQ) * 5;  // this group's rows inside a stage
   if (!prm.swapped) {
-    if (do_p) P.init(tl, (const uint8_t *)g.A + g.a_sb * bt, p0, NP, (int)g.a_si, (int)g.a_sk, g.K);
-    if (do_q) Q.init(tl, (const uint8_t *)g.B + g.b_sb * bt, q0, NQ, (int)g.b_sj, (int)g.b_sk, g.K);
+    P.init(tl, (const uint8_t *)g.A + g.a_sb * bt, p0 + grp * LP, NP, (int)g.a_si, (int)g.a_sk, g.K);
+    Q.init(tl, (const uint8_t *)g.B + g.b_sb * bt, q0 + grp * LQ, NQ, (int)g.b_sj, (int)g.b_sk, g.K);
   } else {
-    if (do_p) P.init(tl, (const uint8_t *)g.B + g.b_sb * bt, p0, NP, (int)g.b_sj, (int)g.b_sk, g.K);
-    if (do_q) Q.init(tl, (const uint8_t *)g.A + g.a_sb * bt, q0, NQ, (int)g.a_si, (int)g.a_sk, g.K);
+    P.init(tl, (const uint8_t *)g.B + g.b_sb * bt, p0 + grp * LP, NP, (int)g.b_sj, (int)g.b_sk, g.K);
+    Q.init(tl, (const uint8_t *)g.A + g.a_sb * bt, q0 + grp * LQ, NQ, (int)g.a_si, (int)g.a_sk, g.K);
   }
   const int KT = (g.K + 63) / 64;
 
   // LDS rows (in v4i units) of this lane's fragment rows
   int prow[TP], qrow[TQ];
 #pragma unroll
-  for (int b = 0; b < TP; b++) prow[b] = tr_rho_of<BP>(wp * WTP + b * 32 + lr) * 5;
+  for (int b = 0; b < TP; b++) {
+    const int i = wp * WTP + b * 32 + lr;
+    prow[b] = (i / LP * LP + tr_rho_of<LP>(i % LP)) * 5;
+  }
 #pragma unroll
-  for (int a = 0; a < TQ; a++) qrow[a] = (BP + tr_rho_of<BQ>(wq * WTQ + a * 32 + lr)) * 5;
+  for (int a = 0; a < TQ; a++) {
+    const int i = wq * WTQ + a * 32 + lr;
+    qrow[a] = (BP + i / LQ * LQ + tr_rho_of<LQ>(i % LQ)) * 5;
+  }
 
   acc_v acc[TQ][TP];
 #pragma unroll
@@ -195,48 +204,114 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_tr_kernel(MfmaParams pr
 #pragma unroll
       for (int v = 0; v < 16; v++) acc[a][b][v] = 0;
 
-  if (do_p) P.load(0);
-  if (do_q) Q.load(0);
-  for (int kt = 0; kt < KT; kt++) {
-    v4i *stage = &lds[(kt & 1) * STAGE_V4];
-    if (do_p) P.store(tl, stage);
-    if (do_q) Q.store(tl, stage + BP * 5);
-    // the other stage is free again: every wave passed this barrier one trip ago, after it had read it
-    __syncthreads();
-    if (do_p) P.load(kt + 1);  // one past the end reads zeros, which nothing consumes
-    if (do_q) Q.load(kt + 1);
+  // fragments of sub-step ks of the stage in `buf`
+  struct Frags { frag_v p[TP], q[TQ]; };
+  auto read_frags = [&](const v4i *buf, int ks, Frags &f) {
+    if constexpr (KIND == KIND_I8) {
+      const int ch = ks * 2 + gsel;
 #pragma unroll
-    for (int ks = 0; ks < KS; ks++) {
-      frag_v fp[TP], fq[TQ];
-      if constexpr (KIND == KIND_I8) {
-        const int ch = ks * 2 + gsel;
+      for (int b = 0; b < TP; b++) f.p[b] = buf[prow[b] + ch];
 #pragma unroll
-        for (int b = 0; b < TP; b++) fp[b] = stage[prow[b] + ch];
+      for (int a = 0; a < TQ; a++) f.q[a] = buf[qrow[a] + ch];
+    } else {
+      const int c0 = gsel * 2;
 #pragma unroll
-        for (int a = 0; a < TQ; a++) fq[a] = stage[qrow[a] + ch];
-      } else {
-        const int c0 = gsel * 2;
-#pragma unroll
-        for (int b = 0; b < TP; b++) {
-          const v4i lo = stage[prow[b] + c0], hi = stage[prow[b] + c0 + 1];
-          fp[b] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        }
-#pragma unroll
-        for (int a = 0; a < TQ; a++) {
-          const v4i lo = stage[qrow[a] + c0], hi = stage[qrow[a] + c0 + 1];
-          fq[a] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        }
+      for (int b = 0; b < TP; b++) {
+        const v4i lo = buf[prow[b] + c0], hi = buf[prow[b] + c0 + 1];
+        f.p[b] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
       }
 #pragma unroll
-      for (int a = 0; a < TQ; a++)
-#pragma unroll
-        for (int b = 0; b < TP; b++) {
-          if constexpr (KIND == KIND_I8)
-            acc[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fq[a], fp[b], acc[a][b], 0, 0, 0);
-          else
-            acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fq[a], fp[b], acc[a][b], FQ, FP, 0, 0, 0, 0);
-        }
+      for (int a = 0; a < TQ; a++) {
+        const v4i lo = buf[qrow[a] + c0], hi = buf[qrow[a] + c0 + 1];
+        f.q[a] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      }
     }
+  };
+  auto mfma_all = [&](const Frags &f) {
+#pragma unroll
+    for (int a = 0; a < TQ; a++)
+#pragma unroll
+      for (int b = 0; b < TP; b++) {
+        if constexpr (KIND == KIND_I8)
+          acc[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.q[a], f.p[b], acc[a][b], 0, 0, 0);
+        else
+          acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.q[a], f.p[b], acc[a][b], FQ, FP, 0, 0, 0, 0);
+      }
+  };
+
+  // One stage (kt), entered with: stage kt complete in `cur`, its sub-step-0 fragments in `f0`, stage
+  // kt+1 in the register sets `sp` / `sq` (loads issued a trip and a half ago), the loads of stage
+  // kt+2 in flight into the other sets.
+  //   first half : MFMAs of sub-step 0, and between them the transposition of stage kt+1 into `nxt`
+  //                (plus the fragment reads of sub-step 1);
+  //   barrier    : `nxt` is complete and nobody reads `cur` any more;
+  //   second half: loads of stage kt+3 into the sets just emptied, fragment reads of stage kt+1's
+  //                sub-step 0, and the MFMAs of sub-step 1 that cover both.
+  // (fp8 stages have a single sub-step: its MFMAs all run in the first half.)
+  auto stage_trip = [&](int kt, const v4i *cur, v4i *nxt, int (&sp)[P.NREG], int (&sq)[Q.NREG], Frags &f0) {
+    Frags f1;
+    if constexpr (KS == 2) read_frags(cur, 1, f1);
+    P.store(tl, nxt + lds_p, sp);
+    Q.store(tl, nxt + lds_q, sq);
+    mfma_all(f0);
+    {
+      // the fragment reads of sub-step 1 go out with the first MFMAs, the byte permutes follow (an LDS
+      // write needs the eight permutes of its 4 x 4 block), the LDS writes come behind the later MFMAs
+      constexpr int NM = TP * TQ, H = NM / 2 > 0 ? NM / 2 : 1;
+      constexpr int NDR = KS == 2 ? (TP + TQ) : 0;
+      constexpr int NPERM = ((PKC ? 0 : P.NREG * 2) + (QKC ? 0 : Q.NREG * 2));
+      constexpr int NDW = (PKC ? P.NCH : P.NREG) + (QKC ? Q.NCH : Q.NREG);
+      static_for<NM>([&](auto i_c) {
+        constexpr int i = decltype(i_c)::value;
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        if constexpr (i < H) {
+          constexpr int nr = NDR * (i + 1) / H - NDR * i / H;
+          if constexpr (nr > 0) __builtin_amdgcn_sched_group_barrier(0x100, nr, 0);
+          constexpr int nv = NPERM * (i + 1) / H - NPERM * i / H;
+          if constexpr (nv > 0) __builtin_amdgcn_sched_group_barrier(0x002, nv, 0);
+        } else {
+          constexpr int nw = NDW * (i - H + 1) / (NM - H) - NDW * (i - H) / (NM - H);
+          if constexpr (nw > 0) __builtin_amdgcn_sched_group_barrier(0x200, nw, 0);
+        }
+      });
+    }
+    // (register-only instructions may otherwise drift across the barrier: keep both halves whole)
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+    P.load(kt + 3, sp);  // past the end: zeros, which multiply nothing
+    Q.load(kt + 3, sq);
+    read_frags(nxt, 0, f0);
+    if constexpr (KS == 2) {
+      mfma_all(f1);
+      constexpr int NM = TP * TQ, NDR = TP + TQ;
+      constexpr int NVM = (PKC ? P.NCH : 4) + (QKC ? Q.NCH : 4);
+      static_for<NM>([&](auto i_c) {
+        constexpr int i = decltype(i_c)::value;
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        constexpr int nr = NDR * (i + 1) / NM - NDR * i / NM;
+        if constexpr (nr > 0) __builtin_amdgcn_sched_group_barrier(0x100, nr, 0);
+        constexpr int nv = NVM * (i + 1) / NM - NVM * i / NM;
+        if constexpr (nv > 0) __builtin_amdgcn_sched_group_barrier(0x020, nv, 0);
+      });
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  // two register sets per operand: stage s travels through set s & 1
+  int rp0[P.NREG], rp1[P.NREG], rq0[Q.NREG], rq1[Q.NREG];
+  v4i *buf0 = &lds[0], *buf1 = &lds[STAGE_V4];
+  Frags f0;
+  P.load(0, rp0); Q.load(0, rq0);
+  P.load(1, rp1); Q.load(1, rq1);
+  P.store(tl, buf0 + lds_p, rp0);
+  Q.store(tl, buf0 + lds_q, rq0);
+  __syncthreads();
+  P.load(2, rp0); Q.load(2, rq0);
+  read_frags(buf0, 0, f0);
+  for (int kt = 0; kt < KT; kt += 2) {
+    stage_trip(kt, buf0, buf1, rp1, rq1, f0);
+    if (kt + 1 < KT) stage_trip(kt + 1, buf1, buf0, rp0, rq0, f0);
   }
 
   // every wave is done with the LDS stages before they become epilogue staging

@@ -329,16 +329,16 @@ static void fill_tr_plan(const Lowered &l, int variant, uint32_t cus, zluda_gemm
   plan->grid_x = ceil_div(np, v.bp) * ceil_div(nq, v.bq); plan->grid_y = g.batch; plan->grid_z = 1;
   plan->block = v.wp * v.wq * 64;
   const uint32_t per_cu = 160u * 1024u / (2u * (v.bp + v.bq) * 80u);  // LDS: two stages of 80-byte rows
-  plan->waves = (float)plan->grid_x * plan->grid_y / (float)(cus * std::min(per_cu, 8u));
+  plan->waves = (float)plan->grid_x * plan->grid_y / (float)(cus * std::min(per_cu, 4u));
   plan->workspace = 0;
 }
 
-// Tile choice of the transposing kernel.  Cost of a variant = rounds over the workgroup slots of the
-// chip x workgroups that share a CU x tile area / relative throughput of a CU running that tile
-// (measured on MI355X, int8: 8192^3 takes 636 / 1050 / 1300 us with the three tiles; one 128x128
-// workgroup alone on a CU runs at two thirds of that rate, hence the slots).
-static const float kTrVariantEfficiency[kNumTrVariants] = {1.00f, 0.60f, 0.48f};
-static const uint32_t kTrVariantPerCu[kNumTrVariants] = {1, 2, 4};
+// Tile choice of the transposing kernel.  A CU runs up to `per_cu` workgroups of a variant side by
+// side; the time it needs for n of them (same K) was measured on MI355X (int8, K = 4096, us):
+// 256x256: 71;  128x128: 37 alone, 48 for two;  64x64: 22 alone, 40 for four  ->  base + slope * n.
+// Cost of a variant = full rounds x time(per_cu) + time(what is left per CU).
+struct TrCost { uint32_t per_cu; float base, slope; };
+static const TrCost kTrCost[kNumTrVariants] = {{1, 0.0f, 71.0f}, {2, 26.0f, 11.0f}, {4, 16.0f, 6.0f}};
 
 static int pick_tr_variant(const Lowered &l, uint32_t cus) {
   const GemmArgs &g = l.g;
@@ -348,10 +348,12 @@ static int pick_tr_variant(const Lowered &l, uint32_t cus) {
   double best_cost = 0;
   for (int v = 0; v < kNumTrVariants; v++) {
     const TrVariant &t = kTrVariants[v];
+    const TrCost &c = kTrCost[v];
     const uint64_t tiles = (uint64_t)ceil_div(np, t.bp) * ceil_div(nq, t.bq) * g.batch;
-    const uint64_t slots = (uint64_t)cus * kTrVariantPerCu[v];
-    const uint64_t rounds = (tiles + slots - 1) / slots;
-    const double cost = (double)rounds * kTrVariantPerCu[v] * t.bp * t.bq / kTrVariantEfficiency[v];
+    const uint64_t slots = (uint64_t)cus * c.per_cu;
+    const uint64_t full = tiles / slots, rem = tiles % slots;
+    double cost = (double)full * (c.base + c.slope * c.per_cu);
+    if (rem) cost += c.base + c.slope * (double)((rem + cus - 1) / cus);
     if (v == 0 || cost < best_cost) { best = v; best_cost = cost; }
   }
   return best;
