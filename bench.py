@@ -7,7 +7,7 @@ synthetic inputs that are already resident in HBM.  The headline line reports BA
 case ride along under "also", each with its own roofline figures and, when the installed hipBLASLt
 has a solution, the time of the reference's hipBLASLt-forwarded path on the same buffers.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c2|c3|c4|c5|i8_8192] [--only]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c2|c3|c4|c5|i8_8192|i8_4096_nt] [--only]
                   [--no-cpu] [--no-hipblaslt] [--copy-probe]
 """
 import argparse
@@ -36,6 +36,8 @@ WORKLOADS = {
                spec=dict(I8, m=256, n=256, k=256, transa=0, transb=1), steps=200),
     "c2": dict(name="int8xint8->int32 M=N=K=4096 A:T B:N (BASELINE config 2)", kind="i8",
                spec=dict(I8, m=4096, n=4096, k=4096), steps=50),
+    "i8_4096_nt": dict(name="int8xint8->int32 M=N=K=4096 A:N B:T (config 1's layout at config 2's size)", kind="i8",
+                       spec=dict(I8, m=4096, n=4096, k=4096, transa=0, transb=1), steps=50),
     "i8_8192": dict(name="int8xint8->int32 M=N=K=8192 A:T B:N", kind="i8", spec=dict(I8, m=8192, n=8192, k=8192), steps=10),
     "c3": dict(name="W8A8 decode M=14336 N=16 K=4096 alpha-vec + per-token scale + fp32 bias -> bf16 (BASELINE config 3)",
                kind="hbm", steps=200,
@@ -59,7 +61,8 @@ WORKLOADS = {
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # script (each counter scaled by what it reads for the 256 MiB copy of --copy-probe: x2.000 and x1.000).
 # The summaries are profiles/<kernel>_<workload>.txt; re-measure after changing a kernel's tiling.
-MEASURED_TRAFFIC = {"c2": 167932106, "i8_8192": 1074777202, "c3": 60076820, "c4": 941640909, "c5": 2250162262}
+MEASURED_TRAFFIC = {"c1": 890804, "c2": 167932243, "i8_4096_nt": 167928019, "i8_8192": 1074786759, "c3": 60073313, "c4": 941586833,
+                    "c5": 2250296529}
 
 
 def algorithmic(spec):
@@ -232,7 +235,7 @@ def cpu_baseline(key, budget_s=12.0):
     from oracle.cases import Case
     spec = dict(WORKLOADS[key]["spec"])
     full_m = spec["m"]
-    rows = {"c1": full_m, "c2": full_m, "i8_8192": 2048, "c3": full_m, "c4": 256, "c5": 64}[key]
+    rows = {"c1": full_m, "c2": full_m, "i8_4096_nt": full_m, "i8_8192": 2048, "c3": full_m, "c4": 256, "c5": 64}[key]
     spec.update(m=rows, batch=1, alpha=1)
     case = Case(spec, 1, int_dist="normal" if key == "c3" else "uniform")
     case.run_oracle()   # page in, spin up the OpenMP team
@@ -281,7 +284,7 @@ def main():
     head = run_workload(torch, api, key, steps, args.warmup, not args.no_hipblaslt)
     also = {}
     if not args.only:
-        for other in ("i8_8192", "c3", "c4", "c5", "c2", "c1"):
+        for other in ("i8_8192", "c3", "c4", "c5", "c2", "c1", "i8_4096_nt"):
             if other == key:
                 continue
             try:
