@@ -71,6 +71,28 @@ def test_decode_shapes_around_the_limits(gpu_api):
         run(gpu_api, dict(dec, c_type=K.CUDA_R_16F, d_type=K.CUDA_R_16F, m=2048, n=8, k=4096, ldd=ld, ldc=ld), 345, int_dist="normal")
 
 
+def test_decode_shapes_outside_the_stream_table_on_mfma_tiles(gpu_api):
+    """K values the LDS-streaming decode kernel has no instantiation for: MFMA tiles when they fill at
+    least half of the CUs (with the K split through the workspace if there is one), with the full decode
+    epilogue: alpha vector, per-token scale, bias"""
+    dec = dict(I8, c_type=K.CUDA_R_16BF, d_type=K.CUDA_R_16BF, scale_type=K.CUDA_R_32F,
+               pointer_mode=K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO,
+               b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F, epilogue=K.CUBLASLT_EPILOGUE_BIAS,
+               bias_type=K.CUDA_R_32F, alpha_range=(0.001, 0.01), scale_range=(0.005, 0.02), bias_std=0.02)
+    assert run(gpu_api, dict(dec, m=8192, n=16, k=2624), 350, int_dist="normal") == K.ZLUDA_KERNEL_MFMA_I8
+    assert run(gpu_api, dict(dec, m=2048, n=16, k=2624), 351, int_dist="normal") == K.ZLUDA_KERNEL_DECODE_W8A8
+    spec = dict(dec, m=4096, n=32, k=11008)
+    print("edge case", spec, "with a 64 MiB workspace", flush=True)
+    case = Case(spec, 352, int_dist="normal")
+    ref = case.run_oracle()
+    st, got, kern, variant = case.run_gpu(gpu_api, workspace_bytes=64 << 20)
+    assert st == 0 and kern == K.ZLUDA_KERNEL_MFMA_I8 and case.last_workspace_needed > 0
+    case.compare(got, ref)
+    st, got, kern, variant = case.run_gpu(gpu_api)          # no workspace: 64 tiles only, decode family
+    assert st == 0 and kern == K.ZLUDA_KERNEL_DECODE_W8A8
+    case.compare(got, ref)
+
+
 def test_in_place_c_equals_d_and_device_scalars(gpu_api):
     """C == D with beta != 0 (allowed: ext/hipblaslt-sys/src/lib.rs:1166-1177), alpha/beta read from device memory"""
     import torch

@@ -146,3 +146,23 @@ def test_split_k_needs_workspace_and_few_tiles(api):
     assert plan_ws(dict(I8, m=4096, n=4096, k=8192, transa=1), 1 << 30)[1].grid_z == 1
     assert plan_ws(dict(I8, m=1024, n=256, k=256, transa=1), 1 << 30)[1].grid_z == 1
     assert plan_ws(dict(MX, m=1024, n=256, k=8192, transa=1), 1 << 30)[1].grid_z == 1
+
+
+def test_decode_shapes_outside_the_stream_table(api):
+    """the LDS-streaming decode kernel serves a table of K values; elsewhere the planner takes MFMA tiles
+    (split along K through the workspace) when they occupy at least half of the CUs, and the
+    register-streaming decode variant otherwise"""
+    dec = dict(I8, transa=1, d_type=K.CUDA_R_16BF, scale_type=K.CUDA_R_32F,
+               pointer_mode=K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO,
+               b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F,
+               epilogue=K.CUBLASLT_EPILOGUE_BIAS, bias_type=K.CUDA_R_32F)
+    st, p = plan(api, dict(dec, m=14336, n=16, k=4096))                       # in the table
+    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.variant == 4
+    st, p = plan(api, dict(dec, m=5120, n=16, k=13824), workspace=64 << 20)   # 80 tiles x 6 K shares
+    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_I8 and p.grid_z > 1 and p.grid_x * p.grid_z >= 128
+    st, p = plan(api, dict(dec, m=5120, n=16, k=13824))                       # no workspace: 80 tiles only
+    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.variant == 0
+    st, p = plan(api, dict(dec, m=18944, n=32, k=3584))                       # 296 tiles without any split
+    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_I8 and p.grid_z == 1
+    st, p = plan(api, dict(dec, m=2048, n=16, k=2560), workspace=64 << 20)    # 32 tiles, short K
+    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8

@@ -247,7 +247,9 @@ bool family_supports(uint32_t kernel, const Lowered &l) {
       const int64_t span = (int64_t)(rows - 1) * s_row + (int64_t)(g.K - 1) * s_k + 1;
       if (span >= 0x7fffffffll) return false;
       if (s_k == 1) return (s_row & 3) == 0 && (g.K & 15) == 0;  // 16-byte pieces along K
-      return s_row == 1 && (s_k & 3) == 0;
+      // (offsets of K rows up to three stages past the end must stay below 2^32, where they are out
+      // of range instead of wrapping into it)
+      return s_row == 1 && (s_k & 3) == 0 && (int64_t)(g.K + 256) * s_k < 0xffffffffll;
     };
     return types && d_fast && g.a_scale_mode != SCALE_BLOCK32_UE8M0 && g.b_scale_mode != SCALE_BLOCK32_UE8M0 &&
            operand_ok(g.A, g.a_si, g.a_sk, g.a_sb, g.M) && operand_ok(g.B, g.b_sj, g.b_sk, g.b_sb, g.N);
@@ -421,7 +423,20 @@ extern "C" uint32_t zluda_gemm_plan_problem(const zluda_gemm_problem *p, uint32_
                                      ZLUDA_KERNEL_MFMA_MXF4, ZLUDA_KERNEL_MFMA_TR8, ZLUDA_KERNEL_GENERIC};
     for (uint32_t k : order) {
       if (k == ZLUDA_KERNEL_DECODE_W8A8 && std::min(l.g.M, l.g.N) > kDecodeAutoMaxTokens) continue;
-      if (family_supports(k, l)) { kernel = k; break; }
+      if (!family_supports(k, l)) continue;
+      if (k == ZLUDA_KERNEL_DECODE_W8A8 && !kDecodeVariants[pick_decode_variant(l)].stream &&
+          family_supports(ZLUDA_KERNEL_MFMA_I8, l)) {
+        // K outside the stream kernel's table: the register-streaming variant measures slower than
+        // 64x64 MFMA tiles (split along K when the workspace allows) as soon as those give at
+        // least half of the CUs a workgroup (5120x16x13824: 37 us against 23; 18944x32x3584: 46
+        // against 25; but 2048x16x2560, 32 tiles: 8 against 12)
+        zluda_gemm_plan mfma;
+        memset(&mfma, 0, sizeof(mfma));
+        fill_mfma_plan(l, pick_mfma_variant(l, cu_count), cu_count, p->workspace_size, &mfma);
+        if ((uint64_t)mfma.grid_x * mfma.grid_y * mfma.grid_z * 2 >= cu_count) continue;
+      }
+      kernel = k;
+      break;
     }
   } else if (!family_supports(kernel, l)) {
     return CUBLAS_STATUS_NOT_SUPPORTED;
