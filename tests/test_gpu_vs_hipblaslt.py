@@ -52,6 +52,34 @@ def test_fp8_scaled_bias_gelu_within_tolerance_of_hipblaslt(gpu_api):
     print("max relative difference to hipBLASLt %.3e" % err)
 
 
+def test_decode_config3_decomposed_through_hipblaslt(gpu_api):
+    """BASELINE config 3 at full size.  hipBLASLt has no int8 -> bf16 algorithm with an alpha vector, so
+    the reference's backend pins the integer part: its int8 -> int32 GEMM of the same operands, followed on
+    the host by the documented epilogue D[i,j] = bf16(alpha[i] * sB[j] * acc[i,j] + bias[i]) in float64,
+    against our fused decode kernel (float bar: 1e-2, bf16 rounding included)."""
+    from oracle.cases import _encode
+    m, n, k = 14336, 16, 4096
+    base = {key: v for key, v in I8.items() if key != "alpha"}      # the decode case draws its alpha vector
+    dec = Case(dict(base, c_type=K.CUDA_R_16BF, d_type=K.CUDA_R_16BF, scale_type=K.CUDA_R_32F, m=m, n=n, k=k,
+                    pointer_mode=K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO,
+                    b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F, epilogue=K.CUBLASLT_EPILOGUE_BIAS,
+                    bias_type=K.CUDA_R_32F, alpha_range=(0.001, 0.01), scale_range=(0.005, 0.02), bias_std=0.02),
+               2, int_dist="normal")
+    print("hipBLASLt decomposition of config 3", flush=True)
+    st, ours, kern, _ = dec.run_gpu(gpu_api)
+    assert st == 0 and kern == K.ZLUDA_KERNEL_DECODE_W8A8
+    plain = Case(dict(I8, m=m, n=n, k=k), 2, int_dist="normal")
+    assert np.array_equal(plain.A, dec.A) and np.array_equal(plain.B, dec.B)
+    acc, why = plain.run_hipblaslt()
+    if acc is None:
+        pytest.skip("hipBLASLt offers no int8 -> int32 algorithm for 14336 x 16 x 4096: " + why)
+    acc = acc.astype(np.float64).reshape(n, m)            # column-major D, ld = m
+    want = dec.alpha.astype(np.float64)[None, :] * dec.b_scale.astype(np.float64)[:, None] * acc + \
+        decode_storage(dec.bias, K.CUDA_R_32F).astype(np.float64)[None, :]
+    err = dec.compare(ours, _encode(want.astype(np.float32).ravel(), K.CUDA_R_16BF), tol=1e-2)
+    print("max relative difference to hipBLASLt int32 GEMM + host epilogue %.3e" % err)
+
+
 def test_gelu_form_of_hipblaslt_is_the_tanh_form(gpu_api):
     """fp32 output, K = 16 with one non-zero product per output: D = GELU(x) for a sweep of x.
     The tanh form 0.5x(1+tanh(sqrt(2/pi)(x+0.044715x^3))) and the erf form 0.5x(1+erf(x/sqrt2)) are
