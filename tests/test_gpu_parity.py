@@ -38,7 +38,7 @@ def check(gpu_api, spec, seed, kernel=None, variant=-1, expect_kernel=None, tol=
 
 
 # ---- int8 -> int32 MFMA, every tile variant --------------------------------
-@pytest.mark.parametrize("variant", range(7))
+@pytest.mark.parametrize("variant", range(8))
 @pytest.mark.parametrize("m,n,k", [(256, 256, 128), (300, 200, 144), (512, 384, 1024)])
 def test_mfma_i8_variants(gpu_api, variant, m, n, k):
     check(gpu_api, dict(I8, m=m, n=n, k=k, lda=k + 16 if k == 144 else k), 10 + variant, K.ZLUDA_KERNEL_MFMA_I8, variant)
@@ -59,7 +59,7 @@ def test_mfma_i8_row_major_output_swaps(gpu_api):
 
 
 # full tiles take the register-direct / vectorised epilogues; cover each of them per tile shape
-@pytest.mark.parametrize("variant", range(7))
+@pytest.mark.parametrize("variant", range(8))
 def test_mfma_full_tile_epilogues(gpu_api, variant):
     full = dict(m=512, n=256, k=384)
     check(gpu_api, dict(I8, **full, alpha=1), 110, K.ZLUDA_KERNEL_MFMA_I8, variant)
@@ -80,7 +80,7 @@ def test_mfma_full_tile_epilogues(gpu_api, variant):
     check(gpu_api, dict(MX, m=512, n=256, k=1024), 116, K.ZLUDA_KERNEL_MFMA_MXF4, variant)
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7])
 def test_mfma_i8_float_epilogue(gpu_api, variant):
     spec = dict(I8F, m=260, n=140, k=512, epilogue=K.CUBLASLT_EPILOGUE_RELU_BIAS, bias_type=K.CUDA_R_32F,
                 pointer_mode=K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_HOST, with_c=True,
@@ -95,7 +95,7 @@ def test_mfma_i8_float_epilogue(gpu_api, variant):
 
 
 # ---- fp8 -------------------------------------------------------------------------------------------
-@pytest.mark.parametrize("variant", range(7))
+@pytest.mark.parametrize("variant", range(8))
 def test_mfma_f8_variants(gpu_api, variant):
     check(gpu_api, dict(F8, m=256, n=256, k=256), 20 + variant, K.ZLUDA_KERNEL_MFMA_F8, variant)
     check(gpu_api, dict(F8, m=320, n=272, k=400, lda=416, ldb=400, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS,
@@ -110,7 +110,7 @@ def test_mfma_f8_mixed_formats(gpu_api, at, bt):
 
 
 # ---- MXFP4 -----------------------------------------------------------------------------------------
-@pytest.mark.parametrize("variant", range(7))
+@pytest.mark.parametrize("variant", range(8))
 def test_mfma_mxf4_variants(gpu_api, variant):
     check(gpu_api, dict(MX, m=256, n=256, k=512), 50 + variant, K.ZLUDA_KERNEL_MFMA_MXF4, variant)
     check(gpu_api, dict(MX, m=288, n=160, k=768, batch=2), 60 + variant, K.ZLUDA_KERNEL_MFMA_MXF4, variant)

@@ -53,6 +53,17 @@ def test_small_problems_get_smaller_tiles(api):
     assert st == 0 and p.variant == 2 and p.grid_x == 16 * 16
 
 
+def test_extents_that_256_divides_badly_get_the_192_row_tile(api):
+    st, p = plan(api, dict(F8, m=6144, n=4096, k=4096, transa=1))
+    assert st == 0 and p.variant == 7 and p.grid_x == 32 * 16          # two full rounds instead of 1.5 -> 2 of 256x256
+    st, p = plan(api, dict(I8, m=3072, n=3072, k=3072, transa=1))
+    assert st == 0 and p.variant == 7 and p.grid_x == 16 * 12
+    st, p = plan(api, dict(I8, m=8192, n=8192, k=8192, transa=1))
+    assert st == 0 and p.variant == 0
+    st, p = plan(api, dict(F8, m=14336, n=4096, k=4096, transa=1))   # 5 rounds of 192x256 lose to 4 of 256x256
+    assert st == 0 and p.variant == 0
+
+
 def test_row_major_output_swaps_operands(api):
     st, p = plan(api, dict(I8, m=512, n=1024, k=512, order_a=1, order_b=1, transb=1, order_c=1, order_d=1))
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_I8 and p.swapped == 1
@@ -120,10 +131,11 @@ def test_fp4_must_be_k_contiguous(api):
 
 def test_forced_variants(api):
     spec = dict(I8, m=4096, n=4096, k=4096, transa=1)
-    for v, (grid, block) in enumerate([(256, 512), (256, 256), (512, 256), (1024, 256), (1024, 256), (2048, 256), (4096, 256)]):
+    for v, (grid, block) in enumerate([(256, 512), (256, 256), (512, 256), (1024, 256), (1024, 256), (2048, 256), (4096, 256),
+                                       (352, 512)]):
         st, p = plan(api, spec, forced=K.ZLUDA_KERNEL_MFMA_I8, variant=v)
         assert st == 0 and p.variant == v and p.grid_x == grid and p.block == block
-    assert plan(api, spec, forced=K.ZLUDA_KERNEL_MFMA_I8, variant=7)[0] == K.CUBLAS_STATUS_INVALID_VALUE
+    assert plan(api, spec, forced=K.ZLUDA_KERNEL_MFMA_I8, variant=8)[0] == K.CUBLAS_STATUS_INVALID_VALUE
     assert plan(api, spec, forced=K.ZLUDA_KERNEL_MFMA_F8)[0] == K.CUBLAS_STATUS_NOT_SUPPORTED
 
 

@@ -88,8 +88,9 @@ __device__ __forceinline__ void mfma_store_tile_general(const MfmaParams &prm, A
   // Each wave stages 16 Q-rows x WTP P-columns per pass in its own LDS region.
   constexpr int SROW = WTP + 8;              // dwords; +8 keeps the two lane halves on distinct banks
   constexpr int LPR = WTP / 4;               // lanes per staged row
-  constexpr int RPI = 64 / LPR;              // staged rows read per instruction
+  constexpr int RPI = 64 / LPR;              // staged rows read per instruction (96-wide wave tiles: 2, lanes 48-63 idle)
   constexpr int ITER = 16 / RPI;
+  static_assert(16 % RPI == 0, "whole passes");
   int *stage = lds_words + wave * (16 * SROW);
 
   Epilogue ep(g, bt);
@@ -133,7 +134,7 @@ __device__ __forceinline__ void mfma_store_tile_general(const MfmaParams &prm, A
       const int ql = it * RPI + qsub;
       const int qi = q0 + wq * WTQ + a * 32 + h * 16 + ql;
       const v4i raw = *(const v4i *)&stage[ql * SROW + pl];
-      if (qi >= NQ || pi0 >= NP) continue;
+      if (qi >= NQ || pi0 >= NP || qsub >= RPI) continue;
       const int64_t dbase = g.d_sb * bt + (int64_t)pi0 * d_sp + (int64_t)qi * d_sq;
       const int64_t cbase = g.c_sb * bt + (int64_t)pi0 * c_sp + (int64_t)qi * c_sq;
       const bool full4 = pi0 + 3 < NP && ((dbase * dbits / 8) & (dbits / 2 - 1)) == 0 &&
@@ -269,6 +270,7 @@ __device__ __forceinline__ void mfma_store_tile_f(const MfmaParams &prm, AccV (&
                                                   int *lds_words, int p0, int q0, int bt) {
   constexpr int TP = WTP / 32, TQ = WTQ / 32;
   constexpr int SROW = WTP + 8, LPR = WTP / 4, RPI = 64 / LPR, ITER = 16 / RPI;
+  static_assert(16 % RPI == 0, "whole passes");
   constexpr int ESZ = DT == 2 ? 4 : 2;
   const GemmArgs &g = prm.g;
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -309,6 +311,7 @@ __device__ __forceinline__ void mfma_store_tile_f(const MfmaParams &prm, AccV (&
     // writes and reads of one wave in program order
 #pragma unroll 2
     for (int it = 0; it < ITER; it++) {
+      if (64 % LPR != 0 && qsub >= RPI) continue;  // 96-wide wave tiles: lanes beyond the last whole staged row
       const v4i raw = *(const v4i *)&stage[it * RPI * SROW + read_off];
       float qs = q_scale_u, qb = 0.0f;
       if (q_vec) {

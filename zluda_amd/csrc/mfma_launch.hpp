@@ -28,6 +28,7 @@ inline uint32_t launch_mfma_variant(const MfmaParams &prm, const zluda_gemm_plan
     ZLUDA_MFMA_CASE(4, 128, 128, 2, 2, 64, 4)
     ZLUDA_MFMA_CASE(5, 128, 64, 2, 2, 128, 3)
     ZLUDA_MFMA_CASE(6, 64, 64, 2, 2, 128, 3)
+    ZLUDA_MFMA_CASE(7, 192, 256, 2, 4, 128, 2)
   default: return CUBLAS_STATUS_INVALID_VALUE;
   }
 #undef ZLUDA_MFMA_CASE

@@ -301,7 +301,7 @@ static void fill_mfma_plan(const Lowered &l, int variant, uint32_t cus, uint64_t
 
 // Relative throughput of one CU running tiles of each variant (measured on MI355X, int8 and fp8, K >= 1024;
 // variant 0 = 1).  Smaller tiles read more LDS and L2 bytes per MFMA.
-static const float kMfmaVariantEfficiency[kNumMfmaVariants] = {1.00f, 0.95f, 0.80f, 0.70f, 0.72f, 0.55f, 0.40f};
+static const float kMfmaVariantEfficiency[kNumMfmaVariants] = {1.00f, 0.95f, 0.80f, 0.70f, 0.72f, 0.55f, 0.40f, 0.85f};
 
 static int pick_mfma_variant(const Lowered &l, uint32_t cus) {
   const GemmArgs &g = l.g;

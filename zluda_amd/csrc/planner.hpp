@@ -17,6 +17,7 @@ constexpr MfmaVariant kMfmaVariants[] = {
     {128, 128, 2, 2, 64, 4},   // 4: same tile, half-line stages, deeper ring (short K)
     {128, 64, 2, 2, 128, 3},   // 5: 4 waves, 64x32 per wave: skinny problems
     {64, 64, 2, 2, 128, 3},    // 6: 4 waves, 32x32 per wave: problems of a few hundred tiles at most
+    {192, 256, 2, 4, 128, 2},  // 7: 8 waves, 96x64 per wave: extents that 256 divides badly (3072, 6144, ...)
 };
 constexpr int kNumMfmaVariants = sizeof(kMfmaVariants) / sizeof(kMfmaVariants[0]);
 
