@@ -40,6 +40,29 @@ def test_int8_bit_exact_with_hipblaslt(gpu_api, n):
     assert np.array_equal(ours, theirs)
 
 
+@pytest.mark.parametrize("n,ta,tb", [(256, 0, 1), (1024, 0, 0), (1024, 0, 1), (1024, 1, 1), (4096, 0, 1)])
+def test_int8_transposed_layouts_bit_exact_with_hipblaslt(gpu_api, n, ta, tb):
+    """BASELINE config 1 (256^3, A:N B:T) and the other layouts in which an operand is not K-contiguous:
+    the transposing MFMA kernel against hipBLASLt called the way the reference forwards it"""
+    spec = dict(I8, m=n, n=n, k=n, transa=ta, transb=tb)
+    case, ours, theirs, why, kern = both(gpu_api, spec, 11)
+    assert kern == K.ZLUDA_KERNEL_MFMA_TR8
+    if theirs is None:
+        pytest.skip("hipBLASLt offers no algorithm here: " + why)
+    assert np.array_equal(ours, theirs)
+
+
+def test_fp8_transposed_layout_within_tolerance_of_hipblaslt(gpu_api):
+    spec = dict(F8, m=1024, n=768, k=512, transa=0, transb=1, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS,
+                bias_type=K.CUDA_R_16BF, with_scalar_scales=True, scale_range=(0.05, 0.06), bias_std=0.5)
+    case, ours, theirs, why, kern = both(gpu_api, spec, 12)
+    assert kern == K.ZLUDA_KERNEL_MFMA_TR8
+    if theirs is None:
+        pytest.skip("hipBLASLt offers no algorithm here: " + why)
+    err = case.compare(ours, theirs, tol=1e-2)
+    print("max relative difference to hipBLASLt %.3e" % err)
+
+
 def test_fp8_scaled_bias_gelu_within_tolerance_of_hipblaslt(gpu_api):
     """BASELINE config 4 at 1024^3: per-tensor scales, bf16 bias, GELU, bf16 output"""
     spec = dict(F8, m=1024, n=1024, k=1024, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS, bias_type=K.CUDA_R_16BF,
