@@ -270,7 +270,8 @@ def test_algorithm_enumeration_and_configuration(api):
     assert api.cublasLtMatmulAlgoGetIds(h, *i8, 1, ids, C.byref(n)) == 0 and n.value == 1
     f8 = (abi.CUBLAS_COMPUTE_32F, abi.CUDA_R_32F, abi.CUDA_R_8F_E4M3, abi.CUDA_R_8F_E4M3, abi.CUDA_R_16BF, abi.CUDA_R_16BF)
     assert api.cublasLtMatmulAlgoGetIds(h, *f8, 8, ids, C.byref(n)) == 0
-    assert sorted(ids[:n.value]) == [abi.ZLUDA_KERNEL_GENERIC, abi.ZLUDA_KERNEL_MFMA_F8, abi.ZLUDA_KERNEL_MFMA_TR8]
+    assert sorted(ids[:n.value]) == [abi.ZLUDA_KERNEL_GENERIC, abi.ZLUDA_KERNEL_MFMA_F8, abi.ZLUDA_KERNEL_DECODE_W8A8,
+                                     abi.ZLUDA_KERNEL_MFMA_TR8]
     f4 = (abi.CUBLAS_COMPUTE_32F, abi.CUDA_R_32F, abi.CUDA_R_4F_E2M1, abi.CUDA_R_4F_E2M1, abi.CUDA_R_16BF, abi.CUDA_R_16BF)
     assert api.cublasLtMatmulAlgoGetIds(h, *f4, 8, ids, C.byref(n)) == 0
     assert sorted(ids[:n.value]) == [abi.ZLUDA_KERNEL_GENERIC, abi.ZLUDA_KERNEL_MFMA_MXF4]

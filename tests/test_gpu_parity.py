@@ -156,6 +156,34 @@ def test_decode_stream_variants(gpu_api, variant, monkeypatch):
             check(gpu_api, dict(I8, m=333, n=tokens - 1, k=k, with_c=True), 180 + variant, K.ZLUDA_KERNEL_DECODE_W8A8, variant)
 
 
+@pytest.mark.parametrize("variant", sorted(STREAM))
+def test_decode_stream_variants_fp8(gpu_api, variant, monkeypatch):
+    """the same kernel for e4m3 x e4m3 (v_mfma_f32_16x16x128_f8f6f4): per-tensor scales, bias, bf16 / f16 / f32
+    outputs, ragged row ranges, 1..64 tokens, a C read"""
+    nw, steps = STREAM[variant]
+    k = nw * steps * 64
+    DEC = K.ZLUDA_KERNEL_DECODE_W8A8
+    f8 = dict(F8, epilogue=K.CUBLASLT_EPILOGUE_BIAS, bias_type=K.CUDA_R_16BF, with_scalar_scales=True, scale_range=(0.05, 0.06))
+    check(gpu_api, dict(f8, m=1000, n=16, k=k), 420 + variant, DEC, variant)
+    monkeypatch.setenv("ZLUDA_DECODE_GRID", "7")
+    check(gpu_api, dict(f8, m=1000, n=5, k=k, lda=k + 64, d_type=K.CUDA_R_16F), 440 + variant, DEC, variant)
+    check(gpu_api, dict(F8, m=333, n=3, k=k, with_c=True, d_type=K.CUDA_R_32F, c_type=K.CUDA_R_32F), 450 + variant, DEC, variant)
+    for blocks, tokens in ((2, 29), (3, 41), (4, 64)):
+        if blocks * steps <= 32:
+            check(gpu_api, dict(f8, m=332, n=tokens, k=k, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS), 460 + variant, DEC, variant)
+
+
+def test_decode_fp8_planner_choice_and_orientation(gpu_api):
+    DEC = K.ZLUDA_KERNEL_DECODE_W8A8
+    check(gpu_api, dict(F8, m=14336, n=16, k=4096, with_scalar_scales=True, scale_range=(0.05, 0.06)), 470, expect_kernel=DEC)
+    # row-major activations [tokens][K] x weights^T: tokens are rows of D
+    check(gpu_api, dict(F8, transa=0, transb=1, order_a=1, order_b=1, order_c=1, order_d=1, m=16, n=2048, k=4096,
+                        epilogue=K.CUBLASLT_EPILOGUE_BIAS, bias_type=K.CUDA_R_16BF), 471, expect_kernel=DEC)
+    # what the family does not take: mixed formats, K outside the table -> the MFMA tiles
+    check(gpu_api, dict(F8, a_type=K.CUDA_R_8F_E5M2, m=2048, n=16, k=4096), 472, expect_kernel=K.ZLUDA_KERNEL_MFMA_F8)
+    check(gpu_api, dict(F8, m=2048, n=16, k=2624 + 64), 473, expect_kernel=K.ZLUDA_KERNEL_MFMA_F8)
+
+
 def test_decode_config3_shape_takes_the_stream_kernel(gpu_api):
     st_spec = dict(DECODE, m=14336, n=16, k=4096)
     check(gpu_api, st_spec, 2, expect_kernel=K.ZLUDA_KERNEL_DECODE_W8A8, int_dist="normal")

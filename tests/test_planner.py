@@ -178,3 +178,17 @@ def test_decode_shapes_outside_the_stream_table(api):
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_I8 and p.grid_z == 1
     st, p = plan(api, dict(dec, m=2048, n=16, k=2560), workspace=64 << 20)    # 32 tiles, short K
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8
+
+
+def test_fp8_decode_takes_the_streaming_kernel_for_table_k_only(api):
+    f8 = dict(F8, transa=1)
+    st, p = plan(api, dict(f8, m=14336, n=16, k=4096))
+    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.variant == 4 and p.grid_x == 256
+    st, p = plan(api, dict(f8, m=14336, n=33, k=4096))                      # beyond 32 tokens: MFMA tiles
+    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_F8
+    st, p = plan(api, dict(f8, m=4096, n=16, k=11008))                      # K outside the table: no fp8 fallback variant
+    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_F8
+    st, p = plan(api, dict(f8, m=4096, n=16, k=4096, b_type=K.CUDA_R_8F_E5M2))
+    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_F8
+    assert plan(api, dict(f8, m=4096, n=16, k=11008), forced=K.ZLUDA_KERNEL_DECODE_W8A8)[0] == K.CUBLAS_STATUS_NOT_SUPPORTED
+    assert plan(api, dict(f8, m=4096, n=16, k=4096), forced=K.ZLUDA_KERNEL_DECODE_W8A8, variant=0)[0] == K.CUBLAS_STATUS_NOT_SUPPORTED

@@ -1,0 +1,75 @@
+// Launchers of the LDS-streaming decode kernel (kernels/decode_stream.hpp), shared by the int8
+// instantiations in launch.hip and the fp8 ones in decode_f8.hip.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "kernels/decode_stream.hpp"
+#include "planner.hpp"
+
+namespace zluda_amd {
+
+template <int N, int I = 0, class F>
+inline void static_for_host(F &&f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for_host<N, I + 1>(f);
+  }
+}
+
+// every output of the problem can leave through the packed 8-byte store of decode_stream_kernel
+inline bool decode_packed_output(const GemmArgs &g, bool swapped) {
+  const int64_t d_sr = swapped ? g.d_sj : g.d_si, d_st = swapped ? g.d_si : g.d_sj;
+  const int rows = swapped ? g.N : g.M;
+  return !g.int_scale && (g.d_type == CUDA_R_16BF || g.d_type == CUDA_R_16F) && d_sr == 1 &&
+         g.beta_mode == SCALAR_VALUE && g.beta_val.f == 0.0f && ((uintptr_t)g.D & 7) == 0 && (d_st & 3) == 0 &&
+         (g.d_sb & 3) == 0 && (rows & 3) == 0;
+}
+
+template <int NW, int SPW, int KIND>
+inline uint32_t launch_decode_stream(const DecodeParams &prm, const zluda_gemm_plan &plan, int nb, hipStream_t s) {
+  dim3 grid(plan.grid_x, plan.grid_y, 1), block(NW * 64);
+  const bool fast = decode_packed_output(prm.g, prm.swapped != 0);
+  bool done = false;
+  static_for_host<4>([&](auto nb_c) {
+    constexpr int NB = decltype(nb_c)::value + 1;
+    if constexpr (NB * SPW <= kDecodeStreamMaxFragments) {
+      if (nb == NB) {
+        if (fast) hipLaunchKernelGGL((decode_stream_kernel<NW, SPW, NB, true, KIND>), grid, block, 0, s, prm);
+        else hipLaunchKernelGGL((decode_stream_kernel<NW, SPW, NB, false, KIND>), grid, block, 0, s, prm);
+        done = true;
+      }
+    }
+  });
+  return done ? CUBLAS_STATUS_SUCCESS : CUBLAS_STATUS_NOT_SUPPORTED;
+}
+
+// plan.variant -> instantiation of the stream kernel for one element kind (the table restates
+// kDecodeVariants, planner.hpp)
+template <int KIND>
+inline uint32_t launch_decode_stream_variant(const DecodeParams &prm, const zluda_gemm_plan &plan, int nb, hipStream_t s) {
+  switch (plan.variant) {
+#define ZLUDA_STREAM_CASE(V, NW, SPW)                                                         \
+  case V:                                                                                     \
+    static_assert(kDecodeVariants[V].nw == NW && kDecodeVariants[V].steps == SPW && kDecodeVariants[V].stream, \
+                  "variant table mismatch");                                                  \
+    return launch_decode_stream<NW, SPW, KIND>(prm, plan, nb, s);
+    ZLUDA_STREAM_CASE(4, 8, 8)
+    ZLUDA_STREAM_CASE(5, 8, 16)
+    ZLUDA_STREAM_CASE(6, 8, 28)
+    ZLUDA_STREAM_CASE(7, 4, 8)
+    ZLUDA_STREAM_CASE(8, 8, 12)
+    ZLUDA_STREAM_CASE(9, 8, 24)
+    ZLUDA_STREAM_CASE(10, 4, 4)
+    ZLUDA_STREAM_CASE(11, 8, 20)
+    ZLUDA_STREAM_CASE(12, 4, 28)
+    ZLUDA_STREAM_CASE(13, 4, 12)
+    ZLUDA_STREAM_CASE(14, 4, 20)
+#undef ZLUDA_STREAM_CASE
+  default: return CUBLAS_STATUS_INVALID_VALUE;
+  }
+}
+
+uint32_t launch_decode_stream_i8(const DecodeParams &prm, const zluda_gemm_plan &plan, int nb, hipStream_t s);
+uint32_t launch_decode_stream_f8(const DecodeParams &prm, const zluda_gemm_plan &plan, int nb, hipStream_t s);
+
+} // namespace zluda_amd

@@ -1,8 +1,12 @@
-// Skinny (<= 32 tokens) W8A8 decode GEMM, streaming form: the weights go from HBM straight into LDS
+// Skinny (<= 64 tokens) W8A8 decode GEMM, streaming form: the weights go from HBM straight into LDS
 // in whole cache lines and are re-read from LDS in the MFMA operand layout.
 //
-//   W : R rows x K int8, K-contiguous (read exactly once)     X : T <= 32 rows x K int8
-//   out(r, t) = sum_k W[r][k] * X[t][k]     int32, then the fused float / integer epilogue
+//   W : R rows x K int8 (or fp8 e4m3), K-contiguous (read exactly once)     X : T <= 64 rows x K, same type
+//   out(r, t) = sum_k W[r][k] * X[t][k]     int32 (fp32), then the fused float / integer epilogue
+//
+// KIND_I8 uses v_mfma_i32_16x16x64_i8 (lane l: row l%16, 16 K-bytes at (l/16)*16 of a 64-byte step),
+// KIND_F8 v_mfma_f32_16x16x128_f8f6f4 (lane l: row l%16, 32 K-bytes at (l/16)*32 of a 128-byte step):
+// the same four 16-byte LDS reads per lane and 256-byte unit, at different chunk positions.
 //
 // Why LDS: v_mfma_i32_16x16x64_i8 wants lane l to hold 16 K-bytes of row l%16, so a 128-bit global
 // load in that layout touches 16 rows x 64 bytes: half a cache line per row.  Measured on MI355X,
@@ -72,8 +76,10 @@ __device__ __forceinline__ void lds_values_ready(v4i (&x)[N]) {
 // epilogue without C, 16-bit D contiguous along the weight rows, 8-byte aligned, row count a multiple
 // of 4); the element-wise epilogue with all its type dispatch is then not even compiled in, which
 // keeps the code the reducing wave runs between two blocks short.
-template <int NW, int SPW, int NB, bool FAST>
+template <int NW, int SPW, int NB, bool FAST, int KIND = KIND_I8>
 __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(DecodeParams prm) {
+  static_assert(KIND == KIND_I8 || KIND == KIND_F8, "int8 or fp8 (e4m3 x e4m3) operands");
+  using acc_t = typename std::conditional<KIND == KIND_I8, v4i, v4f>::type;
   constexpr int SEG = 256;             // bytes of one row per unit
   constexpr int Q = SPW * 64 / SEG;    // units per 16-row block (and wave)
   constexpr int NSLOT = 2;
@@ -136,14 +142,15 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(DecodeParams prm
     }
   }
 
-  // activation fragments of this wave's K slice: lane -> token l16 (+16 per block), 16 bytes at
-  // K = kwave + step*64 + g4*16
+  // activation fragments of this wave's K slice: lane -> token l16 (+16 per block); int8: 16 bytes
+  // at K = kwave + s*64 + g4*16; fp8: the halves (s & 1) of 32 bytes at kwave + (s/2)*128 + g4*32
   v4i xf[NB][SPW];
 #pragma unroll
   for (int nb = 0; nb < NB; nb++) {
-    const uint8_t *xr = Xg + (int64_t)min(nb * 16 + l16, T - 1) * ldx + kwave + g4 * 16;
+    const uint8_t *xr = Xg + (int64_t)min(nb * 16 + l16, T - 1) * ldx + kwave + g4 * (KIND == KIND_I8 ? 16 : 32);
 #pragma unroll
-    for (int s = 0; s < SPW; s++) xf[nb][s] = *(const v4i *)(xr + s * 64);
+    for (int s = 0; s < SPW; s++)
+      xf[nb][s] = *(const v4i *)(xr + (KIND == KIND_I8 ? s * 64 : (s >> 1) * 128 + (s & 1) * 16));
   }
 
   // Pin the wait for the activation loads here, in straight-line code.  Left to its own devices the
@@ -212,9 +219,9 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(DecodeParams prm
           }
       }
     };
-    v4i acc[NB];
+    acc_t acc[NB];
 #pragma unroll
-    for (int nb = 0; nb < NB; nb++) acc[nb] = v4i{0, 0, 0, 0};
+    for (int nb = 0; nb < NB; nb++) acc[nb] = acc_t{0, 0, 0, 0};
 #pragma unroll
     for (int q = 0; q < Q; q++) {
       // the oldest unit in flight has landed (the younger NSLOT-1 may still be on their way)
@@ -222,7 +229,10 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(DecodeParams prm
       const uint32_t src = ring_base + slot * (UNIT_V4 * 16);
       v4i w[4];
 #pragma unroll
-      for (int s = 0; s < 4; s++) w[s] = lds_read16_unordered(src + (((s * 4 + g4) ^ l16) << 4));
+      for (int s = 0; s < 4; s++) {
+        const int chunk = KIND == KIND_I8 ? s * 4 + g4 : (s >> 1) * 8 + g4 * 2 + (s & 1);
+        w[s] = lds_read16_unordered(src + ((chunk ^ l16) << 4));
+      }
       // the fragments are in registers before the slot is overwritten
       frags_ready(w[0], w[1], w[2], w[3]);
       // Issued between the wait for this unit and the refill: the counted wait of the next unit
@@ -244,11 +254,24 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(DecodeParams prm
       issue_unit(fblk, fq, slot);
       if (++fq == Q) { fq = 0; fblk++; }
       slot ^= 1;
+      if constexpr (KIND == KIND_I8) {
 #pragma unroll
-      for (int s = 0; s < 4; s++)
+        for (int s = 0; s < 4; s++)
 #pragma unroll
-        for (int nb = 0; nb < NB; nb++)
-          acc[nb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[s], xf[nb][q * 4 + s], acc[nb], 0, 0, 0);
+          for (int nb = 0; nb < NB; nb++)
+            acc[nb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[s], xf[nb][q * 4 + s], acc[nb], 0, 0, 0);
+      } else {
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+          const v8i wa = {w[2 * s][0], w[2 * s][1], w[2 * s][2], w[2 * s][3], w[2 * s + 1][0], w[2 * s + 1][1], w[2 * s + 1][2], w[2 * s + 1][3]};
+#pragma unroll
+          for (int nb = 0; nb < NB; nb++) {
+            const v4i x0 = xf[nb][q * 4 + 2 * s], x1 = xf[nb][q * 4 + 2 * s + 1];
+            const v8i xb = {x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+            acc[nb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa, xb, acc[nb], 0, 0, 0, 0, 0, 0);
+          }
+        }
+      }
     }
 
     // cross-wave reduction of the finished block (double-buffered: a wave writes its partial sums
@@ -256,7 +279,7 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(DecodeParams prm
     // of block b)
     const int buf = blk & 1;
 #pragma unroll
-    for (int nb = 0; nb < NB; nb++) red[buf][wave][nb][lane] = acc[nb];
+    for (int nb = 0; nb < NB; nb++) red[buf][wave][nb][lane] = __builtin_bit_cast(v4i, acc[nb]);
     lds_barrier();
     if (has_pair) {
 #pragma unroll
@@ -267,9 +290,9 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(DecodeParams prm
         for (int w2 = 0; w2 < NW; w2++)
           part[w2] = lds_read16_unordered(red_base0 + (((buf * NW + w2) * NB + my_nb[pp]) * 64 + src_lane[pp]) * 16);
         lds_values_ready(part);
-        v4i s = part[0];
+        acc_t s = __builtin_bit_cast(acc_t, part[0]);
 #pragma unroll
-        for (int w2 = 1; w2 < NW; w2++) s += part[w2];
+        for (int w2 = 1; w2 < NW; w2++) s += __builtin_bit_cast(acc_t, part[w2]);
         const int tok = my_tok[pp], row0 = my_row0[pp];
         if (FAST || (packed && row0 + 3 < r1)) {
           if (tok < T && row0 < r1) {  // FAST: r1 is a multiple of 4, a quad is inside or outside
@@ -293,7 +316,7 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(DecodeParams prm
             const int row = row0 + v;
             if (row < r1 && tok < T) {
               const int i = prm.swapped ? tok : row, j = prm.swapped ? row : tok;
-              if (g.int_scale) ep.store_int(i, j, s[v]);
+              if (KIND == KIND_I8 && g.int_scale) ep.store_int(i, j, (int)s[v]);
               else ep.store_f(i, j, (float)s[v], f_al[pp][v] * f_sa[pp][v], f_sb[pp][v], f_be[pp][v], ep.bias_from_raw(f_bias[pp][v]));
             }
           }

@@ -209,7 +209,8 @@ static bool decode_variant_ok(const Lowered &l, int variant) {
   const GemmArgs &g = l.g;
   const DecodeVariant &v = kDecodeVariants[variant];
   const int T = std::min(g.M, g.N), nb = (T + 15) / 16;
-  if (!v.stream) return nb == 1 || (nb == 2 && v.steps <= 8);  // token blocks multiply the fragment registers
+  // the register-streaming kernel is int8 only; token blocks multiply its fragment registers
+  if (!v.stream) return g.a_type == CUDA_R_8I && (nb == 1 || (nb == 2 && v.steps <= 8));
   const bool swapped = g.M < g.N;
   const int64_t rows = swapped ? g.N : g.M, ldw = swapped ? g.b_sj : g.a_si;
   return g.K == v.nw * v.steps * 64 && rows * ldw < 0x7fffffffll && nb * v.steps <= kDecodeStreamMaxFragments;
@@ -255,7 +256,10 @@ bool family_supports(uint32_t kernel, const Lowered &l) {
            operand_ok(g.A, g.a_si, g.a_sk, g.a_sb, g.M) && operand_ok(g.B, g.b_sj, g.b_sk, g.b_sb, g.N);
   }
   case ZLUDA_KERNEL_DECODE_W8A8:
-    return fast_layout && g.a_type == CUDA_R_8I && g.b_type == CUDA_R_8I &&
+    // int8, or e4m3 x e4m3 without block scales (the LDS-streaming variants only)
+    return fast_layout && ((g.a_type == CUDA_R_8I && g.b_type == CUDA_R_8I) ||
+                           (g.a_type == CUDA_R_8F_E4M3 && g.b_type == CUDA_R_8F_E4M3 &&
+                            g.a_scale_mode != SCALE_BLOCK32_UE8M0 && g.b_scale_mode != SCALE_BLOCK32_UE8M0)) &&
            std::min(g.M, g.N) <= kDecodeMaxTokens && std::max(g.M, g.N) >= 64 && any_decode_variant_ok(l);
   default: return false;
   }
@@ -425,7 +429,7 @@ extern "C" uint32_t zluda_gemm_plan_problem(const zluda_gemm_problem *p, uint32_
       if (k == ZLUDA_KERNEL_DECODE_W8A8 && std::min(l.g.M, l.g.N) > kDecodeAutoMaxTokens) continue;
       if (!family_supports(k, l)) continue;
       if (k == ZLUDA_KERNEL_DECODE_W8A8 && !kDecodeVariants[pick_decode_variant(l)].stream &&
-          family_supports(ZLUDA_KERNEL_MFMA_I8, l)) {
+          family_supports(ZLUDA_KERNEL_MFMA_I8, l)) {  // (int8 only: fp8 has no such variant)
         // K outside the stream kernel's table: the register-streaming variant measures slower than
         // 64x64 MFMA tiles (split along K when the workspace allows) as soon as those give at
         // least half of the CUs a workgroup (5120x16x13824: 37 us against 23; 18944x32x3584: 46
