@@ -2,8 +2,8 @@
 """Benchmark of the cublasLtMatmul hot path on one MI355X.
 
 A "step" is one cublasLtMatmul call (through the exported C ABI of zluda_amd/lib/libcublaslt.so) on
-synthetic inputs that are already resident in HBM.  The headline line reports BASELINE config 2
-(int8 x int8 -> int32, M=N=K=4096, A:T B:N); the other BASELINE configurations and the 8192^3 int8
+synthetic inputs that are already resident in HBM.  The headline line reports benchmark configuration 2
+(int8 x int8 -> int32, M=N=K=4096, A:T B:N); the other benchmark configurations and the 8192^3 int8
 case ride along under "also", each with its own roofline figures and, when the installed hipBLASLt
 has a solution, the time of the reference's hipBLASLt-forwarded path on the same buffers.
 
@@ -32,25 +32,25 @@ PEAK = {"i8": 5000.0, "f8": 5000.0, "f4": 10100.0, "hbm": 8000.0}  # TOP/s, TFLO
 I8 = dict(a_type=K.CUDA_R_8I, b_type=K.CUDA_R_8I, d_type=K.CUDA_R_32I, compute_type=K.CUBLAS_COMPUTE_32I,
           scale_type=K.CUDA_R_32I, transa=1)
 WORKLOADS = {
-    "c1": dict(name="int8xint8->int32 M=N=K=256 A:N B:T (BASELINE config 1)", kind="i8",
+    "c1": dict(name="int8xint8->int32 M=N=K=256 A:N B:T (benchmark configuration 1)", kind="i8",
                spec=dict(I8, m=256, n=256, k=256, transa=0, transb=1), steps=200),
-    "c2": dict(name="int8xint8->int32 M=N=K=4096 A:T B:N (BASELINE config 2)", kind="i8",
+    "c2": dict(name="int8xint8->int32 M=N=K=4096 A:T B:N (benchmark configuration 2)", kind="i8",
                spec=dict(I8, m=4096, n=4096, k=4096), steps=50),
     "i8_4096_nt": dict(name="int8xint8->int32 M=N=K=4096 A:N B:T (config 1's layout at config 2's size)", kind="i8",
                        spec=dict(I8, m=4096, n=4096, k=4096, transa=0, transb=1), steps=50),
     "i8_8192": dict(name="int8xint8->int32 M=N=K=8192 A:T B:N", kind="i8", spec=dict(I8, m=8192, n=8192, k=8192), steps=10),
-    "c3": dict(name="W8A8 decode M=14336 N=16 K=4096 alpha-vec + per-token scale + fp32 bias -> bf16 (BASELINE config 3)",
+    "c3": dict(name="W8A8 decode M=14336 N=16 K=4096 alpha-vec + per-token scale + fp32 bias -> bf16 (benchmark configuration 3)",
                kind="hbm", steps=200,
                spec=dict(I8, d_type=K.CUDA_R_16BF, scale_type=K.CUDA_R_32F, m=14336, n=16, k=4096,
                          pointer_mode=K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO,
                          b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F,
                          epilogue=K.CUBLASLT_EPILOGUE_BIAS, bias_type=K.CUDA_R_32F)),
-    "c4": dict(name="fp8 e4m3 M=N=K=8192 per-tensor scales, bf16 bias + GELU -> bf16 (BASELINE config 4)", kind="f8",
+    "c4": dict(name="fp8 e4m3 M=N=K=8192 per-tensor scales, bf16 bias + GELU -> bf16 (benchmark configuration 4)", kind="f8",
                steps=10,
                spec=dict(a_type=K.CUDA_R_8F_E4M3, b_type=K.CUDA_R_8F_E4M3, d_type=K.CUDA_R_16BF,
                          compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F, transa=1, m=8192, n=8192, k=8192,
                          epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS, bias_type=K.CUDA_R_16BF)),
-    "c5": dict(name="MXFP4 (E2M1 + UE8M0/32) M=N=K=8192 batch 4 -> bf16 (BASELINE config 5)", kind="f4", steps=5,
+    "c5": dict(name="MXFP4 (E2M1 + UE8M0/32) M=N=K=8192 batch 4 -> bf16 (benchmark configuration 5)", kind="f4", steps=5,
                spec=dict(a_type=K.CUDA_R_4F_E2M1, b_type=K.CUDA_R_4F_E2M1, d_type=K.CUDA_R_16BF,
                          compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F, transa=1, m=8192, n=8192, k=8192,
                          batch=4, a_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_VEC32_UE8M0,

@@ -1,4 +1,4 @@
-"""BASELINE configurations 4 and 5 at their full 8192^3 size.  The CPU oracle cannot finish the whole
+"""benchmark configurations 4 and 5 at their full 8192^3 size.  The CPU oracle cannot finish the whole
 problem in seconds, so it recomputes three 64-row slabs of D (first, an interior tile boundary, last):
 for K-contiguous operands a slab of op(A) is a pointer offset, so the slab is itself a complete
 cublasLtMatmul problem with the same B, scales and epilogue."""

@@ -221,7 +221,7 @@ def test_misaligned_pointers_fall_back(gpu_api):
     case.compare(got, ref)
 
 
-# ---- BASELINE configurations ---------------------------------------------------------------------------
+# ---- benchmark configurations ---------------------------------------------------------------------------
 def test_config1_int8_256_nt(gpu_api):
     check(gpu_api, dict(I8, transa=0, transb=1, m=256, n=256, k=256, alpha=1), 0, expect_kernel=K.ZLUDA_KERNEL_MFMA_TR8)
     check(gpu_api, dict(I8, transa=0, transb=1, m=256, n=256, k=256, alpha=1), 0, K.ZLUDA_KERNEL_GENERIC)

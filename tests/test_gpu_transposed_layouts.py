@@ -1,5 +1,5 @@
 """GPU parity of the transposing 8-bit MFMA family (ZLUDA_KERNEL_MFMA_TR8): int8 and fp8 problems in
-which A, B or both are not K-contiguous -- BASELINE config 1's `A:N, B:T`, the N/N and T/T
+which A, B or both are not K-contiguous -- benchmark configuration 1's `A:N, B:T`, the N/N and T/T
 combinations and their row-major counterparts -- through the exported C ABI, against the CPU oracle
 on the same seeded inputs.  int8 -> int32 bit-exact over the whole D storage; float outputs within
 1e-2 (floor documented in oracle/cases.py)."""

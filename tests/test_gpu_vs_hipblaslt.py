@@ -32,7 +32,7 @@ def both(gpu_api, spec, seed, **kw):
 
 @pytest.mark.parametrize("n", [1024, 4096])
 def test_int8_bit_exact_with_hipblaslt(gpu_api, n):
-    """BASELINE config 2 (and a quarter-size version): every int32 of D identical"""
+    """benchmark configuration 2 (and a quarter-size version): every int32 of D identical"""
     case, ours, theirs, why, kern = both(gpu_api, dict(I8, m=n, n=n, k=n), 1)
     assert kern == K.ZLUDA_KERNEL_MFMA_I8
     if theirs is None:
@@ -42,7 +42,7 @@ def test_int8_bit_exact_with_hipblaslt(gpu_api, n):
 
 @pytest.mark.parametrize("n,ta,tb", [(256, 0, 1), (1024, 0, 0), (1024, 0, 1), (1024, 1, 1), (4096, 0, 1)])
 def test_int8_transposed_layouts_bit_exact_with_hipblaslt(gpu_api, n, ta, tb):
-    """BASELINE config 1 (256^3, A:N B:T) and the other layouts in which an operand is not K-contiguous:
+    """benchmark configuration 1 (256^3, A:N B:T) and the other layouts in which an operand is not K-contiguous:
     the transposing MFMA kernel against hipBLASLt called the way the reference forwards it"""
     spec = dict(I8, m=n, n=n, k=n, transa=ta, transb=tb)
     case, ours, theirs, why, kern = both(gpu_api, spec, 11)
@@ -64,7 +64,7 @@ def test_fp8_transposed_layout_within_tolerance_of_hipblaslt(gpu_api):
 
 
 def test_fp8_scaled_bias_gelu_within_tolerance_of_hipblaslt(gpu_api):
-    """BASELINE config 4 at 1024^3: per-tensor scales, bf16 bias, GELU, bf16 output"""
+    """benchmark configuration 4 at 1024^3: per-tensor scales, bf16 bias, GELU, bf16 output"""
     spec = dict(F8, m=1024, n=1024, k=1024, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS, bias_type=K.CUDA_R_16BF,
                 with_scalar_scales=True, scale_range=(0.05, 0.06), bias_std=0.5)
     case, ours, theirs, why, kern = both(gpu_api, spec, 3)
@@ -76,7 +76,7 @@ def test_fp8_scaled_bias_gelu_within_tolerance_of_hipblaslt(gpu_api):
 
 
 def test_decode_config3_decomposed_through_hipblaslt(gpu_api):
-    """BASELINE config 3 at full size.  hipBLASLt has no int8 -> bf16 algorithm with an alpha vector, so
+    """benchmark configuration 3 at full size.  hipBLASLt has no int8 -> bf16 algorithm with an alpha vector, so
     the reference's backend pins the integer part: its int8 -> int32 GEMM of the same operands, followed on
     the host by the documented epilogue D[i,j] = bf16(alpha[i] * sB[j] * acc[i,j] + bias[i]) in float64,
     against our fused decode kernel (float bar: 1e-2, bf16 rounding included)."""

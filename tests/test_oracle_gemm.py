@@ -97,7 +97,7 @@ def test_int8_layouts_against_numpy(ta, tb, oa, ob, od):
 
 
 def test_int8_config1_shape_identity_and_transpose():
-    # BASELINE config 1: 256^3, A:N B:T column-major, alpha=1 beta=0, seed 0
+    # benchmark configuration 1: 256^3, A:N B:T column-major, alpha=1 beta=0, seed 0
     spec = dict(I8, m=256, n=256, k=256, transa=0, transb=1, alpha=1)
     case = Case(spec, 0)
     d = case.run_oracle().reshape(256, 256).T  # col-major storage -> [i, j]
