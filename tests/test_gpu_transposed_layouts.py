@@ -101,6 +101,31 @@ def test_fp8_mixed_formats(gpu_api, at, bt):
                             order_c=od, order_d=od), 320, TR8, 2 if od else 0)
 
 
+def test_split_k_through_the_workspace(gpu_api):
+    """few tiles and a long K: with a workspace the K range of a tile is shared by several workgroups
+    (raw partial tiles + the reduce kernel with the full epilogue); K shares that are empty or partial"""
+    ws = 64 << 20
+    dec = dict(I8F, transa=0, transb=0, epilogue=K.CUBLASLT_EPILOGUE_BIAS, bias_type=K.CUDA_R_32F,
+               pointer_mode=K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO,
+               b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F, alpha_range=(0.001, 0.002), scale_range=(0.5, 1.5))
+    for spec, seed in ((dict(I8, m=1024, n=16, k=4096, transa=0, transb=0), 340),          # N-contiguous weights, decode shape
+                       (dict(I8, m=300, n=200, k=1104, transa=0, transb=1, with_c=True, batch=2, lda=304, ldb=200,
+                             alpha=2, beta=-1), 341),                                      # 17.25 stages over 8 shares
+                       (dict(dec, m=640, n=16, k=2048), 342),
+                       (dict(F8, m=512, n=64, k=4096, transa=0, transb=1, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS,
+                             with_scalar_scales=True, scale_range=(0.02, 0.03)), 343)):
+        print("TR8 split-K case", spec, flush=True)
+        case = Case(spec, seed)
+        ref = case.run_oracle()
+        st, got, kern, variant = case.run_gpu(gpu_api, workspace_bytes=ws)
+        assert st == 0 and kern == TR8
+        assert case.last_workspace_needed and case.last_workspace_needed <= ws, "the planner did not split K"
+        case.compare(got, ref)
+        st, got, kern, variant = case.run_gpu(gpu_api)       # and without a workspace: unsplit
+        assert st == 0 and kern == TR8 and case.last_workspace_needed == 0
+        case.compare(got, ref)
+
+
 def test_planner_prefers_the_k_contiguous_kernels_when_they_apply(gpu_api):
     check(gpu_api, dict(I8, m=512, n=256, k=512, transa=1, transb=0), 330, expect_kernel=K.ZLUDA_KERNEL_MFMA_I8)
     # K-contiguous but only 4-byte aligned pitches: the LDS DMA kernels need 16

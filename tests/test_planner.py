@@ -192,3 +192,17 @@ def test_fp8_decode_takes_the_streaming_kernel_for_table_k_only(api):
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_F8
     assert plan(api, dict(f8, m=4096, n=16, k=11008), forced=K.ZLUDA_KERNEL_DECODE_W8A8)[0] == K.CUBLAS_STATUS_NOT_SUPPORTED
     assert plan(api, dict(f8, m=4096, n=16, k=4096), forced=K.ZLUDA_KERNEL_DECODE_W8A8, variant=0)[0] == K.CUBLAS_STATUS_NOT_SUPPORTED
+
+
+def test_transposing_kernel_splits_k_when_tiles_are_few(api):
+    spec = dict(I8, transa=0, transb=0, m=4096, n=16, k=14336, ldb=14336)     # N-contiguous weights, decode shape
+    st, p = plan(api, spec)
+    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_TR8 and p.variant == 2 and p.grid_z == 1 and p.workspace == 0
+    st, p = plan(api, spec, workspace=64 << 20)
+    assert st == 0 and p.grid_x == 64 and p.grid_z == 8 and p.workspace == 8 * 4096 * 64 * 4
+    st, p = plan(api, spec, workspace=3 * 4096 * 64 * 4)
+    assert st == 0 and p.grid_z == 3
+    st, p = plan(api, dict(I8, transa=0, transb=1, m=4096, n=4096, k=4096), workspace=1 << 30)
+    assert st == 0 and p.grid_z == 1                                           # enough tiles already
+    st, p = plan(api, dict(I8, transa=0, transb=1, m=256, n=256, k=256), workspace=1 << 30)
+    assert st == 0 and p.grid_z == 1                                           # short K

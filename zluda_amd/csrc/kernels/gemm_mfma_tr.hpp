@@ -88,7 +88,7 @@ struct TrOperand {
       // the operand's extent, up to the end of its last dword (the range check is per dword; base
       // and ld_k are multiples of 4, so that dword lies in the same allocation granule): K rows past
       // the end read as zero
-      rs = __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, ((K - 1) * ld_k + nrows + 3) & ~3, 0x00020000);
+      rs = __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, K > 0 ? (((K - 1) * ld_k + nrows + 3) & ~3) : 0, 0x00020000);
       voff[0] = ((t >> 4) * 4) * ld_k + row0 + (t & 15) * IW;
       kstep = 64 * ld_k;
       ld = ld_k;
@@ -174,14 +174,25 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_tr_kernel(MfmaParams pr
   TrOperand<LQ, QKC> Q;
   const int tl = t & 255, grp = wave >> 2;
   const int lds_p = grp * LP * 5, lds_q = (BP + grp * LQ) * 5;  // this group's rows inside a stage
-  if (!prm.swapped) {
-    P.init(tl, (const uint8_t *)g.A + g.a_sb * bt, p0 + grp * LP, NP, (int)g.a_si, (int)g.a_sk, g.K);
-    Q.init(tl, (const uint8_t *)g.B + g.b_sb * bt, q0 + grp * LQ, NQ, (int)g.b_sj, (int)g.b_sk, g.K);
-  } else {
-    P.init(tl, (const uint8_t *)g.B + g.b_sb * bt, p0 + grp * LP, NP, (int)g.b_sj, (int)g.b_sk, g.K);
-    Q.init(tl, (const uint8_t *)g.A + g.a_sb * bt, q0 + grp * LQ, NQ, (int)g.a_si, (int)g.a_sk, g.K);
+  // split-K (as in gemm_mfma_pipe_kernel): workgroup z of gridDim.z takes stages [z * split_stages, ...)
+  // of K; the operands start k0 further along K and the rest of the kernel sees a shorter K
+  int k0 = 0, Kl = g.K;
+  if (prm.splits > 1) {
+    k0 = (int)blockIdx.z * prm.split_stages * 64;
+    Kl = max(0, min(g.K - k0, prm.split_stages * 64));
   }
-  const int KT = (g.K + 63) / 64;
+  {
+    const uint8_t *a = (const uint8_t *)g.A + g.a_sb * bt + (int64_t)k0 * g.a_sk;
+    const uint8_t *b = (const uint8_t *)g.B + g.b_sb * bt + (int64_t)k0 * g.b_sk;
+    if (!prm.swapped) {
+      P.init(tl, a, p0 + grp * LP, NP, (int)g.a_si, (int)g.a_sk, Kl);
+      Q.init(tl, b, q0 + grp * LQ, NQ, (int)g.b_sj, (int)g.b_sk, Kl);
+    } else {
+      P.init(tl, b, p0 + grp * LP, NP, (int)g.b_sj, (int)g.b_sk, Kl);
+      Q.init(tl, a, q0 + grp * LQ, NQ, (int)g.a_si, (int)g.a_sk, Kl);
+    }
+  }
+  const int KT = (Kl + 63) / 64;
 
   // LDS rows (in v4i units) of this lane's fragment rows
   int prow[TP], qrow[TQ];
@@ -316,6 +327,12 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_tr_kernel(MfmaParams pr
 
   // every wave is done with the LDS stages before they become epilogue staging
   __syncthreads();
+  if (prm.splits > 1) {
+    const int ws_np = prm.tiles_p * BP, ws_nq = prm.tiles_q * BQ;
+    int32_t *ws_tile = (int32_t *)prm.ws + ((int64_t)blockIdx.z * g.batch + bt) * ws_np * ws_nq + (int64_t)q0 * ws_np + p0;
+    mfma_store_tile_raw<WP, WQ, WTP, WTQ>(ws_tile, ws_np, acc);
+    return;
+  }
   mfma_store_tile<KIND, WP, WQ, WTP, WTQ>(prm, acc, (int *)&lds[0], sizeof(lds), p0, q0, NP, NQ, bt);
 }
 

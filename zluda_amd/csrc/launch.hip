@@ -73,7 +73,7 @@ uint32_t launch_mfma(const Lowered &l, const zluda_gemm_plan &plan, const zluda_
   return CUBLAS_STATUS_SUCCESS;
 }
 
-uint32_t launch_tr(const Lowered &l, const zluda_gemm_plan &plan, hipStream_t s) {
+uint32_t launch_tr(const Lowered &l, const zluda_gemm_plan &plan, const zluda_gemm_problem *p, hipStream_t s) {
   if (plan.variant >= (uint32_t)kNumTrVariants) return CUBLAS_STATUS_INVALID_VALUE;
   const TrVariant &v = kTrVariants[plan.variant];
   MfmaParams prm;
@@ -85,11 +85,36 @@ uint32_t launch_tr(const Lowered &l, const zluda_gemm_plan &plan, hipStream_t s)
   prm.group_p = 8;
   prm.splits = 1; prm.split_stages = 0; prm.ws = nullptr;
   if ((uint32_t)(prm.tiles_p * prm.tiles_q) != plan.grid_x) return CUBLAS_STATUS_INVALID_VALUE;
+  if (plan.grid_z > 1) {
+    // split-K: partial tiles go through the caller's workspace (64 K bytes per stage)
+    const uint64_t need = (uint64_t)plan.grid_z * l.g.batch * prm.tiles_p * v.bp * prm.tiles_q * v.bq * 4;
+    if (!p->workspace || (((uintptr_t)p->workspace) & 15) || p->workspace_size < need || plan.workspace != need)
+      return CUBLAS_STATUS_INVALID_VALUE;
+    const int stages = (l.g.K + 63) / 64;
+    prm.splits = (int32_t)plan.grid_z;
+    prm.split_stages = (stages + prm.splits - 1) / prm.splits;
+    prm.ws = p->workspace;
+  }
   // P is op(A) for a column-major D, op(B)^T otherwise
   const bool pkc = plan.swapped ? l.b_kcontig : l.a_kcontig, qkc = plan.swapped ? l.a_kcontig : l.b_kcontig;
-  if (l.g.a_type == CUDA_R_8I) return launch_tr_i8(prm, plan, pkc, qkc, s);
-  const int fa = f8_fmt(l.g.a_type), fb = f8_fmt(l.g.b_type);
-  return launch_tr_f8(prm, plan, plan.swapped ? fa : fb, plan.swapped ? fb : fa, pkc, qkc, s);
+  uint32_t st;
+  if (l.g.a_type == CUDA_R_8I) {
+    st = launch_tr_i8(prm, plan, pkc, qkc, s);
+  } else {
+    const int fa = f8_fmt(l.g.a_type), fb = f8_fmt(l.g.b_type);
+    st = launch_tr_f8(prm, plan, plan.swapped ? fa : fb, plan.swapped ? fb : fa, pkc, qkc, s);
+  }
+  if (st || prm.splits == 1) return st;
+  SplitKReduceParams rp;
+  rp.g = l.g;
+  rp.swapped = plan.swapped;
+  rp.splits = prm.splits;
+  rp.acc_is_int = l.g.a_type == CUDA_R_8I;
+  rp.ws_np = prm.tiles_p * v.bp;
+  rp.ws_nq = prm.tiles_q * v.bq;
+  rp.ws = (const int32_t *)p->workspace;
+  hipLaunchKernelGGL(splitk_reduce_kernel, dim3((np + 1023) / 1024, nq, l.g.batch), dim3(256), 0, s, rp);
+  return CUBLAS_STATUS_SUCCESS;
 }
 
 template <int NW, int STEPS>
@@ -177,7 +202,7 @@ extern "C" uint32_t zluda_gemm_launch(const zluda_gemm_problem *p, const zluda_g
     if ((st = launch_decode(l, *plan, s))) return st;
     break;
   case ZLUDA_KERNEL_MFMA_TR8:
-    if ((st = launch_tr(l, *plan, s))) return st;
+    if ((st = launch_tr(l, *plan, p, s))) return st;
     break;
   default: return CUBLAS_STATUS_NOT_SUPPORTED;
   }

@@ -11,7 +11,7 @@ namespace zluda_amd {
 // plan.variant indexes kTrVariants (planner.hpp); pkc / qkc: operand P / Q has unit stride along K
 template <int KIND, int FQ, int FP>
 inline uint32_t launch_tr_variant(const MfmaParams &prm, const zluda_gemm_plan &plan, bool pkc, bool qkc, hipStream_t s) {
-  const dim3 grid(plan.grid_x, plan.grid_y, 1);
+  const dim3 grid(plan.grid_x, plan.grid_y, plan.grid_z > 1 ? plan.grid_z : 1);  // z: split-K shares
 #define ZLUDA_TR_MODE(BP, BQ, WP, WQ, PK, QK)                                                                   \
   if (pkc == PK && qkc == QK) {                                                                                 \
     hipLaunchKernelGGL((gemm_mfma_tr_kernel<KIND, FQ, FP, BP, BQ, WP, WQ, PK, QK>), grid, dim3(WP * WQ * 64), 0, s, prm); \

@@ -325,7 +325,7 @@ static int pick_mfma_variant(const Lowered &l, uint32_t cus) {
   return best;
 }
 
-static void fill_tr_plan(const Lowered &l, int variant, uint32_t cus, zluda_gemm_plan *plan) {
+static void fill_tr_plan(const Lowered &l, int variant, uint32_t cus, uint64_t workspace_size, zluda_gemm_plan *plan) {
   const GemmArgs &g = l.g;
   const TrVariant &v = kTrVariants[variant];
   const bool swapped = g.d_si != 1;
@@ -337,6 +337,24 @@ static void fill_tr_plan(const Lowered &l, int variant, uint32_t cus, zluda_gemm
   const uint32_t per_cu = 160u * 1024u / (2u * (v.bp + v.bq) * 80u);  // LDS: two stages of 80-byte rows
   plan->waves = (float)plan->grid_x * plan->grid_y / (float)(cus * std::min(per_cu, 4u));
   plan->workspace = 0;
+  // Split-K as for the K-contiguous kernels: grid_z workgroups share a tile's K range through the
+  // caller's workspace when K has at least 16 stages and the tiles leave half of the chip idle --
+  // half of the CUs, or, for skinny problems (<= 64 rows or columns: memory bound, a workgroup keeps
+  // only ~16 KiB in flight), half of the workgroup slots.  N-contiguous weights, 16 tokens, us:
+  // 4096x14336 89 -> 25, 4096x4096 31 -> 14, 14336x4096 31 -> 24; 14336x128x4096 would lose (37 -> 42).
+  const uint64_t tiles = (uint64_t)plan->grid_x * plan->grid_y;
+  const uint64_t slots = (uint64_t)cus * std::min(per_cu, 4u);
+  const bool skinny = std::min(g.M, g.N) <= 64;
+  if (tiles * 2 <= (skinny ? slots : (uint64_t)cus) && g.K >= 1024 && (uint64_t)ceil_div(np, v.bp) * v.bp <= (1u << 20)) {
+    uint32_t s = (uint32_t)std::min<uint64_t>({8, slots / tiles, (uint64_t)g.K / 512});
+    const uint64_t per_split = (uint64_t)g.batch * ceil_div(np, v.bp) * v.bp * ceil_div(nq, v.bq) * v.bq * 4;
+    while (s > 1 && s * per_split > workspace_size) s--;
+    if (s > 1) {
+      plan->grid_z = s;
+      plan->workspace = s * per_split;
+      plan->waves = (float)tiles * s / (float)slots;
+    }
+  }
 }
 
 // Tile choice of the transposing kernel.  A CU runs up to `per_cu` workgroups of a variant side by
@@ -463,7 +481,7 @@ extern "C" uint32_t zluda_gemm_plan_problem(const zluda_gemm_problem *p, uint32_
   case ZLUDA_KERNEL_MFMA_TR8: {
     int v = forced_variant >= 0 ? forced_variant : pick_tr_variant(l, cu_count);
     if (v >= kNumTrVariants) return CUBLAS_STATUS_INVALID_VALUE;
-    fill_tr_plan(l, v, cu_count, plan);
+    fill_tr_plan(l, v, cu_count, p->workspace_size, plan);
     break;
   }
   case ZLUDA_KERNEL_DECODE_W8A8: {
