@@ -291,8 +291,13 @@ static void fill_mfma_plan(const Lowered &l, int variant, uint32_t cus, uint64_t
   const uint32_t kt = ceil_div((uint32_t)((int64_t)g.K * (g.a_type == CUDA_R_4F_E2M1 ? 4 : 8) / 8), v.bkb);
   // (below ~6 KiB of K per row the second kernel and the workspace traffic cost more than the idle CUs)
   const uint32_t kbytes = kt * v.bkb;
-  if (g.a_type != CUDA_R_4F_E2M1 && tiles * 2 <= cus && kbytes >= 6144 && (uint64_t)tp * v.bp <= (1u << 20)) {
-    uint32_t s = (uint32_t)std::min<uint64_t>({8, cus / tiles, kbytes / 2048});
+  // Skinny problems (<= 64 rows or columns) are memory bound: they split from 2 KiB of K per row on
+  // and down to 1 KiB per share, up to two workgroups per CU (fp8 4096x48x4096: 18 -> 13 us; but
+  // 14336x64x4096, 224 tiles, must stay whole: 16.5 us against 23.7 split in three).
+  const bool skinny = std::min(g.M, g.N) <= 64;
+  if (g.a_type != CUDA_R_4F_E2M1 && tiles * 2 <= cus && kbytes >= (skinny ? 2048u : 6144u) &&
+      (uint64_t)tp * v.bp <= (1u << 20)) {
+    uint32_t s = (uint32_t)std::min<uint64_t>({8, (skinny ? 2 * cus : cus) / tiles, kbytes / (skinny ? 1024 : 2048)});
     const uint64_t per_split = (uint64_t)g.batch * tp * v.bp * tq * v.bq * 4;
     while (s > 1 && s * per_split > workspace_size) s--;
     if (s > 1) {
@@ -444,8 +449,12 @@ extern "C" uint32_t zluda_gemm_plan_problem(const zluda_gemm_problem *p, uint32_
     static const uint32_t order[] = {ZLUDA_KERNEL_DECODE_W8A8, ZLUDA_KERNEL_MFMA_I8, ZLUDA_KERNEL_MFMA_F8,
                                      ZLUDA_KERNEL_MFMA_MXF4, ZLUDA_KERNEL_MFMA_TR8, ZLUDA_KERNEL_GENERIC};
     for (uint32_t k : order) {
-      if (k == ZLUDA_KERNEL_DECODE_W8A8 && std::min(l.g.M, l.g.N) > kDecodeAutoMaxTokens) continue;
       if (!family_supports(k, l)) continue;
+      if (k == ZLUDA_KERNEL_DECODE_W8A8) {
+        const int tokens = std::min(l.g.M, l.g.N);
+        const bool stream = kDecodeVariants[pick_decode_variant(l)].stream;
+        if (tokens > (stream ? kDecodeAutoMaxTokensStream : kDecodeAutoMaxTokens)) continue;
+      }
       if (k == ZLUDA_KERNEL_DECODE_W8A8 && !kDecodeVariants[pick_decode_variant(l)].stream &&
           family_supports(ZLUDA_KERNEL_MFMA_I8, l)) {  // (int8 only: fp8 has no such variant)
         // K outside the stream kernel's table: the register-streaming variant measures slower than

@@ -57,7 +57,10 @@ constexpr int kNumDecodeVariants = sizeof(kDecodeVariants) / sizeof(kDecodeVaria
 // registers for the whole kernel.
 constexpr int kDecodeStreamMaxFragments = 32;  // stream kernel: up to 64 tokens at K = 4096
 constexpr int kDecodeMaxTokens = 64;      // what the family can run
-constexpr int kDecodeAutoMaxTokens = 32;  // what the planner gives it: beyond, 64x64 MFMA tiles measure faster
+constexpr int kDecodeAutoMaxTokens = 32;  // what the planner gives it whatever the variant ...
+constexpr int kDecodeAutoMaxTokensStream = 56;  // ... and when the LDS-streaming variant applies: a partial 64-wide MFMA
+                                                // tile pays the general epilogue (14336x48x4096 fp8: 19 us against 23); from
+                                                // 57 tokens on the two measure alike, at 64 the full MFMA tile wins
 
 struct Lowered {
   GemmArgs g;
