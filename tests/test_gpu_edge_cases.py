@@ -62,11 +62,11 @@ def test_decode_shapes_around_the_limits(gpu_api):
     assert run(gpu_api, dict(dec, m=4099, n=32, k=4096), 341, int_dist="normal") == K.ZLUDA_KERNEL_DECODE_W8A8   # rows % 4 != 0
     assert run(gpu_api, dict(dec, m=2048, n=3, k=11008), 342, int_dist="normal") == K.ZLUDA_KERNEL_DECODE_W8A8  # K outside the stream table
     assert run(gpu_api, dict(dec, m=512, n=16, k=4096, batch=3), 343, int_dist="normal") == K.ZLUDA_KERNEL_DECODE_W8A8
-    # beyond 56 tokens the planner prefers small MFMA tiles (the decode family itself runs up to 64)
+    # beyond 48 tokens the planner prefers small MFMA tiles (the decode family itself runs up to 64)
     assert run(gpu_api, dict(dec, m=2048, n=32, k=4096), 344, int_dist="normal") == K.ZLUDA_KERNEL_DECODE_W8A8
     assert run(gpu_api, dict(dec, m=2048, n=33, k=4096), 346, int_dist="normal") == K.ZLUDA_KERNEL_DECODE_W8A8
-    assert run(gpu_api, dict(dec, m=2048, n=56, k=4096), 348, int_dist="normal") == K.ZLUDA_KERNEL_DECODE_W8A8
-    assert run(gpu_api, dict(dec, m=2048, n=57, k=4096), 349, int_dist="normal") == K.ZLUDA_KERNEL_MFMA_I8
+    assert run(gpu_api, dict(dec, m=2048, n=48, k=4096), 348, int_dist="normal") == K.ZLUDA_KERNEL_DECODE_W8A8
+    assert run(gpu_api, dict(dec, m=2048, n=49, k=4096), 349, int_dist="normal") == K.ZLUDA_KERNEL_MFMA_I8
     assert run(gpu_api, dict(dec, m=2048, n=64, k=4096), 347, int_dist="normal") == K.ZLUDA_KERNEL_MFMA_I8
     # f16 output, ld > rows (the packed store needs ld % 4 == 0: 2052 qualifies, 2051 does not)
     for ld in (2052, 2051):

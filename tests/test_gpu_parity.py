@@ -80,6 +80,26 @@ def test_mfma_full_tile_epilogues(gpu_api, variant):
     check(gpu_api, dict(MX, m=512, n=256, k=1024), 116, K.ZLUDA_KERNEL_MFMA_MXF4, variant)
 
 
+@pytest.mark.parametrize("variant", range(8))
+def test_mfma_ragged_token_count_keeps_the_fast_epilogues(gpu_api, variant):
+    """M a multiple of every tile height, N ragged (tokens): the stores of the columns past the end fall
+    outside the buffer window; padding, the next batch and the canary behind D must stay untouched"""
+    rag = dict(m=768, n=203, k=256)
+    check(gpu_api, dict(I8, **rag, alpha=1, batch=2, ldd=784), 410, K.ZLUDA_KERNEL_MFMA_I8, variant)
+    vec = dict(I8F, **rag, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS, bias_type=K.CUDA_R_32F,
+               pointer_mode=K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO,
+               a_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F,
+               b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F,
+               alpha_range=(0.001, 0.002), scale_range=(0.5, 1.5))
+    for dt in (K.CUDA_R_16BF, K.CUDA_R_32F):
+        check(gpu_api, dict(vec, d_type=dt, c_type=dt, batch=2), 411, K.ZLUDA_KERNEL_MFMA_I8, variant)
+    check(gpu_api, dict(F8, **rag, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS, with_scalar_scales=True, batch=2), 412,
+          K.ZLUDA_KERNEL_MFMA_F8, variant)
+    # row-major D: the ragged dimension is M
+    check(gpu_api, dict(F8, m=203, n=768, k=256, order_c=1, order_d=1, d_type=K.CUDA_R_16F, c_type=K.CUDA_R_16F), 413,
+          K.ZLUDA_KERNEL_MFMA_F8, variant)
+
+
 @pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7])
 def test_mfma_i8_float_epilogue(gpu_api, variant):
     spec = dict(I8F, m=260, n=140, k=512, epilogue=K.CUBLASLT_EPILOGUE_RELU_BIAS, bias_type=K.CUDA_R_32F,

@@ -184,9 +184,9 @@ def test_fp8_decode_takes_the_streaming_kernel_for_table_k_only(api):
     f8 = dict(F8, transa=1)
     st, p = plan(api, dict(f8, m=14336, n=16, k=4096))
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.variant == 4 and p.grid_x == 256
-    st, p = plan(api, dict(f8, m=14336, n=48, k=4096))                      # up to 56 tokens while the variant applies
+    st, p = plan(api, dict(f8, m=14336, n=48, k=4096))                      # up to 48 tokens while the variant applies
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8
-    st, p = plan(api, dict(f8, m=14336, n=57, k=4096))                      # beyond: MFMA tiles
+    st, p = plan(api, dict(f8, m=14336, n=49, k=4096))                      # beyond: MFMA tiles
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_F8
     st, p = plan(api, dict(f8, m=14336, n=33, k=8192))                      # 3 token blocks x 16 steps: too many fragments
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_F8

@@ -197,13 +197,22 @@ __device__ __forceinline__ void mfma_store_tile_general(const MfmaParams &prm, A
   static_for<TQ * 2>(do_pass);
 }
 
+// Size of the buffer window of a wave tile whose corner is `base_elems` elements into this batch's D:
+// what is left of the matrix (NQ columns of pitch d_sq, the last one NP long).  Stores of a tile that
+// hangs over the last column fall outside the window and are dropped by the hardware, which is what
+// lets the fast paths below take tiles that are complete along P only.
+__device__ __forceinline__ uint32_t tile_window_bytes(int64_t d_sq, int NP, int NQ, int64_t base_elems, int esz) {
+  const int64_t left = ((int64_t)(NQ - 1) * d_sq + NP - base_elems) * esz;
+  return left <= 0 ? 0u : (left > 0xFFFFFFFFll ? 0xFFFFFFFFu : (uint32_t)left);
+}
+
 // Fast path 1: pure integer epilogue with alpha, beta scalars and beta == 0 on a full tile with
 // 16-byte aligned columns: D = alpha * acc straight from the accumulator registers.  Lanes 0..31 of
 // a store hold 32 consecutive int32 of one D column (one 128-byte line), so no LDS staging is
 // needed; two instructions per output element.
 template <int WP, int WQ, int WTP, int WTQ>
 __device__ __forceinline__ void mfma_store_tile_i32(const MfmaParams &prm, v16i (&acc)[WTQ / 32][WTP / 32],
-                                                    int p0, int q0, int bt, int ialpha) {
+                                                    int p0, int q0, int NP, int NQ, int bt, int ialpha) {
   constexpr int TP = WTP / 32, TQ = WTQ / 32;
   const GemmArgs &g = prm.g;
   // the wave index is uniform by construction; say so, or the buffer descriptor built from it is
@@ -214,8 +223,9 @@ __device__ __forceinline__ void mfma_store_tile_i32(const MfmaParams &prm, v16i 
   const int d_sq = (int)(prm.swapped ? g.d_si : g.d_sj);  // < 2^22 (checked by the dispatcher)
   // Buffer stores: wave-uniform descriptor at the wave tile, per-lane byte offset of (row 4*gsel,
   // column lr) in a VGPR, everything else in the scalar offset.
-  int32_t *Dw = (int32_t *)g.D + g.d_sb * bt + (int64_t)(q0 + wq * WTQ) * d_sq + (p0 + wp * WTP);
-  const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)Dw, 0, 0xFFFFFFFF, 0x00020000);
+  const int64_t corner = (int64_t)(q0 + wq * WTQ) * d_sq + (p0 + wp * WTP);
+  int32_t *Dw = (int32_t *)g.D + g.d_sb * bt + corner;
+  const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)Dw, 0, tile_window_bytes(d_sq, NP, NQ, corner, 4), 0x00020000);
   const int voff = (4 * gsel * d_sq + lr) * 4;
   // alpha == 1 (the usual case) stores the accumulator registers as they are
   if (ialpha == 1) {
@@ -268,7 +278,7 @@ __device__ __forceinline__ void mfma_store_tile_raw(int32_t *ws_tile, int ws_pit
 // one ds_read_b128, the arithmetic and one store.
 template <int KIND, int WP, int WQ, int WTP, int WTQ, int ACT, int DT, class AccV>
 __device__ __forceinline__ void mfma_store_tile_f(const MfmaParams &prm, AccV (&acc)[WTQ / 32][WTP / 32],
-                                                  int *lds_words, int p0, int q0, int bt) {
+                                                  int *lds_words, int p0, int q0, int NP, int NQ, int bt) {
   constexpr int TP = WTP / 32, TQ = WTQ / 32;
   constexpr int SROW = WTP + 8, LPR = WTP / 4, RPI = 64 / LPR, ITER = 16 / RPI;
   static_assert(16 % RPI == 0, "whole passes");
@@ -293,8 +303,9 @@ __device__ __forceinline__ void mfma_store_tile_f(const MfmaParams &prm, AccV (&
   const float q_scale_u = swp ? ep.row_scale(0) : ep.col_scale(0);  // used when !q_vec
   const int d_sq = (int)(swp ? g.d_si : g.d_sj);  // < 2^22 (checked by the dispatcher)
   // buffer stores: uniform descriptor at the wave tile, per-lane byte offset (row qsub, column pl)
-  char *Dw = (char *)g.D + (g.d_sb * bt + (int64_t)(q0 + wq * WTQ) * d_sq + (p0 + wp * WTP)) * ESZ;
-  const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)Dw, 0, 0xFFFFFFFF, 0x00020000);
+  const int64_t corner = (int64_t)(q0 + wq * WTQ) * d_sq + (p0 + wp * WTP);
+  char *Dw = (char *)g.D + (g.d_sb * bt + corner) * ESZ;
+  const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)Dw, 0, tile_window_bytes(d_sq, NP, NQ, corner, ESZ), 0x00020000);
   const int voff = (qsub * d_sq + pl) * ESZ;
   const int read_off = qsub * SROW + pl;
 
@@ -316,7 +327,7 @@ __device__ __forceinline__ void mfma_store_tile_f(const MfmaParams &prm, AccV (&
       const v4i raw = *(const v4i *)&stage[it * RPI * SROW + read_off];
       float qs = q_scale_u, qb = 0.0f;
       if (q_vec) {
-        const int qi = q0 + wq * WTQ + a * 32 + h * 16 + it * RPI + qsub;
+        const int qi = min(q0 + wq * WTQ + a * 32 + h * 16 + it * RPI + qsub, NQ - 1);  // columns past the end: dropped stores
         qs = swp ? ep.row_scale(qi) : ep.col_scale(qi);
         qb = swp ? ep.bias_at(qi) : 0.0f;
       }
@@ -359,7 +370,7 @@ __device__ __forceinline__ void mfma_store_tile_f(const MfmaParams &prm, AccV (&
 // segments.
 template <int KIND, int WP, int WQ, int WTP, int WTQ, int ACT, int DT, class AccV>
 __device__ __forceinline__ void mfma_store_tile_f16_direct(const MfmaParams &prm, AccV (&acc)[WTQ / 32][WTP / 32],
-                                                           int p0, int q0, int bt) {
+                                                           int p0, int q0, int NP, int NQ, int bt) {
   static_assert(DT == 0 || DT == 1, "16-bit outputs");
   constexpr int TP = WTP / 32, TQ = WTQ / 32;
   const GemmArgs &g = prm.g;
@@ -377,8 +388,9 @@ __device__ __forceinline__ void mfma_store_tile_f16_direct(const MfmaParams &prm
     p_bias[b] = swp ? 0.0f : ep.bias_at(pi);
   }
   const int d_sq = (int)(swp ? g.d_si : g.d_sj);  // < 2^22 (checked by the dispatcher)
-  char *Dw = (char *)g.D + (g.d_sb * bt + (int64_t)(q0 + wq * WTQ) * d_sq + (p0 + wp * WTP)) * 2;
-  const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)Dw, 0, 0xFFFFFFFF, 0x00020000);
+  const int64_t corner = (int64_t)(q0 + wq * WTQ) * d_sq + (p0 + wp * WTP);
+  char *Dw = (char *)g.D + (g.d_sb * bt + corner) * 2;
+  const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)Dw, 0, tile_window_bytes(d_sq, NP, NQ, corner, 2), 0x00020000);
   const int voff = ((4 * gsel + odd) * d_sq + (lr & ~1)) * 2;
   auto value = [&](float accf, int b) {
     float y = (swp ? q_scale * p_scale[b] : p_scale[b] * q_scale) * accf + p_bias[b];
@@ -406,8 +418,9 @@ __device__ __forceinline__ void mfma_store_tile_f16_direct(const MfmaParams &prm
     }
 }
 
-// Epilogue dispatch: the fast paths for full tiles of the common configurations, the general path
-// for the rest.  All conditions are workgroup-uniform.
+// Epilogue dispatch: the fast paths for the common configurations on tiles that are complete along
+// P (columns past the end of D are dropped by the store window, so a ragged token count keeps the
+// fast path), the general path for the rest.  All conditions are workgroup-uniform.
 template <int KIND, int WP, int WQ, int WTP, int WTQ, class AccV>
 __device__ __forceinline__ void mfma_store_tile(const MfmaParams &prm, AccV (&acc)[WTQ / 32][WTP / 32],
                                                 int *lds_words, size_t lds_bytes, int p0, int q0, int NP,
@@ -415,7 +428,7 @@ __device__ __forceinline__ void mfma_store_tile(const MfmaParams &prm, AccV (&ac
   const GemmArgs &g = prm.g;
   const bool swp = prm.swapped != 0;
   const int64_t d_sq = swp ? g.d_si : g.d_sj;
-  const bool full = p0 + WP * WTP <= NP && q0 + WQ * WTQ <= NQ;
+  const bool full = p0 + WP * WTP <= NP;  // along Q the store window cuts the tile
   const int dbytes = (g.d_type == CUDA_R_32F || g.d_type == CUDA_R_32I) ? 4 : (g.d_type == CUDA_R_8I ? 1 : 2);
   // columns of the tile start 16-byte aligned and the lane offsets fit 32 bits
   const bool aligned = (((uintptr_t)g.D) & 15) == 0 && ((d_sq * dbytes) & 15) == 0 &&
@@ -424,7 +437,7 @@ __device__ __forceinline__ void mfma_store_tile(const MfmaParams &prm, AccV (&ac
     if (g.int_scale && full && aligned && g.alpha_mode != VECTOR_DEV && g.beta_mode == SCALAR_VALUE &&
         g.beta_val.i == 0) {
       const int ialpha = g.alpha_mode == SCALAR_VALUE ? g.alpha_val.i : *(const int32_t *)g.alpha_ptr;
-      mfma_store_tile_i32<WP, WQ, WTP, WTQ>(prm, acc, p0, q0, bt, ialpha);
+      mfma_store_tile_i32<WP, WQ, WTP, WTQ>(prm, acc, p0, q0, NP, NQ, bt, ialpha);
       return;
     }
   }
@@ -435,7 +448,7 @@ __device__ __forceinline__ void mfma_store_tile(const MfmaParams &prm, AccV (&ac
     const bool q_vec = swp ? (g.alpha_mode == VECTOR_DEV || g.a_scale_mode == SCALE_OUTER_VEC || g.bias != nullptr)
                            : (g.b_scale_mode == SCALE_OUTER_VEC);
     if (!q_vec && dt != 2) {
-#define ZLUDA_EPI_D(ACT_, DT_) mfma_store_tile_f16_direct<KIND, WP, WQ, WTP, WTQ, ACT_, DT_>(prm, acc, p0, q0, bt)
+#define ZLUDA_EPI_D(ACT_, DT_) mfma_store_tile_f16_direct<KIND, WP, WQ, WTP, WTQ, ACT_, DT_>(prm, acc, p0, q0, NP, NQ, bt)
       if (dt == 0) {
         if (g.act == ACT_GELU) ZLUDA_EPI_D(ACT_GELU, 0);
         else if (g.act == ACT_RELU) ZLUDA_EPI_D(ACT_RELU, 0);
@@ -448,7 +461,7 @@ __device__ __forceinline__ void mfma_store_tile(const MfmaParams &prm, AccV (&ac
 #undef ZLUDA_EPI_D
       return;
     }
-#define ZLUDA_EPI(ACT_, DT_) mfma_store_tile_f<KIND, WP, WQ, WTP, WTQ, ACT_, DT_>(prm, acc, lds_words, p0, q0, bt)
+#define ZLUDA_EPI(ACT_, DT_) mfma_store_tile_f<KIND, WP, WQ, WTP, WTQ, ACT_, DT_>(prm, acc, lds_words, p0, q0, NP, NQ, bt)
     if (dt == 0) {
       if (g.act == ACT_GELU) ZLUDA_EPI(ACT_GELU, 0);
       else if (g.act == ACT_RELU) ZLUDA_EPI(ACT_RELU, 0);

@@ -58,9 +58,9 @@ constexpr int kNumDecodeVariants = sizeof(kDecodeVariants) / sizeof(kDecodeVaria
 constexpr int kDecodeStreamMaxFragments = 32;  // stream kernel: up to 64 tokens at K = 4096
 constexpr int kDecodeMaxTokens = 64;      // what the family can run
 constexpr int kDecodeAutoMaxTokens = 32;  // what the planner gives it whatever the variant ...
-constexpr int kDecodeAutoMaxTokensStream = 56;  // ... and when the LDS-streaming variant applies: a partial 64-wide MFMA
-                                                // tile pays the general epilogue (14336x48x4096 fp8: 19 us against 23); from
-                                                // 57 tokens on the two measure alike, at 64 the full MFMA tile wins
+constexpr int kDecodeAutoMaxTokensStream = 48;  // ... and when the LDS-streaming variant applies: 3 token blocks still beat
+                                                // 64-wide MFMA tiles (6144x48x4096 fp8: 13 us against 16), 4 blocks do not
+                                                // (14336x56x4096: 21 us against 19)
 
 struct Lowered {
   GemmArgs g;
