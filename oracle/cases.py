@@ -351,5 +351,12 @@ class Case:
         if s["d_type"] == abi.CUDA_R_8I:
             assert np.max(np.abs(g - r)) <= 1, "int8 outputs differ by more than one step"
             return err
-        assert err <= tol, "max relative error %.3e > %.1e" % (err, tol)
+        if err > tol:
+            rel = np.abs(g - r) / np.maximum(np.abs(r), floor)
+            bad = np.nonzero(rel > tol)[0]
+            m = s["m"]
+            rows, cols = (idx[bad] % (self.dtot // self.batch)) % max(_layout(s, "d", m, s["n"])[1], 1), None
+            raise AssertionError("max relative error %.3e > %.1e: %d of %d outputs off, logical positions %d..%d, "
+                                 "storage offsets mod ld: min %d max %d (%d distinct)" %
+                                 (err, tol, bad.size, rel.size, bad[0], bad[-1], rows.min(), rows.max(), np.unique(rows).size))
         return err

@@ -208,6 +208,16 @@ def test_split_k_through_the_workspace(gpu_api):
         assert st == 0 and kern in (K.ZLUDA_KERNEL_MFMA_I8, K.ZLUDA_KERNEL_MFMA_F8)
         assert case.last_workspace_needed and case.last_workspace_needed <= ws, "the planner did not split K"
         case.compare(got, ref)
+    # MXFP4: the K shares are whole scale chunks (1024 elements); 8960 = 35 stages in 4 shares -> 12 + 12 + 11 + 0
+    for spec, seed in ((dict(MX, m=512, n=64, k=8192), 376), (dict(MX, m=320, n=48, k=8960, batch=2), 377),
+                       (dict(MX, m=1024, n=256, k=16384), 378)):
+        print("split-K case", spec, flush=True)
+        case = Case(spec, seed)
+        ref = case.run_oracle()
+        st, got, kern, variant = case.run_gpu(gpu_api, workspace_bytes=ws)
+        assert st == 0 and kern == K.ZLUDA_KERNEL_MFMA_MXF4
+        assert case.last_workspace_needed and case.last_workspace_needed <= ws, "the planner did not split K"
+        case.compare(got, ref)
     # the same token with too little workspace at call time: the call must not use it
     case = Case(dict(I8, m=1024, n=256, k=8192), 375)
     ref = case.run_oracle()

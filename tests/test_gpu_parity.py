@@ -136,6 +136,23 @@ def test_mfma_mxf4_variants(gpu_api, variant):
     check(gpu_api, dict(MX, m=288, n=160, k=768, batch=2), 60 + variant, K.ZLUDA_KERNEL_MFMA_MXF4, variant)
 
 
+@pytest.mark.parametrize("variant", [4, 5, 6])
+def test_last_real_stage_is_waited_for(gpu_api, variant):
+    """tile variants with three or four LDS stages wait for a stage by counting the younger operations in
+    flight; behind the last stage of K those are padding.  A padding instruction that is out of range as a
+    whole completes without a memory round trip and retires ahead of older loads, so the last stage was
+    read before it had landed, once in a while: padding is a real load now.  K just above the number of
+    LDS stages, repeated, with other work in between."""
+    import torch
+    other = torch.randn(1 << 22, device="cuda:0")
+    bkb = 64 if variant == 4 else 128
+    for rep in range(6):
+        other.mul_(1.0001)
+        check(gpu_api, dict(MX, m=512, n=256, k=1024), 116, K.ZLUDA_KERNEL_MFMA_MXF4, variant)
+        check(gpu_api, dict(I8, m=512, n=256, k=5 * bkb, alpha=1), 117 + rep, K.ZLUDA_KERNEL_MFMA_I8, variant)
+        check(gpu_api, dict(F8, m=512, n=256, k=5 * bkb), 118 + rep, K.ZLUDA_KERNEL_MFMA_F8, variant)
+
+
 def test_mxf4_generic_agrees(gpu_api):
     check(gpu_api, dict(MX, m=96, n=80, k=384), 70, K.ZLUDA_KERNEL_GENERIC)
 

@@ -154,7 +154,7 @@ def test_split_k_needs_workspace_and_few_tiles(api):
     # a workspace that holds only 3 partial matrices limits the split
     st, p3 = plan_ws(spec, 3 * 1024 * 256 * 4)
     assert st == 0 and p3.grid_z == 3 and p3.workspace == 3 * 1024 * 256 * 4
-    # enough tiles already, short K, or MXFP4: no split
+    # enough tiles already or short K: no split (MXFP4 counts its K in bytes: 8192 elements are 4 KiB)
     assert plan_ws(dict(I8, m=4096, n=4096, k=8192, transa=1), 1 << 30)[1].grid_z == 1
     assert plan_ws(dict(I8, m=1024, n=256, k=256, transa=1), 1 << 30)[1].grid_z == 1
     assert plan_ws(dict(MX, m=1024, n=256, k=8192, transa=1), 1 << 30)[1].grid_z == 1

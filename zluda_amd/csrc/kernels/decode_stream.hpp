@@ -110,8 +110,10 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(DecodeParams prm
   const int nblk = (r1 - r0 + 15) >> 4;
   const int kwave = wave * (SPW * 64);
 
-  // 2 GiB raw buffer window over W: an offset with bit 31 set is out of range, reads as zero and
-  // moves no data (rows past r1 of the last block, and the units issued past the last block)
+  // 2 GiB raw buffer window over W.  Rows past r1 of the last block, and the units issued past the
+  // last block, are never used; they read the last row of W instead of going out of range: an
+  // instruction whose lanes are all out of range completes without a memory round trip and can
+  // retire ahead of older loads, which the counted waits below must not see.
   const __amdgpu_buffer_rsrc_t rsW = __builtin_amdgcn_make_buffer_rsrc((void *)Wg, 0, 0x80000000, 0x00020000);
   // DMA instruction i of a unit: lane -> row rho = 4*i + lane/16 at position lane%16, i.e. logical
   // chunk (lane%16) ^ rho
@@ -119,16 +121,15 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(DecodeParams prm
 #pragma unroll
   for (int i = 0; i < NDMA; i++) {
     const int rho = 4 * i + g4;
-    dma_off[i] = rho * ldw + ((l16 ^ rho) << 4) + kwave;
+    dma_off[i] = ((l16 ^ rho) << 4) + kwave;
   }
   auto issue_unit = [&](int blk, int q, int slot) {
     const int rb = r0 + blk * 16;
     v4i *dst = &ring[wave][slot][0];
 #pragma unroll
     for (int i = 0; i < NDMA; i++) {
-      const int rho = 4 * i + g4;
-      const int oob = rb + rho < r1 ? 0 : (int)0x80000000;
-      lds_dma16(rsW, dst + i * 64, (rb * ldw + q * SEG + dma_off[i]) | oob, 0);
+      const int row = min(rb + 4 * i + g4, R - 1);
+      lds_dma16(rsW, dst + i * 64, row * ldw + q * SEG + dma_off[i], 0);
     }
   };
 

@@ -102,16 +102,18 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
     Pg = (const uint8_t *)g.B + g.b_sb * bt * ebits / 8; ldp = (int)(g.b_sj * ebits / 8);
     Qg = (const uint8_t *)g.A + g.a_sb * bt * ebits / 8; ldq = (int)(g.a_si * ebits / 8);
   }
-  // split-K: this workgroup's share of the stages; the pointers move, the rest of the kernel sees a
-  // shorter K
+  // split-K: this workgroup's share of the stages starts k0 bytes into every row; the rest of the
+  // kernel sees a shorter K
   int Kbytes_local = Kbytes;
+  int k0 = 0;
+  int sk0 = 0;  // MX: first scale byte of this workgroup's K range in a row of scales (the host keeps
+                // split_stages a multiple of the CH stages of a scale chunk)
   if (prm.splits > 1) {
-    const int k0 = (int)blockIdx.z * prm.split_stages * BKB_;
-    Pg += k0; Qg += k0;
+    k0 = (int)blockIdx.z * prm.split_stages * BKB_;
     Kbytes_local = max(0, min(Kbytes - k0, prm.split_stages * BKB_));
+    sk0 = k0 / 16;
   }
   const int KT = (Kbytes_local + BKB_ - 1) / BKB_;  // real stages
-  const int KTR = (KT + SPT - 1) / SPT * SPT;     // stages run (padding stages multiply zeros)
 
   // 2 GiB raw buffer windows: an offset with bit 31 set is out of range and reads as zero
   const __amdgpu_buffer_rsrc_t rsP = __builtin_amdgcn_make_buffer_rsrc((void *)Pg, 0, 0x80000000, 0x00020000);
@@ -145,17 +147,22 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
     srowP = p0 + (lane >> 1);
     srowQ = q0 - BP + (lane >> 1);
   }
-  // An out-of-range instruction still writes (zeros) to LDS.  The spare ones (part >= SPARTS) are
-  // pointed at the 1 KiB of data slot `so` that this same wave fills with its very next data
-  // instruction: loads of one wave complete in order, so the zeros never survive.
-  auto issue_scale_part = [&](int c, int part, int so) {
+  // Every wave issues the same number of scale instructions per stage (the vmcnt bookkeeping needs
+  // that), which is more than a chunk has parts.  The surplus ones (part >= SPARTS) fetch a part of
+  // the same chunk once more: the same bytes to the same place, harmless whenever they land.  (They
+  // must not be out-of-range instructions aimed at a data slot: those still write zeros to LDS, and
+  // such a write was seen to land after the data that was issued behind it.)
+  auto issue_scale_part = [&](int c, int part_any, int so) {
+    (void)so;
     if constexpr (MX) {
-      const bool spare = part >= SPARTS;
+      const int part = part_any % SPARTS;
       const bool isq = part >= BP / 32;  // wave-uniform: a part never straddles P and Q
       const int row = isq ? min(srowQ + 32 * part, NQ - 1) : min(srowP + 32 * part, NP - 1);
-      const int oob = (!spare && c * 32 < KB) ? 0 : (int)0x80000000;
-      v4i *dst = spare ? &lds[so + wave * RPW * CPR] : &lds[NSTAGE * STAGE_V4 + (c & 1) * CHUNK_V4 + part * 64];
-      lds_dma16(isq ? rsSQ : rsSP, dst, (row * KB + c * 32 + (lane & 1) * 16) | oob, 0);
+      // a chunk past the end of K is never used: it re-reads the start of the tensor (a real load,
+      // see issue_stage)
+      const int live = c * 32 + sk0 < KB ? -1 : 0;
+      v4i *dst = &lds[NSTAGE * STAGE_V4 + (c & 1) * CHUNK_V4 + part * 64];
+      lds_dma16(isq ? rsSQ : rsSP, dst, (row * KB + sk0 + c * 32 + (lane & 1) * 16) & live, 0);
     }
   };
   // the LS scale instructions a wave issues in front of the data that refills slot `so` during
@@ -165,16 +172,24 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
     for (int i = 0; i < LS; i++) issue_scale_part(kt / CH + 1, ((kt % CH) * LS + i) * NWV + wave, so);
   };
 
-  // stage kt -> LDS slot at 16-byte offset `so`; kt >= KT is a padding stage that is zero-filled
+  // stage kt -> LDS slot at 16-byte offset `so`.  Stages kt >= KT are never multiplied; they are
+  // issued only so that every trip of the loop has the same number of vector memory operations in
+  // flight, which the counted waits rely on.  They must be real loads, though (every lane re-reads
+  // the first 16 bytes of the operand: one cache line per instruction): an instruction whose lanes
+  // are all out of range completes without a memory round trip and was seen to retire ahead of
+  // older loads, so a counted wait for the last real stage passed while its data was still on its
+  // way.  (A partly out-of-range instruction, as in the K tail below, goes to memory like any other.)
   auto issue_stage = [&](int kt, int so) {
-    const int oob = kt >= KT ? (int)0x80000000 : (kt == KT - 1 ? oob_last : 0);
+    const int live = kt < KT ? -1 : 0;  // uniform
+    const int oob = kt == KT - 1 ? oob_last : 0;
+    const int soff = (k0 + kt * BKB_) & live;
     v4i *base = &lds[so];
 #pragma unroll
     for (int i = 0; i < LP; i++)
-      lds_dma16(rsP, base + (wave * RPW + RPP * i) * CPR, voffP[i] | oob, kt * BKB_);
+      lds_dma16(rsP, base + (wave * RPW + RPP * i) * CPR, (voffP[i] | oob) & live, soff);
 #pragma unroll
     for (int i = 0; i < LQ; i++)
-      lds_dma16(rsQ, base + (BP + wave * RPW + RPP * i) * CPR, voffQ[i] | oob, kt * BKB_);
+      lds_dma16(rsQ, base + (BP + wave * RPW + RPP * i) * CPR, (voffQ[i] | oob) & live, soff);
   };
 
   // fragment (and MX scale) loads of sub-step ks of the stage in the LDS slot at offset `so`
@@ -262,7 +277,7 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
 #pragma unroll
   for (int s = 0; s < NSTAGE; s++) {
 #pragma unroll
-    for (int i = 0; i < LS; i++) issue_scale_part(0, SPARTS, s * STAGE_V4);  // spare: moves nothing
+    for (int i = 0; i < LS; i++) issue_scale_part(0, SPARTS + i, s * STAGE_V4);  // surplus: part i of chunk 0 once more
     issue_stage(s, s * STAGE_V4);
   }
   wait_vmcnt_barrier<(NSTAGE - 1) * NLOAD>();
@@ -319,15 +334,20 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
     });
   };
 
-  // K loop: SPT stages per trip, no other control flow
+  // K loop: SPT stages per trip, no other control flow; with two stages per trip (the fragment
+  // roles realign every other stage) an odd last stage follows on its own
   int so = 0;
-  for (int kt = 0; kt < KTR; kt += SPT) {
+  int kt = 0;
+  for (; kt + SPT <= KT; kt += SPT) {
     do_stage(kt, so, fa, fb);
     so = so == (NSTAGE - 1) * STAGE_V4 ? 0 : so + STAGE_V4;
     if constexpr (SPT == 2) {
       do_stage(kt + 1, so, fb, fa);
       so = so == (NSTAGE - 1) * STAGE_V4 ? 0 : so + STAGE_V4;
     }
+  }
+  if constexpr (SPT == 2) {
+    if (kt < KT) do_stage(kt, so, fa, fb);
   }
 
   // every wave is done with the LDS tiles (and every DMA has landed) before they become staging

@@ -38,14 +38,18 @@ uint32_t launch_mfma(const Lowered &l, const zluda_gemm_plan &plan, const zluda_
   if ((uint32_t)(prm.tiles_p * prm.tiles_q) != plan.grid_x) return CUBLAS_STATUS_INVALID_VALUE;
   if (plan.grid_z > 1) {
     // split-K: partial tiles go through the caller's workspace
-    if (plan.kernel == ZLUDA_KERNEL_MFMA_MXF4) return CUBLAS_STATUS_INVALID_VALUE;
     const uint64_t need = (uint64_t)plan.grid_z * l.g.batch * prm.tiles_p * v.bp * prm.tiles_q * v.bq * 4;
     if (!p->workspace || (((uintptr_t)p->workspace) & 15) || p->workspace_size < need || plan.workspace != need)
       return CUBLAS_STATUS_INVALID_VALUE;
-    const int kbytes = l.g.K;  // 8-bit operands
+    const bool mx = plan.kernel == ZLUDA_KERNEL_MFMA_MXF4;
+    const int kbytes = mx ? l.g.K / 2 : l.g.K;
     const int stages = (kbytes + v.bkb - 1) / v.bkb;
     prm.splits = (int32_t)plan.grid_z;
     prm.split_stages = (stages + prm.splits - 1) / prm.splits;
+    if (mx) {  // whole scale chunks (32 scale bytes = 512 fp4 bytes per row) per share
+      const int ch = 512 / v.bkb;
+      prm.split_stages = (prm.split_stages + ch - 1) / ch * ch;
+    }
     prm.ws = p->workspace;
   }
   uint32_t st;

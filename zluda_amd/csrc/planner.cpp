@@ -286,7 +286,7 @@ static void fill_mfma_plan(const Lowered &l, int variant, uint32_t cus, uint64_t
   // Split-K: when even the chosen tiles leave half of the CUs idle and K is long, grid_z workgroups
   // share a tile's K range, write their fp32 / int32 partial tiles to the workspace and a second
   // kernel sums them and applies the epilogue.  Only if the caller's workspace holds the partial
-  // tiles (padded to whole tiles); never for MXFP4 (its scale chunks are tied to absolute K).
+  // tiles (padded to whole tiles).  (MXFP4 shares are whole scale chunks: the launcher rounds.)
   const uint64_t tiles = (uint64_t)plan->grid_x * plan->grid_y;
   const uint32_t kt = ceil_div((uint32_t)((int64_t)g.K * (g.a_type == CUDA_R_4F_E2M1 ? 4 : 8) / 8), v.bkb);
   // (below ~6 KiB of K per row the second kernel and the workspace traffic cost more than the idle CUs)
@@ -295,7 +295,8 @@ static void fill_mfma_plan(const Lowered &l, int variant, uint32_t cus, uint64_t
   // and down to 1 KiB per share, up to two workgroups per CU (fp8 4096x48x4096: 18 -> 13 us; but
   // 14336x64x4096, 224 tiles, must stay whole: 16.5 us against 23.7 split in three).
   const bool skinny = std::min(g.M, g.N) <= 64;
-  if (g.a_type != CUDA_R_4F_E2M1 && tiles * 2 <= cus && kbytes >= (skinny ? 2048u : 6144u) &&
+  const bool mx = g.a_type == CUDA_R_4F_E2M1;  // (a byte of FP4 is worth two K steps: 4096x16x4096 loses when split)
+  if (tiles * 2 <= cus && kbytes >= (skinny ? (mx ? 4096u : 2048u) : 6144u) &&
       (uint64_t)tp * v.bp <= (1u << 20)) {
     uint32_t s = (uint32_t)std::min<uint64_t>({8, (skinny ? 2 * cus : cus) / tiles, kbytes / (skinny ? 1024 : 2048)});
     const uint64_t per_split = (uint64_t)g.batch * tp * v.bp * tq * v.bq * 4;
