@@ -325,7 +325,7 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(DecodeParams prm
       }
     }
   }
-  // the zero-fill units issued past the last block still target this workgroup's LDS
+  // the units issued past the last block still target this workgroup's LDS
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 

@@ -44,8 +44,8 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
   constexpr int LP = BP / RPP, LQ = BQ / RPP;  // data DMA instructions per thread, stage and operand
   // MX block scales travel in chunks of 32 scale bytes per tile row (1024 K elements = CH stages),
   // double buffered behind the data stages.  One DMA instruction copies 32 rows x 32 bytes; every
-  // wave issues LS of them per stage (the instructions a chunk does not need go out of range and
-  // move nothing, so that the vmcnt bookkeeping is the same in every stage).
+  // wave issues LS of them per stage (the instructions a chunk does not need fetch one of its parts
+  // a second time, so that the vmcnt bookkeeping is the same in every stage).
   constexpr bool MX = KIND == KIND_MXF4;
   constexpr int SB = BKB_ / 16;                // scale bytes per row and stage
   constexpr int CH = 32 / SB;                  // stages per scale chunk
@@ -115,7 +115,8 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
   }
   const int KT = (Kbytes_local + BKB_ - 1) / BKB_;  // real stages
 
-  // 2 GiB raw buffer windows: an offset with bit 31 set is out of range and reads as zero
+  // 2 GiB raw buffer windows: an offset with bit 31 set is out of range and reads as zero (the lanes
+  // of a K tail)
   const __amdgpu_buffer_rsrc_t rsP = __builtin_amdgcn_make_buffer_rsrc((void *)Pg, 0, 0x80000000, 0x00020000);
   const __amdgpu_buffer_rsrc_t rsQ = __builtin_amdgcn_make_buffer_rsrc((void *)Qg, 0, 0x80000000, 0x00020000);
 
