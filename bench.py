@@ -61,8 +61,8 @@ WORKLOADS = {
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # script (each counter scaled by what it reads for the 256 MiB copy of --copy-probe: x2.000 and x1.000).
 # The summaries are profiles/<kernel>_<workload>.txt; re-measure after changing a kernel's tiling.
-MEASURED_TRAFFIC = {"c1": 905139, "c2": 167889957, "i8_4096_nt": 167951357, "i8_8192": 1074777866, "c3": 60091205, "c4": 941321048,
-                    "c5": 2249388431}
+MEASURED_TRAFFIC = {"c1": 905137, "c2": 167903219, "i8_4096_nt": 167946194, "i8_8192": 1074657654, "c3": 60098974, "c4": 941239837,
+                    "c5": 2248978449}
 
 
 def algorithmic(spec):
