@@ -44,8 +44,8 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
   constexpr int LP = BP / RPP, LQ = BQ / RPP;  // data DMA instructions per thread, stage and operand
   // MX block scales travel in chunks of 32 scale bytes per tile row (1024 K elements = CH stages),
   // double buffered behind the data stages.  One DMA instruction copies 32 rows x 32 bytes; every
-  // wave issues LS of them per stage (the instructions a chunk does not need fetch one of its parts
-  // a second time, so that the vmcnt bookkeeping is the same in every stage).
+  // wave issues LS of them per stage (the instructions a chunk does not need read a single cache line,
+  // so that the vmcnt bookkeeping is the same in every stage).
   constexpr bool MX = KIND == KIND_MXF4;
   constexpr int SB = BKB_ / 16;                // scale bytes per row and stage
   constexpr int CH = 32 / SB;                  // stages per scale chunk
@@ -149,20 +149,19 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
     srowQ = q0 - BP + (lane >> 1);
   }
   // Every wave issues the same number of scale instructions per stage (the vmcnt bookkeeping needs
-  // that), which is more than a chunk has parts.  The surplus ones (part >= SPARTS) fetch a part of
-  // the same chunk once more: the same bytes to the same place, harmless whenever they land.  (They
-  // must not be out-of-range instructions aimed at a data slot: those still write zeros to LDS, and
-  // such a write was seen to land after the data that was issued behind it.)
-  auto issue_scale_part = [&](int c, int part_any, int so) {
-    (void)so;
+  // that), which is more than a chunk has parts.  The surplus ones (part >= SPARTS) are real loads
+  // of one cache line (every lane reads the first 16 bytes of the tensor) into the 1 KiB of data slot
+  // `so` that this same wave fills with its very next data instruction: loads of one wave return in
+  // order, so the bytes never survive.  (Not out-of-range instructions: those complete without a
+  // memory round trip and can retire ahead of older loads, see issue_stage.)
+  auto issue_scale_part = [&](int c, int part, int so) {
     if constexpr (MX) {
-      const int part = part_any % SPARTS;
+      const bool surplus = part >= SPARTS;
       const bool isq = part >= BP / 32;  // wave-uniform: a part never straddles P and Q
       const int row = isq ? min(srowQ + 32 * part, NQ - 1) : min(srowP + 32 * part, NP - 1);
-      // a chunk past the end of K is never used: it re-reads the start of the tensor (a real load,
-      // see issue_stage)
-      const int live = c * 32 + sk0 < KB ? -1 : 0;
-      v4i *dst = &lds[NSTAGE * STAGE_V4 + (c & 1) * CHUNK_V4 + part * 64];
+      // a chunk past the end of K is never used either: it re-reads the start of the tensor
+      const int live = (!surplus && c * 32 + sk0 < KB) ? -1 : 0;
+      v4i *dst = surplus ? &lds[so + wave * RPW * CPR] : &lds[NSTAGE * STAGE_V4 + (c & 1) * CHUNK_V4 + part * 64];
       lds_dma16(isq ? rsSQ : rsSP, dst, (row * KB + sk0 + c * 32 + (lane & 1) * 16) & live, 0);
     }
   };
@@ -278,7 +277,7 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
 #pragma unroll
   for (int s = 0; s < NSTAGE; s++) {
 #pragma unroll
-    for (int i = 0; i < LS; i++) issue_scale_part(0, SPARTS + i, s * STAGE_V4);  // surplus: part i of chunk 0 once more
+    for (int i = 0; i < LS; i++) issue_scale_part(0, SPARTS, s * STAGE_V4);  // surplus: one line, overwritten by the data
     issue_stage(s, s * STAGE_V4);
   }
   wait_vmcnt_barrier<(NSTAGE - 1) * NLOAD>();
