@@ -63,6 +63,18 @@ def test_fp8_transposed_layout_within_tolerance_of_hipblaslt(gpu_api):
     print("max relative difference to hipBLASLt %.3e" % err)
 
 
+def test_fp8_decode_shape_within_tolerance_of_hipblaslt(gpu_api):
+    """a decode-shaped fp8 problem (16 tokens) runs on the streaming kernel; hipBLASLt has algorithms for it"""
+    spec = dict(F8, m=6144, n=16, k=4096, epilogue=K.CUBLASLT_EPILOGUE_BIAS, bias_type=K.CUDA_R_16BF,
+                with_scalar_scales=True, scale_range=(0.05, 0.06), bias_std=0.5)
+    case, ours, theirs, why, kern = both(gpu_api, spec, 13)
+    assert kern == K.ZLUDA_KERNEL_DECODE_W8A8
+    if theirs is None:
+        pytest.skip("hipBLASLt offers no algorithm here: " + why)
+    err = case.compare(ours, theirs, tol=1e-2)
+    print("max relative difference to hipBLASLt %.3e" % err)
+
+
 def test_fp8_scaled_bias_gelu_within_tolerance_of_hipblaslt(gpu_api):
     """benchmark configuration 4 at 1024^3: per-tensor scales, bf16 bias, GELU, bf16 output"""
     spec = dict(F8, m=1024, n=1024, k=1024, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS, bias_type=K.CUDA_R_16BF,
