@@ -174,7 +174,7 @@ def test_decode_two_token_blocks_and_long_k(gpu_api, variant):
 
 
 STREAM = {4: (8, 8), 5: (8, 16), 6: (8, 28), 7: (4, 8), 8: (8, 12), 9: (8, 24), 10: (4, 4), 11: (8, 20), 12: (4, 28),
-          13: (4, 12), 14: (4, 20)}
+          13: (4, 12), 14: (4, 20), 15: (8, 32)}
 
 
 @pytest.mark.parametrize("variant", sorted(STREAM))

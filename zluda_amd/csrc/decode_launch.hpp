@@ -64,6 +64,7 @@ inline uint32_t launch_decode_stream_variant(const DecodeParams &prm, const zlud
     ZLUDA_STREAM_CASE(12, 4, 28)
     ZLUDA_STREAM_CASE(13, 4, 12)
     ZLUDA_STREAM_CASE(14, 4, 20)
+    ZLUDA_STREAM_CASE(15, 8, 32)
 #undef ZLUDA_STREAM_CASE
   default: return CUBLAS_STATUS_INVALID_VALUE;
   }

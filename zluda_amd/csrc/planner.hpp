@@ -51,6 +51,7 @@ constexpr DecodeVariant kDecodeVariants[] = {
     {4, 28, 1},  // 12: K = 7168
     {4, 12, 1},  // 13: K = 3072
     {4, 20, 1},  // 14: K = 5120
+    {8, 32, 1},  // 15: K = 16384 (one block of 16 tokens: 32 fragments)
 };
 constexpr int kNumDecodeVariants = sizeof(kDecodeVariants) / sizeof(kDecodeVariants[0]);
 // Tokens come in blocks of 16; a wave keeps blocks x steps activation fragments (4 VGPRs each) in
