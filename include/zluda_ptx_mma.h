@@ -38,6 +38,13 @@ extern "C" {
 uint32_t zluda_ptx_mma_run(uint32_t kind, const uint32_t *a, const uint32_t *b, const void *c, void *d,
                            uint32_t threads, uint32_t block, uint32_t masked_warps, void *stream);
 
+/* Measurement aid: every thread runs c <- mma(a, b, c) `iters` times in a dependent chain and writes
+ * the last c to d.  Whole wavefronts only (`block` a multiple of 64); `per_lane` != 0 forces the form
+ * that a half-present wavefront falls back to, so that the two can be timed side by side. */
+uint32_t zluda_ptx_mma_chain(uint32_t kind, const uint32_t *a, const uint32_t *b, const void *c, void *d,
+                             uint32_t threads, uint32_t block, uint32_t iters, uint32_t per_lane,
+                             void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -89,3 +89,22 @@ def test_random_fragments_against_the_oracle(lib, kind, block, masked):
         want[odd] = c[odd]
     got = run_gpu(lib, kind, a, b, c, block, masked)
     np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("per_lane", [0, 1])
+def test_chained_instructions(lib, per_lane):
+    """the measurement entry point: c <- mma(a, b, c) three times, both forms, int8 (wraps exactly)"""
+    import torch
+    warps = 16
+    a, b, c = random_fragments(ref.S8, warps, 7100)
+    want = c
+    for _ in range(3):
+        want = ref.mma_sync(ref.S8, a, b, want)
+    ta, tb, tc = (torch.from_numpy(x.view(np.int32).reshape(-1)).cuda() for x in (a, b, c))
+    td = torch.zeros_like(tc)
+    st = lib.zluda_ptx_mma_chain(ref.S8, ta.data_ptr(), tb.data_ptr(), tc.data_ptr(), td.data_ptr(), warps * 32, 128, 3,
+                                 per_lane, torch.cuda.current_stream().cuda_stream)
+    assert st == 0
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(td.cpu().numpy().reshape(warps, 32, 4), want)

@@ -32,6 +32,39 @@ __global__ void ptx_mma_run_kernel(const u32x4 *a, const u32x2 *b, const u32x4 *
   d[i] = dv;
 }
 
+// c <- mma(a, b, c) `iters` times in a dependent chain: the cost of one instruction, for measurement
+template <int KIND, bool PER_LANE>
+__global__ void ptx_mma_chain_kernel(const u32x4 *a, const u32x2 *b, const u32x4 *c, u32x4 *d, uint32_t iters) {
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  const u32x4 av = a[i];
+  const u32x2 bv = b[i];
+  typename Acc<KIND>::type acc = __builtin_bit_cast(typename Acc<KIND>::type, c[i]);
+  const int lane = lane_id();
+  for (uint32_t it = 0; it < iters; it++) acc = PER_LANE ? mma_per_lane<KIND>(av, bv, acc, lane) : mma_wave64<KIND>(av, bv, acc, lane);
+  d[i] = __builtin_bit_cast(u32x4, acc);
+}
+
+extern "C" uint32_t zluda_ptx_mma_chain(uint32_t kind, const uint32_t *a, const uint32_t *b, const void *c, void *d,
+                                        uint32_t threads, uint32_t block, uint32_t iters, uint32_t per_lane, void *stream) {
+  if (!a || !b || !c || !d || kind > ZLUDA_PTX_MMA_BF16) return 7;
+  if (block == 0 || block > 1024 || block % 64 || threads == 0 || threads % block) return 7;
+  const dim3 grid(threads / block), blk(block);
+  hipStream_t s = (hipStream_t)stream;
+  const u32x4 *av = (const u32x4 *)a, *cv = (const u32x4 *)c;
+  const u32x2 *bv = (const u32x2 *)b;
+  u32x4 *dv = (u32x4 *)d;
+#define ZLUDA_CHAIN(K)                                                                                       \
+  if (per_lane) hipLaunchKernelGGL((ptx_mma_chain_kernel<K, true>), grid, blk, 0, s, av, bv, cv, dv, iters); \
+  else hipLaunchKernelGGL((ptx_mma_chain_kernel<K, false>), grid, blk, 0, s, av, bv, cv, dv, iters)
+  switch (kind) {
+  case ZLUDA_PTX_MMA_S8: ZLUDA_CHAIN(S8); break;
+  case ZLUDA_PTX_MMA_F16: ZLUDA_CHAIN(F16); break;
+  default: ZLUDA_CHAIN(BF16); break;
+  }
+#undef ZLUDA_CHAIN
+  return hipGetLastError() == hipSuccess ? 0 : 13;
+}
+
 extern "C" uint32_t zluda_ptx_mma_run(uint32_t kind, const uint32_t *a, const uint32_t *b, const void *c, void *d,
                                       uint32_t threads, uint32_t block, uint32_t masked_warps, void *stream) {
   if (!a || !b || !c || !d || kind > ZLUDA_PTX_MMA_BF16) return 7;
