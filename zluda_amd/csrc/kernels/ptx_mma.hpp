@@ -24,8 +24,8 @@
 //   B register r: rows t*E .. +E-1 (+ 4E if r == 1), column g
 //   C/D register r: row g + 8*(r>>1), column 2*t + (r&1)
 //
-// Data movement per wavefront (two mma instructions' worth): 4 ds_permute for A, 4 ds_bpermute for
-// B, 4 ds_permute for D -- each ds_permute is a permutation of the 64 lanes in which the SENDER picks
+// Data movement per wavefront (two mma instructions' worth): 4 ds_permute for A, 2 ds_permute (and two
+// DPP rotates) for B, 4 ds_permute for D -- each ds_permute is a permutation of the 64 lanes in which the SENDER picks
 // which of its registers goes out, which halves the count against pulling (a lane holds two rows of
 // A but an MFMA lane wants one) -- plus one MFMA, against 16 ds_bpermute and 32 dot instructions per
 // warp in the per-lane form.
@@ -116,12 +116,17 @@ __device__ __forceinline__ typename Acc<KIND>::type mma_wave64(u32x4 a, u32x2 b,
   }
   const i32x4 cols = {(int)(hi ? ta[1] : ta[0]), (int)(hi ? ta[3] : ta[2]), (int)(hi ? ta[0] : ta[1]), (int)(hi ? ta[2] : ta[3])};
 
-  // B -> src0.  MFMA row idx = 8*w' + n takes column n of warp w' from lanes (g = n, t = 2h, 2h+1) of
-  // that warp, and only in that warp's K-groups.
-  const int s0 = 32 * (kq >> 1) + 4 * (idx & 7) + 2 * (kq & 1);
+  // B -> src0.  MFMA row 8*w + n takes column n of warp w, and only in that warp's K-groups; the other
+  // half of the MFMA lanes (row of the other warp) holds zeros.  Lanes with even t send their two
+  // registers to the MFMA lane that uses them (row 8w + g, K-group 2w + t/2), lanes with odd t to
+  // its idle neighbour 8 lanes further in the same row of 16, from where a DPP rotate brings them
+  // over: 2 permutations instead of 4.
+  const int dst_b = ((8 * w + g) ^ (t_odd << 3)) + 16 * (2 * w + (t >> 1));
+  const uint32_t e0 = push(dst_b, b[0]), e1 = push(dst_b, b[1]);
+  const uint32_t o0 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)e0, 0x128, 0xf, 0xf, false);  // row_ror:8
+  const uint32_t o1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)e1, 0x128, 0xf, 0xf, false);
   const bool mine = (idx >> 3) == (kq >> 1);
-  const uint32_t r0 = pull(s0, b[0]), r1 = pull(s0, b[1]), r2 = pull(s0 + 1, b[0]), r3 = pull(s0 + 1, b[1]);
-  const i32x4 rows = {mine ? (int)r0 : 0, mine ? (int)r1 : 0, mine ? (int)r2 : 0, mine ? (int)r3 : 0};
+  const i32x4 rows = {mine ? (int)e0 : 0, mine ? (int)e1 : 0, mine ? (int)o0 : 0, mine ? (int)o1 : 0};
 
   acc_t acc;
   if constexpr (KIND == S8) acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(rows, cols, i32x4{0, 0, 0, 0}, 0, 0, 0);
