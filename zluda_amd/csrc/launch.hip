@@ -1,5 +1,6 @@
 // The extern "C" launch layer: lowers a problem, picks the template instantiation the plan names
 // and enqueues it on the caller's stream.  Only the HIP runtime is used (hipLaunchKernelGGL).
+#include <atomic>
 #include <hip/hip_runtime.h>
 
 #include <cstring>
@@ -173,11 +174,14 @@ uint32_t launch_decode(const Lowered &l, const zluda_gemm_plan &plan, hipStream_
 extern "C" uint32_t zluda_gemm_device_cu_count(void) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return 0;
-  static int cached[64];
-  if (dev >= 0 && dev < 64 && cached[dev]) return (uint32_t)cached[dev];
+  static std::atomic<int> cached[64];  // zero-initialised; any thread may fill an entry (same value)
+  if (dev >= 0 && dev < 64) {
+    const int c = cached[dev].load(std::memory_order_relaxed);
+    if (c) return (uint32_t)c;
+  }
   int cus = 0;
   if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
-  if (dev >= 0 && dev < 64) cached[dev] = cus;
+  if (dev >= 0 && dev < 64) cached[dev].store(cus, std::memory_order_relaxed);
   return (uint32_t)cus;
 }
 
