@@ -2,12 +2,19 @@
 """Benchmark of the cublasLtMatmul hot path on one MI355X.
 
 A "step" is one cublasLtMatmul call (through the exported C ABI of zluda_amd/lib/libcublaslt.so) on
-synthetic inputs that are already resident in HBM.  The headline line reports benchmark configuration 2
-(int8 x int8 -> int32, M=N=K=4096, A:T B:N); the other benchmark configurations and the 8192^3 int8
-case ride along under "also", each with its own roofline figures and, when the installed hipBLASLt
-has a solution, the time of the reference's hipBLASLt-forwarded path on the same buffers.
+synthetic inputs that are already resident in HBM.  The headline line reports benchmark configuration 4
+(fp8 e4m3, M=N=K=8192, per-tensor scales, bf16 bias + GELU, bf16 D): the 8192^3 size the metric is quoted
+on.  The other benchmark configurations, the 8192^3 int8 case and configuration 5's problem at batch 1
+ride along under "also", each with its own roofline figures and, when the installed hipBLASLt has a
+solution, the time of the reference's hipBLASLt-forwarded path on the same buffers.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c2|c3|c4|c5|i8_8192|i8_4096_nt] [--only]
+Timing: W warm-up calls, then exactly K calls between two synchronisations (wall clock -> `value`); HIP
+events on the launch stream split the K calls into five batches, and `roofline.kernel_ms` is the median
+batch.  A one-wave probe kernel on a second stream samples the shader cycle counter against the real-time
+counter during one more (untimed) batch: `clock_mhz_observed`, and `frac_at_observed_clock` = the
+roofline fraction against the datasheet peak scaled to that clock (the peak assumes 2400 MHz).
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c2|c3|c4|c5|c5_b1|i8_8192|i8_4096_nt] [--only]
                   [--no-cpu] [--no-hipblaslt] [--copy-probe]
 """
 import argparse
@@ -28,6 +35,7 @@ from zluda_amd.cublaslt import MatmulCall  # noqa: E402
 
 K = abi
 PEAK = {"i8": 5000.0, "f8": 5000.0, "f4": 10100.0, "hbm": 8000.0}  # TOP/s, TFLOP/s, GB/s (MI355X datasheet)
+PEAK_CLOCK_MHZ = 2400.0   # the shader clock the datasheet's matrix peaks are quoted at
 
 I8 = dict(a_type=K.CUDA_R_8I, b_type=K.CUDA_R_8I, d_type=K.CUDA_R_32I, compute_type=K.CUBLAS_COMPUTE_32I,
           scale_type=K.CUDA_R_32I, transa=1)
@@ -38,7 +46,7 @@ WORKLOADS = {
                spec=dict(I8, m=4096, n=4096, k=4096), steps=50),
     "i8_4096_nt": dict(name="int8xint8->int32 M=N=K=4096 A:N B:T (config 1's layout at config 2's size)", kind="i8",
                        spec=dict(I8, m=4096, n=4096, k=4096, transa=0, transb=1), steps=50),
-    "i8_8192": dict(name="int8xint8->int32 M=N=K=8192 A:T B:N", kind="i8", spec=dict(I8, m=8192, n=8192, k=8192), steps=10),
+    "i8_8192": dict(name="int8xint8->int32 M=N=K=8192 A:T B:N", kind="i8", spec=dict(I8, m=8192, n=8192, k=8192), steps=25),
     "c3": dict(name="W8A8 decode M=14336 N=16 K=4096 alpha-vec + per-token scale + fp32 bias -> bf16 (benchmark configuration 3)",
                kind="hbm", steps=200,
                spec=dict(I8, d_type=K.CUDA_R_16BF, scale_type=K.CUDA_R_32F, m=14336, n=16, k=4096,
@@ -46,23 +54,47 @@ WORKLOADS = {
                          b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F,
                          epilogue=K.CUBLASLT_EPILOGUE_BIAS, bias_type=K.CUDA_R_32F)),
     "c4": dict(name="fp8 e4m3 M=N=K=8192 per-tensor scales, bf16 bias + GELU -> bf16 (benchmark configuration 4)", kind="f8",
-               steps=10,
+               steps=50,
                spec=dict(a_type=K.CUDA_R_8F_E4M3, b_type=K.CUDA_R_8F_E4M3, d_type=K.CUDA_R_16BF,
                          compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F, transa=1, m=8192, n=8192, k=8192,
                          epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS, bias_type=K.CUDA_R_16BF)),
-    "c5": dict(name="MXFP4 (E2M1 + UE8M0/32) M=N=K=8192 batch 4 -> bf16 (benchmark configuration 5)", kind="f4", steps=5,
+    "c5": dict(name="MXFP4 (E2M1 + UE8M0/32) M=N=K=8192 batch 4 -> bf16 (benchmark configuration 5)", kind="f4", steps=10,
                spec=dict(a_type=K.CUDA_R_4F_E2M1, b_type=K.CUDA_R_4F_E2M1, d_type=K.CUDA_R_16BF,
                          compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F, transa=1, m=8192, n=8192, k=8192,
                          batch=4, a_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_VEC32_UE8M0,
                          b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_VEC32_UE8M0)),
+    "c5_b1": dict(name="MXFP4 (E2M1 + UE8M0/32) M=N=K=8192 batch 1 -> bf16 (configuration 5's problem at the one batch "
+                       "count the installed hipBLASLt takes)", kind="f4", steps=10,
+                  spec=dict(a_type=K.CUDA_R_4F_E2M1, b_type=K.CUDA_R_4F_E2M1, d_type=K.CUDA_R_16BF,
+                            compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F, transa=1, m=8192, n=8192, k=8192,
+                            a_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_VEC32_UE8M0,
+                            b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_VEC32_UE8M0)),
 }
+for _w in WORKLOADS.values():   # five equal batches
+    _w["steps"] = max(5, _w["steps"] // 5 * 5)
 
 
-# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
-# script (each counter scaled by what it reads for the 256 MiB copy of --copy-probe: x2.000 and x1.000).
-# The summaries are profiles/<kernel>_<workload>.txt; re-measure after changing a kernel's tiling.
-MEASURED_TRAFFIC = {"c1": 905137, "c2": 167903219, "i8_4096_nt": 167946194, "i8_8192": 1074657654, "c3": 60098974, "c4": 941239837,
-                    "c5": 2248978449}
+# HBM bytes per launch of the dominant kernel come from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# this script whose summaries are committed under profiles/ (each counter scaled by what it reads for the
+# 256 MiB copy of --copy-probe).  The line carries the figure and the file it was read from; a workload
+# without a summary reports null.
+PROFILE_OF = {"c1": "gemm_mfma_tr_i8_c1_256", "c2": "gemm_mfma_pipe_i8_c2_4096", "i8_4096_nt": "gemm_mfma_tr_i8_4096_nt",
+              "i8_8192": "gemm_mfma_pipe_i8_8192", "c3": "decode_stream_c3", "c4": "gemm_mfma_pipe_f8_c4_8192",
+              "c5": "gemm_mfma_pipe_mxf4_c5_8192x4"}
+
+
+def measured_traffic(key):
+    """(bytes per launch or None, file name or None) from profiles/<kernel>_<workload>.txt"""
+    import re
+    name = PROFILE_OF.get(key)
+    if not name:
+        return None, None
+    path = os.path.join(ROOT, "profiles", name + ".txt")
+    try:
+        m = re.search(r"traffic = (\d+) bytes per dispatch", open(path).read())
+    except OSError:
+        return None, None
+    return (int(m.group(1)), "profiles/%s.txt" % name) if m else (None, None)
 
 
 def algorithmic(spec):
@@ -89,7 +121,7 @@ class Buffers:
     def __init__(self, torch, key, spec, copies=1):
         dev = "cuda:0"
         g = torch.Generator(device=dev)
-        g.manual_seed({"c2": 1, "c3": 2, "c4": 3, "c5": 4}.get(key, 5))
+        g.manual_seed({"c2": 1, "c3": 2, "c4": 3, "c5": 4, "c5_b1": 4}.get(key, 5))
         m, n, k, b = spec["m"], spec["n"], spec["k"], spec.get("batch", 1)
         self.keep = []
         self.bias = self.a_scale = self.b_scale = self.alpha_dev = None
@@ -137,20 +169,59 @@ class Buffers:
             self.bias = (torch.randn(m, device=dev, generator=g) * 0.02).to(torch.bfloat16)
 
 
+NBATCH = 5
+
+
 def time_calls(torch, fn, steps, warmup):
-    """returns (wall seconds for `steps` calls, seconds per call by HIP events on the launch stream)"""
+    """`warmup` untimed calls, then exactly `steps` calls between two synchronisations.  Returns (wall seconds
+    for the `steps` calls, median over NBATCH equal batches of the seconds per call by HIP events on the launch
+    stream, [seconds per call of each batch])."""
     for i in range(warmup):
         fn(i)
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    nb = NBATCH if steps % NBATCH == 0 else 1
+    per = steps // nb
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(nb + 1)]
     t0 = time.perf_counter()
-    e0.record()
-    for i in range(steps):
-        fn(i)
-    e1.record()
+    ev[0].record()
+    for b in range(nb):
+        for i in range(per):
+            fn(b * per + i)
+        ev[b + 1].record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    return wall, e0.elapsed_time(e1) * 1e-3 / steps
+    batches = sorted(ev[b].elapsed_time(ev[b + 1]) * 1e-3 / per for b in range(nb))
+    return wall, batches[len(batches) // 2], batches
+
+
+_probe = None
+
+
+def observed_clock_mhz(torch, fn, calls, seconds_per_call):
+    """Shader clock held while `calls` more calls of `fn` run: a one-wave kernel on a second stream reads the
+    shader cycle counter and the constant-rate real-time counter at both ends of ~80 % of that stretch.
+    None when the helper library is missing."""
+    global _probe
+    path = os.path.join(ROOT, "zluda_amd", "lib", "libzluda_bench_probe.so")
+    if _probe is None:
+        if not os.path.exists(path):
+            return None
+        _probe = C.CDLL(path)
+        _probe.zluda_bench_clock_probe.argtypes = [C.c_void_p, C.c_uint64, C.c_void_p]
+    khz = _probe.zluda_bench_wall_clock_khz()
+    if khz <= 0:
+        return None
+    out = torch.zeros(2, dtype=torch.int64, device="cuda:0")
+    side = torch.cuda.Stream()
+    ticks = int(max(calls * seconds_per_call * 0.8, 20e-6) * khz * 1e3)
+    fn(0)   # the load is already running when the probe takes its first sample
+    if _probe.zluda_bench_clock_probe(out.data_ptr(), ticks, side.cuda_stream) != 0:
+        return None
+    for i in range(calls):
+        fn(i)
+    torch.cuda.synchronize()
+    cycles, rt = (int(x) for x in out.tolist())
+    return cycles / (rt / (khz * 1e3)) / 1e6 if rt > 0 else None
 
 
 def run_workload(torch, api, key, steps, warmup, with_hipblaslt):
@@ -179,18 +250,23 @@ def run_workload(torch, api, key, steps, warmup, with_hipblaslt):
         st = call.run(alpha, a_ptrs[i % copies], bp, zero, None, dp, None, 0, stream)
         if st:
             raise RuntimeError("cublasLtMatmul status %d on workload %s" % (st, key))
-    wall, per_call = time_calls(torch, ours, steps, warmup)
+    wall, per_call, batches = time_calls(torch, ours, steps, warmup)
     bound = "hbm" if w["kind"] == "hbm" else "mfma"
     achieved = (nbytes / per_call / 1e9) if bound == "hbm" else (ops / per_call / 1e12)
     peak = PEAK[w["kind"]]
+    traffic, traffic_file = measured_traffic(key)
+    clock = observed_clock_mhz(torch, ours, max(steps // NBATCH, 4), per_call)
     res = {
         "workload": w["name"], "steps": steps, "ms_per_step": wall / steps * 1e3,
         "tops": ops / (wall / steps) / 1e12, "gbps": nbytes / (wall / steps) / 1e9,
         "kernel": {"family": call.kernel, "variant": call.variant},
         "roofline": {"bound": bound, "achieved": achieved, "peak": peak, "unit": "GB/s" if bound == "hbm" else "TFLOP/s",
-                     "frac": achieved / peak, "traffic": MEASURED_TRAFFIC.get(key), "kernel_ms": per_call * 1e3,
-                     "algorithmic_ops": ops, "algorithmic_bytes": nbytes},
+                     "frac": achieved / peak, "traffic": traffic, "traffic_source": traffic_file,
+                     "kernel_ms": per_call * 1e3, "kernel_ms_batches": [b * 1e3 for b in batches],
+                     "algorithmic_ops": ops, "algorithmic_bytes": nbytes, "clock_mhz_observed": clock},
     }
+    if clock and bound == "mfma":   # what the datasheet peak comes to at the clock the part actually held
+        res["roofline"]["frac_at_observed_clock"] = achieved / (peak * clock / PEAK_CLOCK_MHZ)
     if with_hipblaslt:
         res["hipblaslt_forwarded"] = time_hipblaslt(torch, spec, buf, alpha, zero, a_ptrs, copies, steps, warmup, ops, nbytes)
     call.close()
@@ -219,7 +295,7 @@ def time_hipblaslt(torch, spec, buf, alpha, zero, a_ptrs, copies, steps, warmup,
             st = rp.run(alpha, a_ptrs[i % copies], bp, zero, None, dp, stream)
             if st:
                 raise RuntimeError("hipblasLtMatmul status %d" % st)
-        wall, per_call = time_calls(torch, theirs, steps, warmup)
+        wall, per_call, _ = time_calls(torch, theirs, steps, warmup)
         rp.close()
         return {"available": True, "ms_per_step": wall / steps * 1e3, "kernel_ms": per_call * 1e3,
                 "tops": ops / per_call / 1e12, "gbps": nbytes / per_call / 1e9}
@@ -230,12 +306,13 @@ def time_hipblaslt(torch, spec, buf, alpha, zero, a_ptrs, copies, steps, warmup,
 def cpu_baseline(key, budget_s=12.0):
     """The CPU oracle (oracle/ref_gemm.c, OpenMP over all host cores) timed on a bounded sample of the
     workload: a slab of rows of D (full N and K, one batch), repeated until `budget_s` seconds of CPU
-    work have been spent."""
+    work have been spent.  For a slab the rate is extrapolated to the whole problem (every row of D costs the
+    same) and the sample text says so."""
     import oracle  # noqa: F401
     from oracle.cases import Case
     spec = dict(WORKLOADS[key]["spec"])
     full_m = spec["m"]
-    rows = {"c1": full_m, "c2": full_m, "i8_4096_nt": full_m, "i8_8192": 2048, "c3": full_m, "c4": 256, "c5": 64}[key]
+    rows = {"c1": full_m, "c2": full_m, "i8_4096_nt": full_m, "i8_8192": 2048, "c3": full_m, "c4": 256, "c5": 64, "c5_b1": 64}[key]
     spec.update(m=rows, batch=1, alpha=1)
     case = Case(spec, 1, int_dist="normal" if key == "c3" else "uniform")
     case.run_oracle()   # page in, spin up the OpenMP team
@@ -250,16 +327,17 @@ def cpu_baseline(key, budget_s=12.0):
     val = (algorithmic(spec)[1] * reps / dt / 1e9) if key == "c3" else ops / dt / 1e12
     return {"value": val, "unit": unit, "cores": int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)),
             "kind": "port", "seconds": dt,
-            "sample": "%d passes over %d of %d rows of D (full N=%d, K=%d, batch 1), oracle/ref_gemm.c with OpenMP, "
-                      "%.1f s of CPU time" % (reps, rows, full_m, spec["n"], spec["k"], dt)}
+            "sample": "%d passes over %d of %d rows of D (full N=%d, K=%d, batch 1)%s, oracle/ref_gemm.c with OpenMP, "
+                      "%.1f s of CPU time" % (reps, rows, full_m, spec["n"], spec["k"],
+                                              "; rate of the slab, extrapolated to the whole problem" if rows < full_m else "", dt)}
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=0)
-    ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS))
     ap.add_argument("--only", action="store_true", help="skip the other workloads")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-hipblaslt", action="store_true")
@@ -284,7 +362,7 @@ def main():
     head = run_workload(torch, api, key, steps, args.warmup, not args.no_hipblaslt)
     also = {}
     if not args.only:
-        for other in ("i8_8192", "c3", "c4", "c5", "c2", "c1", "i8_4096_nt"):
+        for other in ("c4", "i8_8192", "c3", "c5", "c5_b1", "c2", "c1", "i8_4096_nt"):
             if other == key:
                 continue
             try:
@@ -300,6 +378,8 @@ def main():
         "vs_baseline": None, "dtype": {"i8": "int8", "hbm": "int8", "f8": "fp8_e4m3", "f4": "fp4_e2m1"}[WORKLOADS[key]["kind"]],
         "data": "synthetic", "config": {"workload": head["workload"], "kernel": head["kernel"]},
         "roofline": head["roofline"],
+        "clock_mhz_observed": head["roofline"].get("clock_mhz_observed"),
+        "frac_at_observed_clock": head["roofline"].get("frac_at_observed_clock"),
         "cpu_baseline": None if args.no_cpu else cpu_baseline(key),
         "hipblaslt_forwarded": head.get("hipblaslt_forwarded"),
         "device": torch.cuda.get_device_name(0), "cu_count": api.zluda_gemm_device_cu_count(),

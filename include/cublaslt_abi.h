@@ -23,6 +23,10 @@
 #ifdef __cplusplus
 extern "C" {
 #endif
+/* the declarations below are the library's exported symbols (it is built with -fvisibility=hidden) */
+#if defined(__GNUC__)
+#pragma GCC visibility push(default)
+#endif
 
 /* ---- cublasStatus_t : cuda_types/src/cublas.rs:322-350 ---------------------------------- */
 typedef uint32_t cublasStatus_t;
@@ -356,6 +360,9 @@ cublasStatus_t cublasLtLoggerSetLevel(int level);
 cublasStatus_t cublasLtLoggerSetMask(int mask);
 cublasStatus_t cublasLtLoggerForceDisable(void);
 
+#if defined(__GNUC__)
+#pragma GCC visibility pop
+#endif
 #ifdef __cplusplus
 }
 #endif

@@ -18,6 +18,10 @@
 #ifdef __cplusplus
 extern "C" {
 #endif
+/* the declarations below are the library's exported symbols (it is built with -fvisibility=hidden) */
+#if defined(__GNUC__)
+#pragma GCC visibility push(default)
+#endif
 
 /* One matrix operand as cublasLtMatrixLayout_t describes it
  * (cuda_types/src/cublaslt.rs:3981-4058; created by zluda_blaslt/src/impl.rs:360-386). */
@@ -119,6 +123,9 @@ uint32_t zluda_gemm_variant_count(uint32_t kernel);
 /* Number of compute units of the current HIP device (0 when no device is usable). */
 uint32_t zluda_gemm_device_cu_count(void);
 
+#if defined(__GNUC__)
+#pragma GCC visibility pop
+#endif
 #ifdef __cplusplus
 }
 #endif

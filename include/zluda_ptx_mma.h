@@ -22,6 +22,10 @@
 #ifdef __cplusplus
 extern "C" {
 #endif
+/* the declarations below are the library's exported symbols (it is built with -fvisibility=hidden) */
+#if defined(__GNUC__)
+#pragma GCC visibility push(default)
+#endif
 
 #define ZLUDA_PTX_MMA_S8 0u   /* m16n8k32.row.col.s32.s8.s8.s32 */
 #define ZLUDA_PTX_MMA_F16 1u  /* m16n8k16.row.col.f32.f16.f16.f32 */
@@ -45,6 +49,9 @@ uint32_t zluda_ptx_mma_chain(uint32_t kind, const uint32_t *a, const uint32_t *b
                              uint32_t threads, uint32_t block, uint32_t iters, uint32_t per_lane,
                              void *stream);
 
+#if defined(__GNUC__)
+#pragma GCC visibility pop
+#endif
 #ifdef __cplusplus
 }
 #endif

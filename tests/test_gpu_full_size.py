@@ -49,8 +49,10 @@ def slab_check(gpu_api, spec, seed, slabs, rows=64, **kw):
 def test_config4_fp8_8192_gelu_bias(gpu_api):
     spec = dict(a_type=K.CUDA_R_8F_E4M3, b_type=K.CUDA_R_8F_E4M3, d_type=K.CUDA_R_16BF, c_type=K.CUDA_R_16BF,
                 compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F, transa=1, m=8192, n=8192, k=8192,
-                epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS, bias_type=K.CUDA_R_16BF, with_scalar_scales=True,
-                alpha=1.0, scale_range=(0.1, 0.12), bias_std=0.5)
+                epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS, bias_type=K.CUDA_R_16BF, f8_amax_quant=True,
+                alpha=1.0, bias_std=0.02)
+    # the configuration's own recipe: x ~ N(0,1), q = e4m3(x * 448 / max|x|), per-tensor scale = max|x| / 448,
+    # bf16 bias ~ N(0, 0.02)
     kern = slab_check(gpu_api, spec, 3, [0, 4064, 8128])
     assert kern == K.ZLUDA_KERNEL_MFMA_F8
 

@@ -178,14 +178,23 @@ STREAM = {4: (8, 8), 5: (8, 16), 6: (8, 28), 7: (4, 8), 8: (8, 12), 9: (8, 24), 
 
 
 @pytest.mark.parametrize("variant", sorted(STREAM))
-def test_decode_stream_variants(gpu_api, variant, monkeypatch):
+def check_small_grid(gpu_api, spec, seed, variant, grid_x, **case_kw):
+    """through the inner launch layer with a grid of `grid_x` workgroups: several 16-row blocks per workgroup"""
+    print("case", spec, "seed", seed, "variant", variant, "grid_x", grid_x, flush=True)
+    case = Case(spec, seed, **case_kw)
+    st, got, plan = case.run_gpu_plan(gpu_api, K.ZLUDA_KERNEL_DECODE_W8A8, variant, grid_x=grid_x)
+    assert st == 0 and plan.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and plan.variant == variant
+    case.compare(got, case.run_oracle())
+
+
+def test_decode_stream_variants(gpu_api, variant):
     """weights streamed through LDS: every K the variant table serves, ragged row ranges (row count
     neither a multiple of 16 nor of the grid), several 16-row blocks per workgroup, 1..32 tokens"""
     nw, steps = STREAM[variant]
     k = nw * steps * 64
     check(gpu_api, dict(DECODE, m=1000, n=16, k=k), 120 + variant, K.ZLUDA_KERNEL_DECODE_W8A8, variant, int_dist="normal")
-    monkeypatch.setenv("ZLUDA_DECODE_GRID", "7")      # 142.86 rows per workgroup: 9 blocks, the last partial
-    check(gpu_api, dict(DECODE, m=1000, n=5, k=k, lda=k + 64), 140 + variant, K.ZLUDA_KERNEL_DECODE_W8A8, variant, int_dist="normal")
+    # 7 workgroups: 142.86 rows each, 9 blocks, the last partial
+    check_small_grid(gpu_api, dict(DECODE, m=1000, n=5, k=k, lda=k + 64), 140 + variant, variant, 7, int_dist="normal")
     # more tokens: blocks of 16, as many as the activation registers allow (blocks x steps <= 32)
     for blocks, tokens in ((2, 29), (3, 41), (4, 64)):
         if blocks * steps <= 32:
@@ -194,7 +203,7 @@ def test_decode_stream_variants(gpu_api, variant, monkeypatch):
 
 
 @pytest.mark.parametrize("variant", sorted(STREAM))
-def test_decode_stream_variants_fp8(gpu_api, variant, monkeypatch):
+def test_decode_stream_variants_fp8(gpu_api, variant):
     """the same kernel for e4m3 x e4m3 (v_mfma_f32_16x16x128_f8f6f4): per-tensor scales, bias, bf16 / f16 / f32
     outputs, ragged row ranges, 1..64 tokens, a C read"""
     nw, steps = STREAM[variant]
@@ -202,8 +211,7 @@ def test_decode_stream_variants_fp8(gpu_api, variant, monkeypatch):
     DEC = K.ZLUDA_KERNEL_DECODE_W8A8
     f8 = dict(F8, epilogue=K.CUBLASLT_EPILOGUE_BIAS, bias_type=K.CUDA_R_16BF, with_scalar_scales=True, scale_range=(0.05, 0.06))
     check(gpu_api, dict(f8, m=1000, n=16, k=k), 420 + variant, DEC, variant)
-    monkeypatch.setenv("ZLUDA_DECODE_GRID", "7")
-    check(gpu_api, dict(f8, m=1000, n=5, k=k, lda=k + 64, d_type=K.CUDA_R_16F), 440 + variant, DEC, variant)
+    check_small_grid(gpu_api, dict(f8, m=1000, n=5, k=k, lda=k + 64, d_type=K.CUDA_R_16F), 440 + variant, variant, 7)
     check(gpu_api, dict(F8, m=333, n=3, k=k, with_c=True, d_type=K.CUDA_R_32F, c_type=K.CUDA_R_32F), 450 + variant, DEC, variant)
     for blocks, tokens in ((2, 29), (3, 41), (4, 64)):
         if blocks * steps <= 32:

@@ -59,7 +59,7 @@ def test_fp8_transposed_layout_within_tolerance_of_hipblaslt(gpu_api):
     assert kern == K.ZLUDA_KERNEL_MFMA_TR8
     if theirs is None:
         pytest.skip("hipBLASLt offers no algorithm here: " + why)
-    err = case.compare(ours, theirs, tol=1e-2)
+    err = case.compare(ours, theirs, tol=1e-2, floor_frac=1e-2)   # both sides use the fp8 MFMA: strict floor
     print("max relative difference to hipBLASLt %.3e" % err)
 
 
@@ -71,7 +71,7 @@ def test_fp8_decode_shape_within_tolerance_of_hipblaslt(gpu_api):
     assert kern == K.ZLUDA_KERNEL_DECODE_W8A8
     if theirs is None:
         pytest.skip("hipBLASLt offers no algorithm here: " + why)
-    err = case.compare(ours, theirs, tol=1e-2)
+    err = case.compare(ours, theirs, tol=1e-2, floor_frac=1e-2)   # both sides use the fp8 MFMA: strict floor
     print("max relative difference to hipBLASLt %.3e" % err)
 
 
@@ -83,7 +83,7 @@ def test_fp8_scaled_bias_gelu_within_tolerance_of_hipblaslt(gpu_api):
     assert kern == K.ZLUDA_KERNEL_MFMA_F8
     if theirs is None:
         pytest.skip("hipBLASLt offers no algorithm here: " + why)
-    err = case.compare(ours, theirs, tol=1e-2)
+    err = case.compare(ours, theirs, tol=1e-2, floor_frac=1e-2)   # both sides use the fp8 MFMA: strict floor
     print("max relative difference to hipBLASLt %.3e" % err)
 
 
@@ -140,4 +140,106 @@ def test_gelu_form_of_hipblaslt_is_the_tanh_form(gpu_api):
           "to the erf form %.3e; max |diff| overall %.3e / %.3e" % (apart.sum(), d_tanh, d_erf,
                                                                    np.abs(t - tanh_form).max(), np.abs(t - erf_form).max()))
     assert d_tanh < d_erf, "hipBLASLt applies the erf form: the oracle's GELU must follow"
-    case.compare(ours, theirs, tol=1e-2)
+    case.compare(ours, theirs, tol=1e-2, floor_frac=1e-2)
+
+
+def test_hipblaslt_fp8_deviates_from_the_fp64_oracle_like_we_do(gpu_api):
+    """Why the comparison with the float64 oracle uses floor = 1e-1 * rms for fp8 inputs: the reference's own
+    backend, on the same inputs, misses the strict bound (floor 1e-2 * rms) against the exact sum by the same
+    order as our kernel does, while the two GPU results agree with each other under the strict floor.  The
+    figures of all three comparisons are printed."""
+    spec = dict(F8, m=1024, n=1024, k=4096, with_scalar_scales=True, scale_range=(0.05, 0.06))
+    case, ours, theirs, why, kern = both(gpu_api, spec, 21)
+    assert kern == K.ZLUDA_KERNEL_MFMA_F8
+    if theirs is None:
+        pytest.skip("hipBLASLt offers no algorithm here: " + why)
+    ref = case.run_oracle()
+    case.compare(ours, ref)
+    e_ours = dict(case.last_errors)
+    case.compare(theirs, ref)
+    e_theirs = dict(case.last_errors)
+    case.compare(ours, theirs, tol=1e-2, floor_frac=1e-2)
+    e_both = dict(case.last_errors)
+    print("vs float64 oracle: ours %s, hipBLASLt %s; ours vs hipBLASLt %s" % (e_ours, e_theirs, e_both))
+    # same order of magnitude: neither implementation is more than 4x further from the exact sum than the other
+    hi, lo = max(e_ours["max_abs_over_rms"], e_theirs["max_abs_over_rms"]), min(e_ours["max_abs_over_rms"], e_theirs["max_abs_over_rms"])
+    assert hi <= 4 * lo, "one implementation is much further from the exact result than the other"
+
+
+MX = dict(a_type=K.CUDA_R_4F_E2M1, b_type=K.CUDA_R_4F_E2M1, compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F,
+          transa=1, alpha=1.0, a_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_VEC32_UE8M0,
+          b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_VEC32_UE8M0)
+
+
+def test_mxfp4_scale_tensor_layout_of_hipblaslt(gpu_api):
+    """Which byte of the scale tensors does the reference's backend read for (row i, K block kb)?  Answered
+    by impulse responses at 256^3, batch 1, fp32 D: every FP4 element of the probed operand is 0 except K
+    block kb (all 1.0), the other operand is all 1.0 under unit scales, and byte p of the probed scale tensor
+    holds a code that encodes p (two runs: 64 + p % 128 and 64 + p // 128).  D(i, 0) = 32 * 2^(code - 127)
+    then names the byte used for (i, kb).  The tensor is four times larger than [256][8] so that a padded or
+    tiled layout would show.  Expected: p = i * (K/32) + kb for both operands -- one UE8M0 byte per 32
+    elements along K, rows of K/32 bytes, no swizzle (cuda_types/src/cublaslt.rs:3813-3818 read literally)."""
+    import ctypes as C
+    import torch
+    from oracle.hipblaslt_replay import Replay
+    n = 256
+    kb_count = n // 32
+    spec = dict(MX, m=n, n=n, k=n, d_type=K.CUDA_R_32F, c_type=K.CUDA_R_32F)
+    print("hipBLASLt MXFP4 scale layout probe", spec, flush=True)
+    rp = Replay(spec)
+    if rp.why:
+        pytest.skip("hipBLASLt cannot describe the problem: " + rp.why)
+    dev = torch.device("cuda:0")
+    total = 4 * n * kb_count
+    d_t = torch.zeros(n * n, dtype=torch.float32, device=dev)
+    ones = torch.full((n * n // 2,), 0x22, dtype=torch.uint8, device=dev)       # E2M1 code 2 = 1.0, twice per byte
+    flat = torch.full((total,), 127, dtype=torch.uint8, device=dev)              # 2^0
+    p = np.arange(total)
+    codes = [torch.from_numpy((64 + p % 128).astype(np.uint8)).to(dev), torch.from_numpy((64 + (p // 128) % 128).astype(np.uint8)).to(dev)]
+    have_algo = False
+    stream = torch.cuda.current_stream().cuda_stream
+    try:
+        for which in ("A", "B"):
+            used = np.zeros((n, kb_count), np.int64)
+            for kb in (0, 1, 5, 7):
+                data = torch.zeros(n, n // 2, dtype=torch.uint8, device=dev)
+                data[:, kb * 16:(kb + 1) * 16] = 0x22
+                digits = []
+                for enc in range(2):
+                    a_s, b_s = (codes[enc], flat) if which == "A" else (flat, codes[enc])
+                    assert rp.set_pointers(a_scale=a_s.data_ptr(), b_scale=b_s.data_ptr()), rp.why
+                    if not have_algo:
+                        if not rp.find_algo():
+                            pytest.skip("hipBLASLt offers no MXFP4 algorithm at batch 1: " + rp.why)
+                        have_algo = True
+                    a_d, b_d = (data, ones) if which == "A" else (ones, data)
+                    st = rp.run(C.c_float(1.0), a_d.data_ptr(), b_d.data_ptr(), C.c_float(0.0), None, d_t.data_ptr(), stream)
+                    torch.cuda.synchronize()
+                    assert st == 0, "hipblasLtMatmul status %d" % st
+                    d = d_t.cpu().numpy().astype(np.float64).reshape(n, n)    # [j][i]
+                    v = d[0, :] if which == "A" else d[:, 0]
+                    assert (v > 0).all()
+                    digits.append(np.rint(np.log2(v / 32.0)).astype(np.int64) + 127 - 64)
+                used[:, kb] = digits[0] + 128 * digits[1]
+                want = np.arange(n) * kb_count + kb
+                assert np.array_equal(used[:, kb], want), "operand %s, K block %d: hipBLASLt reads scale bytes %s..., the plain " \
+                    "[row][K/32] layout says %s..." % (which, kb, used[:6, kb], want[:6])
+    finally:
+        rp.close()
+
+
+@pytest.mark.parametrize("n,dt", [(256, K.CUDA_R_32F), (1024, K.CUDA_R_16BF), (8192, K.CUDA_R_16BF)])
+def test_mxfp4_batch1_within_tolerance_of_hipblaslt(gpu_api, n, dt):
+    """benchmark configuration 5's problem at batch 1 (the installed hipBLASLt takes block-scaled FP4 for one
+    batch only), A:T B:N: random E2M1 codes under scale bytes drawn independently per row and per K block
+    (a transposed, tiled or swizzled scale tensor could not agree by accident), ours against hipBLASLt
+    called the way the reference forwards it, element by element at the float bar of 1e-2."""
+    spec = dict(MX, m=n, n=n, k=n, d_type=dt, c_type=dt, mx_scale_range=(122, 133))
+    case, ours, theirs, why, kern = both(gpu_api, spec, 40 + n)
+    assert kern == K.ZLUDA_KERNEL_MFMA_MXF4
+    if theirs is None:
+        pytest.skip("hipBLASLt offers no algorithm here: " + why)
+    err = case.compare(ours, theirs, tol=1e-2)
+    print("max relative difference to hipBLASLt %.3e" % err)
+    if n <= 1024:   # and both against the float64 oracle
+        case.compare(theirs, case.run_oracle(), tol=1e-2)

@@ -301,13 +301,24 @@ bool unpack_algo(const cublasLtMatmulAlgo_t *algo, uint32_t *kernel, int32_t *va
   return *kernel >= ZLUDA_KERNEL_GENERIC && *kernel <= ZLUDA_KERNEL_MFMA_TR8;
 }
 
-// A/B forcing for measurements: ZLUDA_FORCE_KERNEL=<family>[:<variant>]
+// A/B forcing for measurements: ZLUDA_FORCE_KERNEL=<family>[:<variant>], read once per process (the
+// first call that needs it), never on the per-call path afterwards
 void env_force(uint32_t *kernel, int32_t *variant) {
-  const char *e = getenv("ZLUDA_FORCE_KERNEL");
-  if (!e || !*e) return;
-  *kernel = (uint32_t)atoi(e);
-  const char *c = strchr(e, ':');
-  *variant = c ? atoi(c + 1) : -1;
+  struct Forced { bool on; uint32_t kernel; int32_t variant; };
+  static const Forced f = [] {
+    Forced r{false, 0, -1};
+    const char *e = getenv("ZLUDA_FORCE_KERNEL");
+    if (e && *e) {
+      r.on = true;
+      r.kernel = (uint32_t)atoi(e);
+      const char *c = strchr(e, ':');
+      r.variant = c ? atoi(c + 1) : -1;
+    }
+    return r;
+  }();
+  if (!f.on) return;
+  *kernel = f.kernel;
+  *variant = f.variant;
 }
 
 } // namespace
@@ -566,6 +577,8 @@ cublasStatus_t cublasLtMatmul(cublasLtHandle_t lightHandle, cublasLtMatmulDesc_t
   p.alpha = alpha; p.beta = beta;
   p.A = A; p.B = B; p.C = C; p.D = D;
   p.workspace = workspace; p.workspace_size = workspaceSizeInBytes;
+  // split-K needs 16-byte aligned scratch: without it the problem is planned unsplit instead of refused
+  if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 15)) { p.workspace = nullptr; p.workspace_size = 0; }
 
   uint32_t kernel = ZLUDA_KERNEL_AUTO;
   int32_t variant = -1;

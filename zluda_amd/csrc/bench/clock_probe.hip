@@ -1,0 +1,35 @@
+// Measurement helper of bench.py, not part of libcublaslt.so: one wavefront that samples the shader
+// cycle counter (s_memtime) against the constant-rate real-time counter (s_memrealtime) while other
+// kernels run, so that the benchmark can state the shader clock the GPU actually held under the
+// measured load.  The wave sleeps between samples and leaves after `ticks` real-time ticks
+// (at most ~1 s worth, whatever the caller passes), so it always exits.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+__global__ void clock_probe_kernel(uint64_t *out, uint64_t ticks) {
+  if (threadIdx.x != 0) return;
+  if (ticks > 100000000ull) ticks = 100000000ull;
+  const uint64_t r0 = wall_clock64(), c0 = clock64();
+  uint64_t r1 = r0;
+  for (uint32_t spins = 0; spins < 40000000u && r1 - r0 < ticks; spins++) {
+    __builtin_amdgcn_s_sleep(64);
+    r1 = wall_clock64();
+  }
+  const uint64_t c1 = clock64();
+  out[0] = c1 - c0;  // shader cycles
+  out[1] = r1 - r0;  // real-time ticks
+}
+
+// out: two uint64 in device memory; ticks: length of the sample in real-time ticks; returns hipError_t
+extern "C" __attribute__((visibility("default"))) int zluda_bench_clock_probe(uint64_t *out, uint64_t ticks, void *stream) {
+  void *args[] = {&out, &ticks};
+  return (int)hipLaunchKernel((const void *)clock_probe_kernel, dim3(1), dim3(64), args, 0, (hipStream_t)stream);
+}
+
+// real-time counter rate in kHz (0 on failure)
+extern "C" __attribute__((visibility("default"))) int zluda_bench_wall_clock_khz(void) {
+  int dev = 0, khz = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 0;
+  if (hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev) != hipSuccess) return 0;
+  return khz;
+}

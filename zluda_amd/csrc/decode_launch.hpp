@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 
 #include "kernels/decode_stream.hpp"
+#include "launch_util.hpp"
 #include "planner.hpp"
 
 namespace zluda_amd {
@@ -29,18 +30,17 @@ template <int NW, int SPW, int KIND>
 inline uint32_t launch_decode_stream(const DecodeParams &prm, const zluda_gemm_plan &plan, int nb, hipStream_t s) {
   dim3 grid(plan.grid_x, plan.grid_y, 1), block(NW * 64);
   const bool fast = decode_packed_output(prm.g, prm.swapped != 0);
-  bool done = false;
+  uint32_t st = CUBLAS_STATUS_NOT_SUPPORTED;
   static_for_host<4>([&](auto nb_c) {
     constexpr int NB = decltype(nb_c)::value + 1;
     if constexpr (NB * SPW <= kDecodeStreamMaxFragments) {
       if (nb == NB) {
-        if (fast) hipLaunchKernelGGL((decode_stream_kernel<NW, SPW, NB, true, KIND>), grid, block, 0, s, prm);
-        else hipLaunchKernelGGL((decode_stream_kernel<NW, SPW, NB, false, KIND>), grid, block, 0, s, prm);
-        done = true;
+        st = fast ? launch_kernel(decode_stream_kernel<NW, SPW, NB, true, KIND>, grid, block, s, prm)
+                  : launch_kernel(decode_stream_kernel<NW, SPW, NB, false, KIND>, grid, block, s, prm);
       }
     }
   });
-  return done ? CUBLAS_STATUS_SUCCESS : CUBLAS_STATUS_NOT_SUPPORTED;
+  return st;
 }
 
 // plan.variant -> instantiation of the stream kernel for one element kind (the table restates

@@ -1,11 +1,12 @@
 // The extern "C" launch layer: lowers a problem, picks the template instantiation the plan names
-// and enqueues it on the caller's stream.  Only the HIP runtime is used (hipLaunchKernelGGL).
+// and enqueues it on the caller's stream.  Only the HIP runtime is used (hipLaunchKernel).
 #include <atomic>
 #include <hip/hip_runtime.h>
 
 #include <cstring>
 
 #include "decode_launch.hpp"
+#include "launch_util.hpp"
 #include "kernels/decode_w8a8.hpp"
 #include "kernels/gemm_generic.hpp"
 #include "kernels/splitk_reduce.hpp"
@@ -25,7 +26,8 @@ namespace {
 
 inline int f8_fmt(uint32_t t) { return t == CUDA_R_8F_E5M2 ? 1 : 0; }
 
-uint32_t launch_mfma(const Lowered &l, const zluda_gemm_plan &plan, const zluda_gemm_problem *p, hipStream_t s) {
+// `ws` / `ws_size`: the scratch that holds split-K partial tiles (the caller's workspace, or the library's own)
+uint32_t launch_mfma(const Lowered &l, const zluda_gemm_plan &plan, void *ws, uint64_t ws_size, hipStream_t s) {
   MfmaParams prm;
   prm.g = l.g;
   prm.swapped = plan.swapped;
@@ -40,8 +42,7 @@ uint32_t launch_mfma(const Lowered &l, const zluda_gemm_plan &plan, const zluda_
   if (plan.grid_z > 1) {
     // split-K: partial tiles go through the caller's workspace
     const uint64_t need = (uint64_t)plan.grid_z * l.g.batch * prm.tiles_p * v.bp * prm.tiles_q * v.bq * 4;
-    if (!p->workspace || (((uintptr_t)p->workspace) & 15) || p->workspace_size < need || plan.workspace != need)
-      return CUBLAS_STATUS_INVALID_VALUE;
+    if (!ws || (((uintptr_t)ws) & 15) || ws_size < need || plan.workspace != need) return CUBLAS_STATUS_INVALID_VALUE;
     const bool mx = plan.kernel == ZLUDA_KERNEL_MFMA_MXF4;
     const int kbytes = mx ? l.g.K / 2 : l.g.K;
     const int stages = (kbytes + v.bkb - 1) / v.bkb;
@@ -51,7 +52,7 @@ uint32_t launch_mfma(const Lowered &l, const zluda_gemm_plan &plan, const zluda_
       const int ch = 512 / v.bkb;
       prm.split_stages = (prm.split_stages + ch - 1) / ch * ch;
     }
-    prm.ws = p->workspace;
+    prm.ws = ws;
   }
   uint32_t st;
   switch (plan.kernel) {
@@ -73,12 +74,11 @@ uint32_t launch_mfma(const Lowered &l, const zluda_gemm_plan &plan, const zluda_
   rp.acc_is_int = plan.kernel == ZLUDA_KERNEL_MFMA_I8;
   rp.ws_np = prm.tiles_p * v.bp;
   rp.ws_nq = prm.tiles_q * v.bq;
-  rp.ws = (const int32_t *)p->workspace;
-  hipLaunchKernelGGL(splitk_reduce_kernel, dim3((np + 1023) / 1024, nq, l.g.batch), dim3(256), 0, s, rp);
-  return CUBLAS_STATUS_SUCCESS;
+  rp.ws = (const int32_t *)ws;
+  return launch_kernel(splitk_reduce_kernel, dim3((np + 1023) / 1024, nq, l.g.batch), dim3(256), s, rp);
 }
 
-uint32_t launch_tr(const Lowered &l, const zluda_gemm_plan &plan, const zluda_gemm_problem *p, hipStream_t s) {
+uint32_t launch_tr(const Lowered &l, const zluda_gemm_plan &plan, void *ws, uint64_t ws_size, hipStream_t s) {
   if (plan.variant >= (uint32_t)kNumTrVariants) return CUBLAS_STATUS_INVALID_VALUE;
   const TrVariant &v = kTrVariants[plan.variant];
   MfmaParams prm;
@@ -93,12 +93,11 @@ uint32_t launch_tr(const Lowered &l, const zluda_gemm_plan &plan, const zluda_ge
   if (plan.grid_z > 1) {
     // split-K: partial tiles go through the caller's workspace (64 K bytes per stage)
     const uint64_t need = (uint64_t)plan.grid_z * l.g.batch * prm.tiles_p * v.bp * prm.tiles_q * v.bq * 4;
-    if (!p->workspace || (((uintptr_t)p->workspace) & 15) || p->workspace_size < need || plan.workspace != need)
-      return CUBLAS_STATUS_INVALID_VALUE;
+    if (!ws || (((uintptr_t)ws) & 15) || ws_size < need || plan.workspace != need) return CUBLAS_STATUS_INVALID_VALUE;
     const int stages = (l.g.K + 63) / 64;
     prm.splits = (int32_t)plan.grid_z;
     prm.split_stages = (stages + prm.splits - 1) / prm.splits;
-    prm.ws = p->workspace;
+    prm.ws = ws;
   }
   // P is op(A) for a column-major D, op(B)^T otherwise
   const bool pkc = plan.swapped ? l.b_kcontig : l.a_kcontig, qkc = plan.swapped ? l.a_kcontig : l.b_kcontig;
@@ -117,21 +116,21 @@ uint32_t launch_tr(const Lowered &l, const zluda_gemm_plan &plan, const zluda_ge
   rp.acc_is_int = l.g.a_type == CUDA_R_8I;
   rp.ws_np = prm.tiles_p * v.bp;
   rp.ws_nq = prm.tiles_q * v.bq;
-  rp.ws = (const int32_t *)p->workspace;
-  hipLaunchKernelGGL(splitk_reduce_kernel, dim3((np + 1023) / 1024, nq, l.g.batch), dim3(256), 0, s, rp);
-  return CUBLAS_STATUS_SUCCESS;
+  rp.ws = (const int32_t *)ws;
+  return launch_kernel(splitk_reduce_kernel, dim3((np + 1023) / 1024, nq, l.g.batch), dim3(256), s, rp);
 }
 
 template <int NW, int STEPS>
-void launch_decode_variant(const DecodeParams &prm, const zluda_gemm_plan &plan, int nb, bool full, hipStream_t s) {
+uint32_t launch_decode_variant(const DecodeParams &prm, const zluda_gemm_plan &plan, int nb, bool full, hipStream_t s) {
   dim3 grid(plan.grid_x, plan.grid_y, 1), block(NW * 64);
   if (nb == 1) {
-    if (full) hipLaunchKernelGGL((decode_w8a8_kernel<NW, STEPS, 1, true>), grid, block, 0, s, prm);
-    else hipLaunchKernelGGL((decode_w8a8_kernel<NW, STEPS, 1, false>), grid, block, 0, s, prm);
+    return full ? launch_kernel(decode_w8a8_kernel<NW, STEPS, 1, true>, grid, block, s, prm)
+                : launch_kernel(decode_w8a8_kernel<NW, STEPS, 1, false>, grid, block, s, prm);
   } else if constexpr (STEPS <= 8) {  // two token blocks double the fragment registers
-    if (full) hipLaunchKernelGGL((decode_w8a8_kernel<NW, STEPS, 2, true>), grid, block, 0, s, prm);
-    else hipLaunchKernelGGL((decode_w8a8_kernel<NW, STEPS, 2, false>), grid, block, 0, s, prm);
+    return full ? launch_kernel(decode_w8a8_kernel<NW, STEPS, 2, true>, grid, block, s, prm)
+                : launch_kernel(decode_w8a8_kernel<NW, STEPS, 2, false>, grid, block, s, prm);
   }
+  return CUBLAS_STATUS_NOT_SUPPORTED;
 }
 
 uint32_t launch_decode(const Lowered &l, const zluda_gemm_plan &plan, hipStream_t s) {
@@ -160,13 +159,12 @@ uint32_t launch_decode(const Lowered &l, const zluda_gemm_plan &plan, hipStream_
   if (l.g.a_type != CUDA_R_8I) return CUBLAS_STATUS_NOT_SUPPORTED;  // the register-streaming kernel is int8 only
   if (nb > 2 || (nb == 2 && v.steps > 8)) return CUBLAS_STATUS_NOT_SUPPORTED;
   switch (plan.variant) {
-  case 0: launch_decode_variant<8, 8>(prm, plan, nb, full, s); break;
-  case 1: launch_decode_variant<8, 16>(prm, plan, nb, full, s); break;
-  case 2: launch_decode_variant<4, 16>(prm, plan, nb, full, s); break;
-  case 3: launch_decode_variant<4, 8>(prm, plan, nb, full, s); break;
+  case 0: return launch_decode_variant<8, 8>(prm, plan, nb, full, s);
+  case 1: return launch_decode_variant<8, 16>(prm, plan, nb, full, s);
+  case 2: return launch_decode_variant<4, 16>(prm, plan, nb, full, s);
+  case 3: return launch_decode_variant<4, 8>(prm, plan, nb, full, s);
   default: return CUBLAS_STATUS_INVALID_VALUE;
   }
-  return CUBLAS_STATUS_SUCCESS;
 }
 
 } // namespace
@@ -185,36 +183,36 @@ extern "C" uint32_t zluda_gemm_device_cu_count(void) {
   return (uint32_t)cus;
 }
 
-extern "C" uint32_t zluda_gemm_launch(const zluda_gemm_problem *p, const zluda_gemm_plan *plan,
-                                      void *stream) {
-  if (!p || !plan) return CUBLAS_STATUS_INVALID_VALUE;
+namespace zluda_amd {
+
+uint32_t launch_planned(const zluda_gemm_problem *p, const zluda_gemm_plan *plan, void *ws, uint64_t ws_size, void *stream) {
+  hipStream_t s = (hipStream_t)stream;
   Lowered l;
   uint32_t st = lower_problem(p, false, &l);
   if (st) return st;
   if (!family_supports(plan->kernel, l)) return CUBLAS_STATUS_INVALID_VALUE;
-  if (p->workspace_size < plan->workspace) return CUBLAS_STATUS_INVALID_VALUE;
+  if (ws_size < plan->workspace) return CUBLAS_STATUS_INVALID_VALUE;
   if (zluda_gemm_device_cu_count() == 0) return CUBLAS_STATUS_NOT_INITIALIZED;
-  hipStream_t s = (hipStream_t)stream;
   switch (plan->kernel) {
   case ZLUDA_KERNEL_GENERIC: {
     dim3 grid(plan->grid_x, plan->grid_y, plan->grid_z);
     const bool int_acc = l.g.a_type == CUDA_R_8I;
-    if (int_acc) hipLaunchKernelGGL(gemm_generic_kernel<true>, grid, dim3(256), 0, s, l.g);
-    else hipLaunchKernelGGL(gemm_generic_kernel<false>, grid, dim3(256), 0, s, l.g);
-    break;
+    return int_acc ? launch_kernel(gemm_generic_kernel<true>, grid, dim3(256), s, l.g)
+                   : launch_kernel(gemm_generic_kernel<false>, grid, dim3(256), s, l.g);
   }
-  case ZLUDA_KERNEL_MFMA_I8: case ZLUDA_KERNEL_MFMA_F8: case ZLUDA_KERNEL_MFMA_MXF4:
-    if ((st = launch_mfma(l, *plan, p, s))) return st;
-    break;
-  case ZLUDA_KERNEL_DECODE_W8A8:
-    if ((st = launch_decode(l, *plan, s))) return st;
-    break;
-  case ZLUDA_KERNEL_MFMA_TR8:
-    if ((st = launch_tr(l, *plan, p, s))) return st;
-    break;
+  case ZLUDA_KERNEL_MFMA_I8: case ZLUDA_KERNEL_MFMA_F8: case ZLUDA_KERNEL_MFMA_MXF4: return launch_mfma(l, *plan, ws, ws_size, s);
+  case ZLUDA_KERNEL_DECODE_W8A8: return launch_decode(l, *plan, s);
+  case ZLUDA_KERNEL_MFMA_TR8: return launch_tr(l, *plan, ws, ws_size, s);
   default: return CUBLAS_STATUS_NOT_SUPPORTED;
   }
-  return hipGetLastError() == hipSuccess ? CUBLAS_STATUS_SUCCESS : CUBLAS_STATUS_EXECUTION_FAILED;
+}
+
+} // namespace zluda_amd
+
+extern "C" uint32_t zluda_gemm_launch(const zluda_gemm_problem *p, const zluda_gemm_plan *plan,
+                                      void *stream) {
+  if (!p || !plan) return CUBLAS_STATUS_INVALID_VALUE;
+  return launch_planned(p, plan, p->workspace, p->workspace_size, stream);
 }
 
 // ---- cublasGemmEx-shaped entry points --------------------------------------------------------

@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 
 #include "kernels/gemm_mfma_pipe.hpp"
+#include "launch_util.hpp"
 #include "planner.hpp"
 
 namespace zluda_amd {
@@ -17,9 +18,8 @@ inline uint32_t launch_mfma_variant(const MfmaParams &prm, const zluda_gemm_plan
     static_assert(kMfmaVariants[V].bp == BP && kMfmaVariants[V].bq == BQ && kMfmaVariants[V].wp == WP &&   \
                   kMfmaVariants[V].wq == WQ && kMfmaVariants[V].bkb == BKB && kMfmaVariants[V].stages == NS, \
                   "variant table mismatch");                                                               \
-    hipLaunchKernelGGL((gemm_mfma_pipe_kernel<KIND, FQ, FP, BP, BQ, WP, WQ, BKB, NS>), grid,               \
-                       dim3(WP * WQ * 64), 0, s, prm);                                                     \
-    break;
+    return launch_kernel(gemm_mfma_pipe_kernel<KIND, FQ, FP, BP, BQ, WP, WQ, BKB, NS>, grid,               \
+                         dim3(WP * WQ * 64), s, prm);
   switch (plan.variant) {
     ZLUDA_MFMA_CASE(0, 256, 256, 2, 4, 128, 2)
     ZLUDA_MFMA_CASE(1, 256, 256, 2, 2, 128, 2)
@@ -32,7 +32,7 @@ inline uint32_t launch_mfma_variant(const MfmaParams &prm, const zluda_gemm_plan
   default: return CUBLAS_STATUS_INVALID_VALUE;
   }
 #undef ZLUDA_MFMA_CASE
-  return CUBLAS_STATUS_SUCCESS;
+  return CUBLAS_STATUS_INVALID_VALUE;
 }
 
 uint32_t launch_mfma_i8(const MfmaParams &prm, const zluda_gemm_plan &plan, hipStream_t s);

@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 
 #include "kernels/gemm_mfma_tr.hpp"
+#include "launch_util.hpp"
 #include "planner.hpp"
 
 namespace zluda_amd {
@@ -14,8 +15,7 @@ inline uint32_t launch_tr_variant(const MfmaParams &prm, const zluda_gemm_plan &
   const dim3 grid(plan.grid_x, plan.grid_y, plan.grid_z > 1 ? plan.grid_z : 1);  // z: split-K shares
 #define ZLUDA_TR_MODE(BP, BQ, WP, WQ, PK, QK)                                                                   \
   if (pkc == PK && qkc == QK) {                                                                                 \
-    hipLaunchKernelGGL((gemm_mfma_tr_kernel<KIND, FQ, FP, BP, BQ, WP, WQ, PK, QK>), grid, dim3(WP * WQ * 64), 0, s, prm); \
-    return CUBLAS_STATUS_SUCCESS;                                                                               \
+    return launch_kernel(gemm_mfma_tr_kernel<KIND, FQ, FP, BP, BQ, WP, WQ, PK, QK>, grid, dim3(WP * WQ * 64), s, prm); \
   }
 #define ZLUDA_TR_CASE(V, BP, BQ, WP, WQ)                                                                        \
   case V:                                                                                                       \

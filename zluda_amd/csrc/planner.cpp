@@ -402,7 +402,6 @@ static void fill_decode_plan(const Lowered &l, int variant, uint32_t cus, zluda_
   uint32_t grid;
   if (v.stream) grid = std::min(nrb, resident);  // contiguous, balanced row ranges
   else grid = nrb <= resident ? nrb : ceil_div(nrb, ceil_div(nrb, resident));
-  if (const char *e = getenv("ZLUDA_DECODE_GRID")) { int x = atoi(e); if (x > 0) grid = std::min<uint32_t>(x, nrb); }
   plan->variant = variant;
   plan->swapped = swapped;
   plan->grid_x = grid; plan->grid_y = g.batch; plan->grid_z = 1;

@@ -77,4 +77,8 @@ uint32_t lower_problem(const zluda_gemm_problem *p, bool dry, Lowered *out);
 // which kernel families can run the lowered problem
 bool family_supports(uint32_t kernel, const Lowered &l);
 
+// Lowers `p` with its real pointers and enqueues the kernel `plan` names on `stream` (a hipStream_t).
+// `ws` / `ws_size`: device scratch for split-K partial tiles, at least plan->workspace bytes.
+uint32_t launch_planned(const zluda_gemm_problem *p, const zluda_gemm_plan *plan, void *ws, uint64_t ws_size, void *stream);
+
 } // namespace zluda_amd

@@ -2,6 +2,7 @@
 // compiler calls, and the host entry point of include/zluda_ptx_mma.h.
 #include "../../include/zluda_ptx_mma.h"
 #include "kernels/ptx_mma.hpp"
+#include "launch_util.hpp"
 
 using namespace zluda_amd::ptx_mma;
 
@@ -53,16 +54,17 @@ extern "C" uint32_t zluda_ptx_mma_chain(uint32_t kind, const uint32_t *a, const 
   const u32x4 *av = (const u32x4 *)a, *cv = (const u32x4 *)c;
   const u32x2 *bv = (const u32x2 *)b;
   u32x4 *dv = (u32x4 *)d;
-#define ZLUDA_CHAIN(K)                                                                                       \
-  if (per_lane) hipLaunchKernelGGL((ptx_mma_chain_kernel<K, true>), grid, blk, 0, s, av, bv, cv, dv, iters); \
-  else hipLaunchKernelGGL((ptx_mma_chain_kernel<K, false>), grid, blk, 0, s, av, bv, cv, dv, iters)
+  uint32_t st;
+#define ZLUDA_CHAIN(K)                                                                                \
+  st = per_lane ? zluda_amd::launch_kernel(ptx_mma_chain_kernel<K, true>, grid, blk, s, av, bv, cv, dv, iters) \
+                : zluda_amd::launch_kernel(ptx_mma_chain_kernel<K, false>, grid, blk, s, av, bv, cv, dv, iters)
   switch (kind) {
   case ZLUDA_PTX_MMA_S8: ZLUDA_CHAIN(S8); break;
   case ZLUDA_PTX_MMA_F16: ZLUDA_CHAIN(F16); break;
   default: ZLUDA_CHAIN(BF16); break;
   }
 #undef ZLUDA_CHAIN
-  return hipGetLastError() == hipSuccess ? 0 : 13;
+  return st;  // 0 or 13 (CUBLAS_STATUS_EXECUTION_FAILED)
 }
 
 extern "C" uint32_t zluda_ptx_mma_run(uint32_t kind, const uint32_t *a, const uint32_t *b, const void *c, void *d,
@@ -75,9 +77,8 @@ extern "C" uint32_t zluda_ptx_mma_run(uint32_t kind, const uint32_t *a, const ui
   const u32x2 *bv = (const u32x2 *)b;
   u32x4 *dv = (u32x4 *)d;
   switch (kind) {
-  case ZLUDA_PTX_MMA_S8: hipLaunchKernelGGL(ptx_mma_run_kernel<S8>, grid, blk, 0, s, av, bv, cv, dv, masked_warps); break;
-  case ZLUDA_PTX_MMA_F16: hipLaunchKernelGGL(ptx_mma_run_kernel<F16>, grid, blk, 0, s, av, bv, cv, dv, masked_warps); break;
-  default: hipLaunchKernelGGL(ptx_mma_run_kernel<BF16>, grid, blk, 0, s, av, bv, cv, dv, masked_warps); break;
+  case ZLUDA_PTX_MMA_S8: return zluda_amd::launch_kernel(ptx_mma_run_kernel<S8>, grid, blk, s, av, bv, cv, dv, masked_warps);
+  case ZLUDA_PTX_MMA_F16: return zluda_amd::launch_kernel(ptx_mma_run_kernel<F16>, grid, blk, s, av, bv, cv, dv, masked_warps);
+  default: return zluda_amd::launch_kernel(ptx_mma_run_kernel<BF16>, grid, blk, s, av, bv, cv, dv, masked_warps);
   }
-  return hipGetLastError() == hipSuccess ? 0 : 13;
 }
