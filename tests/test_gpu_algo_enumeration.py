@@ -65,9 +65,11 @@ def run_enumerated(api, spec, seed, want_family, variants):
         vmax, wrote = C.c_int32(), C.c_size_t()
         assert api.cublasLtMatmulAlgoCapGetAttribute(C.byref(algo), ALGO_CAP_CUSTOM_OPTION_MAX, C.byref(vmax), 4, C.byref(wrote)) == 0
         for variant in variants:
-            assert variant < vmax.value
-            print("enumerated algorithm: family %d, CUSTOM_OPTION %d" % (want_family, variant), spec, flush=True)
-            v = C.c_uint32(variant)
+            # CUSTOM_OPTION: 0 leaves the tile variant to the planner, v + 1 selects variant v; the capability
+            # attribute reports the largest value
+            assert variant + 1 <= vmax.value
+            print("enumerated algorithm: family %d, CUSTOM_OPTION %d" % (want_family, variant + 1), spec, flush=True)
+            v = C.c_uint32(variant + 1)
             assert api.cublasLtMatmulAlgoConfigSetAttribute(C.byref(algo), ALGO_CONFIG_CUSTOM_OPTION, C.byref(v), 4) == 0
             res = abi.cublasLtMatmulHeuristicResult_t()
             assert api.cublasLtMatmulAlgoCheck(handle, desc, lay["a"], lay["b"], lay["c"], lay["d"], C.byref(algo), C.byref(res)) == 0

@@ -177,7 +177,6 @@ STREAM = {4: (8, 8), 5: (8, 16), 6: (8, 28), 7: (4, 8), 8: (8, 12), 9: (8, 24), 
           13: (4, 12), 14: (4, 20), 15: (8, 32)}
 
 
-@pytest.mark.parametrize("variant", sorted(STREAM))
 def check_small_grid(gpu_api, spec, seed, variant, grid_x, **case_kw):
     """through the inner launch layer with a grid of `grid_x` workgroups: several 16-row blocks per workgroup"""
     print("case", spec, "seed", seed, "variant", variant, "grid_x", grid_x, flush=True)
@@ -187,6 +186,7 @@ def check_small_grid(gpu_api, spec, seed, variant, grid_x, **case_kw):
     case.compare(got, case.run_oracle())
 
 
+@pytest.mark.parametrize("variant", sorted(STREAM))
 def test_decode_stream_variants(gpu_api, variant):
     """weights streamed through LDS: every K the variant table serves, ragged row ranges (row count
     neither a multiple of 16 nor of the grid), several 16-row blocks per workgroup, 1..32 tokens"""
