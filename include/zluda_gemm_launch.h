@@ -99,6 +99,20 @@ uint32_t zluda_gemm_plan_problem(const zluda_gemm_problem *p, uint32_t forced_ke
 uint32_t zluda_gemm_launch(const zluda_gemm_problem *p, const zluda_gemm_plan *plan,
                            void *stream);
 
+/* zluda_gemm_launch for callers that cannot hand over device scratch and cannot allocate any (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the
+ * reference.  Same arguments and results as zluda_gemm_launch, but split-K partial tiles go to an array of
+ * ZLUDA_GEMM_STATIC_SCRATCH_BYTES of device memory that is part of the library image (every device the
+ * library runs on holds its own copy until the process ends); `p->workspace` is ignored.  Plan with
+ * p->workspace_size = ZLUDA_GEMM_STATIC_SCRATCH_BYTES so that zluda_gemm_plan_problem sizes the split for it;
+ * a plan that needs more returns CUBLAS_STATUS_ALLOC_FAILED (3) and launches nothing.  The call allocates and
+ * frees nothing (the first call on a device looks up the array's address).  All calls on one device share that
+ * device's array: calls that may overlap on one device (two streams, two threads) race on it and must be
+ * serialised by the caller; nothing in it needs clearing between calls. */
+#define ZLUDA_GEMM_STATIC_SCRATCH_BYTES (32u << 20)
+uint32_t zluda_gemm_launch_noalloc(const zluda_gemm_problem *p, const zluda_gemm_plan *plan,
+                                   void *stream);
+
 /* cublasGemmEx / cublasGemmStridedBatchedEx on the same kernels: column-major operands, C is read
  * (when beta != 0) and overwritten, alpha and beta are host scalars of the type the compute type
  * implies (int32 for CUBLAS_COMPUTE_32I*, float for CUBLAS_COMPUTE_32F*).  This is what

@@ -76,6 +76,7 @@ LAUNCH_SIGNATURES = {
     "zluda_gemm_plan_problem": (_u32, [C.POINTER(abi.zluda_gemm_problem), _u32, C.c_int32, _u32,
                                        C.POINTER(abi.zluda_gemm_plan)]),
     "zluda_gemm_launch": (_u32, [C.POINTER(abi.zluda_gemm_problem), C.POINTER(abi.zluda_gemm_plan), _vp]),
+    "zluda_gemm_launch_noalloc": (_u32, [C.POINTER(abi.zluda_gemm_problem), C.POINTER(abi.zluda_gemm_plan), _vp]),
     "zluda_gemm_variant_count": (_u32, [_u32]),
     "zluda_gemm_ex": (_u32, [_u32, _u32, C.c_int32, C.c_int32, C.c_int32, _vp, _vp, _u32, C.c_int64, _vp, _u32, C.c_int64,
                              _vp, _vp, _u32, C.c_int64, _u32, _vp]),
