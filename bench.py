@@ -296,8 +296,9 @@ def time_hipblaslt(torch, spec, buf, alpha, zero, a_ptrs, copies, steps, warmup,
             if st:
                 raise RuntimeError("hipblasLtMatmul status %d" % st)
         wall, per_call, _ = time_calls(torch, theirs, steps, warmup)
+        clock = observed_clock_mhz(torch, theirs, max(steps // NBATCH, 4), per_call)
         rp.close()
-        return {"available": True, "ms_per_step": wall / steps * 1e3, "kernel_ms": per_call * 1e3,
+        return {"available": True, "ms_per_step": wall / steps * 1e3, "kernel_ms": per_call * 1e3, "clock_mhz_observed": clock,
                 "tops": ops / per_call / 1e12, "gbps": nbytes / per_call / 1e9}
     except Exception as e:  # the comparison point is optional; the product numbers are not
         return {"available": False, "why": "%s: %s" % (type(e).__name__, e)}

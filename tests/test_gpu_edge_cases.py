@@ -60,7 +60,7 @@ def test_decode_shapes_around_the_limits(gpu_api):
     dec = dict(I8, c_type=K.CUDA_R_16BF, d_type=K.CUDA_R_16BF, scale_type=K.CUDA_R_32F, alpha_range=(0.001, 0.01))
     assert run(gpu_api, dict(dec, m=64, n=1, k=4096), 340, int_dist="normal") == K.ZLUDA_KERNEL_DECODE_W8A8
     assert run(gpu_api, dict(dec, m=4099, n=32, k=4096), 341, int_dist="normal") == K.ZLUDA_KERNEL_DECODE_W8A8   # rows % 4 != 0
-    assert run(gpu_api, dict(dec, m=2048, n=3, k=11008), 342, int_dist="normal") == K.ZLUDA_KERNEL_DECODE_W8A8  # K outside the stream table
+    assert run(gpu_api, dict(dec, m=2048, n=3, k=11008), 342, int_dist="normal") == K.ZLUDA_KERNEL_DECODE_W8A8  # K under the 12288 cover
     assert run(gpu_api, dict(dec, m=512, n=16, k=4096, batch=3), 343, int_dist="normal") == K.ZLUDA_KERNEL_DECODE_W8A8
     # beyond 48 tokens the planner prefers small MFMA tiles (the decode family itself runs up to 64)
     assert run(gpu_api, dict(dec, m=2048, n=32, k=4096), 344, int_dist="normal") == K.ZLUDA_KERNEL_DECODE_W8A8
@@ -73,17 +73,28 @@ def test_decode_shapes_around_the_limits(gpu_api):
         run(gpu_api, dict(dec, c_type=K.CUDA_R_16F, d_type=K.CUDA_R_16F, m=2048, n=8, k=4096, ldd=ld, ldc=ld), 345, int_dist="normal")
 
 
-def test_decode_shapes_outside_the_stream_table_on_mfma_tiles(gpu_api):
-    """K values the LDS-streaming decode kernel has no instantiation for: MFMA tiles when they fill at
-    least half of the CUs (with the K split through the workspace if there is one), with the full decode
-    epilogue: alpha vector, per-token scale, bias"""
+def test_decode_k_between_the_stream_instantiations(gpu_api):
+    """K values between the covers of the LDS-streaming decode kernel's instantiations run on the next larger one
+    with the lanes past the end of K reading zero (whole 256-byte units past it are never multiplied), with the full
+    decode epilogue: alpha vector, per-token scale, bias.  K outside every cover, or more activation fragments than
+    the registers hold: MFMA tiles when they fill at least half of the CUs (with the K split through the workspace
+    if there is one), the register-streaming decode kernel otherwise."""
     dec = dict(I8, c_type=K.CUDA_R_16BF, d_type=K.CUDA_R_16BF, scale_type=K.CUDA_R_32F,
                pointer_mode=K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO,
                b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F, epilogue=K.CUBLASLT_EPILOGUE_BIAS,
                bias_type=K.CUDA_R_32F, alpha_range=(0.001, 0.01), scale_range=(0.005, 0.02), bias_std=0.02)
-    assert run(gpu_api, dict(dec, m=8192, n=16, k=2624), 350, int_dist="normal") == K.ZLUDA_KERNEL_MFMA_I8
-    assert run(gpu_api, dict(dec, m=2048, n=16, k=2624), 351, int_dist="normal") == K.ZLUDA_KERNEL_DECODE_W8A8
-    spec = dict(dec, m=4096, n=32, k=11008)
+    DEC = K.ZLUDA_KERNEL_DECODE_W8A8
+    assert run(gpu_api, dict(dec, m=8192, n=16, k=2624), 350, int_dist="normal") == DEC      # 3072 cover: tail inside a unit
+    assert run(gpu_api, dict(dec, m=2048, n=16, k=2560), 351, int_dist="normal") == DEC      # 3072 cover: two whole units missing
+    assert run(gpu_api, dict(dec, m=1000, n=5, k=3584, lda=3584 + 64), 353, int_dist="normal") == DEC    # 4096 cover
+    assert run(gpu_api, dict(dec, m=5120, n=16, k=13824), 354, int_dist="normal") == DEC     # 14336 cover
+    assert run(gpu_api, dict(dec, m=2048, n=29, k=3584), 355, int_dist="normal") == DEC      # two token blocks
+    f8 = dict(a_type=K.CUDA_R_8F_E4M3, b_type=K.CUDA_R_8F_E4M3, c_type=K.CUDA_R_16BF, d_type=K.CUDA_R_16BF,
+              compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F, transa=1, epilogue=K.CUBLASLT_EPILOGUE_BIAS,
+              bias_type=K.CUDA_R_16BF, with_scalar_scales=True, scale_range=(0.05, 0.06))
+    assert run(gpu_api, dict(f8, m=4096, n=16, k=11008), 356) == DEC                           # fp8, 12288 cover
+    assert run(gpu_api, dict(f8, m=1000, n=7, k=2736), 357) == DEC                             # fp8, tail inside a 128-byte step
+    spec = dict(dec, m=4096, n=32, k=11008)      # two token blocks x 24 steps: more fragments than the registers hold
     print("edge case", spec, "with a 64 MiB workspace", flush=True)
     case = Case(spec, 352, int_dist="normal")
     ref = case.run_oracle()

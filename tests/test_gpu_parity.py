@@ -224,9 +224,10 @@ def test_decode_fp8_planner_choice_and_orientation(gpu_api):
     # row-major activations [tokens][K] x weights^T: tokens are rows of D
     check(gpu_api, dict(F8, transa=0, transb=1, order_a=1, order_b=1, order_c=1, order_d=1, m=16, n=2048, k=4096,
                         epilogue=K.CUBLASLT_EPILOGUE_BIAS, bias_type=K.CUDA_R_16BF), 471, expect_kernel=DEC)
-    # what the family does not take: mixed formats, K outside the table -> the MFMA tiles
+    # what the family does not take: mixed formats, K under no instantiation's cover -> the MFMA tiles
     check(gpu_api, dict(F8, a_type=K.CUDA_R_8F_E5M2, m=2048, n=16, k=4096), 472, expect_kernel=K.ZLUDA_KERNEL_MFMA_F8)
-    check(gpu_api, dict(F8, m=2048, n=16, k=2624 + 64), 473, expect_kernel=K.ZLUDA_KERNEL_MFMA_F8)
+    check(gpu_api, dict(F8, m=2048, n=16, k=1536), 473, expect_kernel=K.ZLUDA_KERNEL_MFMA_F8)
+    check(gpu_api, dict(F8, m=2048, n=16, k=2624 + 64), 474, expect_kernel=DEC)     # under the 3072 cover
 
 
 def test_decode_config3_shape_takes_the_stream_kernel(gpu_api):

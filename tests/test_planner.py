@@ -160,27 +160,35 @@ def test_split_k_needs_workspace_and_few_tiles(api):
     assert plan_ws(dict(MX, m=1024, n=256, k=8192, transa=1), 1 << 30)[1].grid_z == 1
 
 
-def test_decode_shapes_outside_the_stream_table(api):
-    """the LDS-streaming decode kernel serves a table of K values; elsewhere the planner takes MFMA tiles
-    (split along K through the workspace) when they occupy at least half of the CUs, and the
-    register-streaming decode variant otherwise"""
+def test_decode_k_between_the_stream_instantiations(api):
+    """an instantiation of the LDS-streaming decode kernel covers nw * steps * 64 bytes of K and takes any K (a
+    multiple of 16) down to three quarters of that; K outside every cover goes to MFMA tiles (split along K through
+    the workspace) when they occupy at least half of the CUs, and to the register-streaming decode variant otherwise"""
     dec = dict(I8, transa=1, d_type=K.CUDA_R_16BF, scale_type=K.CUDA_R_32F,
                pointer_mode=K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO,
                b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F,
                epilogue=K.CUBLASLT_EPILOGUE_BIAS, bias_type=K.CUDA_R_32F)
-    st, p = plan(api, dict(dec, m=14336, n=16, k=4096))                       # in the table
+    st, p = plan(api, dict(dec, m=14336, n=16, k=4096))                       # exactly one instantiation's cover
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.variant == 4
-    st, p = plan(api, dict(dec, m=5120, n=16, k=13824), workspace=64 << 20)   # 80 tiles x 6 K shares
+    for ws in (0, 64 << 20):
+        st, p = plan(api, dict(dec, m=5120, n=16, k=13824), workspace=ws)     # under the 14336 cover
+        assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.variant == 6 and p.workspace == 0
+    st, p = plan(api, dict(dec, m=18944, n=32, k=3584))                       # under the 4096 cover, two token blocks
+    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.variant == 4
+    st, p = plan(api, dict(dec, m=2048, n=16, k=2560), workspace=64 << 20)    # under the 3072 cover
+    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.variant == 13
+    st, p = plan(api, dict(dec, m=4096, n=16, k=11008))                       # under the 12288 cover
+    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.variant == 9
+    # no cover: K = 1536 lies between 1024 and three quarters of 2048, K = 20480 beyond the largest
+    st, p = plan(api, dict(dec, m=8192, n=16, k=20480), workspace=64 << 20)
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_I8 and p.grid_z > 1 and p.grid_x * p.grid_z >= 128
-    st, p = plan(api, dict(dec, m=5120, n=16, k=13824))                       # no workspace: 80 tiles only
+    st, p = plan(api, dict(dec, m=4096, n=16, k=20480))                       # 64 tiles only, no workspace
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.variant == 0
-    st, p = plan(api, dict(dec, m=18944, n=32, k=3584))                       # 296 tiles without any split
+    st, p = plan(api, dict(dec, m=16384, n=16, k=1536))                       # 256 tiles without any split
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_I8 and p.grid_z == 1
-    st, p = plan(api, dict(dec, m=2048, n=16, k=2560), workspace=64 << 20)    # 32 tiles, short K
-    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8
 
 
-def test_fp8_decode_takes_the_streaming_kernel_for_table_k_only(api):
+def test_fp8_decode_takes_the_streaming_kernel_under_a_cover_only(api):
     f8 = dict(F8, transa=1)
     st, p = plan(api, dict(f8, m=14336, n=16, k=4096))
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.variant == 4 and p.grid_x == 256
@@ -190,11 +198,13 @@ def test_fp8_decode_takes_the_streaming_kernel_for_table_k_only(api):
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_F8
     st, p = plan(api, dict(f8, m=14336, n=33, k=8192))                      # 3 token blocks x 16 steps: too many fragments
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_F8
-    st, p = plan(api, dict(f8, m=4096, n=16, k=11008))                      # K outside the table: no fp8 fallback variant
+    st, p = plan(api, dict(f8, m=4096, n=16, k=11008))                      # under the 12288 cover
+    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.variant == 9
+    st, p = plan(api, dict(f8, m=4096, n=16, k=20480))                      # no cover: no fp8 fallback variant
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_F8
     st, p = plan(api, dict(f8, m=4096, n=16, k=4096, b_type=K.CUDA_R_8F_E5M2))
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_F8
-    assert plan(api, dict(f8, m=4096, n=16, k=11008), forced=K.ZLUDA_KERNEL_DECODE_W8A8)[0] == K.CUBLAS_STATUS_NOT_SUPPORTED
+    assert plan(api, dict(f8, m=4096, n=16, k=20480), forced=K.ZLUDA_KERNEL_DECODE_W8A8)[0] == K.CUBLAS_STATUS_NOT_SUPPORTED
     assert plan(api, dict(f8, m=4096, n=16, k=4096), forced=K.ZLUDA_KERNEL_DECODE_W8A8, variant=0)[0] == K.CUBLAS_STATUS_NOT_SUPPORTED
 
 

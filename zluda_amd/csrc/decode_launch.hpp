@@ -35,8 +35,13 @@ inline uint32_t launch_decode_stream(const DecodeParams &prm, const zluda_gemm_p
     constexpr int NB = decltype(nb_c)::value + 1;
     if constexpr (NB * SPW <= kDecodeStreamMaxFragments) {
       if (nb == NB) {
-        st = fast ? launch_kernel(decode_stream_kernel<NW, SPW, NB, true, KIND>, grid, block, s, prm)
-                  : launch_kernel(decode_stream_kernel<NW, SPW, NB, false, KIND>, grid, block, s, prm);
+        const bool tail = prm.g.K < NW * SPW * 64;
+        if (tail)
+          st = fast ? launch_kernel(decode_stream_kernel<NW, SPW, NB, true, KIND, true>, grid, block, s, prm)
+                    : launch_kernel(decode_stream_kernel<NW, SPW, NB, false, KIND, true>, grid, block, s, prm);
+        else
+          st = fast ? launch_kernel(decode_stream_kernel<NW, SPW, NB, true, KIND>, grid, block, s, prm)
+                    : launch_kernel(decode_stream_kernel<NW, SPW, NB, false, KIND>, grid, block, s, prm);
       }
     }
   });

@@ -15,6 +15,9 @@
 // bytes, occupies no VGPRs while in flight, and the ds_read_b128 that follows is free to use any
 // layout.
 //
+// K: an instantiation covers NW * SPW * 64 bytes of K; any shorter K (a multiple of 16) runs on it with the
+// lanes past the end reading zero, so the host takes the smallest instantiation that covers K.
+//
 // Work split: workgroup w owns the contiguous rows [w*R/G, (w+1)*R/G) (balanced to one row across
 // the grid, whatever R is) and walks them in blocks of 16.  K is split across the NW waves of the
 // workgroup: wave v streams bytes [v*SPW*64, (v+1)*SPW*64) of every row and keeps the matching
@@ -76,7 +79,9 @@ __device__ __forceinline__ void lds_values_ready(v4i (&x)[N]) {
 // epilogue without C, 16-bit D contiguous along the weight rows, 8-byte aligned, row count a multiple
 // of 4); the element-wise epilogue with all its type dispatch is then not even compiled in, which
 // keeps the code the reducing wave runs between two blocks short.
-template <int NW, int SPW, int NB, bool FAST, int KIND = KIND_I8>
+// TAIL: K is shorter than the NW * SPW * 64 bytes the instantiation covers (the checks cost ~3 % on an exact K,
+// so that case has its own instantiation without them).
+template <int NW, int SPW, int NB, bool FAST, int KIND = KIND_I8, bool TAIL = false>
 __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(DecodeParams prm) {
   static_assert(KIND == KIND_I8 || KIND == KIND_F8, "int8 or fp8 (e4m3 x e4m3) operands");
   using acc_t = typename std::conditional<KIND == KIND_I8, v4i, v4f>::type;
@@ -124,17 +129,41 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(DecodeParams prm
     const int rho = 4 * i + g4;
     dma_off[i] = ((l16 ^ rho) << 4) + kwave;
   }
+  // K may be shorter than the NW * SPW * 64 bytes the instantiation covers: the lanes of a unit that lie past
+  // the end of K go out of range (bit 31) and read as zero; a unit that lies past it entirely (a uniform
+  // condition: its first byte is kwave + q * SEG) is fetched like the rows past r1 and never multiplied.
+  const int K = g.K;
   auto issue_unit = [&](int blk, int q, int slot) {
     const int rb = r0 + blk * 16;
     v4i *dst = &ring[wave][slot][0];
+    const bool inside = !TAIL || kwave + q * SEG < K;  // uniform
 #pragma unroll
     for (int i = 0; i < NDMA; i++) {
       const int row = rb + 4 * i + g4;
-      lds_dma16(rsW, dst + i * 64, row < r1 ? row * ldw + q * SEG + dma_off[i] : 0, 0);
+      const int koff = q * SEG + dma_off[i];
+      lds_dma16(rsW, dst + i * 64, (inside && row < r1) ? ((!TAIL || koff < K) ? row * ldw + koff : (int)0x80000000) : 0, 0);
     }
   };
 
-  // prologue: the first NSLOT units, before anything else touches memory
+  // activation fragments of this wave's K slice: lane -> token l16 (+16 per block); int8: 16 bytes
+  // at K = kwave + s*64 + g4*16; fp8: the halves (s & 1) of 32 bytes at kwave + (s/2)*128 + g4*32.
+  // Issued BEFORE the first weight units: the wait for them below then leaves those units in flight
+  // (memory operations are counted in issue order).  The other way round the wave would sit out the
+  // arrival of everything it has issued and restart the weight stream from empty: 1.3 us of 14.3 on a
+  // 14336 x 4096 matrix.
+  v4i xf[NB][SPW];
+#pragma unroll
+  for (int nb = 0; nb < NB; nb++) {
+    const uint8_t *xr = Xg + (int64_t)min(nb * 16 + l16, T - 1) * ldx + kwave + g4 * (KIND == KIND_I8 ? 16 : 32);
+#pragma unroll
+    for (int s = 0; s < SPW; s++) {
+      const int ko = KIND == KIND_I8 ? s * 64 : (s >> 1) * 128 + (s & 1) * 16;
+      // (past the end of K: zero, and no load: the bytes behind a row are the next token's, or nobody's)
+      xf[nb][s] = (!TAIL || kwave + g4 * (KIND == KIND_I8 ? 16 : 32) + ko < K) ? *(const v4i *)(xr + ko) : v4i{0, 0, 0, 0};
+    }
+  }
+
+  // prologue: the first NSLOT units
   {
     int blk = 0, q = 0;
 #pragma unroll
@@ -144,21 +173,9 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(DecodeParams prm
     }
   }
 
-  // activation fragments of this wave's K slice: lane -> token l16 (+16 per block); int8: 16 bytes
-  // at K = kwave + s*64 + g4*16; fp8: the halves (s & 1) of 32 bytes at kwave + (s/2)*128 + g4*32
-  v4i xf[NB][SPW];
-#pragma unroll
-  for (int nb = 0; nb < NB; nb++) {
-    const uint8_t *xr = Xg + (int64_t)min(nb * 16 + l16, T - 1) * ldx + kwave + g4 * (KIND == KIND_I8 ? 16 : 32);
-#pragma unroll
-    for (int s = 0; s < SPW; s++)
-      xf[nb][s] = *(const v4i *)(xr + (KIND == KIND_I8 ? s * 64 : (s >> 1) * 128 + (s & 1) * 16));
-  }
-
-  // Pin the wait for the activation loads here, in straight-line code.  Left to its own devices the
-  // compiler waits at their first use inside the loop, where all it can prove is vmcnt(0): that
-  // drains the stream per block.  Here the wait costs nothing: the first units were issued at the
-  // same moment and are needed next.
+  // Pin the wait for the activation loads here, in straight-line code, where the compiler can count the
+  // NSLOT * NDMA younger operations.  Left to its own devices it waits at their first use inside the loop,
+  // where all it can prove is vmcnt(0): that drains the stream per block.
 #pragma unroll
   for (int nb = 0; nb < NB; nb++)
 #pragma unroll
@@ -256,6 +273,7 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(DecodeParams prm
       issue_unit(fblk, fq, slot);
       if (++fq == Q) { fq = 0; fblk++; }
       slot ^= 1;
+      if (TAIL && kwave + q * SEG >= K) continue;  // (uniform) a unit past the end of K holds no data
       if constexpr (KIND == KIND_I8) {
 #pragma unroll
         for (int s = 0; s < 4; s++)

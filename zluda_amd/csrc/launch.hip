@@ -147,9 +147,9 @@ uint32_t launch_decode(const Lowered &l, const zluda_gemm_plan &plan, hipStream_
   const bool full = l.g.K == v.nw * v.steps * 64;
   const int nb = (T + 15) / 16;
   if (v.stream) {
-    // the kernel addresses W through one 2 GiB buffer window and assumes K == nw * steps * 64
+    // the kernel addresses W through one 2 GiB buffer window and covers K <= nw * steps * 64
     const int64_t rows = plan.swapped ? l.g.N : l.g.M, ldw = plan.swapped ? l.g.b_sj : l.g.a_si;
-    if (!full || rows * ldw >= 0x7fffffffll || plan.grid_x > (uint32_t)((rows + 15) / 16))
+    if (l.g.K > v.nw * v.steps * 64 || (l.g.K & 15) || rows * ldw >= 0x7fffffffll || plan.grid_x > (uint32_t)((rows + 15) / 16))
       return CUBLAS_STATUS_NOT_SUPPORTED;
     const int64_t quads = (rows + 3) / 4;  // the kernel splits the rows in quads of 4
     prm.rows_base = (int32_t)(quads / plan.grid_x);

@@ -213,7 +213,11 @@ static bool decode_variant_ok(const Lowered &l, int variant) {
   if (!v.stream) return g.a_type == CUDA_R_8I && (nb == 1 || (nb == 2 && v.steps <= 8));
   const bool swapped = g.M < g.N;
   const int64_t rows = swapped ? g.N : g.M, ldw = swapped ? g.b_sj : g.a_si;
-  return g.K == v.nw * v.steps * 64 && rows * ldw < 0x7fffffffll && nb * v.steps <= kDecodeStreamMaxFragments;
+  // a stream instantiation covers nw * steps * 64 bytes of K and takes any K up to that (lanes past the end read
+  // zero); more than a quarter of idle lanes is left to the smaller instantiations or to the MFMA tiles
+  const int cover = v.nw * v.steps * 64;
+  return g.K <= cover && g.K * 4 > cover * 3 && (g.K & 15) == 0 && rows * ldw < 0x7fffffffll &&
+         nb * v.steps <= kDecodeStreamMaxFragments;
 }
 
 static bool any_decode_variant_ok(const Lowered &l) {
@@ -412,8 +416,13 @@ static void fill_decode_plan(const Lowered &l, int variant, uint32_t cus, zluda_
 
 static int pick_decode_variant(const Lowered &l) {
   const int K = l.g.K;
+  // the stream instantiation with the least cover that takes K
+  int best = -1;
   for (int v = 0; v < kNumDecodeVariants; v++)
-    if (kDecodeVariants[v].stream && decode_variant_ok(l, v)) return v;
+    if (kDecodeVariants[v].stream && decode_variant_ok(l, v) &&
+        (best < 0 || kDecodeVariants[v].nw * kDecodeVariants[v].steps < kDecodeVariants[best].nw * kDecodeVariants[best].steps))
+      best = v;
+  if (best >= 0) return best;
   for (int v = 0; v < kNumDecodeVariants; v++)
     if (!kDecodeVariants[v].stream && K == kDecodeVariants[v].nw * kDecodeVariants[v].steps * 64 && decode_variant_ok(l, v))
       return v;

@@ -33,7 +33,8 @@ constexpr int kNumTrVariants = sizeof(kTrVariants) / sizeof(kTrVariants[0]);
 
 // decode configurations (index = plan.variant for ZLUDA_KERNEL_DECODE_W8A8).
 // stream == 0: weights loaded straight into registers, any K (grid-stride over 16-row blocks).
-// stream == 1: weights streamed through LDS in whole cache lines; K must equal nw * steps * 64.
+// stream == 1: weights streamed through LDS in whole cache lines; covers K <= nw * steps * 64 (the planner
+// gives an instantiation the K values down to three quarters of its cover).
 struct DecodeVariant { int nw, steps, stream; };
 constexpr DecodeVariant kDecodeVariants[] = {
     {8, 8, 0},   // 0: 8 waves x 512 B of K per pass
