@@ -302,12 +302,16 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
       constexpr bool last = s + 1 == KS;
       if constexpr (!last) {
         load_frags(so, std::integral_constant<int, (s + 1 < KS ? s + 1 : 1)>{}, nxt);
+        // MX: the next stage's scales, early (their chunk landed at least one barrier ago: the last parts
+        // of a chunk are issued CH - NSTAGE stages into the chunk before it), so that the last sub-step is
+        // left with the fragment reads and the refill
+        if constexpr (s == 0) load_scales(kt + 1, sc_nxt);
       } else {
         wait_vmcnt_barrier<(NSTAGE - 2) * NLOAD>();
         // reads first: the compiler cannot prove that the DMA (an LDS write) and these reads hit
         // different slots, so whatever comes second in the source stays second in the schedule
         load_frags(so_next, std::integral_constant<int, 0>{}, nxt);
-        load_scales(kt + 1, sc_nxt);
+        if constexpr (KS == 1) load_scales(kt + 1, sc_nxt);
         issue_scales_for(kt, so);
         issue_stage(kt + NSTAGE, so);
       }
@@ -317,7 +321,7 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
       // first half of them and the LDS DMA of the refill behind the second half.  Without the
       // pattern the scheduler either sinks every ds_read to its first use (the wave then stalls on
       // it) or keeps the loads in one block in front of the MFMAs (the matrix pipe idles meanwhile).
-      constexpr int NM = TP * TQ, NDS = (TP + TQ) * (KIND == KIND_F8 ? 2 : 1) + (KIND == KIND_MXF4 && last ? TP + TQ : 0);
+      constexpr int NM = TP * TQ, NDS = (TP + TQ) * (KIND == KIND_F8 ? 2 : 1) + (KIND == KIND_MXF4 && (KS == 1 ? last : s == 0) ? TP + TQ : 0);
       constexpr int NVM = last ? NLOAD : 0, H1 = NM / 2 > 0 ? NM / 2 : 1, H2 = NM - H1 > 0 ? NM - H1 : 1;
       static_for<NM>([&](auto i_c) {
         constexpr int i = decltype(i_c)::value;
