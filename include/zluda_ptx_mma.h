@@ -36,8 +36,9 @@ extern "C" {
  * memory): thread i reads a[4i..4i+3], b[2i..2i+1], c[4i..4i+3] and writes d[4i..4i+3], all device
  * pointers to 32-bit words (c and d hold int32 for S8, float otherwise).  `threads` lanes in blocks of
  * `block` threads (a multiple of 32, at most 1024; `threads` a multiple of `block`), enqueued on
- * `stream` (a hipStream_t).  `masked_warps` != 0 lets only the even warps of each block execute the
- * instruction (the odd ones copy c to d), which exercises wavefronts that are only half there.
+ * `stream` (a hipStream_t).  `masked_warps` 1 lets only the even warps of each block execute the
+ * instruction, 2 only the odd ones (the others copy c to d), which exercises wavefronts of which only
+ * the low or only the high half is there.
  * Returns 0, or 7 (invalid value) / 13 (launch failed) with cublasStatus_t numbering. */
 uint32_t zluda_ptx_mma_run(uint32_t kind, const uint32_t *a, const uint32_t *b, const void *c, void *d,
                            uint32_t threads, uint32_t block, uint32_t masked_warps, void *stream);

@@ -45,8 +45,8 @@ def unpack(regs, kind):
     return (h.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
 
 
-def mma_sync(kind, a, b, c):
-    """a: uint32 [W, 32, 4], b: uint32 [W, 32, 2], c: int32 / float32 [W, 32, 4] -> d like c"""
+def _matrices(kind, a, b, c):
+    """fragments -> (A [W,16,K], B [W,K,8], C [W,16,8]) in float64"""
     a, b = np.asarray(a, np.uint32), np.asarray(b, np.uint32)
     W = a.shape[0]
     E = 4 if kind == S8 else 2
@@ -61,13 +61,34 @@ def mma_sync(kind, a, b, c):
     for r in range(2):
         for e in range(E):
             B[:, t * E + e + 4 * E * r, g] = bv[:, :, r, e]
-    D = A @ B + C   # exact in float64 for int8 and for the value ranges the float tests use
-    d = np.zeros((W, 32, 4))
+    return A, B, C
+
+
+def _fragment(D):
+    """D [W,16,8] -> the accumulator fragment [W,32,4]"""
+    lane = np.arange(32); g, t = lane >> 2, lane & 3
+    d = np.zeros((D.shape[0], 32, 4))
     for r in range(4):
         d[:, :, r] = D[:, g + 8 * (r >> 1), 2 * t + (r & 1)]
+    return d
+
+
+def mma_sync(kind, a, b, c):
+    """a: uint32 [W, 32, 4], b: uint32 [W, 32, 2], c: int32 / float32 [W, 32, 4] -> d like c"""
+    A, B, C = _matrices(kind, a, b, c)
+    d = _fragment(A @ B + C)   # exact in float64 for int8 and for the value ranges the exact float tests use
     if kind == S8:
         return (d.astype(np.int64) & 0xFFFFFFFF).astype(np.uint32).view(np.int32)
     return d.astype(np.float32)
+
+
+def mma_sync_exact(kind, a, b, c):
+    """(d, mag) in float64, unrounded: d = A * B + C and mag = |A| * |B| + |C|, the sum of the magnitudes
+    of the terms of each element.  Any fp32 accumulation of the K + 1 terms, in whatever order and with
+    or without fused multiply-adds, stays within (K + 1) * 2^-24 * mag of d; the PTX ISA leaves the order
+    open, so this is the bound a result for arbitrary float inputs is held to."""
+    A, B, C = _matrices(kind, a, b, c)
+    return _fragment(A @ B + C), _fragment(np.abs(A) @ np.abs(B) + np.abs(C))
 
 
 def program_inputs(name, threads=64):

@@ -36,7 +36,10 @@
  *   - which GELU hipBLASLt applies: the tanh form is restated here.  No CPU-side fixture pins it;
  *     on a GPU box tests/test_gpu_vs_hipblaslt.py tells the tanh and erf forms apart against
  *     hipBLASLt itself (it applies the tanh form)
- *   - the memory layout of the UE8M0 scale tensors (restated as plain [row][K/32] bytes)
+ *   - the batch stride of the UE8M0 scale tensors for batch counts above 1 (restated as batches back to
+ *     back, rows * K/32 bytes each): hipBLASLt takes MXFP4 at batch 1 only.  The layout inside a batch,
+ *     plain [row][K/32] bytes for both operands, is pinned on a GPU box against hipBLASLt itself by the
+ *     impulse responses of tests/test_gpu_vs_hipblaslt.py
  */
 #include <math.h>
 #include <stdint.h>

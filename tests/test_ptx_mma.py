@@ -78,17 +78,44 @@ def random_fragments(kind, warps, seed):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("kind", [ref.S8, ref.F16, ref.BF16])
-@pytest.mark.parametrize("block,masked", [(64, 0), (256, 0), (32, 0), (128, 1)])
+@pytest.mark.parametrize("block,masked", [(64, 0), (256, 0), (32, 0), (128, 1), (128, 2)])
 def test_random_fragments_against_the_oracle(lib, kind, block, masked):
     print("kind", kind, "block", block, "masked", masked, flush=True)
     warps = 64
     a, b, c = random_fragments(kind, warps, 7000 + kind)
     want = ref.mma_sync(kind, a, b, c)
-    if masked:   # odd warps of each block skip the instruction: d = c
-        odd = (np.arange(warps) % (block // 32)) % 2 == 1
-        want[odd] = c[odd]
+    if masked:   # masked 1: the odd warps of each block skip the instruction (d = c), masked 2: the even ones
+        skip = (np.arange(warps) % (block // 32)) % 2 == (1 if masked == 1 else 0)
+        want[skip] = c[skip]
     got = run_gpu(lib, kind, a, b, c, block, masked)
     np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", [ref.F16, ref.BF16])
+@pytest.mark.parametrize("block,masked", [(64, 0), (32, 0), (128, 2)])
+def test_arbitrary_floats_within_the_accumulation_bound(lib, kind, block, masked):
+    """Non-integer f16 / bf16 fragments: the sum is no longer exact in fp32, the PTX ISA does not fix the
+    order of accumulation, and the MFMA form (products summed by the matrix unit, c added last) and the
+    per-lane form (c first, then a chain of fused multiply-adds) round differently.  Tolerance: the bound
+    every fp32 accumulation order meets, (K + 1) * 2^-24 * (|A| * |B| + |C|) per element, K = 16."""
+    print("kind", kind, "block", block, "masked", masked, flush=True)
+    warps = 64
+    rng = np.random.default_rng(7200 + kind)
+    bits = ref.bf16_bits_rne if kind == ref.BF16 else ref.f16_bits
+    pack = lambda x: (bits(x[..., 1]) << 16 | bits(x[..., 0])).astype(np.uint32)
+    a = pack(rng.normal(0, 1, (warps, 32, 4, 2)).astype(np.float32))
+    b = pack(rng.normal(0, 1, (warps, 32, 2, 2)).astype(np.float32))
+    c = rng.normal(0, 4, (warps, 32, 4)).astype(np.float32)
+    want, mag = ref.mma_sync_exact(kind, a, b, c)
+    if masked:
+        skip = (np.arange(warps) % (block // 32)) % 2 == 0
+        want[skip] = c[skip]
+    got = run_gpu(lib, kind, a, b, c, block, masked).astype(np.float64)
+    err = np.abs(got - want)
+    print("largest error / bound: %.3f" % float((err / (17 * 2.0**-24 * mag)).max()), flush=True)
+    assert (err <= 17 * 2.0**-24 * mag).all()
+    assert err.max() > 0   # the inputs do exercise rounding: an all-exact result means the case is too easy
 
 
 @pytest.mark.gpu

@@ -23,7 +23,7 @@ __global__ void ptx_mma_run_kernel(const u32x4 *a, const u32x2 *b, const u32x4 *
   const u32x4 av = a[i], cv = c[i];
   const u32x2 bv = b[i];
   u32x4 dv = cv;
-  if (!masked_warps || ((threadIdx.x >> 5) & 1) == 0) {
+  if (!masked_warps || ((threadIdx.x >> 5) & 1) == ((masked_warps - 1) & 1)) {   // 1: the even warps run, 2: the odd ones
     if constexpr (KIND == S8) dv = __zluda_ptx_impl_mma_sync_aligned_m16n8k32_row_col_s32_s8_s8_s32(av, bv, cv);
     else if constexpr (KIND == F16)
       dv = __builtin_bit_cast(u32x4, __zluda_ptx_impl_mma_sync_aligned_m16n8k16_row_col_f32_f16_f16_f32(av, bv, __builtin_bit_cast(f32x4, cv)));
