@@ -42,7 +42,8 @@ typedef struct zluda_matmul_desc {
   int32_t pointer_mode;  /* cublasLtPointerMode_t */
   uint32_t transa, transb;
   uint32_t epilogue;     /* cublasLtEpilogue_t */
-  const void *bias;      /* device, length = rows of D */
+  const void *bias;      /* device, length = rows of D; with the BGRADA / BGRADB epilogues it is written instead:
+                          * the sums over K of op(A)'s rows (rows of D values) / of op(B)'s columns (columns of D) */
   int32_t bias_type;     /* cudaDataType or -1 (= default for the D type) */
   int64_t bias_batch_stride;
   int64_t alpha_vector_batch_stride;

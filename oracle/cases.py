@@ -188,6 +188,18 @@ class Case:
             nb = m + s.get("bias_batch_stride", 0) * (batch - 1)
             bvals = (rng.standard_normal(nb) * s.get("bias_std", 0.5)).astype(np.float32)
             self.bias = _encode(bvals, bt)
+        # bias-gradient epilogues: the bias buffer is an output (M sums for BGRADA, N for BGRADB); it starts as a
+        # canary, the oracle's result lands in self.bgrad_ref and the GPU's in self.bgrad_got
+        self.bgrad = {abi.CUBLASLT_EPILOGUE_BGRADA: 1, abi.CUBLASLT_EPILOGUE_BGRADB: 2}.get(epi, 0)
+        if self.bgrad:
+            bt = s.get("bias_type", -1)
+            if bt < 0:
+                bt = abi.CUDA_R_32F if s["d_type"] in (abi.CUDA_R_8I, abi.CUDA_R_32I, abi.CUDA_R_8F_E4M3,
+                                                       abi.CUDA_R_8F_E5M2) else s["d_type"]
+            self.bgrad_type = bt
+            nb = (m if self.bgrad == 1 else n) + s.get("bias_batch_stride", 0) * (batch - 1)
+            self.bias = np.frombuffer(bytes([0xCD]) * (nb * (4 if bt == abi.CUDA_R_32F else 2)),
+                                      dtype=np.float32 if bt == abi.CUDA_R_32F else np.uint16).copy()
 
     def new_d(self):
         """output storage pre-filled with a canary pattern"""
@@ -227,8 +239,11 @@ class Case:
     def run_oracle(self):
         d = self.new_d()
         hp = lambda x: x.ctypes.data if x is not None else None
+        bias = self.bias
+        if self.bgrad:   # the oracle writes it: keep the canary for the GPU run
+            bias = self.bgrad_ref = self.bias.copy()
         ptrs = {"A": hp(self.A), "B": hp(self.B), "C": hp(self.Cm), "D": hp(d), "alpha": hp(self.alpha),
-                "beta": hp(self.beta), "bias": hp(self.bias), "a_scale": hp(self.a_scale),
+                "beta": hp(self.beta), "bias": hp(bias), "a_scale": hp(self.a_scale),
                 "b_scale": hp(self.b_scale), "c_scale": hp(self.c_scale), "d_scale": hp(self.d_scale)}
         p = self.problem(ptrs)
         st = oracle.gemm(p)
@@ -306,6 +321,8 @@ class Case:
             st = call.run(alpha, ptr["A"], ptr["B"], beta, ptr["C"], ptr["D"],
                           ws.data_ptr() if ws is not None else None, workspace_bytes, stream)
             torch.cuda.synchronize()
+            if self.bgrad:
+                self.bgrad_got = keep[3][:self.bias.nbytes].cpu().numpy().view(self.bias.dtype).copy()
             return st, self.download(dt), call.kernel, call.variant
         finally:
             call.close()
@@ -351,11 +368,27 @@ class Case:
             torch.cuda.synchronize()
             if st:
                 return None, "hipblasLtMatmul status %d" % st
+            if self.bgrad:
+                self.bgrad_theirs = keep[3][:self.bias.nbytes].cpu().numpy().view(self.bias.dtype).copy()
             return self.download(dt), ""
         finally:
             rp.close()
 
     # ---- comparison -------------------------------------------------------------------------------
+    def compare_bgrad(self, got, ref, exact=False):
+        """bias gradients as stored (bias data type): bit-exact when `exact` (integer operands: the sums are
+        exact in int32 and convert the same way), else within 1e-2 of max(|ref|, 1e-2 * rms(ref)) -- the fp32
+        summation order of the GPU kernel is its own and the output may be a 16-bit float"""
+        g, r = decode_storage(got, self.bgrad_type), decode_storage(ref, self.bgrad_type)
+        assert g.shape == r.shape
+        if exact:
+            np.testing.assert_array_equal(got, ref)
+            return
+        floor = 1e-2 * float(np.sqrt(np.mean(r * r))) + 1e-30
+        err = np.abs(g - r) / np.maximum(np.abs(r), floor)
+        print("bias gradient: max relative error %.3g" % float(err.max()), flush=True)
+        assert err.max() <= 1e-2
+
     def logical_index(self):
         """flat storage indices of D(i, j, batch) as an int64 array [batch, m, n]"""
         s = self.spec

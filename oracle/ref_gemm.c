@@ -358,8 +358,12 @@ uint32_t oracle_gemm(const zluda_gemm_problem *p) {
                        epi == CUBLASLT_EPILOGUE_GELU_BIAS;
   const int relu = epi == CUBLASLT_EPILOGUE_RELU || epi == CUBLASLT_EPILOGUE_RELU_BIAS;
   const int gelu = epi == CUBLASLT_EPILOGUE_GELU || epi == CUBLASLT_EPILOGUE_GELU_BIAS;
-  if (!(epi == CUBLASLT_EPILOGUE_DEFAULT || has_bias || relu || gelu))
+  /* BGRADA / BGRADB (cuda_types/src/cublaslt.rs:4636-4654): D as with DEFAULT; the bias buffer receives the
+   * sums over K of op(A)'s rows (M values) / of op(B)'s columns (N values), in the bias data type */
+  const int bgrad = epi == CUBLASLT_EPILOGUE_BGRADA ? 1 : epi == CUBLASLT_EPILOGUE_BGRADB ? 2 : 0;
+  if (!(epi == CUBLASLT_EPILOGUE_DEFAULT || has_bias || relu || gelu || bgrad))
     return CUBLAS_STATUS_NOT_SUPPORTED;
+  if (bgrad && (a_blk || b_blk || op->a_scale || op->b_scale || !op->bias)) return CUBLAS_STATUS_NOT_SUPPORTED;
   uint32_t bias_type = op->bias_type >= 0 ? (uint32_t)op->bias_type
                        : (p->d.type == CUDA_R_8I || p->d.type == CUDA_R_32I ||
                           p->d.type == CUDA_R_8F_E4M3 || p->d.type == CUDA_R_8F_E5M2)
@@ -410,6 +414,16 @@ uint32_t oracle_gemm(const zluda_gemm_problem *p) {
           fb[j * K + k] = v;
         }
       }
+
+    if (bgrad) {
+      const int64_t R = bgrad == 1 ? M : N;
+      for (int64_t r = 0; r < R; r++) {
+        double s = 0.0;
+        for (int64_t k = 0; k < K; k++)
+          s += int_path ? (double)(bgrad == 1 ? ia : ib)[r * K + k] : (double)(bgrad == 1 ? fa : fb)[r * K + k];
+        store_from_float((void *)op->bias, bias_type, r + op->bias_batch_stride * bt, (float)s);
+      }
+    }
 
 #pragma omp parallel for schedule(dynamic, 1)
     for (int64_t j = 0; j < N; j++) {

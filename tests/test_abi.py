@@ -95,6 +95,9 @@ def test_matmul_desc_attributes(api):
     assert api.desc_set(d, D.CUBLASLT_MATMUL_DESC_TRANSA, C.c_int32, D.CUBLAS_OP_T) == 0
     assert api.desc_set(d, D.CUBLASLT_MATMUL_DESC_TRANSB, C.c_int32, 7) == IV
     assert api.desc_set(d, D.CUBLASLT_MATMUL_DESC_EPILOGUE, C.c_uint32, D.CUBLASLT_EPILOGUE_GELU_BIAS) == 0
+    assert api.desc_set(d, D.CUBLASLT_MATMUL_DESC_EPILOGUE, C.c_uint32, D.CUBLASLT_EPILOGUE_BGRADA) == 0
+    assert api.desc_set(d, D.CUBLASLT_MATMUL_DESC_EPILOGUE, C.c_uint32, D.CUBLASLT_EPILOGUE_BGRADB) == 0
+    assert api.desc_set(d, D.CUBLASLT_MATMUL_DESC_EPILOGUE, C.c_uint32, D.CUBLASLT_EPILOGUE_GELU_BIAS) == 0
     assert api.desc_set(d, D.CUBLASLT_MATMUL_DESC_EPILOGUE, C.c_uint32, D.CUBLASLT_EPILOGUE_DGELU) == NS
     assert api.desc_set(d, D.CUBLASLT_MATMUL_DESC_BIAS_DATA_TYPE, C.c_int32, D.CUDA_R_16BF) == 0
     assert api.desc_set(d, D.CUBLASLT_MATMUL_DESC_BIAS_POINTER, C.c_void_p, 0x1000) == 0

@@ -246,3 +246,30 @@ def test_oracle_rejects_bad_shapes():
     p = case.problem({"A": hp(case.A), "B": hp(case.B), "D": hp(d), "alpha": hp(case.alpha), "beta": hp(case.beta)})
     p.b.rows = 5
     assert oracle.gemm(p) == abi.CUBLAS_STATUS_INVALID_VALUE
+
+
+@pytest.mark.parametrize("which", ["a", "b"])
+@pytest.mark.parametrize("typ", [abi.CUDA_R_8I, abi.CUDA_R_16BF, abi.CUDA_R_8F_E4M3])
+@pytest.mark.parametrize("ta,tb,oa,ob", [(1, 0, 0, 0), (0, 1, 0, 0), (0, 0, 1, 1)])
+def test_bias_gradient_epilogues_against_numpy(which, typ, ta, tb, oa, ob):
+    """BGRADA / BGRADB: the bias buffer receives the sums over K of op(A)'s rows / op(B)'s columns (numpy sums of
+    the matrices read straight from the layout definition), per batch at the bias batch stride, in the bias data
+    type; D is what the DEFAULT epilogue gives."""
+    epi = abi.CUBLASLT_EPILOGUE_BGRADA if which == "a" else abi.CUBLASLT_EPILOGUE_BGRADB
+    base = dict(a_type=typ, b_type=typ, d_type=abi.CUDA_R_32F, compute_type=abi.CUBLAS_COMPUTE_32F, scale_type=abi.CUDA_R_32F,
+                alpha=1.0, m=19, n=11, k=48, transa=ta, transb=tb, order_a=oa, order_b=ob, batch=2, bias_batch_stride=24)
+    if typ == abi.CUDA_R_8I:
+        base.update(compute_type=abi.CUBLAS_COMPUTE_32I)
+    case = Case(dict(base, epilogue=epi, bias_type=abi.CUDA_R_32F), 77)
+    d = case.run_oracle()
+    plain = Case(dict(base), 77)
+    np.testing.assert_array_equal(d, plain.run_oracle())
+    rows = 19 if which == "a" else 11
+    for b in range(2):
+        A, B = op_matrices(case, b)
+        src = decode_storage(A, typ) if which == "a" else decode_storage(B, typ).T
+        want = src.sum(axis=1)
+        got = case.bgrad_ref[24 * b:24 * b + rows].astype(np.float64)
+        assert np.max(np.abs(got - want)) <= 1e-6 * max(1.0, np.max(np.abs(want)))
+    # what lies between the batches' vectors stays untouched
+    assert (case.bgrad_ref[rows:24].view(np.uint32) == 0xCDCDCDCD).all()

@@ -220,3 +220,23 @@ def test_transposing_kernel_splits_k_when_tiles_are_few(api):
     assert st == 0 and p.grid_z == 1                                           # enough tiles already
     st, p = plan(api, dict(I8, transa=0, transb=1, m=256, n=256, k=256), workspace=1 << 30)
     assert st == 0 and p.grid_z == 1                                           # short K
+
+
+def test_bias_gradient_epilogues_are_planned_like_the_plain_problem(api):
+    """BGRADA / BGRADB leave the matmul itself as with DEFAULT (the reduction is a second kernel behind it), so
+    the plan is the plain problem's; block-scaled and per-tensor-scaled operands are refused (a sum of stored
+    codes is not the gradient of anything then)."""
+    bf = dict(a_type=K.CUDA_R_16BF, b_type=K.CUDA_R_16BF, d_type=K.CUDA_R_16BF, compute_type=K.CUBLAS_COMPUTE_32F,
+              scale_type=K.CUDA_R_32F, m=512, n=384, k=1024, transa=1)
+    for spec in (bf, dict(F8, m=4096, n=4096, k=4096, transa=1), dict(I8, m=4096, n=4096, k=4096, transa=1, scale_type=K.CUDA_R_32F)):
+        st0, p0 = plan(api, spec)
+        for epi in (K.CUBLASLT_EPILOGUE_BGRADA, K.CUBLASLT_EPILOGUE_BGRADB):
+            st, p = plan(api, dict(spec, epilogue=epi))
+            assert st == 0 and st0 == 0
+            assert (p.kernel, p.variant, p.grid_x, p.grid_y, p.grid_z) == (p0.kernel, p0.variant, p0.grid_x, p0.grid_y, p0.grid_z)
+    st, _ = plan(api, dict(MX, m=512, n=512, k=512, transa=1, epilogue=K.CUBLASLT_EPILOGUE_BGRADA))
+    assert st == K.CUBLAS_STATUS_NOT_SUPPORTED
+    st, _ = plan(api, dict(I8, m=512, n=512, k=512, transa=1, epilogue=K.CUBLASLT_EPILOGUE_BGRADB))   # int32 scale type: DEFAULT only
+    assert st == K.CUBLAS_STATUS_NOT_SUPPORTED
+    st, _ = plan(api, dict(F8, m=512, n=512, k=512, transa=1, epilogue=K.CUBLASLT_EPILOGUE_DGELU))
+    assert st == K.CUBLAS_STATUS_NOT_SUPPORTED

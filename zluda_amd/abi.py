@@ -107,6 +107,7 @@ CUBLASLT_EPILOGUE_RELU_AUX = 130
 CUBLASLT_EPILOGUE_GELU_AUX = 160
 CUBLASLT_EPILOGUE_DGELU = 192
 CUBLASLT_EPILOGUE_BGRADA = 256
+CUBLASLT_EPILOGUE_BGRADB = 512
 
 # cublasLtMatmulPreferenceAttributes_t -- cuda_types/src/cublaslt.rs:4725-4820
 CUBLASLT_MATMUL_PREF_SEARCH_MODE = 0

@@ -103,6 +103,7 @@ bool epilogue_supported(uint32_t e) {
   switch (e) {
   case CUBLASLT_EPILOGUE_DEFAULT: case CUBLASLT_EPILOGUE_RELU: case CUBLASLT_EPILOGUE_BIAS:
   case CUBLASLT_EPILOGUE_RELU_BIAS: case CUBLASLT_EPILOGUE_GELU: case CUBLASLT_EPILOGUE_GELU_BIAS:
+  case CUBLASLT_EPILOGUE_BGRADA: case CUBLASLT_EPILOGUE_BGRADB:
     return true;
   default: return false;
   }

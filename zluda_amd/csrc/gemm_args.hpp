@@ -35,6 +35,10 @@ struct GemmArgs {
   uint32_t bias_type;
   int64_t bias_sb;
   int32_t act;                             // Activation
+  // bias-gradient epilogues: the K sums of op(A)'s rows (bgrad_src 1, M values) or of op(B)'s columns
+  // (2, N values) go to `bgrad` in bias_type, batches bias_sb apart; `bias` is NULL then
+  void *bgrad;
+  int32_t bgrad_src;
 };
 
 } // namespace zluda_amd

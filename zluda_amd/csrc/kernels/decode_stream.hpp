@@ -186,9 +186,9 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(DecodeParams prm
   // contiguous along the weight rows and suitably aligned, and no C is read, they leave as one
   // 8-byte store instead of four scattered 2-byte ones.
   const int64_t d_sr = prm.swapped ? g.d_sj : g.d_si, d_st = prm.swapped ? g.d_si : g.d_sj;
-  const bool packed = FAST || !g.int_scale && (g.d_type == CUDA_R_16BF || g.d_type == CUDA_R_16F) && d_sr == 1 &&
-                      g.beta_mode == SCALAR_VALUE && g.beta_val.f == 0.0f && ((uintptr_t)g.D & 7) == 0 &&
-                      (d_st & 3) == 0 && (g.d_sb & 3) == 0;
+  const bool packed = FAST || (!g.int_scale && (g.d_type == CUDA_R_16BF || g.d_type == CUDA_R_16F) && d_sr == 1 &&
+                               g.beta_mode == SCALAR_VALUE && g.beta_val.f == 0.0f && ((uintptr_t)g.D & 7) == 0 &&
+                               (d_st & 3) == 0 && (g.d_sb & 3) == 0);
   uint16_t *const Dp = (uint16_t *)g.D + g.d_sb * bt;
   const uint32_t red_base0 = lds_addr(&red[0][0][0][0]);
   const uint32_t ring_base = lds_addr(&ring[wave][0][l16 * 16]);  // this lane's row in slot 0

@@ -7,6 +7,7 @@
 
 #include "decode_launch.hpp"
 #include "launch_util.hpp"
+#include "kernels/bgrad_reduce.hpp"
 #include "kernels/decode_w8a8.hpp"
 #include "kernels/gemm_generic.hpp"
 #include "kernels/splitk_reduce.hpp"
@@ -185,6 +186,25 @@ extern "C" uint32_t zluda_gemm_device_cu_count(void) {
 
 namespace zluda_amd {
 
+// BGRADA / BGRADB: the K sums of one operand into the bias buffer, behind the matmul on its stream
+static uint32_t launch_bgrad(const GemmArgs &g, hipStream_t s) {
+  BgradParams b;
+  const bool of_a = g.bgrad_src == 1;
+  b.src = of_a ? g.A : g.B;
+  b.type = of_a ? g.a_type : g.b_type;
+  b.rows = of_a ? g.M : g.N;
+  b.K = g.K;
+  b.batch = g.batch;
+  b.s_row = of_a ? g.a_si : g.b_sj;
+  b.s_k = of_a ? g.a_sk : g.b_sk;
+  b.s_b = of_a ? g.a_sb : g.b_sb;
+  b.out = g.bgrad;
+  b.out_type = g.bias_type;
+  b.out_sb = g.bias_sb;
+  if (b.s_k <= b.s_row) return launch_kernel(bgrad_rows_kernel, dim3(b.rows, b.batch), dim3(256), s, b);
+  return launch_kernel(bgrad_cols_kernel, dim3((b.rows + 255) / 256, b.batch), dim3(256), s, b);
+}
+
 uint32_t launch_planned(const zluda_gemm_problem *p, const zluda_gemm_plan *plan, void *ws, uint64_t ws_size, void *stream) {
   hipStream_t s = (hipStream_t)stream;
   Lowered l;
@@ -197,14 +217,17 @@ uint32_t launch_planned(const zluda_gemm_problem *p, const zluda_gemm_plan *plan
   case ZLUDA_KERNEL_GENERIC: {
     dim3 grid(plan->grid_x, plan->grid_y, plan->grid_z);
     const bool int_acc = l.g.a_type == CUDA_R_8I;
-    return int_acc ? launch_kernel(gemm_generic_kernel<true>, grid, dim3(256), s, l.g)
-                   : launch_kernel(gemm_generic_kernel<false>, grid, dim3(256), s, l.g);
+    st = int_acc ? launch_kernel(gemm_generic_kernel<true>, grid, dim3(256), s, l.g)
+                 : launch_kernel(gemm_generic_kernel<false>, grid, dim3(256), s, l.g);
+    break;
   }
-  case ZLUDA_KERNEL_MFMA_I8: case ZLUDA_KERNEL_MFMA_F8: case ZLUDA_KERNEL_MFMA_MXF4: return launch_mfma(l, *plan, ws, ws_size, s);
-  case ZLUDA_KERNEL_DECODE_W8A8: return launch_decode(l, *plan, s);
-  case ZLUDA_KERNEL_MFMA_TR8: return launch_tr(l, *plan, ws, ws_size, s);
+  case ZLUDA_KERNEL_MFMA_I8: case ZLUDA_KERNEL_MFMA_F8: case ZLUDA_KERNEL_MFMA_MXF4: st = launch_mfma(l, *plan, ws, ws_size, s); break;
+  case ZLUDA_KERNEL_DECODE_W8A8: st = launch_decode(l, *plan, s); break;
+  case ZLUDA_KERNEL_MFMA_TR8: st = launch_tr(l, *plan, ws, ws_size, s); break;
   default: return CUBLAS_STATUS_NOT_SUPPORTED;
   }
+  if (st == CUBLAS_STATUS_SUCCESS && l.g.bgrad_src) st = launch_bgrad(l.g, s);
+  return st;
 }
 
 } // namespace zluda_amd

@@ -172,11 +172,21 @@ uint32_t lower_problem(const zluda_gemm_problem *p, bool dry, Lowered *out) {
   case CUBLASLT_EPILOGUE_BIAS: g.act = ACT_NONE; has_bias = true; break;
   case CUBLASLT_EPILOGUE_RELU_BIAS: g.act = ACT_RELU; has_bias = true; break;
   case CUBLASLT_EPILOGUE_GELU_BIAS: g.act = ACT_GELU; has_bias = true; break;
+  // the bias buffer is an output here: sums over K of op(A)'s rows / op(B)'s columns, D as with DEFAULT
+  case CUBLASLT_EPILOGUE_BGRADA: g.act = ACT_NONE; g.bgrad_src = 1; break;
+  case CUBLASLT_EPILOGUE_BGRADB: g.act = ACT_NONE; g.bgrad_src = 2; break;
   default: return CUBLAS_STATUS_NOT_SUPPORTED;
   }
-  if (has_bias) {
+  if (g.bgrad_src) {
+    // sums of the stored elements: defined here for unscaled operands only
+    if (a.type == CUDA_R_4F_E2M1 || b.type == CUDA_R_4F_E2M1 || g.a_scale_mode || g.b_scale_mode)
+      return CUBLAS_STATUS_NOT_SUPPORTED;
     if (!dry && !op.bias) return CUBLAS_STATUS_INVALID_VALUE;
-    g.bias = op.bias;
+    g.bgrad = const_cast<void *>(op.bias);
+  }
+  if (has_bias || g.bgrad_src) {
+    if (has_bias && !dry && !op.bias) return CUBLAS_STATUS_INVALID_VALUE;
+    if (has_bias) g.bias = op.bias;
     g.bias_sb = op.bias_batch_stride;
     if (op.bias_type >= 0) g.bias_type = (uint32_t)op.bias_type;
     else  // cuda_types/src/cublaslt.rs:4395-4403
