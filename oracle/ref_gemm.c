@@ -371,6 +371,7 @@ uint32_t oracle_gemm(const zluda_gemm_problem *p) {
                            : p->d.type;
 
   const int batch = p->d.batch_count > 0 ? p->d.batch_count : 1;
+  if (bgrad && batch > 1 && op->bias_batch_stride == 0) return CUBLAS_STATUS_NOT_SUPPORTED; /* aliased outputs */
   const zluda_matrix_layout *cl = p->C ? &p->c : &p->d;
 
   /* dense K-contiguous copies of op(A) [M][K] and op(B) [N][K] for one batch */

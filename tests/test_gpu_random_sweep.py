@@ -1,126 +1,158 @@
-"""Seeded random sweep over what cublasLtMatmul admits for the quantized types: shapes, transposes,
-orders, leading dimensions, batches, epilogues, scale modes, pointer modes, C reads, with and without a
-workspace -- every case through the planner's own choice and against the CPU oracle (int8 -> int32
-bit-exact, floats within 1e-2).  The point is the seams between the kernel families (LDS-DMA MFMA tiles,
-transposing tiles, streaming decode, split-K, generic) rather than any one of them."""
+"""Seeded random sweep on the GPU: problems drawn over every family of the library (int8 with integer and with
+float scaling, fp8 in its three operand mixes, MXFP4, 16/32-bit floats), transposes, orders, padded and
+unaligned leading dimensions, batches, pointer modes, scale modes, every epilogue incl. the bias gradients,
+decode-like and split-K-like shapes, with and without a workspace -- each through the planner's choice and
+then through up to three other tile variants of the family it chose, all against the CPU oracle.  The draw
+is deterministic (fixed seed), so a failure names a case that can be rerun."""
+import json
+
 import numpy as np
 import pytest
 
 from oracle.cases import Case
-from zluda_amd import abi
+from zluda_amd import abi as K, cublaslt
 
 pytestmark = pytest.mark.gpu
-K = abi
+BIG = True   # include shapes of several tiles of the large variants
+NVAR = {K.ZLUDA_KERNEL_MFMA_I8: 8, K.ZLUDA_KERNEL_MFMA_F8: 8, K.ZLUDA_KERNEL_MFMA_MXF4: 8, K.ZLUDA_KERNEL_MFMA_TR8: 3,
+        K.ZLUDA_KERNEL_DECODE_W8A8: 16}
+RNG = None
 
 
-def random_spec(rng):
-    kind = rng.choice(["i8", "i8f", "f8", "mx"], p=[0.3, 0.25, 0.3, 0.15])
-    shape = rng.choice(["small", "skinny", "tiles"])
-    if shape == "small":
-        m, n = int(rng.integers(1, 200)), int(rng.integers(1, 200))
-    elif shape == "skinny":
-        m, n = int(rng.choice([256, 512, 1000, 2048])), int(rng.integers(1, 70))
-        if rng.random() < 0.3:
-            m, n = n, m
-    else:
-        m, n = int(rng.choice([128, 192, 256, 320, 512])), int(rng.choice([64, 128, 203, 256, 384]))
-    kq = int(rng.choice([16, 64, 256]))                      # K granularity of the case
-    k = kq * int(rng.integers(1, max(2, 2048 // kq)))
-    if shape == "skinny" and rng.random() < 0.5:
-        k = int(rng.choice([1024, 2048, 3072, 4096, 2624, 1104]))
-    spec = dict(m=m, n=n, k=k)
-    if kind == "mx":
+EPIS = [K.CUBLASLT_EPILOGUE_DEFAULT, K.CUBLASLT_EPILOGUE_RELU, K.CUBLASLT_EPILOGUE_GELU, K.CUBLASLT_EPILOGUE_BIAS,
+        K.CUBLASLT_EPILOGUE_RELU_BIAS, K.CUBLASLT_EPILOGUE_GELU_BIAS, K.CUBLASLT_EPILOGUE_BGRADA, K.CUBLASLT_EPILOGUE_BGRADB]
+
+
+def pick(xs):
+    return xs[int(RNG.integers(len(xs)))]
+
+
+def dims():
+    r = RNG.random()
+    if r < 0.2:   # decode-like
+        return int(RNG.integers(16, 3000)), int(RNG.integers(1, 49)), pick([1024, 2048, 2560, 3072, 3584, 4096, 960, 1536, 5120, 272])
+    if r < 0.4:   # few tiles, long K (split-K)
+        return int(RNG.integers(1, 200)), int(RNG.integers(1, 200)), pick([2048, 4096, 6144, 8192, 3000, 4112])
+    if r < 0.5:
+        return pick([256, 320, 512, 640]), pick([256, 384, 512]), pick([256, 512, 768, 1024])
+    if r < 0.75 and BIG:
+        return int(RNG.integers(200, 1500)), int(RNG.integers(200, 1500)), int(RNG.integers(64, 1200))
+    return int(RNG.integers(1, 400)), int(RNG.integers(1, 400)), int(RNG.integers(1, 700))
+
+
+def make():
+    fam = pick(["i8i", "i8f", "i8f", "f8", "f8", "mx", "fl"])
+    m, n, k = dims()
+    s = dict(m=m, n=n, k=k)
+    s["transa"], s["transb"] = int(RNG.integers(2)), int(RNG.integers(2))
+    if RNG.random() < 0.5: s["transa"], s["transb"] = 1, 0
+    for t in "abcd":
+        if RNG.random() < 0.25: s["order_" + t] = 1
+    if fam == "i8i":
+        s.update(a_type=K.CUDA_R_8I, b_type=K.CUDA_R_8I, d_type=K.CUDA_R_32I, compute_type=K.CUBLAS_COMPUTE_32I, scale_type=K.CUDA_R_32I)
+        if RNG.random() < 0.4: s["with_c"] = True
+    elif fam == "i8f":
+        s.update(a_type=K.CUDA_R_8I, b_type=K.CUDA_R_8I, d_type=pick([K.CUDA_R_16BF, K.CUDA_R_16F, K.CUDA_R_32F, K.CUDA_R_8I, K.CUDA_R_32I]),
+                 compute_type=K.CUBLAS_COMPUTE_32I, scale_type=K.CUDA_R_32F, alpha_range=(0.001, 0.002))
+    elif fam == "f8":
+        at, bt = pick([(K.CUDA_R_8F_E4M3, K.CUDA_R_8F_E4M3), (K.CUDA_R_8F_E5M2, K.CUDA_R_8F_E4M3), (K.CUDA_R_8F_E4M3, K.CUDA_R_8F_E5M2)])
+        s.update(a_type=at, b_type=bt, d_type=pick([K.CUDA_R_16BF, K.CUDA_R_16F, K.CUDA_R_32F, K.CUDA_R_8F_E4M3]), compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F)
+    elif fam == "mx":
         k = max(32, k // 32 * 32)
-        spec.update(k=k, a_type=K.CUDA_R_4F_E2M1, b_type=K.CUDA_R_4F_E2M1, compute_type=K.CUBLAS_COMPUTE_32F,
-                    scale_type=K.CUDA_R_32F, transa=1, transb=0,
-                    a_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_VEC32_UE8M0,
-                    b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_VEC32_UE8M0)
-        spec["d_type"] = int(rng.choice([K.CUDA_R_16BF, K.CUDA_R_16F, K.CUDA_R_32F]))
+        if RNG.random() < 0.6: k = max(256, k // 256 * 256)
+        s.update(k=k, transa=1, transb=0, a_type=K.CUDA_R_4F_E2M1, b_type=K.CUDA_R_4F_E2M1, d_type=pick([K.CUDA_R_16BF, K.CUDA_R_32F]),
+                 compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F, a_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_VEC32_UE8M0,
+                 b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_VEC32_UE8M0)
+        s.pop("order_a", None); s.pop("order_b", None)
     else:
-        ta, tb = int(rng.integers(0, 2)), int(rng.integers(0, 2))
-        if rng.random() < 0.4:
-            ta, tb = 1, 0                                    # the K-contiguous combination is the common one
-        spec.update(transa=ta, transb=tb)
-        if rng.random() < 0.25:
-            spec.update(order_a=1, order_b=1)
-        if kind == "i8":
-            spec.update(a_type=K.CUDA_R_8I, b_type=K.CUDA_R_8I, d_type=K.CUDA_R_32I, compute_type=K.CUBLAS_COMPUTE_32I,
-                        scale_type=K.CUDA_R_32I)
-        elif kind == "i8f":
-            spec.update(a_type=K.CUDA_R_8I, b_type=K.CUDA_R_8I, compute_type=K.CUBLAS_COMPUTE_32I, scale_type=K.CUDA_R_32F,
-                        d_type=int(rng.choice([K.CUDA_R_16BF, K.CUDA_R_16F, K.CUDA_R_32F])), alpha_range=(0.001, 0.002))
-        else:
-            at, bt = K.CUDA_R_8F_E4M3, K.CUDA_R_8F_E4M3
-            r = rng.random()
-            if r < 0.1:
-                at = K.CUDA_R_8F_E5M2
-            elif r < 0.2:
-                bt = K.CUDA_R_8F_E5M2
-            spec.update(a_type=at, b_type=bt, compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F,
-                        d_type=int(rng.choice([K.CUDA_R_16BF, K.CUDA_R_16F, K.CUDA_R_32F])))
-    spec["c_type"] = spec["d_type"]
-    if rng.random() < 0.3:
-        spec.update(order_c=1, order_d=1)
-    if rng.random() < 0.3:
-        spec["batch"] = int(rng.integers(2, 4))
-    if rng.random() < 0.3:
-        spec["with_c"] = True
-    # padded leading dimensions (multiples of 4 or 16 bytes, or odd ones: the planner must cope)
-    def pad(x):
-        return x + int(rng.choice([0, 0, 4, 16, 48, 3]))
-    ta, tb = spec.get("transa", 0), spec.get("transb", 0)
-    row_a, row_b = spec.get("order_a", 0) == 1, spec.get("order_b", 0) == 1
-    a_rows, a_cols = (k, m) if ta else (m, k)
-    b_rows, b_cols = (n, k) if tb else (k, n)
-    if kind != "mx" and rng.random() < 0.4:
-        spec["lda"] = pad(a_cols if row_a else a_rows)
-        spec["ldb"] = pad(b_cols if row_b else b_rows)
-    if rng.random() < 0.3:
-        row_d = spec.get("order_d", 0) == 1
-        spec["ldd"] = (n if row_d else m) + int(rng.choice([0, 8, 16, 5]))
-        spec["ldc"] = (n if row_d else m) + int(rng.choice([0, 8, 16, 5]))
-    if kind != "i8":
-        epi = rng.choice(["none", "bias", "relu_bias", "gelu_bias", "gelu", "relu"])
-        code = {"none": K.CUBLASLT_EPILOGUE_DEFAULT, "bias": K.CUBLASLT_EPILOGUE_BIAS, "relu_bias": K.CUBLASLT_EPILOGUE_RELU_BIAS,
-                "gelu_bias": K.CUBLASLT_EPILOGUE_GELU_BIAS, "gelu": K.CUBLASLT_EPILOGUE_GELU, "relu": K.CUBLASLT_EPILOGUE_RELU}[epi]
-        spec["epilogue"] = code
-        if "bias" in epi:
-            spec["bias_type"] = int(rng.choice([K.CUDA_R_32F, K.CUDA_R_16BF]))
-        if kind != "mx":
-            r = rng.random()
-            if r < 0.3:
-                spec.update(with_scalar_scales=True, scale_range=(0.05, 0.06) if kind == "f8" else (0.5, 1.5))
-            elif r < 0.55:
-                spec.update(a_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F,
-                            b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F,
-                            scale_range=(0.05, 0.06) if kind == "f8" else (0.5, 1.5))
-            elif r < 0.7:
-                spec.update(b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F,
-                            scale_range=(0.05, 0.06) if kind == "f8" else (0.5, 1.5))
-        pm = rng.random()
-        if pm < 0.25:
-            spec["pointer_mode"] = (K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_HOST if spec.get("with_c")
-                                    else K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO)
-        elif pm < 0.4 and spec.get("with_c"):    # a device-side beta may be non-zero: the call needs a C then
-            spec["pointer_mode"] = K.CUBLASLT_POINTER_MODE_DEVICE
-    elif rng.random() < 0.3 and spec.get("with_c"):
-        spec["pointer_mode"] = K.CUBLASLT_POINTER_MODE_DEVICE
-    return spec
+        t = pick([K.CUDA_R_16BF, K.CUDA_R_16F, K.CUDA_R_32F])
+        s.update(a_type=t, b_type=t, d_type=pick([t, K.CUDA_R_32F]), compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F)
+        s["m"], s["n"], s["k"] = min(m, 300), min(n, 300), min(s["k"], 600)
+    m, n, k = s["m"], s["n"], s["k"]
+    ta, tb = s["transa"], s["transb"]
+    # leading dimensions: sometimes padded
+    def ld(tag, rows, cols, mult):
+        order = s.get("order_" + tag, 0)
+        base = rows if order == 0 else cols
+        r = RNG.random()
+        if r < 0.5: return
+        pad = int(RNG.integers(1, 40)) if r < 0.6 else (16 * int(RNG.integers(1, 4)) if r < 0.9 else 4 * int(RNG.integers(1, 9)))
+        if mode16: pad = (pad + 15) // 16 * 16; v16 = (base + 15) // 16 * 16 - base; pad += v16
+        v = base + pad
+        if mult > 1: v = (v + mult - 1) // mult * mult
+        s["ld" + tag] = v
+    mult = 2 if fam == "mx" else 1
+    mode16 = RNG.random() < 0.6
+    if mode16 and fam != "fl":   # K-contiguous operands need K % 16 == 0 for the MFMA kernels
+        s["k"] = k = max(16, k // 16 * 16) if fam != "mx" else k
+    ld("a", k if ta else m, m if ta else k, mult); ld("b", n if tb else k, k if tb else n, mult)
+    ld("c", m, n, 1); ld("d", m, n, 1)
+    if RNG.random() < 0.25:
+        s["batch"] = int(RNG.integers(2, 4))
+    if fam != "i8i":
+        if RNG.random() < 0.4: s["with_c"] = True
+        epi = pick(EPIS)
+        if fam == "mx" and epi in (K.CUBLASLT_EPILOGUE_BGRADA, K.CUBLASLT_EPILOGUE_BGRADB): epi = K.CUBLASLT_EPILOGUE_GELU_BIAS
+        s["epilogue"] = epi
+        if epi != K.CUBLASLT_EPILOGUE_DEFAULT and RNG.random() < 0.5:
+            s["bias_type"] = pick([K.CUDA_R_32F, K.CUDA_R_16BF, K.CUDA_R_16F])
+        bg = epi in (K.CUBLASLT_EPILOGUE_BGRADA, K.CUBLASLT_EPILOGUE_BGRADB)
+        if s.get("batch", 1) > 1 and epi not in (K.CUBLASLT_EPILOGUE_DEFAULT, K.CUBLASLT_EPILOGUE_RELU, K.CUBLASLT_EPILOGUE_GELU) and RNG.random() < 0.5:
+            s["bias_batch_stride"] = max(m, n) + int(RNG.integers(0, 9))
+        pm = pick([K.CUBLASLT_POINTER_MODE_HOST] * 3 + [K.CUBLASLT_POINTER_MODE_DEVICE, K.CUBLASLT_POINTER_MODE_DEVICE_VECTOR,
+                  K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO, K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_HOST])
+        s["pointer_mode"] = pm
+        if pm == K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO: s.pop("with_c", None)
+        if pm in (K.CUBLASLT_POINTER_MODE_DEVICE, K.CUBLASLT_POINTER_MODE_DEVICE_VECTOR): s["with_c"] = True
+        if bg and s.get("batch", 1) > 1: s["bias_batch_stride"] = max(m, n) + int(RNG.integers(0, 9))
+        if fam in ("i8f", "f8") and not bg:
+            r = RNG.random()
+            if r < 0.3: s["with_scalar_scales"] = True
+            elif r < 0.5 and fam == "i8f": s["b_scale_mode"] = K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F
+            elif r < 0.6 and fam == "i8f": s["a_scale_mode"] = K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F
+            if RNG.random() < 0.2 and fam == "f8": s["with_cd_scales"] = True
+    return fam, s
 
 
-@pytest.mark.parametrize("chunk", range(8))
+@pytest.mark.parametrize("chunk", range(6))
 def test_random_problems_against_the_oracle(gpu_api, chunk):
-    rng = np.random.default_rng(9000 + chunk)
-    families = {}
-    for i in range(24):
-        spec = random_spec(rng)
-        seed = 9000 + chunk * 100 + i
-        ws = int(rng.choice([0, 0, 64 << 20]))
-        print("random case", chunk, i, spec, "workspace", ws, flush=True)
-        case = Case(spec, seed, int_dist="normal" if rng.random() < 0.3 else "uniform")
+    global RNG
+    RNG = np.random.default_rng(4200 + chunk)
+    ran = 0
+    for it in range(40):
+        fam, spec = make()
+        seed = 420000 + chunk * 1000 + it
+        ws = pick([0, 0, 1 << 24])
+        forced = pick([None, None, None, K.ZLUDA_KERNEL_GENERIC])
+        print("case", chunk, it, "seed", seed, "workspace", ws, "forced family", forced, json.dumps(spec), flush=True)
+        case = Case(spec, seed)
         ref = case.run_oracle()
-        st, got, kern, variant = case.run_gpu(gpu_api, workspace_bytes=ws)
+        try:
+            st, got, kern, var = case.run_gpu(gpu_api, forced_kernel=forced, workspace_bytes=ws)
+        except cublaslt.CublasLtError as e:   # a combination the API refuses when the descriptors are built
+            print("  refused:", e, flush=True)
+            continue
         assert st == 0, "cublasLtMatmul status %d" % st
-        case.compare(got, ref)
-        families[kern] = families.get(kern, 0) + 1
-    print("kernel families used:", families)
+        ran += 1
+        # one e4m3 step is 2^-3 of the value; int32 outputs of float-scaled problems may sit on a rounding boundary
+        tol = 0.13 if spec["d_type"] == K.CUDA_R_8F_E4M3 else None
+        check(case, spec, got, ref, tol)
+        if case.bgrad:
+            ints = spec["a_type"] == K.CUDA_R_8I and case.bgrad_type == K.CUDA_R_32F
+            case.compare_bgrad(case.bgrad_got, case.bgrad_ref, exact=ints)
+        if kern in NVAR and forced is None:
+            for fv in RNG.permutation(NVAR[kern])[:3]:
+                st, got, _, _ = case.run_gpu(gpu_api, forced_kernel=kern, forced_variant=int(fv), workspace_bytes=ws)
+                print("  forced variant", int(fv), "status", st, flush=True)
+                if st == 0:
+                    check(case, spec, got, ref, tol)
+    assert ran >= 30
+
+
+def check(case, spec, got, ref, tol):
+    if spec["d_type"] == K.CUDA_R_32I and spec["scale_type"] == K.CUDA_R_32F:
+        # float epilogue rounded to int32: association differences may move a value across a .5 boundary
+        idx = case.logical_index().ravel()
+        assert np.max(np.abs(got[idx].astype(np.int64) - ref[idx].astype(np.int64))) <= 1
+        return
+    case.compare(got, ref, tol=tol)

@@ -238,5 +238,9 @@ def test_bias_gradient_epilogues_are_planned_like_the_plain_problem(api):
     assert st == K.CUBLAS_STATUS_NOT_SUPPORTED
     st, _ = plan(api, dict(I8, m=512, n=512, k=512, transa=1, epilogue=K.CUBLASLT_EPILOGUE_BGRADB))   # int32 scale type: DEFAULT only
     assert st == K.CUBLAS_STATUS_NOT_SUPPORTED
+    st, _ = plan(api, dict(bf, batch=2, epilogue=K.CUBLASLT_EPILOGUE_BGRADA))   # batches would share one output vector
+    assert st == K.CUBLAS_STATUS_NOT_SUPPORTED
+    st, _ = plan(api, dict(bf, batch=2, bias_batch_stride=512, epilogue=K.CUBLASLT_EPILOGUE_BGRADA))
+    assert st == 0
     st, _ = plan(api, dict(F8, m=512, n=512, k=512, transa=1, epilogue=K.CUBLASLT_EPILOGUE_DGELU))
     assert st == K.CUBLAS_STATUS_NOT_SUPPORTED

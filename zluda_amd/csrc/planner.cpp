@@ -181,6 +181,8 @@ uint32_t lower_problem(const zluda_gemm_problem *p, bool dry, Lowered *out) {
     // sums of the stored elements: defined here for unscaled operands only
     if (a.type == CUDA_R_4F_E2M1 || b.type == CUDA_R_4F_E2M1 || g.a_scale_mode || g.b_scale_mode)
       return CUBLAS_STATUS_NOT_SUPPORTED;
+    // batches with no stride between their gradient vectors would all write the same one
+    if (g.batch > 1 && op.bias_batch_stride == 0) return CUBLAS_STATUS_NOT_SUPPORTED;
     if (!dry && !op.bias) return CUBLAS_STATUS_INVALID_VALUE;
     g.bgrad = const_cast<void *>(op.bias);
   }
