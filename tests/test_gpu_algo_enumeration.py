@@ -88,7 +88,7 @@ def run_enumerated(api, spec, seed, want_family, variants):
 def test_int8_through_enumerated_algorithms(gpu_api):
     spec = dict(a_type=K.CUDA_R_8I, b_type=K.CUDA_R_8I, c_type=K.CUDA_R_32I, d_type=K.CUDA_R_32I,
                 compute_type=K.CUBLAS_COMPUTE_32I, scale_type=K.CUDA_R_32I, transa=1, m=512, n=384, k=1024, alpha=1)
-    run_enumerated(gpu_api, spec, 501, K.ZLUDA_KERNEL_MFMA_I8, [0, 3, 6])
+    run_enumerated(gpu_api, spec, 501, K.ZLUDA_KERNEL_MFMA_I8, [0, 3, 6, 8])
     run_enumerated(gpu_api, dict(spec, transa=0, transb=1), 502, K.ZLUDA_KERNEL_MFMA_TR8, [1, 2])
     run_enumerated(gpu_api, spec, 503, K.ZLUDA_KERNEL_GENERIC, [0])
 
@@ -97,4 +97,4 @@ def test_fp8_through_enumerated_algorithms(gpu_api):
     spec = dict(a_type=K.CUDA_R_8F_E4M3, b_type=K.CUDA_R_8F_E4M3, c_type=K.CUDA_R_16BF, d_type=K.CUDA_R_16BF,
                 compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F, transa=1, m=512, n=256, k=768, alpha=1.0,
                 epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS, bias_type=K.CUDA_R_16BF, with_scalar_scales=True)
-    run_enumerated(gpu_api, spec, 511, K.ZLUDA_KERNEL_MFMA_F8, [0, 2, 5])
+    run_enumerated(gpu_api, spec, 511, K.ZLUDA_KERNEL_MFMA_F8, [0, 2, 5, 8])

@@ -32,7 +32,7 @@ def test_baseline_configs_pick_the_intended_kernels(api):
     st, p = plan(api, dict(I8, m=256, n=256, k=256, transa=0, transb=1))            # config 1: A:N B:T
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_TR8 and p.variant == 2 and p.grid_x == 16 and p.block == 256
     st, p = plan(api, dict(I8, m=4096, n=4096, k=4096, transa=1))                   # config 2
-    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_I8 and p.variant == 0 and p.grid_x == 256 and p.block == 512
+    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_I8 and p.variant == 8 and p.grid_x == 256 and p.block == 512   # 256x256 on the 16x16 MFMA shapes
     st, p = plan(api, dict(I8, m=14336, n=16, k=4096, transa=1, d_type=K.CUDA_R_16BF, scale_type=K.CUDA_R_32F,
                            pointer_mode=K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO,
                            b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F,
@@ -59,9 +59,13 @@ def test_extents_that_256_divides_badly_get_the_192_row_tile(api):
     st, p = plan(api, dict(I8, m=3072, n=3072, k=3072, transa=1))
     assert st == 0 and p.variant == 7 and p.grid_x == 16 * 12
     st, p = plan(api, dict(I8, m=8192, n=8192, k=8192, transa=1))
-    assert st == 0 and p.variant == 0
+    assert st == 0 and p.variant == 8
     st, p = plan(api, dict(F8, m=14336, n=4096, k=4096, transa=1))   # 5 rounds of 192x256 lose to 4 of 256x256
+    assert st == 0 and p.variant == 8
+    st, p = plan(api, dict(MX, m=8192, n=8192, k=8192, transa=1))      # MXFP4 has no 16x16-shape variant
     assert st == 0 and p.variant == 0
+    assert plan(api, dict(MX, m=8192, n=8192, k=8192, transa=1), forced=K.ZLUDA_KERNEL_MFMA_MXF4, variant=8)[0] == K.CUBLAS_STATUS_INVALID_VALUE
+    assert api.zluda_gemm_variant_count(K.ZLUDA_KERNEL_MFMA_I8) == 9 and api.zluda_gemm_variant_count(K.ZLUDA_KERNEL_MFMA_MXF4) == 8
 
 
 def test_row_major_output_swaps_operands(api):
@@ -132,10 +136,10 @@ def test_fp4_must_be_k_contiguous(api):
 def test_forced_variants(api):
     spec = dict(I8, m=4096, n=4096, k=4096, transa=1)
     for v, (grid, block) in enumerate([(256, 512), (256, 256), (512, 256), (1024, 256), (1024, 256), (2048, 256), (4096, 256),
-                                       (352, 512)]):
+                                       (352, 512), (256, 512)]):
         st, p = plan(api, spec, forced=K.ZLUDA_KERNEL_MFMA_I8, variant=v)
         assert st == 0 and p.variant == v and p.grid_x == grid and p.block == block
-    assert plan(api, spec, forced=K.ZLUDA_KERNEL_MFMA_I8, variant=8)[0] == K.CUBLAS_STATUS_INVALID_VALUE
+    assert plan(api, spec, forced=K.ZLUDA_KERNEL_MFMA_I8, variant=9)[0] == K.CUBLAS_STATUS_INVALID_VALUE
     assert plan(api, spec, forced=K.ZLUDA_KERNEL_MFMA_F8)[0] == K.CUBLAS_STATUS_NOT_SUPPORTED
 
 

@@ -56,6 +56,16 @@ __device__ __forceinline__ void lds_dma16(__amdgpu_buffer_rsrc_t rs, void *lds_d
 #endif
 }
 
+// 128-bit buffer store whose data registers stay untouched for the wait states that follow it.  Observed on
+// MI355X: when the instruction right behind a buffer_store_dwordx4 (offen, scalar offset in an SGPR) is a
+// VALU write to the first data register, the store now and then writes the new value instead (element 0 of
+// the four, in a few hundred of 131072 outputs); the compiler's hazard table does not list this case, so it
+// puts no wait state there.  The asm keeps the data registers live across an s_nop that follows the store.
+__device__ __forceinline__ void buffer_store_b128_guarded(v4i data, __amdgpu_buffer_rsrc_t rs, int voff, int soff) {
+  __builtin_amdgcn_raw_buffer_store_b128(data, rs, voff, soff, 0);
+  asm volatile("s_nop 1" : "+v"(data)::"memory");
+}
+
 struct MfmaParams {
   GemmArgs g;
   int32_t swapped;           // P = op(B)^T rows, Q = op(A) rows
@@ -344,7 +354,7 @@ __device__ __forceinline__ void mfma_store_tile_f(const MfmaParams &prm, AccV (&
       const int soff = (a * 32 + h * 16 + it * RPI) * d_sq * ESZ;  // uniform
       if constexpr (DT == 2) {
         const v4i pk = {(int)f2bits(x[0]), (int)f2bits(x[1]), (int)f2bits(x[2]), (int)f2bits(x[3])};
-        __builtin_amdgcn_raw_buffer_store_b128(pk, rs, voff, soff, 0);
+        buffer_store_b128_guarded(pk, rs, voff, soff);
       } else {
         v2i pk;
         if constexpr (DT == 0) {

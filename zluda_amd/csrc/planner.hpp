@@ -8,16 +8,17 @@ namespace zluda_amd {
 
 // MFMA tile configurations (index = plan.variant for the MFMA families): workgroup tile bp x bq,
 // wp x wq waves, `bkb` bytes of K per LDS stage, `stages` LDS stages
-struct MfmaVariant { int bp, bq, wp, wq, bkb, stages; };
+struct MfmaVariant { int bp, bq, wp, wq, bkb, stages, m16; };  // m16: the 16x16 MFMA shapes (gemm_mfma_pipe16.hpp; int8 and fp8)
 constexpr MfmaVariant kMfmaVariants[] = {
-    {256, 256, 2, 4, 128, 2},  // 0: 8 waves, 128x64 per wave
-    {256, 256, 2, 2, 128, 2},  // 1: 4 waves, 128x128 per wave
-    {256, 128, 2, 2, 128, 2},  // 2: 4 waves, 128x64 per wave
-    {128, 128, 2, 2, 128, 2},  // 3: 4 waves, 64x64 per wave, two workgroups per CU
-    {128, 128, 2, 2, 64, 4},   // 4: same tile, half-line stages, deeper ring (short K)
-    {128, 64, 2, 2, 128, 3},   // 5: 4 waves, 64x32 per wave: skinny problems
-    {64, 64, 2, 2, 128, 3},    // 6: 4 waves, 32x32 per wave: problems of a few hundred tiles at most
-    {192, 256, 2, 4, 128, 2},  // 7: 8 waves, 96x64 per wave: extents that 256 divides badly (3072, 6144, ...)
+    {256, 256, 2, 4, 128, 2, 0},  // 0: 8 waves, 128x64 per wave
+    {256, 256, 2, 2, 128, 2, 0},  // 1: 4 waves, 128x128 per wave
+    {256, 128, 2, 2, 128, 2, 0},  // 2: 4 waves, 128x64 per wave
+    {128, 128, 2, 2, 128, 2, 0},  // 3: 4 waves, 64x64 per wave, two workgroups per CU
+    {128, 128, 2, 2, 64, 4, 0},   // 4: same tile, half-line stages, deeper ring (short K)
+    {128, 64, 2, 2, 128, 3, 0},   // 5: 4 waves, 64x32 per wave: skinny problems
+    {64, 64, 2, 2, 128, 3, 0},    // 6: 4 waves, 32x32 per wave: problems of a few hundred tiles at most
+    {192, 256, 2, 4, 128, 2, 0},  // 7: 8 waves, 96x64 per wave: extents that 256 divides badly (3072, 6144, ...)
+    {256, 256, 2, 4, 128, 2, 1},  // 8: variant 0 on v_mfma_*_16x16x*: less energy per multiply-add, and large GEMMs are power bound
 };
 constexpr int kNumMfmaVariants = sizeof(kMfmaVariants) / sizeof(kMfmaVariants[0]);
 
