@@ -54,10 +54,15 @@ def test_small_problems_get_smaller_tiles(api):
 
 
 def test_extents_that_256_divides_badly_get_the_192_row_tile(api):
+    # (variants 9 and 8 are 7's and 0's tiles on the 16x16 MFMA shapes: taken when the grid fills the chip)
     st, p = plan(api, dict(F8, m=6144, n=4096, k=4096, transa=1))
-    assert st == 0 and p.variant == 7 and p.grid_x == 32 * 16          # two full rounds instead of 1.5 -> 2 of 256x256
+    assert st == 0 and p.variant == 9 and p.grid_x == 32 * 16          # two full rounds instead of 1.5 -> 2 of 256x256
     st, p = plan(api, dict(I8, m=3072, n=3072, k=3072, transa=1))
-    assert st == 0 and p.variant == 7 and p.grid_x == 16 * 12
+    assert st == 0 and p.variant == 9 and p.grid_x == 16 * 12
+    st, p = plan(api, dict(F8, m=3072, n=3072, k=3072, transa=1))       # fp8 gains little: only from two rounds on
+    assert st == 0 and p.variant == 7
+    st, p = plan(api, dict(I8, m=2048, n=2048, k=2048, transa=1, batch=2))   # 128 tiles of 256x256: half of the chip idles
+    assert st == 0 and not (p.variant in (8, 9))
     st, p = plan(api, dict(I8, m=8192, n=8192, k=8192, transa=1))
     assert st == 0 and p.variant == 8
     st, p = plan(api, dict(F8, m=14336, n=4096, k=4096, transa=1))   # 5 rounds of 192x256 lose to 4 of 256x256
@@ -65,7 +70,7 @@ def test_extents_that_256_divides_badly_get_the_192_row_tile(api):
     st, p = plan(api, dict(MX, m=8192, n=8192, k=8192, transa=1))      # MXFP4 has no 16x16-shape variant
     assert st == 0 and p.variant == 0
     assert plan(api, dict(MX, m=8192, n=8192, k=8192, transa=1), forced=K.ZLUDA_KERNEL_MFMA_MXF4, variant=8)[0] == K.CUBLAS_STATUS_INVALID_VALUE
-    assert api.zluda_gemm_variant_count(K.ZLUDA_KERNEL_MFMA_I8) == 9 and api.zluda_gemm_variant_count(K.ZLUDA_KERNEL_MFMA_MXF4) == 8
+    assert api.zluda_gemm_variant_count(K.ZLUDA_KERNEL_MFMA_I8) == 10 and api.zluda_gemm_variant_count(K.ZLUDA_KERNEL_MFMA_MXF4) == 8
 
 
 def test_row_major_output_swaps_operands(api):
@@ -136,10 +141,10 @@ def test_fp4_must_be_k_contiguous(api):
 def test_forced_variants(api):
     spec = dict(I8, m=4096, n=4096, k=4096, transa=1)
     for v, (grid, block) in enumerate([(256, 512), (256, 256), (512, 256), (1024, 256), (1024, 256), (2048, 256), (4096, 256),
-                                       (352, 512), (256, 512)]):
+                                       (352, 512), (256, 512), (352, 512)]):
         st, p = plan(api, spec, forced=K.ZLUDA_KERNEL_MFMA_I8, variant=v)
         assert st == 0 and p.variant == v and p.grid_x == grid and p.block == block
-    assert plan(api, spec, forced=K.ZLUDA_KERNEL_MFMA_I8, variant=9)[0] == K.CUBLAS_STATUS_INVALID_VALUE
+    assert plan(api, spec, forced=K.ZLUDA_KERNEL_MFMA_I8, variant=10)[0] == K.CUBLAS_STATUS_INVALID_VALUE
     assert plan(api, spec, forced=K.ZLUDA_KERNEL_MFMA_F8)[0] == K.CUBLAS_STATUS_NOT_SUPPORTED
 
 

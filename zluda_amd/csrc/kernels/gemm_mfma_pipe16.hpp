@@ -355,12 +355,16 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe16_kernel(MfmaParam
       for (int v = 0; v < 4; v++) acc[a][b][v] = 0;
 
   Frag pf[2][HP], qf[2][HQ];  // [half of the wave tile][fragment]
-  auto load_p_half = [&](int so, auto h_c) {
-    constexpr int h = decltype(h_c)::value;
-    static_for<HP>([&](auto i_c) {
-      constexpr int i = decltype(i_c)::value;
+  // fragments [I0, I1) of P half h
+  auto load_p_part = [&](int so, auto h_c, auto i0_c, auto i1_c) {
+    constexpr int h = decltype(h_c)::value, I0 = decltype(i0_c)::value, I1 = decltype(i1_c)::value;
+    static_for<I1 - I0>([&](auto i_c) {
+      constexpr int i = I0 + decltype(i_c)::value;
       load_frag(so, fragP, std::integral_constant<int, h * HP + i>{}, pf[h][i]);
     });
+  };
+  auto load_p_half = [&](int so, auto h_c) {
+    load_p_part(so, h_c, std::integral_constant<int, 0>{}, std::integral_constant<int, HP>{});
   };
   auto load_q_half = [&](int so, auto h_c) {
     constexpr int h = decltype(h_c)::value;
@@ -423,26 +427,36 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe16_kernel(MfmaParam
     using QAc = std::integral_constant<int, QA>;
     using QBc = std::integral_constant<int, QB_>;
     constexpr int DSP = 2 * HP, DSQ = 2 * HQ;  // ds_read_b128 per half
+    // The fragment reads are spread over the four sub-steps (the LDS is the busiest unit of the loop: 24 KiB
+    // per wave and stage): EARLY fragments of P half 1 come with QB, LATE fragments of the next stage's P
+    // half 0 with its first Q half.
+    constexpr int EARLY = 1, LATE = 1;  // (0 / 0: 1.5 % slower at 8192^3 int8; 2 / 1: no better; whole halves early: far slower)
+    using I0 = std::integral_constant<int, 0>;
+    using IE = std::integral_constant<int, EARLY>;
+    using IL = std::integral_constant<int, HP - LATE>;
+    using IH = std::integral_constant<int, HP>;
     // (P0, QA) while QB arrives
     load_q_half(so, QBc{});
+    load_p_part(so, P1{}, I0{}, IE{});
     mfma_halves(P0{}, QAc{});
-    pattern(std::integral_constant<int, DSQ>{}, std::integral_constant<int, 0>{});
+    pattern(std::integral_constant<int, DSQ + 2 * EARLY>{}, std::integral_constant<int, 0>{});
     // (P0, QB) while P1 arrives
-    load_p_half(so, P1{});
+    load_p_part(so, P1{}, IE{}, IH{});
     mfma_halves(P0{}, QBc{});
-    pattern(std::integral_constant<int, DSP>{}, std::integral_constant<int, 0>{});
+    pattern(std::integral_constant<int, DSP - 2 * EARLY>{}, std::integral_constant<int, 0>{});
     // every fragment of the stage has been requested: wait for them and for this wave's share of stage
     // kt+1, meet the other waves; then the slot is free and the other one readable
     wait_vmcnt_barrier<0>();
     // (P1, QB): refill this slot with stage kt+2, P half 0 of stage kt+1 arrives
-    load_p_half(so_next, P0{});
+    load_p_part(so_next, P0{}, I0{}, IL{});
     issue_stage(kt + NSTAGE, so);
     mfma_halves(P1{}, QBc{});
-    pattern(std::integral_constant<int, DSP>{}, std::integral_constant<int, NLOAD>{});
+    pattern(std::integral_constant<int, DSP - 2 * LATE>{}, std::integral_constant<int, NLOAD>{});
     // (P1, QA): Q half QB of stage kt+1 arrives (that stage starts with it)
+    load_p_part(so_next, P0{}, IL{}, IH{});
     load_q_half(so_next, QBc{});
     mfma_halves(P1{}, QAc{});
-    pattern(std::integral_constant<int, DSQ>{}, std::integral_constant<int, 0>{});
+    pattern(std::integral_constant<int, DSQ + 2 * LATE>{}, std::integral_constant<int, 0>{});
   };
 
   int kt = 0;

@@ -326,10 +326,15 @@ static void fill_mfma_plan(const Lowered &l, int variant, uint32_t cus, uint64_t
 }
 
 // Relative throughput of one CU running tiles of each variant (measured on MI355X, int8 and fp8, K >= 1024;
-// variant 0 = 1).  Smaller tiles read more LDS and L2 bytes per MFMA.  Variant 8 (variant 0's tile on the
-// 16x16 MFMA shapes) measures 7-8 % faster than variant 0 for int8 and 1-2 % faster for fp8 at 4096^3 and
-// 8192^3 with the board at its power cap.
-static const float kMfmaVariantEfficiency[kNumMfmaVariants] = {1.00f, 0.95f, 0.80f, 0.70f, 0.72f, 0.55f, 0.40f, 0.85f, 1.02f};
+// variant 0 = 1).  Smaller tiles read more LDS and L2 bytes per MFMA.
+// The variants on the 16x16 MFMA shapes (8, 9) need less energy per multiply-add, which is what bounds a GEMM
+// that keeps the whole chip busy (the board sits at its power cap): at 4096^3 and 8192^3 they take 8-10 % less
+// time than their 32x32 counterparts for int8 and 1-3 % less for fp8.  On a chip that is partly idle the clock
+// is the bound instead and they lose (their epilogue is ~3 us per tile slower: 2048^3 int8 30.5 us against
+// 27.5), so they are only chosen for grids that fill the chip; the same tiles at 256x128 and 128x128 measured
+// no better than the 32x32 ones anywhere and are not instantiated.
+static const float kMfmaVariantEfficiency[kNumMfmaVariants] = {1.00f, 0.95f, 0.80f, 0.70f, 0.72f, 0.55f, 0.40f, 0.85f,
+                                                               1.05f, 0.89f};
 
 static int pick_mfma_variant(const Lowered &l, uint32_t cus) {
   const GemmArgs &g = l.g;
@@ -341,8 +346,13 @@ static int pick_mfma_variant(const Lowered &l, uint32_t cus) {
   double best_cost = 0;
   for (int v = 0; v < kNumMfmaVariants; v++) {
     const MfmaVariant &t = kMfmaVariants[v];
-    if (t.m16 && g.a_type == CUDA_R_4F_E2M1) continue;  // the 16x16 shapes serve int8 and fp8
     const uint64_t tiles = (uint64_t)ceil_div(np, t.bp) * ceil_div(nq, t.bq) * g.batch;
+    if (t.m16) {
+      if (g.a_type == CUDA_R_4F_E2M1) continue;  // the 16x16 shapes serve int8 and fp8
+      // power bound or not: int8 gains from three quarters of the CUs busy on, fp8 (a small gain) from two
+      // full rounds on
+      if (g.a_type == CUDA_R_8I ? tiles * 4 < (uint64_t)cus * 3 : tiles < 2ull * cus) continue;
+    }
     const uint64_t rounds = (tiles + cus - 1) / cus;
     const double cost = (double)rounds * t.bp * t.bq / kMfmaVariantEfficiency[v];
     if (v == 0 || cost < best_cost) { best = v; best_cost = cost; }
@@ -452,7 +462,7 @@ extern "C" uint32_t zluda_gemm_variant_count(uint32_t kernel) {
   switch (kernel) {
   case ZLUDA_KERNEL_GENERIC: return 1;
   case ZLUDA_KERNEL_MFMA_I8: case ZLUDA_KERNEL_MFMA_F8: return kNumMfmaVariants;
-  case ZLUDA_KERNEL_MFMA_MXF4: return kNumMfmaVariants - 1;  // all but the last, which is the 16x16-shape one
+  case ZLUDA_KERNEL_MFMA_MXF4: return kNumMfmaVariants32;  // the 16x16-shape ones serve int8 and fp8
   case ZLUDA_KERNEL_DECODE_W8A8: return kNumDecodeVariants;
   case ZLUDA_KERNEL_MFMA_TR8: return kNumTrVariants;
   default: return 0;

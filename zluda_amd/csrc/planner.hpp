@@ -18,8 +18,12 @@ constexpr MfmaVariant kMfmaVariants[] = {
     {128, 64, 2, 2, 128, 3, 0},   // 5: 4 waves, 64x32 per wave: skinny problems
     {64, 64, 2, 2, 128, 3, 0},    // 6: 4 waves, 32x32 per wave: problems of a few hundred tiles at most
     {192, 256, 2, 4, 128, 2, 0},  // 7: 8 waves, 96x64 per wave: extents that 256 divides badly (3072, 6144, ...)
-    {256, 256, 2, 4, 128, 2, 1},  // 8: variant 0 on v_mfma_*_16x16x*: less energy per multiply-add, and large GEMMs are power bound
+    // the same tiles on v_mfma_*_16x16x* (int8 and fp8): less energy per multiply-add, and GEMMs that keep the
+    // chip busy are power bound
+    {256, 256, 2, 4, 128, 2, 1},  // 8: variant 0's
+    {192, 256, 2, 4, 128, 2, 1},  // 9: variant 7's
 };
+constexpr int kNumMfmaVariants32 = 8;  // the first ones, on the 32x32 shapes: what MXFP4 has
 constexpr int kNumMfmaVariants = sizeof(kMfmaVariants) / sizeof(kMfmaVariants[0]);
 
 // tile configurations of the transposing 8-bit MFMA kernel (index = plan.variant for
