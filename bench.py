@@ -15,7 +15,7 @@ counter during one more (untimed) batch: `clock_mhz_observed`, and `frac_at_obse
 roofline fraction against the datasheet peak scaled to that clock (the peak assumes 2400 MHz).
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c2|c3|c4|c5|c5_b1|i8_8192|i8_4096_nt] [--only]
-                  [--no-cpu] [--no-hipblaslt] [--copy-probe]
+                  [--no-cpu] [--no-hipblaslt] [--copy-probe] [--sustained SECONDS]
 """
 import argparse
 import ctypes as C
@@ -78,8 +78,8 @@ for _w in WORKLOADS.values():   # five equal batches
 # this script whose summaries are committed under profiles/ (each counter scaled by what it reads for the
 # 256 MiB copy of --copy-probe).  The line carries the figure and the file it was read from; a workload
 # without a summary reports null.
-PROFILE_OF = {"c1": "gemm_mfma_tr_i8_c1_256", "c2": "gemm_mfma_pipe_i8_c2_4096", "i8_4096_nt": "gemm_mfma_tr_i8_4096_nt",
-              "i8_8192": "gemm_mfma_pipe_i8_8192", "c3": "decode_stream_c3", "c4": "gemm_mfma_pipe_f8_c4_8192",
+PROFILE_OF = {"c1": "gemm_mfma_tr_i8_c1_256", "c2": "gemm_mfma_pipe16_i8_c2_4096", "i8_4096_nt": "gemm_mfma_tr_i8_4096_nt",
+              "i8_8192": "gemm_mfma_pipe16_i8_8192", "c3": "decode_stream_c3", "c4": "gemm_mfma_pipe16_f8_c4_8192",
               "c5": "gemm_mfma_pipe_mxf4_c5_8192x4", "c5_b1": "gemm_mfma_pipe_mxf4_c5_8192_b1"}
 
 
@@ -224,6 +224,48 @@ def observed_clock_mhz(torch, fn, calls, seconds_per_call):
     return cycles / (rt / (khz * 1e3)) / 1e6 if rt > 0 else None
 
 
+SUSTAIN_SECONDS = 0.0   # --sustained: seconds of back-to-back calls per measurement (0 = off)
+
+
+def sustained(torch, fn, seconds, per_batch=10):
+    """The same call back to back for `seconds`, with the board power sampled from hwmon meanwhile: under matrix
+    load the part sits at its power cap after a few hundred milliseconds, so what a long-running job sees is the
+    time a kernel's ENERGY allows, not what a burst of a few dozen calls shows.  Returns microseconds per call,
+    watts and millijoules per call over the second half of the run (watts None where hwmon is not readable)."""
+    import glob
+    import threading
+    files = glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input")
+    samples, stop = [], []
+
+    def sampler():
+        while not stop:
+            try:
+                samples.append((time.perf_counter(), int(open(files[0]).read()) / 1e6))
+            except (OSError, ValueError, IndexError):
+                return
+            time.sleep(0.002)
+    th = threading.Thread(target=sampler, daemon=True)
+    torch.cuda.synchronize()
+    th.start()
+    t0, marks, n = time.perf_counter(), [], 0
+    while time.perf_counter() - t0 < seconds:
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(per_batch):
+            fn(n + i)
+        e1.record()
+        n += per_batch
+        e1.synchronize()
+        marks.append((time.perf_counter(), e0.elapsed_time(e1) / per_batch * 1e3))
+    stop.append(1)
+    th.join()
+    half = marks[len(marks) // 2:]
+    us = sum(m[1] for m in half) / len(half)
+    pw = [p for (t, p) in samples if half[0][0] <= t <= half[-1][0]]
+    watts = sum(pw) / len(pw) if pw else None
+    return {"seconds": seconds, "us_per_call": us, "watts": watts, "mj_per_call": us * watts * 1e-3 if watts else None}
+
+
 def run_workload(torch, api, key, steps, warmup, with_hipblaslt):
     w = WORKLOADS[key]
     spec = w["spec"]
@@ -265,6 +307,8 @@ def run_workload(torch, api, key, steps, warmup, with_hipblaslt):
                      "kernel_ms": per_call * 1e3, "kernel_ms_batches": [b * 1e3 for b in batches],
                      "algorithmic_ops": ops, "algorithmic_bytes": nbytes, "clock_mhz_observed": clock},
     }
+    if SUSTAIN_SECONDS > 0:
+        res["sustained"] = sustained(torch, ours, SUSTAIN_SECONDS)
     if clock and bound == "mfma":   # what the datasheet peak comes to at the clock the part actually held
         res["roofline"]["frac_at_observed_clock"] = achieved / (peak * clock / PEAK_CLOCK_MHZ)
     if with_hipblaslt:
@@ -297,8 +341,9 @@ def time_hipblaslt(torch, spec, buf, alpha, zero, a_ptrs, copies, steps, warmup,
                 raise RuntimeError("hipblasLtMatmul status %d" % st)
         wall, per_call, _ = time_calls(torch, theirs, steps, warmup)
         clock = observed_clock_mhz(torch, theirs, max(steps // NBATCH, 4), per_call)
+        sus = sustained(torch, theirs, SUSTAIN_SECONDS) if SUSTAIN_SECONDS > 0 else None
         rp.close()
-        return {"available": True, "ms_per_step": wall / steps * 1e3, "kernel_ms": per_call * 1e3, "clock_mhz_observed": clock,
+        return {"available": True, "sustained": sus, "ms_per_step": wall / steps * 1e3, "kernel_ms": per_call * 1e3, "clock_mhz_observed": clock,
                 "tops": ops / per_call / 1e12, "gbps": nbytes / per_call / 1e9}
     except Exception as e:  # the comparison point is optional; the product numbers are not
         return {"available": False, "why": "%s: %s" % (type(e).__name__, e)}
@@ -342,6 +387,9 @@ def main():
     ap.add_argument("--only", action="store_true", help="skip the other workloads")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-hipblaslt", action="store_true")
+    ap.add_argument("--sustained", type=float, default=0.0, metavar="SECONDS",
+                    help="also run every workload (and its hipBLASLt counterpart) back to back for this long with the "
+                         "board power sampled from hwmon: time, watts and energy per call at the power cap")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch one plain elementwise copy of 256 MiB (int32 in, int32 out): the known-size "
                          "kernel that calibrates FETCH_SIZE / WRITE_SIZE in a rocprofv3 --pmc run")
@@ -352,6 +400,8 @@ def main():
         sys.exit("bench.py needs a HIP device; there is no CPU path to benchmark")
     api = cublaslt.load()
     torch.cuda.init()
+    global SUSTAIN_SECONDS
+    SUSTAIN_SECONDS = args.sustained
     key = args.workload
     steps = args.steps or WORKLOADS[key]["steps"]
     if args.copy_probe:
@@ -382,6 +432,7 @@ def main():
         "clock_mhz_observed": head["roofline"].get("clock_mhz_observed"),
         "frac_at_observed_clock": head["roofline"].get("frac_at_observed_clock"),
         "cpu_baseline": None if args.no_cpu else cpu_baseline(key),
+        "sustained": head.get("sustained"),
         "hipblaslt_forwarded": head.get("hipblaslt_forwarded"),
         "device": torch.cuda.get_device_name(0), "cu_count": api.zluda_gemm_device_cu_count(),
         "also": also,
