@@ -8,7 +8,8 @@ on.  The other benchmark configurations, the 8192^3 int8 case and configuration 
 ride along under "also", each with its own roofline figures and, when the installed hipBLASLt has a
 solution, the time of the reference's hipBLASLt-forwarded path on the same buffers.
 
-Timing: W warm-up calls, then exactly K calls between two synchronisations (wall clock -> `value`); HIP
+Timing: W warm-up calls (default: half a second's worth, so that the power management has settled), then
+exactly K calls between two synchronisations (wall clock -> `value`); HIP
 events on the launch stream split the K calls into five batches, and `roofline.kernel_ms` is the median
 batch.  A one-wave probe kernel on a second stream samples the shader cycle counter against the real-time
 counter during one more (untimed) batch: `clock_mhz_observed`, and `frac_at_observed_clock` = the
@@ -172,11 +173,28 @@ class Buffers:
 NBATCH = 5
 
 
+AUTO_WARMUP_SECONDS = 0.5
+
+
 def time_calls(torch, fn, steps, warmup):
-    """`warmup` untimed calls, then exactly `steps` calls between two synchronisations.  Returns (wall seconds
-    for the `steps` calls, median over NBATCH equal batches of the seconds per call by HIP events on the launch
-    stream, [seconds per call of each batch])."""
-    for i in range(warmup):
+    """`warmup` untimed calls, then exactly `steps` calls between two synchronisations.  warmup < 0: as many
+    calls as take AUTO_WARMUP_SECONDS (at least 10) -- the power management needs a few hundred milliseconds
+    of load to settle, and a burst measured before that is up to 15 % slower than what a long-running job sees.
+    Returns (wall seconds for the `steps` calls, median over NBATCH equal batches of the seconds per call by HIP
+    events on the launch stream, [seconds per call of each batch], warm-up calls made)."""
+    if warmup < 0:
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(10):
+            fn(i)
+        e1.record()
+        e1.synchronize()
+        per = max(e0.elapsed_time(e1) * 1e-3 / 10, 1e-6)
+        warmup = 10 + min(int(AUTO_WARMUP_SECONDS / per), 100000)
+        first = 10
+    else:
+        first = 0
+    for i in range(first, warmup):
         fn(i)
     torch.cuda.synchronize()
     nb = NBATCH if steps % NBATCH == 0 else 1
@@ -191,7 +209,7 @@ def time_calls(torch, fn, steps, warmup):
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     batches = sorted(ev[b].elapsed_time(ev[b + 1]) * 1e-3 / per for b in range(nb))
-    return wall, batches[len(batches) // 2], batches
+    return wall, batches[len(batches) // 2], batches, warmup
 
 
 _probe = None
@@ -292,14 +310,14 @@ def run_workload(torch, api, key, steps, warmup, with_hipblaslt):
         st = call.run(alpha, a_ptrs[i % copies], bp, zero, None, dp, None, 0, stream)
         if st:
             raise RuntimeError("cublasLtMatmul status %d on workload %s" % (st, key))
-    wall, per_call, batches = time_calls(torch, ours, steps, warmup)
+    wall, per_call, batches, warmed = time_calls(torch, ours, steps, warmup)
     bound = "hbm" if w["kind"] == "hbm" else "mfma"
     achieved = (nbytes / per_call / 1e9) if bound == "hbm" else (ops / per_call / 1e12)
     peak = PEAK[w["kind"]]
     traffic, traffic_file = measured_traffic(key)
     clock = observed_clock_mhz(torch, ours, max(steps // NBATCH, 4), per_call)
     res = {
-        "workload": w["name"], "steps": steps, "ms_per_step": wall / steps * 1e3,
+        "workload": w["name"], "steps": steps, "warmup": warmed, "ms_per_step": wall / steps * 1e3,
         "tops": ops / (wall / steps) / 1e12, "gbps": nbytes / (wall / steps) / 1e9,
         "kernel": {"family": call.kernel, "variant": call.variant},
         "roofline": {"bound": bound, "achieved": achieved, "peak": peak, "unit": "GB/s" if bound == "hbm" else "TFLOP/s",
@@ -339,7 +357,7 @@ def time_hipblaslt(torch, spec, buf, alpha, zero, a_ptrs, copies, steps, warmup,
             st = rp.run(alpha, a_ptrs[i % copies], bp, zero, None, dp, stream)
             if st:
                 raise RuntimeError("hipblasLtMatmul status %d" % st)
-        wall, per_call, _ = time_calls(torch, theirs, steps, warmup)
+        wall, per_call, _, _ = time_calls(torch, theirs, steps, warmup)
         clock = observed_clock_mhz(torch, theirs, max(steps // NBATCH, 4), per_call)
         sus = sustained(torch, theirs, SUSTAIN_SECONDS) if SUSTAIN_SECONDS > 0 else None
         rp.close()
@@ -382,7 +400,8 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=0)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=-1,
+                    help="untimed calls before the timed ones; default: as many as take %.1f s (at least 10)" % AUTO_WARMUP_SECONDS)
     ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS))
     ap.add_argument("--only", action="store_true", help="skip the other workloads")
     ap.add_argument("--no-cpu", action="store_true")
@@ -425,7 +444,7 @@ def main():
     line = {
         "metric": "cublasLtMatmul TOPS (int8/fp8/MXFP4, 8192^3) + decode GEMM HBM GB/s",
         "value": head["gbps"] if unit == "GB/s" else head["tops"], "unit": unit, "n_gpus": 1, "steps": steps,
-        "warmup": args.warmup, "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak",
+        "warmup": head["warmup"], "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": {"i8": "int8", "hbm": "int8", "f8": "fp8_e4m3", "f4": "fp4_e2m1"}[WORKLOADS[key]["kind"]],
         "data": "synthetic", "config": {"workload": head["workload"], "kernel": head["kernel"]},
         "roofline": head["roofline"],
