@@ -66,7 +66,11 @@ def test_extents_that_256_divides_badly_get_the_192_row_tile(api):
     st, p = plan(api, dict(I8, m=8192, n=8192, k=8192, transa=1))
     assert st == 0 and p.variant == 8
     st, p = plan(api, dict(F8, m=14336, n=4096, k=4096, transa=1))   # 5 rounds of 192x256 lose to 4 of 256x256
+    assert st == 0 and p.variant == 0                                # (fp8 takes the 16x16-shape 256x256 tile from four full rounds on)
+    st, p = plan(api, dict(F8, m=8192, n=8192, k=8192, transa=1))
     assert st == 0 and p.variant == 8
+    st, p = plan(api, dict(F8, m=8192, n=4096, k=4096, transa=1))
+    assert st == 0 and p.variant == 0
     st, p = plan(api, dict(MX, m=8192, n=8192, k=8192, transa=1))      # MXFP4 has no 16x16-shape variant
     assert st == 0 and p.variant == 0
     assert plan(api, dict(MX, m=8192, n=8192, k=8192, transa=1), forced=K.ZLUDA_KERNEL_MFMA_MXF4, variant=8)[0] == K.CUBLAS_STATUS_INVALID_VALUE

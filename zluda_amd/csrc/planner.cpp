@@ -349,9 +349,11 @@ static int pick_mfma_variant(const Lowered &l, uint32_t cus) {
     const uint64_t tiles = (uint64_t)ceil_div(np, t.bp) * ceil_div(nq, t.bq) * g.batch;
     if (t.m16) {
       if (g.a_type == CUDA_R_4F_E2M1) continue;  // the 16x16 shapes serve int8 and fp8
-      // power bound or not: int8 gains from three quarters of the CUs busy on, fp8 (a small gain) from two
-      // full rounds on
-      if (g.a_type == CUDA_R_8I ? tiles * 4 < (uint64_t)cus * 3 : tiles < 2ull * cus) continue;
+      // power bound or not: int8 gains from three quarters of the CUs busy on.  fp8 gains little and only on
+      // long runs: the 192x256 tile from two full rounds on (6144^3: 190 us against 198), the 256x256 tile
+      // from four (8192^3: 405 against 408; at two rounds, 8192x4096x4096, it loses 3 %)
+      const uint64_t need = g.a_type == CUDA_R_8I ? ((uint64_t)cus * 3 + 3) / 4 : (uint64_t)cus * (t.bp == 256 ? 4 : 2);
+      if (tiles < need) continue;
     }
     const uint64_t rounds = (tiles + cus - 1) / cus;
     const double cost = (double)rounds * t.bp * t.bq / kMfmaVariantEfficiency[v];
