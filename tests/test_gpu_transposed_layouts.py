@@ -37,7 +37,7 @@ def test_baseline_config_1_runs_on_the_transposing_kernel(gpu_api):
     check(gpu_api, dict(I8, m=256, n=256, k=256, transa=0, transb=1, alpha=1), 0, expect_kernel=TR8)
 
 
-@pytest.mark.parametrize("variant", range(3))
+@pytest.mark.parametrize("variant", range(4))
 @pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 1), (1, 0)])
 def test_int8_every_transpose_combination(gpu_api, variant, ta, tb):
     # full tiles, ragged edges (rows not a multiple of 4 or 8, K not a multiple of 64), padded lds
@@ -60,7 +60,7 @@ def test_int8_k_tail_of_the_transposed_operand(gpu_api, ta, tb):
                             ldb=(k + (-k) % 4 if tb == 0 else 64)), 230 + k, TR8, 0)
 
 
-@pytest.mark.parametrize("variant", range(3))
+@pytest.mark.parametrize("variant", range(4))
 def test_int8_row_major_operands_and_output(gpu_api, variant):
     # row-major A (m x k, K-contiguous) with row-major B (k x n, N-contiguous) -> row-major D: the
     # everyday "activations x weights" layout of row-major frameworks
@@ -70,7 +70,7 @@ def test_int8_row_major_operands_and_output(gpu_api, variant):
     check(gpu_api, dict(spec, transa=1, order_c=0, order_d=0), 242, TR8, variant)
 
 
-@pytest.mark.parametrize("variant", range(3))
+@pytest.mark.parametrize("variant", range(4))
 def test_int8_batched_float_epilogue(gpu_api, variant):
     spec = dict(I8F, transa=0, transb=1, m=260, n=140, k=320, batch=3, epilogue=K.CUBLASLT_EPILOGUE_RELU_BIAS,
                 bias_type=K.CUDA_R_32F, pointer_mode=K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_HOST,

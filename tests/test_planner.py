@@ -104,16 +104,20 @@ def test_misaligned_or_strided_operands_leave_the_dma_kernels(api):
     assert plan(api, dict(spec, transa=0, transb=0, k=112, ldb=112))[1].kernel == TR8
     assert plan(api, dict(spec, transa=0, lda=518))[1].kernel == GEN                   # stride of a K row % 4
     # tile choice: 256x256 once every CU gets one, 64x64 for what would leave CUs idle
+    # (variant 3 is variant 0's tile on the 16x16 MFMA shape: int8 grids that fill the chip)
     st, p = plan(api, dict(spec, transa=0, transb=1, m=4096, n=4096))
-    assert st == 0 and p.kernel == TR8 and p.variant == 0 and p.grid_x == 256 and p.block == 512
+    assert st == 0 and p.kernel == TR8 and p.variant == 3 and p.grid_x == 256 and p.block == 512
     st, p = plan(api, dict(spec, transa=0, transb=1, m=4096, n=1024, k=4096))
     assert st == 0 and p.variant == 1 and p.grid_x == 256 and p.block == 256
     st, p = plan(api, dict(spec, transa=0, transb=1, m=1024, n=1024, k=1024))
     assert st == 0 and p.variant == 2 and p.grid_x == 256 and p.block == 256
     st, p = plan(api, dict(spec, transa=0, transb=1, m=8192, n=4096, k=1024))
-    assert st == 0 and p.variant == 0 and p.grid_x == 512
-    assert api.zluda_gemm_variant_count(TR8) == 3
-    assert plan(api, dict(spec, transa=0, transb=1), forced=TR8, variant=3)[0] == K.CUBLAS_STATUS_INVALID_VALUE
+    assert st == 0 and p.variant == 3 and p.grid_x == 512
+    st, p = plan(api, dict(spec, transa=0, transb=1, m=8192, n=4096, k=1024, a_type=K.CUDA_R_8F_E4M3, b_type=K.CUDA_R_8F_E4M3,
+                           d_type=K.CUDA_R_16BF, compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F))
+    assert st == 0 and p.kernel == TR8 and p.variant == 0                      # fp8 stays on the 32x32 shape
+    assert api.zluda_gemm_variant_count(TR8) == 4
+    assert plan(api, dict(spec, transa=0, transb=1), forced=TR8, variant=4)[0] == K.CUBLAS_STATUS_INVALID_VALUE
     assert plan(api, dict(MX, m=256, n=256, k=512, transa=1), forced=TR8)[0] == K.CUBLAS_STATUS_NOT_SUPPORTED
     # MXFP4 needs whole 256-element K stages for the MFMA kernel
     assert plan(api, dict(MX, m=256, n=256, k=384, transa=1))[1].kernel == GEN

@@ -25,7 +25,7 @@
 //     of 4 mod 64) and every ds_read_b128 of 16 consecutive matrix rows hits 16 distinct 16-byte
 //     groups (pitch 5 groups, 5 coprime to 16, rho of 16 consecutive rows distinct mod 16).
 #pragma once
-#include "gemm_mfma.hpp"
+#include "gemm_mfma_pipe16.hpp"
 
 namespace zluda_amd {
 
@@ -139,9 +139,14 @@ struct TrOperand {
   }
 };
 
-template <int KIND, int FQ, int FP, int BP, int BQ, int WP, int WQ, bool PKC, bool QKC>
+// M16 (int8 only): the MFMAs are v_mfma_i32_16x16x64_i8 with P as operand "A" and the epilogues of
+// gemm_mfma_pipe16.hpp -- the shape that needs less energy per multiply-add, for problems that keep the whole
+// chip busy (see there).  A fragment is then 16 rows x the 64 K bytes of a stage (lane l: row l%16, 16-byte
+// chunk l/16), one MFMA per pair of fragments and stage.
+template <int KIND, int FQ, int FP, int BP, int BQ, int WP, int WQ, bool PKC, bool QKC, bool M16 = false>
 __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_tr_kernel(MfmaParams prm) {
   static_assert(KIND == KIND_I8 || KIND == KIND_F8, "8-bit operands");
+  static_assert(!M16 || KIND == KIND_I8, "the 16x16 form is instantiated for int8");
   constexpr int NT = WP * WQ * 64;
   static_assert(NT == 256 || NT == 512, "operand rows are dealt to groups of 256 threads");
   constexpr int LP = BP * 256 / NT, LQ = BQ * 256 / NT;  // rows of P / Q one group loads
@@ -216,13 +221,57 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_tr_kernel(MfmaParams pr
     qrow[a] = (BP + i / LQ * LQ + tr_rho_of<LQ>(i % LQ)) * 5;
   }
 
-  acc_v acc[TQ][TP];
+  acc_v acc[M16 ? 1 : TQ][M16 ? 1 : TP];
+  if constexpr (!M16) {
 #pragma unroll
-  for (int a = 0; a < TQ; a++)
+    for (int a = 0; a < TQ; a++)
 #pragma unroll
-    for (int b = 0; b < TP; b++)
+      for (int b = 0; b < TP; b++)
 #pragma unroll
-      for (int v = 0; v < 16; v++) acc[a][b][v] = 0;
+        for (int v = 0; v < 16; v++) acc[a][b][v] = 0;
+  }
+  // ---- the 16x16 form ------------------------------------------------------------------------------
+  constexpr int TP16 = WTP / 16, TQ16 = WTQ / 16, HP16 = TP16 / 2;
+  v4i acc16[M16 ? TP16 : 1][M16 ? TQ16 : 1];
+  int prow16[M16 ? TP16 : 1], qrow16[M16 ? TQ16 : 1];  // this lane's 16-byte piece of each fragment (v4i units)
+  if constexpr (M16) {
+    const int r16 = lane & 15, g4 = lane >> 4;
+#pragma unroll
+    for (int b = 0; b < TP16; b++) {
+      const int i = wp * WTP + b * 16 + r16;
+      prow16[b] = (i / LP * LP + tr_rho_of<LP>(i % LP)) * 5 + g4;
+    }
+#pragma unroll
+    for (int a = 0; a < TQ16; a++) {
+      const int i = wq * WTQ + a * 16 + r16;
+      qrow16[a] = (BP + i / LQ * LQ + tr_rho_of<LQ>(i % LQ)) * 5 + g4;
+    }
+#pragma unroll
+    for (int b = 0; b < TP16; b++)
+#pragma unroll
+      for (int a = 0; a < TQ16; a++) acc16[b][a] = v4i{0, 0, 0, 0};
+  }
+  // fragment registers: both halves of P (the second is read while the first is multiplied) and the Q
+  // fragments of two stages (the next stage's arrive while this stage's are still in use)
+  v4i fp16[2][M16 ? HP16 : 1], fq16[2][M16 ? TQ16 : 1];
+  auto read_p16 = [&](const v4i *buf, auto h_c) {
+    constexpr int h = decltype(h_c)::value;
+#pragma unroll
+    for (int i = 0; i < HP16; i++) fp16[h][i] = buf[prow16[h * HP16 + i]];
+  };
+  auto read_q16 = [&](const v4i *buf, auto s_c) {
+    constexpr int sidx = decltype(s_c)::value;
+#pragma unroll
+    for (int a = 0; a < TQ16; a++) fq16[sidx][a] = buf[qrow16[a]];
+  };
+  auto mfma16 = [&](auto h_c, auto s_c) {
+    constexpr int h = decltype(h_c)::value, sidx = decltype(s_c)::value;
+#pragma unroll
+    for (int i = 0; i < HP16; i++)
+#pragma unroll
+      for (int a = 0; a < TQ16; a++)
+        acc16[h * HP16 + i][a] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fp16[h][i], fq16[sidx][a], acc16[h * HP16 + i][a], 0, 0, 0);
+  };
 
   // fragments of sub-step ks of the stage in `buf`
   struct Frags { frag_v p[TP], q[TQ]; };
@@ -324,6 +373,64 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_tr_kernel(MfmaParams pr
     __builtin_amdgcn_sched_barrier(0);
   };
 
+  // The same trip on the 16x16 form.  PAR = kt & 1 selects the Q register set.  Entered with P half 0 and the
+  // Q fragments of stage kt in registers.
+  //   first half : MFMAs of P half 0; P half 1 is read and stage kt+1 transposed into `nxt` between them;
+  //   barrier;
+  //   second half: MFMAs of P half 1 cover the loads of stage kt+3 and the reads of stage kt+1's P half 0 and Q.
+  auto stage_trip16 = [&](int kt, const v4i *cur, v4i *nxt, int (&sp)[P.NREG], int (&sq)[Q.NREG], auto par_c) {
+    constexpr int PAR = decltype(par_c)::value;
+    using H0 = std::integral_constant<int, 0>;
+    using H1 = std::integral_constant<int, 1>;
+    using SC = std::integral_constant<int, PAR>;
+    using SN = std::integral_constant<int, 1 - PAR>;
+    if (kt >= tail_from) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    read_p16(cur, H1{});
+    P.store(tl, nxt + lds_p, sp);
+    Q.store(tl, nxt + lds_q, sq);
+    mfma16(H0{}, SC{});
+    {
+      constexpr int NM = HP16 * TQ16, H = NM / 2 > 0 ? NM / 2 : 1;
+      constexpr int NDR = HP16;
+      constexpr int NPERM = ((PKC ? 0 : P.NREG * 2) + (QKC ? 0 : Q.NREG * 2));
+      constexpr int NDW = (PKC ? P.NCH : P.NREG) + (QKC ? Q.NCH : Q.NREG);
+      static_for<NM>([&](auto i_c) {
+        constexpr int i = decltype(i_c)::value;
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        if constexpr (i < H) {
+          constexpr int nr = NDR * (i + 1) / H - NDR * i / H;
+          if constexpr (nr > 0) __builtin_amdgcn_sched_group_barrier(0x100, nr, 0);
+          constexpr int nv = NPERM * (i + 1) / H - NPERM * i / H;
+          if constexpr (nv > 0) __builtin_amdgcn_sched_group_barrier(0x002, nv, 0);
+        } else {
+          constexpr int nw = NDW * (i - H + 1) / (NM - H) - NDW * (i - H) / (NM - H);
+          if constexpr (nw > 0) __builtin_amdgcn_sched_group_barrier(0x200, nw, 0);
+        }
+      });
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+    P.load(min(kt + 3, KL), sp);
+    Q.load(min(kt + 3, KL), sq);
+    read_p16(nxt, H0{});
+    read_q16(nxt, SN{});
+    mfma16(H1{}, SC{});
+    {
+      constexpr int NM = HP16 * TQ16, NDR = HP16 + TQ16;
+      constexpr int NVM = (PKC ? P.NCH : 4) + (QKC ? Q.NCH : 4);
+      static_for<NM>([&](auto i_c) {
+        constexpr int i = decltype(i_c)::value;
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        constexpr int nr = NDR * (i + 1) / NM - NDR * i / NM;
+        if constexpr (nr > 0) __builtin_amdgcn_sched_group_barrier(0x100, nr, 0);
+        constexpr int nv = NVM * (i + 1) / NM - NVM * i / NM;
+        if constexpr (nv > 0) __builtin_amdgcn_sched_group_barrier(0x020, nv, 0);
+      });
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
   // two register sets per operand: stage s travels through set s & 1
   int rp0[P.NREG], rp1[P.NREG], rq0[Q.NREG], rq1[Q.NREG];
   v4i *buf0 = &lds[0], *buf1 = &lds[STAGE_V4];
@@ -335,14 +442,33 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_tr_kernel(MfmaParams pr
   Q.store(tl, buf0 + lds_q, rq0);
   __syncthreads();
   P.load(min(2, KL), rp0); Q.load(min(2, KL), rq0);
-  read_frags(buf0, 0, f0);
-  for (int kt = 0; kt < KT; kt += 2) {
-    stage_trip(kt, buf0, buf1, rp1, rq1, f0);
-    if (kt + 1 < KT) stage_trip(kt + 1, buf1, buf0, rp0, rq0, f0);
+  if constexpr (M16) {
+    read_p16(buf0, std::integral_constant<int, 0>{});
+    read_q16(buf0, std::integral_constant<int, 0>{});
+    for (int kt = 0; kt < KT; kt += 2) {
+      stage_trip16(kt, buf0, buf1, rp1, rq1, std::integral_constant<int, 0>{});
+      if (kt + 1 < KT) stage_trip16(kt + 1, buf1, buf0, rp0, rq0, std::integral_constant<int, 1>{});
+    }
+  } else {
+    read_frags(buf0, 0, f0);
+    for (int kt = 0; kt < KT; kt += 2) {
+      stage_trip(kt, buf0, buf1, rp1, rq1, f0);
+      if (kt + 1 < KT) stage_trip(kt + 1, buf1, buf0, rp0, rq0, f0);
+    }
   }
 
   // every wave is done with the LDS stages before they become epilogue staging
   __syncthreads();
+  if constexpr (M16) {
+    if (prm.splits > 1) {
+      const int ws_np = prm.tiles_p * BP, ws_nq = prm.tiles_q * BQ;
+      int32_t *ws_tile = (int32_t *)prm.ws + ((int64_t)blockIdx.z * g.batch + bt) * ws_np * ws_nq + (int64_t)(q0 + wq * WTQ) * ws_np + p0 + wp * WTP;
+      const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)ws_tile, 0, 0xFFFFFFFF, 0x00020000);
+      mfma16_store_raw<TP16, TQ16>(rs, ws_np, acc16, 1);
+      return;
+    }
+    mfma16_store_tile<KIND, WP, WQ, TP16, TQ16, (int)sizeof(lds)>(prm, acc16, (int *)&lds[0], p0, q0, NP, NQ, bt);
+  } else {
   if (prm.splits > 1) {
     const int ws_np = prm.tiles_p * BP, ws_nq = prm.tiles_q * BQ;
     int32_t *ws_tile = (int32_t *)prm.ws + ((int64_t)blockIdx.z * g.batch + bt) * ws_np * ws_nq + (int64_t)q0 * ws_np + p0;
@@ -350,6 +476,7 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_tr_kernel(MfmaParams pr
     return;
   }
   mfma_store_tile<KIND, WP, WQ, WTP, WTQ>(prm, acc, (int *)&lds[0], sizeof(lds), p0, q0, NP, NQ, bt);
+  }
 }
 
 } // namespace zluda_amd

@@ -20,7 +20,7 @@ inline uint32_t launch_tr_variant(const MfmaParams &prm, const zluda_gemm_plan &
 #define ZLUDA_TR_CASE(V, BP, BQ, WP, WQ)                                                                        \
   case V:                                                                                                       \
     static_assert(kTrVariants[V].bp == BP && kTrVariants[V].bq == BQ && kTrVariants[V].wp == WP &&              \
-                  kTrVariants[V].wq == WQ, "variant table mismatch");                                           \
+                  kTrVariants[V].wq == WQ && !kTrVariants[V].m16, "variant table mismatch");                                           \
     ZLUDA_TR_MODE(BP, BQ, WP, WQ, false, false) ZLUDA_TR_MODE(BP, BQ, WP, WQ, false, true)                      \
     ZLUDA_TR_MODE(BP, BQ, WP, WQ, true, false) ZLUDA_TR_MODE(BP, BQ, WP, WQ, true, true)                        \
     break;
@@ -28,6 +28,17 @@ inline uint32_t launch_tr_variant(const MfmaParams &prm, const zluda_gemm_plan &
     ZLUDA_TR_CASE(0, 256, 256, 2, 4)
     ZLUDA_TR_CASE(1, 128, 128, 2, 2)
     ZLUDA_TR_CASE(2, 64, 64, 2, 2)
+  case 3:  // variant 0's tile on the 16x16 MFMA shape (int8)
+    static_assert(kTrVariants[3].bp == 256 && kTrVariants[3].bq == 256 && kTrVariants[3].wp == 2 && kTrVariants[3].wq == 4 &&
+                  kTrVariants[3].m16, "variant table mismatch");
+    if constexpr (KIND == KIND_I8) {
+#define ZLUDA_TR16_MODE(PK, QK)                                                                                  \
+  if (pkc == PK && qkc == QK)                                                                                    \
+    return launch_kernel(gemm_mfma_tr_kernel<KIND, FQ, FP, 256, 256, 2, 4, PK, QK, true>, grid, dim3(512), s, prm);
+      ZLUDA_TR16_MODE(false, false) ZLUDA_TR16_MODE(false, true) ZLUDA_TR16_MODE(true, false) ZLUDA_TR16_MODE(true, true)
+#undef ZLUDA_TR16_MODE
+    }
+    break;
   default: break;
   }
 #undef ZLUDA_TR_CASE

@@ -399,7 +399,7 @@ static void fill_tr_plan(const Lowered &l, int variant, uint32_t cus, uint64_t w
 // 256x256: 71;  128x128: 37 alone, 48 for two;  64x64: 22 alone, 40 for four  ->  base + slope * n.
 // Cost of a variant = full rounds x time(per_cu) + time(what is left per CU).
 struct TrCost { uint32_t per_cu; float base, slope; };
-static const TrCost kTrCost[kNumTrVariants] = {{1, 0.0f, 71.0f}, {2, 26.0f, 11.0f}, {4, 16.0f, 6.0f}};
+static const TrCost kTrCost[kNumTrVariants] = {{1, 0.0f, 71.0f}, {2, 26.0f, 11.0f}, {4, 16.0f, 6.0f}, {1, 0.0f, 67.0f}};
 
 static int pick_tr_variant(const Lowered &l, uint32_t cus) {
   const GemmArgs &g = l.g;
@@ -411,6 +411,8 @@ static int pick_tr_variant(const Lowered &l, uint32_t cus) {
     const TrVariant &t = kTrVariants[v];
     const TrCost &c = kTrCost[v];
     const uint64_t tiles = (uint64_t)ceil_div(np, t.bp) * ceil_div(nq, t.bq) * g.batch;
+    // the 16x16 shape: int8 only, and only where the chip is full enough to sit at its power cap
+    if (t.m16 && (g.a_type != CUDA_R_8I || tiles * 4 < (uint64_t)cus * 3)) continue;
     const uint64_t slots = (uint64_t)cus * c.per_cu;
     const uint64_t full = tiles / slots, rem = tiles % slots;
     double cost = (double)full * (c.base + c.slope * c.per_cu);
@@ -526,7 +528,7 @@ extern "C" uint32_t zluda_gemm_plan_problem(const zluda_gemm_problem *p, uint32_
   }
   case ZLUDA_KERNEL_MFMA_TR8: {
     int v = forced_variant >= 0 ? forced_variant : pick_tr_variant(l, cu_count);
-    if (v >= kNumTrVariants) return CUBLAS_STATUS_INVALID_VALUE;
+    if (v >= kNumTrVariants || (kTrVariants[v].m16 && l.g.a_type != CUDA_R_8I)) return CUBLAS_STATUS_INVALID_VALUE;
     fill_tr_plan(l, v, cu_count, p->workspace_size, plan);
     break;
   }
