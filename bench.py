@@ -215,17 +215,39 @@ def time_calls(torch, fn, steps, warmup):
 _probe = None
 
 
+def load_probe():
+    """the measurement helpers of zluda_amd/csrc/bench (None when not built)"""
+    global _probe
+    path = os.path.join(ROOT, "zluda_amd", "lib", "libzluda_bench_probe.so")
+    if _probe is None and os.path.exists(path):
+        _probe = C.CDLL(path)
+        _probe.zluda_bench_clock_probe.argtypes = [C.c_void_p, C.c_uint64, C.c_void_p]
+        _probe.zluda_bench_flat_read.argtypes = [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]
+    return _probe
+
+
+def flat_read_seconds(torch, buffers, steps, warmup):
+    """A plain read of the same weight buffers, rotated the same way, one kernel launch each: the practical
+    ceiling of a memory-bound kernel over these bytes on this GPU.  Seconds per launch, or None."""
+    probe = load_probe()
+    if probe is None:
+        return None
+    sink = torch.zeros(1, dtype=torch.int32, device="cuda:0")
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def fn(i):
+        t = buffers[i % len(buffers)]
+        if probe.zluda_bench_flat_read(t.data_ptr(), t.numel() * t.element_size(), sink.data_ptr(), stream) != 0:
+            raise RuntimeError("flat read launch failed")
+    return time_calls(torch, fn, steps, warmup)[1]
+
+
 def observed_clock_mhz(torch, fn, calls, seconds_per_call):
     """Shader clock held while `calls` more calls of `fn` run: a one-wave kernel on a second stream reads the
     shader cycle counter and the constant-rate real-time counter at both ends of ~80 % of that stretch.
     None when the helper library is missing."""
-    global _probe
-    path = os.path.join(ROOT, "zluda_amd", "lib", "libzluda_bench_probe.so")
-    if _probe is None:
-        if not os.path.exists(path):
-            return None
-        _probe = C.CDLL(path)
-        _probe.zluda_bench_clock_probe.argtypes = [C.c_void_p, C.c_uint64, C.c_void_p]
+    if load_probe() is None:
+        return None
     khz = _probe.zluda_bench_wall_clock_khz()
     if khz <= 0:
         return None
@@ -325,6 +347,11 @@ def run_workload(torch, api, key, steps, warmup, with_hipblaslt):
                      "kernel_ms": per_call * 1e3, "kernel_ms_batches": [b * 1e3 for b in batches],
                      "algorithmic_ops": ops, "algorithmic_bytes": nbytes, "clock_mhz_observed": clock},
     }
+    if bound == "hbm":   # beside the streaming kernel: what a plain read of the same weights takes
+        flat = flat_read_seconds(torch, buf.A, steps, warmup)
+        if flat:
+            res["roofline"]["flat_read_ms"] = flat * 1e3
+            res["roofline"]["flat_read_gbps"] = sum(a.numel() for a in buf.A[:1]) / flat / 1e9
     if SUSTAIN_SECONDS > 0:
         res["sustained"] = sustained(torch, ours, SUSTAIN_SECONDS)
     if clock and bound == "mfma":   # what the datasheet peak comes to at the clock the part actually held

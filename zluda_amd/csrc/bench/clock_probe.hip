@@ -33,3 +33,24 @@ extern "C" __attribute__((visibility("default"))) int zluda_bench_wall_clock_khz
   if (hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev) != hipSuccess) return 0;
   return khz;
 }
+
+// A flat read of `bytes` (a multiple of 16) bytes: every lane walks the buffer 16 bytes at a time, the whole
+// grid one contiguous stripe per step -- the shortest time in which this GPU can pull that many bytes out of
+// HBM with one kernel launch, i.e. the practical ceiling of a memory-bound kernel over the same data.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(512) void flat_read_kernel(const u32x4 *src, uint64_t n16, uint32_t *sink) {
+  uint32_t acc = 0;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (uint64_t)gridDim.x * blockDim.x) {
+    const u32x4 v = src[i];
+    acc ^= v[0] ^ v[1] ^ v[2] ^ v[3];
+  }
+  if (acc == 0x9e3779b9u) sink[0] = acc;  // (keeps the loads alive; practically never taken)
+}
+
+// src: device buffer of `bytes` bytes, sink: one device dword; returns hipError_t
+extern "C" __attribute__((visibility("default"))) int zluda_bench_flat_read(const void *src, uint64_t bytes, uint32_t *sink, void *stream) {
+  const u32x4 *s4 = (const u32x4 *)src;
+  uint64_t n16 = bytes / 16;
+  void *args[] = {&s4, &n16, &sink};
+  return (int)hipLaunchKernel((const void *)flat_read_kernel, dim3(1024), dim3(512), args, 0, (hipStream_t)stream);
+}
