@@ -37,8 +37,8 @@ def test_baseline_configs_pick_the_intended_kernels(api):
                            pointer_mode=K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO,
                            b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F,
                            epilogue=K.CUBLASLT_EPILOGUE_BIAS, bias_type=K.CUDA_R_32F))       # config 3
-    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.swapped == 0 and p.block == 512
-    assert p.variant == 4 and p.grid_x == 256      # streamed through LDS, one 8-wave workgroup per CU
+    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.swapped == 0 and p.block == 256
+    assert p.variant == 16 and p.grid_x == 224     # streamed through LDS in slabs: 896 blocks of 16 rows, 4 per workgroup
     st, p = plan(api, dict(F8, m=8192, n=8192, k=8192, transa=1, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS))  # config 4
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_F8 and p.grid_x == 1024
     st, p = plan(api, dict(MX, m=8192, n=8192, k=8192, transa=1, batch=4))          # config 5
@@ -185,14 +185,14 @@ def test_decode_k_between_the_stream_instantiations(api):
                pointer_mode=K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO,
                b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F,
                epilogue=K.CUBLASLT_EPILOGUE_BIAS, bias_type=K.CUDA_R_32F)
-    st, p = plan(api, dict(dec, m=14336, n=16, k=4096))                       # exactly one instantiation's cover
+    st, p = plan(api, dict(dec, m=14336, n=17, k=4096))                       # exactly one instantiation's cover
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.variant == 4
     for ws in (0, 64 << 20):
         st, p = plan(api, dict(dec, m=5120, n=16, k=13824), workspace=ws)     # under the 14336 cover
         assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.variant == 6 and p.workspace == 0
     st, p = plan(api, dict(dec, m=18944, n=32, k=3584))                       # under the 4096 cover, two token blocks
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.variant == 4
-    st, p = plan(api, dict(dec, m=2048, n=16, k=2560), workspace=64 << 20)    # under the 3072 cover
+    st, p = plan(api, dict(dec, m=2048, n=17, k=2560), workspace=64 << 20)    # under the 3072 cover
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.variant == 13
     st, p = plan(api, dict(dec, m=4096, n=16, k=11008))                       # under the 12288 cover
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.variant == 9
@@ -205,9 +205,37 @@ def test_decode_k_between_the_stream_instantiations(api):
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_I8 and p.grid_z == 1
 
 
+def test_decode_slab_form_takes_one_token_block_under_4096(api):
+    """the slab form of the stream kernel: up to 16 tokens, 2048 < K <= 4096, int8 or e4m3, as long as 4 blocks of 16 rows
+    per CU hold the matrix; its grid is the fewest rounds of blocks shared out evenly"""
+    dec = dict(I8, transa=1, d_type=K.CUDA_R_16BF, scale_type=K.CUDA_R_32F,
+               pointer_mode=K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO,
+               b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F,
+               epilogue=K.CUBLASLT_EPILOGUE_BIAS, bias_type=K.CUDA_R_32F)
+    DEC = K.ZLUDA_KERNEL_DECODE_W8A8
+    for spec, grid in ((dict(dec, m=14336, n=16, k=4096), 224), (dict(dec, m=14336, n=1, k=3584), 224),
+                       (dict(dec, m=2048, n=16, k=2560), 128), (dict(dec, m=16384, n=9, k=4096), 256),
+                       (dict(F8, transa=1, m=14336, n=16, k=4096), 224), (dict(dec, m=4100, n=16, k=2064), 129)):
+        st, p = plan(api, spec)
+        assert st == 0 and p.kernel == DEC and p.variant == 16 and p.grid_x == grid and p.block == 256 and p.workspace == 0, (spec, p.variant, p.grid_x)
+    # tokens along M: the weights are operand B
+    st, p = plan(api, dict(dec, transa=0, transb=1, order_a=1, order_b=1, order_c=1, order_d=1, m=16, n=4096, k=4096))
+    assert st == 0 and p.kernel == DEC and p.variant == 16 and p.swapped == 1
+    # outside its range: a second token block, K of at most half the cover or beyond it, more rows than 64 per CU
+    for spec, variant in ((dict(dec, m=14336, n=17, k=4096), 4), (dict(dec, m=4096, n=16, k=2048), 7),
+                          (dict(dec, m=4096, n=16, k=4112), 14), (dict(dec, m=16400, n=16, k=4096), 4)):
+        st, p = plan(api, spec)
+        assert st == 0 and p.kernel == DEC and p.variant == variant, (spec, p.variant)
+        assert plan(api, spec, forced=DEC, variant=16)[0] == (0 if spec["m"] == 16400 else K.CUBLAS_STATUS_NOT_SUPPORTED)
+    st, p = plan(api, dict(dec, m=16400, n=16, k=4096), forced=DEC, variant=16)   # forced: more workgroups than CUs
+    assert st == 0 and p.grid_x == 257
+    st, p = plan(api, dict(dec, m=14336, n=16, k=4096), cus=64)                   # a smaller device: too many rows
+    assert st == 0 and p.kernel == DEC and p.variant == 4
+
+
 def test_fp8_decode_takes_the_streaming_kernel_under_a_cover_only(api):
     f8 = dict(F8, transa=1)
-    st, p = plan(api, dict(f8, m=14336, n=16, k=4096))
+    st, p = plan(api, dict(f8, m=14336, n=17, k=4096))
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.variant == 4 and p.grid_x == 256
     st, p = plan(api, dict(f8, m=14336, n=48, k=4096))                      # up to 48 tokens while the variant applies
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8

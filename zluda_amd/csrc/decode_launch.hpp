@@ -3,7 +3,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
-#include "kernels/decode_stream.hpp"
+#include "kernels/decode_slab.hpp"
 #include "launch_util.hpp"
 #include "planner.hpp"
 
@@ -55,7 +55,7 @@ inline uint32_t launch_decode_stream_variant(const DecodeParams &prm, const zlud
   switch (plan.variant) {
 #define ZLUDA_STREAM_CASE(V, NW, SPW)                                                         \
   case V:                                                                                     \
-    static_assert(kDecodeVariants[V].nw == NW && kDecodeVariants[V].steps == SPW && kDecodeVariants[V].stream, \
+    static_assert(kDecodeVariants[V].nw == NW && kDecodeVariants[V].steps == SPW && kDecodeVariants[V].stream == 1, \
                   "variant table mismatch");                                                  \
     return launch_decode_stream<NW, SPW, KIND>(prm, plan, nb, s);
     ZLUDA_STREAM_CASE(4, 8, 8)
@@ -70,11 +70,31 @@ inline uint32_t launch_decode_stream_variant(const DecodeParams &prm, const zlud
     ZLUDA_STREAM_CASE(13, 4, 12)
     ZLUDA_STREAM_CASE(14, 4, 20)
     ZLUDA_STREAM_CASE(15, 8, 32)
+    static_assert(kDecodeVariants[16].stream == 2, "variant 16 is the slab kernel, launched by launch_decode_slab");
 #undef ZLUDA_STREAM_CASE
   default: return CUBLAS_STATUS_INVALID_VALUE;
   }
 }
 
+// the slab form of the stream kernel (kernels/decode_slab.hpp): up to 16 tokens, K <= 4096
+template <int KIND>
+inline uint32_t launch_decode_slab(const DecodeParams &prm, const zluda_gemm_plan &plan, hipStream_t s) {
+  dim3 grid(plan.grid_x, plan.grid_y, 1), block(kSlabWaves * 64);
+  // 0: element-wise epilogue, 1: packed store, 2: packed store behind a GELU
+  const int fast = !decode_packed_output(prm.g, prm.swapped != 0) ? 0 : prm.g.act == ACT_GELU ? 2 : 1;
+  const bool tail = prm.g.K < kSlabWaves * 1024;
+  uint32_t st = CUBLAS_STATUS_NOT_SUPPORTED;
+  static_for_host<3>([&](auto fast_c) {
+    constexpr int FAST = decltype(fast_c)::value;
+    if (fast == FAST)
+      st = tail ? launch_kernel(decode_slab_kernel<FAST, KIND, true>, grid, block, s, prm)
+                : launch_kernel(decode_slab_kernel<FAST, KIND, false>, grid, block, s, prm);
+  });
+  return st;
+}
+
+uint32_t launch_decode_slab_i8(const DecodeParams &prm, const zluda_gemm_plan &plan, hipStream_t s);
+uint32_t launch_decode_slab_f8(const DecodeParams &prm, const zluda_gemm_plan &plan, hipStream_t s);
 uint32_t launch_decode_stream_i8(const DecodeParams &prm, const zluda_gemm_plan &plan, int nb, hipStream_t s);
 uint32_t launch_decode_stream_f8(const DecodeParams &prm, const zluda_gemm_plan &plan, int nb, hipStream_t s);
 

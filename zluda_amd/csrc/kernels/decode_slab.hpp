@@ -1,0 +1,259 @@
+// Skinny (<= 16 tokens) W8A8 decode GEMM, slab form of the LDS-streaming kernel (decode_stream.hpp) for
+// 2048 < K <= 4096: the same math and epilogue, a different road for the bytes.
+//
+//   W : R rows x K int8 (or fp8 e4m3), K-contiguous (read exactly once)     X : T <= 16 rows x K, same type
+//   out(r, t) = sum_k W[r][k] * X[t][k]     int32 (fp32), then the fused float / integer epilogue
+//
+// What differs from decode_stream_kernel, and what each point bought on a 14336 x 4096 int8 matrix with 16
+// tokens (MI355X, 58.7 MB, a flat read of the same bytes takes 9.95 us; decode_stream_kernel 14.8 us):
+//   * One DMA instruction fetches ONE row x 1 KiB (64 lanes x 16 contiguous bytes) instead of 4 rows x 256
+//     bytes, a 16-row block of a wave's K slab is 16 instructions into a 16 KiB slot, two slots per wave.
+//     A workgroup is 4 waves, wave v owning K bytes [v*kw, (v+1)*kw) with kw <= 1024.
+//   * The activations take the same road once (one token x 1 KiB per instruction into the second slot, whole
+//     cache lines) and are copied to registers before that slot joins the weight ring; loading them in the
+//     MFMA layout straight from global memory asks for 64-byte pieces and costs ~1 us more.
+//   * A workgroup runs at most 4 blocks, keeps their accumulators in registers and meets the other waves
+//     ONCE, at the end: one barrier and one LDS round trip per workgroup instead of one per block.
+//   * Blocks are dealt out round-robin (block b of workgroup w = rows 16 * (b*G + w)), so that at any moment
+//     the grid reads one contiguous stripe of W; the rows left over after the last full round of G blocks are
+//     split evenly in quads of 4.  ~0.4 us against contiguous row ranges per workgroup.
+//   * The epilogue factors are fetched without a branch (a null vector reads a dummy address and is replaced
+//     by its scalar afterwards; a bias is read once as 16 and once as 32 bits).  With the usual
+//     "pointer ? load : scalar" and per-type bias loads the same kernel measures ~0.55 us slower, wherever
+//     in the kernel those loads are issued.
+// Together: 12.2-12.5 us.
+//
+// LDS slot layout: row rho (0..15) x 64 chunks of 16 bytes; chunk c of row rho sits at position
+// (c & 48) | ((c ^ rho) & 15) of the row's KiB: the DMA of a row lands linearly (lane l fetches the chunk whose
+// position is l) and the 16-rows-same-chunk fragment reads hit 16 different bank groups.
+#pragma once
+#include "decode_stream.hpp"
+
+namespace zluda_amd {
+
+constexpr int kSlabWaves = 4;       // K slabs (waves) per workgroup
+constexpr int kSlabMaxBlocks = 4;   // 16-row blocks a workgroup can run
+
+// FAST != 0 as in decode_stream_kernel: every output leaves through the packed 8-byte store (1: no activation or
+// ReLU, 2: GELU; whatever code sits between the last weights and the store is exposed in full, so the path of
+// the plain epilogue is kept free of branches).  TAIL = K < 4096 (lanes past a wave's slab or past K fetch
+// nothing and read as zero).
+constexpr int kSlabFactorLoads = 21;  // vector memory loads of the packed epilogue's factors, per lane
+template <int FAST, int KIND, bool TAIL>
+__global__ __launch_bounds__(kSlabWaves * 64) void decode_slab_kernel(DecodeParams prm) {
+  static_assert(KIND == KIND_I8 || KIND == KIND_F8, "int8 or fp8 (e4m3 x e4m3) operands");
+  using acc_t = typename std::conditional<KIND == KIND_I8, v4i, v4f>::type;
+  constexpr int NW = kSlabWaves, MAXB = kSlabMaxBlocks;
+  constexpr int NFRAG = 16;            // 16-byte fragments per lane and block (1 KiB / 64 lanes)
+  constexpr int SLOT_V4 = 16 * 64;     // 16 rows x 1 KiB
+  static_assert(MAXB <= NW, "one wave per block runs the epilogue");
+  __shared__ v4i ring[NW][2][SLOT_V4];
+  __shared__ v4i red[NW][MAXB][64];
+
+  const GemmArgs &g = prm.g;
+  const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int l16 = lane & 15, g4 = lane >> 4;
+  const int bt = blockIdx.y;
+
+  const int R = prm.swapped ? g.N : g.M, T = prm.swapped ? g.M : g.N;
+  const uint8_t *Wg = (const uint8_t *)(prm.swapped ? g.B : g.A) + (prm.swapped ? g.b_sb : g.a_sb) * bt;
+  const uint8_t *Xg = (const uint8_t *)(prm.swapped ? g.A : g.B) + (prm.swapped ? g.a_sb : g.b_sb) * bt;
+  const int ldw = (int)(prm.swapped ? g.b_sj : g.a_si);
+  const int ldx = (int)(prm.swapped ? g.a_si : g.b_sj);
+  const int K = g.K;
+
+  // Blocks of this workgroup: full_rounds round-robin blocks, then its share [rr0, rr1) (at most 16 rows, a
+  // whole number of quads except at the very end of W) of the rows behind the last full round.  The split is
+  // done on the host.
+  const int G = (int)gridDim.x, wg = (int)blockIdx.x, F = prm.full_rounds;
+  const int rr0 = 16 * F * G + 4 * (wg * prm.rows_base + min(wg, prm.rows_rem));
+  const int rr1 = min(R, rr0 + 4 * (prm.rows_base + (wg < prm.rows_rem ? 1 : 0)));
+  const int nblk = F + (rr1 > rr0 ? 1 : 0);  // <= MAXB (host)
+  if (nblk == 0) return;                      // (the whole workgroup)
+  auto row_base = [&](int b) { return b < F ? 16 * (b * G + wg) : rr0; };
+  auto row_end = [&](int b) { return b < F ? 16 * (b * G + wg) + 16 : rr1; };
+
+  // 2 GiB raw buffer windows; bit 31 of an offset puts a lane out of range: it fetches nothing and its 16
+  // bytes of LDS read as zero
+  const __amdgpu_buffer_rsrc_t rsW = __builtin_amdgcn_make_buffer_rsrc((void *)Wg, 0, 0x80000000, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsX = __builtin_amdgcn_make_buffer_rsrc((void *)Xg, 0, 0x80000000, 0x00020000);
+  const int kw = prm.spw * 64;          // bytes of K per wave (a multiple of 128, at most 1024)
+  const int kwave = wave * kw;
+  // DMA instruction i of a block (row rho = i): this lane's chunk and its byte offset inside the row
+  int dma_off[16];
+#pragma unroll
+  for (int i = 0; i < 16; i++) {
+    const int off = ((lane & 48) | ((lane ^ i) & 15)) << 4;
+    dma_off[i] = (!TAIL || (off < kw && kwave + off < K)) ? kwave + off : (int)0x80000000;
+  }
+  auto issue_block = [&](int b, int slot) {
+    const int rb = row_base(b), re = row_end(b);
+    v4i *dst = &ring[wave][slot][0];
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+      // (rows past the end of a short block repeat its last row: in range, a cache hit, never used; the row
+      // goes into the scalar offset, which leaves one scalar multiply per instruction and no vector work)
+      lds_dma16(rsW, dst + i * 64, dma_off[i], min(rb + i, re - 1) * ldw);
+    }
+  };
+  // fragment f (0..15) of this lane: int8: K step f, 16 bytes at f*64 + g4*16; fp8: half (f & 1) of the 32
+  // bytes at (f/2)*128 + g4*32 of K step f/2
+  const uint32_t ring_base = lds_addr(&ring[wave][0][l16 * 64]);
+  auto frag_addr = [&](int slot, int f) {
+    const int c = KIND == KIND_I8 ? 4 * f + g4 : 8 * (f >> 1) + 2 * g4 + (f & 1);
+    return ring_base + slot * (SLOT_V4 * 16) + (((c & 48) | ((c ^ l16) & 15)) << 4);
+  };
+
+  // Activations into slot 1 (token rho = i; tokens past T repeat the last one and are never stored), the first
+  // weights behind them, and as soon as the activations are in registers the second block: nothing that needs
+  // more of the kernel arguments than pointers and sizes stands in front of the stream.
+#pragma unroll
+  for (int i = 0; i < 16; i++) lds_dma16(rsX, &ring[wave][1][i * 64], dma_off[i], min(i, T - 1) * ldx);
+  issue_block(0, 0);
+  asm volatile("s_waitcnt vmcnt(16)" ::: "memory");  // all but the 16 youngest operations: the activations
+  v4i xf[NFRAG];
+#pragma unroll
+  for (int f = 0; f < NFRAG; f++) xf[f] = lds_read16_unordered(frag_addr(1, f));
+  lds_values_ready(xf);
+  // (issued even when there is no second block -- then it fetches the first one again, never used -- so that
+  // the number of operations in flight is the same on every path)
+  issue_block(nblk > 1 ? 1 : 0, 1);
+
+  // Who runs the epilogue: wave b takes block b, lane l the 4 rows (l/16)*4.. of token l%16, i.e. exactly the
+  // accumulator registers lane l holds.
+  const bool has_pair = wave < nblk;
+  const int ptok = l16;
+  const int prow0 = row_base(has_pair ? wave : 0) + g4 * 4, pend = row_end(has_pair ? wave : 0);
+  // Factor loads of the packed epilogue: every factor that lives in device memory -- alpha (scalar or vector),
+  // the operand scales (scalar or per row / token), the bias (16 or 32 bits), the scale of D -- is read per
+  // lane here, behind the second block, and nothing waits for it before the last block does.  Exactly
+  // kSlabFactorLoads loads per lane, whatever the problem: a factor that is an immediate or absent reads a
+  // dummy address instead, and the index passes through an empty asm so that equal addresses are not merged.
+  // The wait for the first block counts them.
+  float f_al[4], f_sa[4], f_sb[4], f_sd = 1.0f;
+  uint32_t f_b16[4], f_b32[4];
+  const bool al_mem = g.alpha_mode != SCALAR_VALUE, al_vec = g.alpha_mode == VECTOR_DEV;
+  const bool sa_mem = g.a_scale_mode == SCALE_SCALAR || g.a_scale_mode == SCALE_OUTER_VEC, sa_vec = g.a_scale_mode == SCALE_OUTER_VEC;
+  const bool sb_mem = g.b_scale_mode == SCALE_SCALAR || g.b_scale_mode == SCALE_OUTER_VEC, sb_vec = g.b_scale_mode == SCALE_OUTER_VEC;
+  const bool bias16 = g.bias && g.bias_type != CUDA_R_32F, bias32 = g.bias && g.bias_type == CUDA_R_32F;
+  const bool counted = FAST && has_pair;
+  if (counted) {
+    const float *dummy = (const float *)Wg;  // (16-byte aligned, at least 64 rows long)
+    const float *al_p = al_mem ? (const float *)g.alpha_ptr + (al_vec ? g.alpha_sb * bt : 0) : dummy;
+    const float *sa_p = sa_mem ? (const float *)g.a_scale : dummy, *sb_p = sb_mem ? (const float *)g.b_scale : dummy;
+    const uint16_t *b16_p = bias16 ? (const uint16_t *)g.bias + g.bias_sb * bt : (const uint16_t *)dummy;
+    const uint32_t *b32_p = bias32 ? (const uint32_t *)g.bias + g.bias_sb * bt : (const uint32_t *)dummy;
+#pragma unroll
+    for (int v = 0; v < 4; v++) {
+      const int row = min(prow0 + v, pend - 1), tok = min(ptok, T - 1);
+      int i = prm.swapped ? tok : row, j = prm.swapped ? row : tok;
+      asm volatile("" : "+v"(i), "+v"(j));
+      f_al[v] = al_p[al_vec ? i : 0];
+      f_sa[v] = sa_p[sa_vec ? i : 0];
+      f_sb[v] = sb_p[sb_vec ? j : 0];
+      f_b16[v] = b16_p[bias16 ? i : 0];
+      f_b32[v] = b32_p[bias32 ? i : 0];
+    }
+    f_sd = *(g.d_scale ? (const float *)g.d_scale : dummy);
+    static_assert(kSlabFactorLoads == 4 * 5 + 1, "five loads per output row and the scale of D");
+  }
+  asm volatile("" ::: "memory");
+  // (what the packed store needs of the kernel arguments, read here rather than behind the last weights)
+  const bool relu = g.act == ACT_RELU, out_bf16 = g.d_type == CUDA_R_16BF;
+  uint16_t *const Dq = (uint16_t *)g.D + g.d_sb * bt + (int64_t)ptok * (prm.swapped ? g.d_si : g.d_sj) + prow0;
+
+  acc_t acc[MAXB];
+#pragma unroll
+  for (int b = 0; b < MAXB; b++) acc[b] = acc_t{0, 0, 0, 0};
+#pragma unroll
+  for (int b = 0; b < MAXB; b++) {
+    if (b < nblk) {
+      // Block b has landed when at most the next one is in flight -- and, for the first block, the factor loads
+      // issued behind the second.  The last block waits for everything, those loads included (they are as old
+      // as the second block): they are folded into one scale and one bias per row here, where the compiler's
+      // own wait for them (vmcnt(0), all it can prove) costs nothing.
+      if (b + 1 == nblk) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (counted) {
+#pragma unroll
+          for (int v = 0; v < 4; v++) {
+            const float al = al_mem ? f_al[v] : g.alpha_val.f, sa = sa_mem ? f_sa[v] : 1.0f, sb = sb_mem ? f_sb[v] : 1.0f;
+            const float b16 = g.bias_type == CUDA_R_16F ? dec_f16((uint16_t)f_b16[v]) : dec_bf16((uint16_t)f_b16[v]);
+            f_al[v] = (al * sa) * sb;
+            f_sa[v] = bias32 ? bits2f(f_b32[v]) : bias16 ? b16 : 0.0f;
+          }
+          f_sd = g.d_scale ? f_sd : 1.0f;
+        }
+      } else if (b == 0 && counted) {
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(16 + kSlabFactorLoads) : "memory");
+      } else {
+        asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+      }
+      v4i w[NFRAG];
+#pragma unroll
+      for (int f = 0; f < NFRAG; f++) w[f] = lds_read16_unordered(frag_addr(b & 1, f));
+      lds_values_ready(w);  // in registers before the slot is refilled
+      if (b + 2 < nblk) issue_block(b + 2, b & 1);
+      if constexpr (KIND == KIND_I8) {
+#pragma unroll
+        for (int f = 0; f < NFRAG; f++) acc[b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[f], xf[f], acc[b], 0, 0, 0);
+      } else {
+#pragma unroll
+        for (int f = 0; f < NFRAG; f += 2) {
+          const v8i wa = {w[f][0], w[f][1], w[f][2], w[f][3], w[f + 1][0], w[f + 1][1], w[f + 1][2], w[f + 1][3]};
+          const v8i xb = {xf[f][0], xf[f][1], xf[f][2], xf[f][3], xf[f + 1][0], xf[f + 1][1], xf[f + 1][2], xf[f + 1][3]};
+          acc[b] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa, xb, acc[b], 0, 0, 0, 0, 0, 0);
+        }
+      }
+    }
+  }
+
+  // the one meeting of the workgroup's waves: wave b sums the NW partial tiles of block b
+#pragma unroll
+  for (int b = 0; b < MAXB; b++) red[wave][b][lane] = __builtin_bit_cast(v4i, acc[b]);
+  lds_barrier();
+  if (!has_pair) return;
+  v4i part[NW];
+  const uint32_t red_base = lds_addr(&red[0][wave][lane]);
+#pragma unroll
+  for (int w2 = 0; w2 < NW; w2++) part[w2] = lds_read16_unordered(red_base + w2 * (MAXB * 64 * 16));
+  lds_values_ready(part);
+  acc_t s = __builtin_bit_cast(acc_t, part[0]);
+#pragma unroll
+  for (int w2 = 1; w2 < NW; w2++) s += __builtin_bit_cast(acc_t, part[w2]);
+
+  if constexpr (FAST != 0) {
+    if (ptok < T && prow0 < pend) {  // the row count is a multiple of 4: a quad is inside or outside
+      float y[4];
+#pragma unroll
+      for (int v = 0; v < 4; v++) {
+        float x = f_al[v] * (float)s[v] + f_sa[v];  // (scale and bias of the row, folded above)
+        if constexpr (FAST == 2) x = gelu_tanh(x);
+        else x = relu ? (x > 0.0f ? x : 0.0f) : x;
+        y[v] = x * f_sd;
+      }
+      uint2 pk;
+      if (out_bf16) {
+        pk.x = pack_bf16x2(y[0], y[1]);
+        pk.y = pack_bf16x2(y[2], y[3]);
+      } else {
+        pk.x = pack_f16x2(y[0], y[1]);
+        pk.y = pack_f16x2(y[2], y[3]);
+      }
+      *(uint2 *)Dq = pk;
+    }
+  } else {
+    const Epilogue ep(g, bt);  // (reads its device scalars on the spot: nothing is in flight any more)
+#pragma unroll
+    for (int v = 0; v < 4; v++) {
+      const int row = prow0 + v;
+      if (row < pend && ptok < T) {
+        const int i = prm.swapped ? ptok : row, j = prm.swapped ? row : ptok;
+        if (KIND == KIND_I8 && g.int_scale) ep.store_int(i, j, (int)s[v]);
+        else ep.store_f(i, j, (float)s[v]);
+      }
+    }
+  }
+}
+
+} // namespace zluda_amd

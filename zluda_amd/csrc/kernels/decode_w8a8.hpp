@@ -23,6 +23,7 @@ struct DecodeParams {
   int32_t spw;      // MFMA K-steps (64 bytes of K each) per wave
   int32_t nchunks;  // ceil(spw / STEPS)
   int32_t rows_base, rows_rem;  // stream kernel: rows per workgroup and how many workgroups take one more
+  int32_t full_rounds;          // slab kernel: round-robin rounds of one 16-row block per workgroup in front of those rows
 };
 
 template <int NW, int STEPS, int NB, bool FULL>

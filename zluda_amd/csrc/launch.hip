@@ -21,6 +21,9 @@ namespace zluda_amd {
 uint32_t launch_decode_stream_i8(const DecodeParams &prm, const zluda_gemm_plan &plan, int nb, hipStream_t s) {
   return launch_decode_stream_variant<KIND_I8>(prm, plan, nb, s);
 }
+uint32_t launch_decode_slab_i8(const DecodeParams &prm, const zluda_gemm_plan &plan, hipStream_t s) {
+  return launch_decode_slab<KIND_I8>(prm, plan, s);
+}
 } // namespace zluda_amd
 
 namespace {
@@ -140,13 +143,31 @@ uint32_t launch_decode(const Lowered &l, const zluda_gemm_plan &plan, hipStream_
   DecodeParams prm;
   prm.g = l.g;
   prm.swapped = plan.swapped;
-  prm.rows_base = prm.rows_rem = 0;
+  prm.rows_base = prm.rows_rem = prm.full_rounds = 0;
   const int T = plan.swapped ? l.g.M : l.g.N;
   const int ksteps = (l.g.K + 63) / 64;
   prm.spw = (ksteps + v.nw - 1) / v.nw;
   prm.nchunks = (prm.spw + v.steps - 1) / v.steps;
   const bool full = l.g.K == v.nw * v.steps * 64;
   const int nb = (T + 15) / 16;
+  if (v.stream == 2) {
+    // slab kernel: one block of tokens, 4 slabs of at most 1 KiB of K, W and X through 2 GiB buffer windows,
+    // at most kSlabMaxBlocks blocks per workgroup: full_rounds round-robin blocks, then an even share (in
+    // quads of 4) of the rows that are left
+    const int64_t rows = plan.swapped ? l.g.N : l.g.M, ldw = plan.swapped ? l.g.b_sj : l.g.a_si;
+    const int64_t ldx = plan.swapped ? l.g.a_si : l.g.b_sj;
+    if (nb != 1 || l.g.K > kSlabWaves * 1024 || (l.g.K & 15) || rows * ldw >= 0x7fffffffll ||
+        (int64_t)(T - 1) * ldx + l.g.K >= 0x7fffffffll || plan.grid_x == 0)
+      return CUBLAS_STATUS_NOT_SUPPORTED;
+    const int64_t G = plan.grid_x;
+    prm.full_rounds = (int32_t)(rows / (16 * G));
+    const int64_t left = rows - 16 * G * prm.full_rounds, quads = (left + 3) / 4;
+    if (prm.full_rounds + (left > 0 ? 1 : 0) > kSlabMaxBlocks) return CUBLAS_STATUS_NOT_SUPPORTED;
+    prm.rows_base = (int32_t)(quads / G);
+    prm.rows_rem = (int32_t)(quads % G);
+    prm.spw = ((l.g.K + 511) / 512) * 2;  // a wave's slab: a quarter of K, rounded up to 128 bytes
+    return l.g.a_type == CUDA_R_8I ? launch_decode_slab_i8(prm, plan, s) : launch_decode_slab_f8(prm, plan, s);
+  }
   if (v.stream) {
     // the kernel addresses W through one 2 GiB buffer window and covers K <= nw * steps * 64
     const int64_t rows = plan.swapped ? l.g.N : l.g.M, ldw = plan.swapped ? l.g.b_sj : l.g.a_si;

@@ -225,6 +225,12 @@ static bool decode_variant_ok(const Lowered &l, int variant) {
   if (!v.stream) return g.a_type == CUDA_R_8I && (nb == 1 || (nb == 2 && v.steps <= 8));
   const bool swapped = g.M < g.N;
   const int64_t rows = swapped ? g.N : g.M, ldw = swapped ? g.b_sj : g.a_si;
+  if (v.stream == 2) {
+    const int64_t ldx = swapped ? g.a_si : g.b_sj;
+    const int cover = v.nw * v.steps * 64;
+    return nb == 1 && g.K <= cover && g.K * 2 > cover && (g.K & 15) == 0 && rows * ldw < 0x7fffffffll &&
+           (int64_t)(T - 1) * ldx + g.K < 0x7fffffffll;
+  }
   // a stream instantiation covers nw * steps * 64 bytes of K and takes any K up to that (lanes past the end read
   // zero); more than a quarter of idle lanes is left to the smaller instantiations or to the MFMA tiles
   const int cover = v.nw * v.steps * 64;
@@ -431,9 +437,14 @@ static void fill_decode_plan(const Lowered &l, int variant, uint32_t cus, zluda_
   // Stream kernel: 8 waves x 2 slots x 4 KiB = 64 KiB in flight per CU is the measured optimum on
   // MI355X (14.8 us for 58.7 MB; 128 KiB in flight: 15.8-16.8 us, 32 KiB: 15.9 us), so one 8-wave
   // workgroup per CU, two 4-wave ones.
-  const uint32_t resident = v.stream ? cus * (v.nw == 8 ? 1 : 2) : cus * (v.nw == 8 ? 2 : 4);
+  const uint32_t resident = v.stream == 2 ? cus : v.stream ? cus * (v.nw == 8 ? 1 : 2) : cus * (v.nw == 8 ? 2 : 4);
   uint32_t grid;
-  if (v.stream) grid = std::min(nrb, resident);  // contiguous, balanced row ranges
+  // slab kernel: at most one workgroup per CU (its LDS ring fills the CU), more only when the rows would not fit
+  // into 4 blocks per workgroup otherwise
+  // (a short block costs its workgroup as many DMA instructions as a full one: the fewest rounds of blocks that
+  // fit the CUs, shared out evenly -- 896 blocks on 256 CUs: 224 workgroups x 4)
+  if (v.stream == 2) grid = std::max(ceil_div(nrb, ceil_div(nrb, cus)), ceil_div(rows, 64));
+  else if (v.stream) grid = std::min(nrb, resident);  // contiguous, balanced row ranges
   else grid = nrb <= resident ? nrb : ceil_div(nrb, ceil_div(nrb, resident));
   plan->variant = variant;
   plan->swapped = swapped;
@@ -443,12 +454,16 @@ static void fill_decode_plan(const Lowered &l, int variant, uint32_t cus, zluda_
   plan->workspace = 0;
 }
 
-static int pick_decode_variant(const Lowered &l) {
+static int pick_decode_variant(const Lowered &l, uint32_t cus) {
   const int K = l.g.K;
+  // the slab form where it applies and one workgroup per CU holds the rows (14336 x 16 x 4096 int8: 12.4 us
+  // against 14.8 for the stream kernel proper)
+  for (int v = 0; v < kNumDecodeVariants; v++)
+    if (kDecodeVariants[v].stream == 2 && decode_variant_ok(l, v) && (uint32_t)std::max(l.g.M, l.g.N) <= 64 * cus) return v;
   // the stream instantiation with the least cover that takes K
   int best = -1;
   for (int v = 0; v < kNumDecodeVariants; v++)
-    if (kDecodeVariants[v].stream && decode_variant_ok(l, v) &&
+    if (kDecodeVariants[v].stream == 1 && decode_variant_ok(l, v) &&
         (best < 0 || kDecodeVariants[v].nw * kDecodeVariants[v].steps < kDecodeVariants[best].nw * kDecodeVariants[best].steps))
       best = v;
   if (best >= 0) return best;
@@ -491,10 +506,10 @@ extern "C" uint32_t zluda_gemm_plan_problem(const zluda_gemm_problem *p, uint32_
       if (!family_supports(k, l)) continue;
       if (k == ZLUDA_KERNEL_DECODE_W8A8) {
         const int tokens = std::min(l.g.M, l.g.N);
-        const bool stream = kDecodeVariants[pick_decode_variant(l)].stream;
+        const bool stream = kDecodeVariants[pick_decode_variant(l, cu_count)].stream;
         if (tokens > (stream ? kDecodeAutoMaxTokensStream : kDecodeAutoMaxTokens)) continue;
       }
-      if (k == ZLUDA_KERNEL_DECODE_W8A8 && !kDecodeVariants[pick_decode_variant(l)].stream &&
+      if (k == ZLUDA_KERNEL_DECODE_W8A8 && !kDecodeVariants[pick_decode_variant(l, cu_count)].stream &&
           family_supports(ZLUDA_KERNEL_MFMA_I8, l)) {  // (int8 only: fp8 has no such variant)
         // K outside the stream kernel's table: the register-streaming variant measures slower than
         // 64x64 MFMA tiles (split along K when the workspace allows) as soon as those give at
@@ -533,7 +548,7 @@ extern "C" uint32_t zluda_gemm_plan_problem(const zluda_gemm_problem *p, uint32_
     break;
   }
   case ZLUDA_KERNEL_DECODE_W8A8: {
-    int v = forced_variant >= 0 ? forced_variant : pick_decode_variant(l);
+    int v = forced_variant >= 0 ? forced_variant : pick_decode_variant(l, cu_count);
     if (v >= kNumDecodeVariants) return CUBLAS_STATUS_INVALID_VALUE;
     if (!decode_variant_ok(l, v)) return CUBLAS_STATUS_NOT_SUPPORTED;
     fill_decode_plan(l, v, cu_count, plan);

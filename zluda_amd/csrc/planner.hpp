@@ -41,6 +41,8 @@ constexpr int kNumTrVariants = sizeof(kTrVariants) / sizeof(kTrVariants[0]);
 // stream == 0: weights loaded straight into registers, any K (grid-stride over 16-row blocks).
 // stream == 1: weights streamed through LDS in whole cache lines; covers K <= nw * steps * 64 (the planner
 // gives an instantiation the K values down to three quarters of its cover).
+// stream == 2: the slab form of the stream kernel (4 waves x 1 KiB of K, whole-KiB row segments, one reduction per
+// workgroup): one block of tokens, K down to half of its cover, at most 4 blocks of 16 rows per workgroup.
 struct DecodeVariant { int nw, steps, stream; };
 constexpr DecodeVariant kDecodeVariants[] = {
     {8, 8, 0},   // 0: 8 waves x 512 B of K per pass
@@ -59,6 +61,7 @@ constexpr DecodeVariant kDecodeVariants[] = {
     {4, 12, 1},  // 13: K = 3072
     {4, 20, 1},  // 14: K = 5120
     {8, 32, 1},  // 15: K = 16384 (one block of 16 tokens: 32 fragments)
+    {4, 16, 2},  // 16: slab form, 2048 < K <= 4096, up to 16 tokens, up to 64 rows per workgroup
 };
 constexpr int kNumDecodeVariants = sizeof(kDecodeVariants) / sizeof(kDecodeVariants[0]);
 // Tokens come in blocks of 16; a wave keeps blocks x steps activation fragments (4 VGPRs each) in
