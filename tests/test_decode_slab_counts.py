@@ -1,0 +1,39 @@
+"""The slab decode kernel waits for its first weight block with a counted s_waitcnt that assumes a fixed number of
+epilogue factor loads in flight behind it (kSlabFactorLoads, kernels/decode_slab.hpp).  A compiler that merged or
+dropped one of those loads would make that wait too lax, silently.  This compiles every packed-epilogue
+instantiation for gfx950 (device code only, a few seconds) and counts the loads it really issues."""
+import os
+import re
+import shutil
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+KERNELS = os.path.join(ROOT, "zluda_amd", "csrc", "kernels")
+
+
+@pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")
+def test_every_packed_instantiation_issues_exactly_the_counted_factor_loads(tmp_path):
+    header = open(os.path.join(KERNELS, "decode_slab.hpp")).read()
+    counted = int(re.search(r"constexpr int kSlabFactorLoads = (\d+);", header).group(1))
+    insts = [(fast, kind, tail) for fast in (1, 2) for kind in ("KIND_I8", "KIND_F8") for tail in ("false", "true")]
+    src = tmp_path / "slab_counts.hip"
+    src.write_text('#include <hip/hip_runtime.h>\n#include "decode_slab.hpp"\nusing namespace zluda_amd;\n' + "".join(
+        "template __global__ void zluda_amd::decode_slab_kernel<%d, %s, %s>(DecodeParams);\n" % i for i in insts))
+    out = tmp_path / "slab_counts.s"
+    subprocess.run(["hipcc", "--offload-arch=gfx950", "-O3", "-std=c++17", "-I", KERNELS, "-Wno-unused-value",
+                    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-S", "--cuda-device-only",
+                    str(src), "-o", str(out)], check=True, stderr=subprocess.DEVNULL)
+    found, name, n = {}, None, 0
+    for line in open(out):
+        m = re.match(r"^(_ZN9zluda_amd18decode_slab_kernel\w+):", line)
+        if m:
+            name, n = m.group(1), 0
+        elif name:
+            if "global_load_" in line:
+                n += 1
+            if "s_barrier" in line:      # everything in front of the reduction: the factor loads and nothing else
+                found[name], name = n, None
+    assert len(found) == len(insts), sorted(found)
+    assert all(v == counted for v in found.values()), (counted, found)
