@@ -221,48 +221,56 @@ def test_decode_stream_variants_fp8(gpu_api, variant):
             check(gpu_api, dict(f8, m=332, n=tokens, k=k, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS), 460 + variant, DEC, variant)
 
 
-SLAB = 16   # the slab form of the stream kernel: 4 waves x 1 KiB of K, up to 16 tokens, up to 4 blocks per workgroup
+# The slab form of the stream kernel, up to 16 tokens and 4 blocks per workgroup: variant 16 = 4 waves x one 1 KiB unit
+# (2048 < K <= 4096), variants 17..19 = 8 waves x 2..4 units of 512 bytes (K up to 8192, 12288, 16384).
+SLAB_K = [(16, 4096), (16, 3072), (16, 2064), (16, 3600), (17, 8192), (17, 5120), (17, 4112), (18, 12288), (18, 11008),
+          (18, 8208), (19, 16384), (19, 13824), (19, 12304)]
 
 
-@pytest.mark.parametrize("k", [4096, 3072, 2064, 3600])
-def test_decode_slab_variant(gpu_api, k):
-    """whole-KiB row segments through LDS: exact and short K (slabs that end inside a KiB, a last slab shorter than
-    the others), ragged row ranges, 1..16 tokens, round-robin blocks plus a split remainder, both epilogues"""
+@pytest.mark.parametrize("variant,k", SLAB_K)
+def test_decode_slab_variant(gpu_api, variant, k):
+    """whole row segments through LDS: exact and short K (slabs that end inside a unit, a last slab shorter than the
+    others, units that lie past the end altogether), ragged row ranges, 1..16 tokens, round-robin blocks plus a split
+    remainder, both epilogues"""
     DEC = K.ZLUDA_KERNEL_DECODE_W8A8
-    check(gpu_api, dict(DECODE, m=1000, n=16, k=k), 520, DEC, SLAB, int_dist="normal")
-    check(gpu_api, dict(DECODE, m=1000, n=1, k=k, bias_type=K.CUDA_R_16BF), 521, DEC, SLAB, int_dist="normal")
+    check(gpu_api, dict(DECODE, m=1000, n=16, k=k), 520, DEC, variant, int_dist="normal")
+    check(gpu_api, dict(DECODE, m=1000, n=1, k=k, bias_type=K.CUDA_R_16BF), 521, DEC, variant, int_dist="normal")
     # 17 workgroups: 3 round-robin blocks each and 184 rows left, 2-3 quads per workgroup
-    check_small_grid(gpu_api, dict(DECODE, m=1000, n=5, k=k, lda=k + 64), 522, SLAB, 17, int_dist="normal")
+    check_small_grid(gpu_api, dict(DECODE, m=1000, n=5, k=k, lda=k + 64), 522, variant, 17, int_dist="normal")
     # 16 workgroups, 1024 rows: exactly 4 rounds, nothing left
-    check_small_grid(gpu_api, dict(DECODE, m=1024, n=16, k=k, d_type=K.CUDA_R_16F), 523, SLAB, 16, int_dist="normal")
+    check_small_grid(gpu_api, dict(DECODE, m=1024, n=16, k=k, d_type=K.CUDA_R_16F), 523, variant, 16, int_dist="normal")
     # element-wise epilogue: int32 with C, a row count that is no multiple of 4, f32 output with scalar factors
-    check(gpu_api, dict(I8, m=333, n=15, k=k, with_c=True), 524, DEC, SLAB)
-    check_small_grid(gpu_api, dict(I8, m=333, n=7, k=k, with_c=True, batch=2), 525, SLAB, 6)
-    check(gpu_api, dict(I8F, m=402, n=9, k=k, d_type=K.CUDA_R_32F, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS, alpha_range=(0.001, 0.002)), 526, DEC, SLAB)
+    check(gpu_api, dict(I8, m=333, n=15, k=k, with_c=True), 524, DEC, variant)
+    check_small_grid(gpu_api, dict(I8, m=333, n=7, k=k, with_c=True, batch=2), 525, variant, 6)
+    check(gpu_api, dict(I8F, m=402, n=9, k=k, d_type=K.CUDA_R_32F, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS, alpha_range=(0.001, 0.002)), 526, DEC, variant)
     # scalar alpha, no bias, packed store; tokens along M (weights are operand B)
-    check(gpu_api, dict(I8F, m=640, n=12, k=k, alpha_range=(0.001, 0.002), batch=3), 527, DEC, SLAB)
+    check(gpu_api, dict(I8F, m=640, n=12, k=k, alpha_range=(0.001, 0.002), batch=3), 527, DEC, variant)
     check(gpu_api, dict(I8F, transa=0, transb=1, order_a=1, order_b=1, order_c=1, order_d=1, m=11, n=2048, k=k,
-                        epilogue=K.CUBLASLT_EPILOGUE_RELU_BIAS, bias_type=K.CUDA_R_16F, alpha_range=(0.001, 0.002)), 528, DEC, SLAB, int_dist="normal")
+                        epilogue=K.CUBLASLT_EPILOGUE_RELU_BIAS, bias_type=K.CUDA_R_16F, alpha_range=(0.001, 0.002)), 528, DEC, variant, int_dist="normal")
 
 
-@pytest.mark.parametrize("k", [4096, 3072, 2176])
-def test_decode_slab_variant_fp8(gpu_api, k):
+@pytest.mark.parametrize("variant,k", [(16, 4096), (16, 3072), (16, 2176), (17, 8192), (17, 4224), (18, 11008), (19, 13824), (19, 16384)])
+def test_decode_slab_variant_fp8(gpu_api, variant, k):
     DEC = K.ZLUDA_KERNEL_DECODE_W8A8
     f8 = dict(F8, epilogue=K.CUBLASLT_EPILOGUE_BIAS, bias_type=K.CUDA_R_16BF, with_scalar_scales=True, scale_range=(0.05, 0.06))
-    check(gpu_api, dict(f8, m=1000, n=16, k=k), 540, DEC, SLAB)
-    check_small_grid(gpu_api, dict(f8, m=1000, n=5, k=k, lda=k + 64, d_type=K.CUDA_R_16F), 541, SLAB, 17)
-    check(gpu_api, dict(F8, m=333, n=3, k=k, with_c=True, d_type=K.CUDA_R_32F, c_type=K.CUDA_R_32F), 542, DEC, SLAB)
-    check(gpu_api, dict(f8, m=332, n=13, k=k, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS, bias_type=K.CUDA_R_32F), 543, DEC, SLAB)
+    check(gpu_api, dict(f8, m=1000, n=16, k=k), 540, DEC, variant)
+    check_small_grid(gpu_api, dict(f8, m=1000, n=5, k=k, lda=k + 64, d_type=K.CUDA_R_16F), 541, variant, 17)
+    check(gpu_api, dict(F8, m=333, n=3, k=k, with_c=True, d_type=K.CUDA_R_32F, c_type=K.CUDA_R_32F), 542, DEC, variant)
+    check(gpu_api, dict(f8, m=332, n=13, k=k, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS, bias_type=K.CUDA_R_32F), 543, DEC, variant)
 
 
 def test_decode_slab_is_refused_outside_its_range(gpu_api):
-    """more than 16 tokens, K beyond 4 KiB or at most half of it, more rows than 4 blocks per workgroup hold"""
+    """more than 16 tokens, K beyond the cover or under the next smaller one, more rows than 4 blocks per workgroup hold"""
     DEC = K.ZLUDA_KERNEL_DECODE_W8A8
-    for spec in (dict(DECODE, m=512, n=17, k=4096), dict(DECODE, m=512, n=16, k=4112), dict(DECODE, m=512, n=16, k=2048)):
-        st, _, _ = Case(spec, 550).run_gpu_plan(gpu_api, DEC, SLAB)
+    for variant, spec in ((16, dict(DECODE, m=512, n=17, k=4096)), (16, dict(DECODE, m=512, n=16, k=4112)),
+                          (16, dict(DECODE, m=512, n=16, k=2048)), (17, dict(DECODE, m=512, n=16, k=4096)),
+                          (17, dict(DECODE, m=512, n=16, k=8208)), (19, dict(DECODE, m=512, n=16, k=12288)),
+                          (19, dict(DECODE, m=512, n=17, k=16384))):
+        st, _, _ = Case(spec, 550).run_gpu_plan(gpu_api, DEC, variant)
+        assert st == K.CUBLAS_STATUS_NOT_SUPPORTED, (variant, spec, st)
+    for variant, k in ((16, 4096), (18, 11008)):
+        st, _, _ = Case(dict(DECODE, m=1000, n=4, k=k), 551).run_gpu_plan(gpu_api, DEC, variant, grid_x=12)   # 1000 > 12 * 64 rows
         assert st == K.CUBLAS_STATUS_NOT_SUPPORTED, st
-    st, _, _ = Case(dict(DECODE, m=1000, n=4, k=4096), 551).run_gpu_plan(gpu_api, DEC, SLAB, grid_x=12)   # 1000 > 12 * 64 rows
-    assert st == K.CUBLAS_STATUS_NOT_SUPPORTED, st
 
 
 def test_decode_fp8_planner_choice_and_orientation(gpu_api):

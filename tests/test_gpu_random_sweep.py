@@ -15,7 +15,7 @@ from zluda_amd import abi as K, cublaslt
 pytestmark = pytest.mark.gpu
 BIG = True   # include shapes of several tiles of the large variants
 NVAR = {K.ZLUDA_KERNEL_MFMA_I8: 10, K.ZLUDA_KERNEL_MFMA_F8: 10, K.ZLUDA_KERNEL_MFMA_MXF4: 8, K.ZLUDA_KERNEL_MFMA_TR8: 4,
-        K.ZLUDA_KERNEL_DECODE_W8A8: 17}
+        K.ZLUDA_KERNEL_DECODE_W8A8: 20}
 RNG = None
 
 
@@ -30,7 +30,7 @@ def pick(xs):
 def dims():
     r = RNG.random()
     if r < 0.2:   # decode-like
-        return int(RNG.integers(16, 3000)), int(RNG.integers(1, 49)), pick([1024, 2048, 2560, 3072, 3584, 4096, 960, 1536, 5120, 272])
+        return int(RNG.integers(16, 3000)), int(RNG.integers(1, 49)), pick([1024, 2048, 2560, 3072, 3584, 4096, 960, 1536, 5120, 272, 8192, 11008, 13824])
     if r < 0.4:   # few tiles, long K (split-K)
         return int(RNG.integers(1, 200)), int(RNG.integers(1, 200)), pick([2048, 4096, 6144, 8192, 3000, 4112])
     if r < 0.5:

@@ -188,14 +188,16 @@ def test_decode_k_between_the_stream_instantiations(api):
     st, p = plan(api, dict(dec, m=14336, n=17, k=4096))                       # exactly one instantiation's cover
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.variant == 4
     for ws in (0, 64 << 20):
-        st, p = plan(api, dict(dec, m=5120, n=16, k=13824), workspace=ws)     # under the 14336 cover
-        assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.variant == 6 and p.workspace == 0
+        st, p = plan(api, dict(dec, m=5120, n=16, k=13824), workspace=ws)     # one block of tokens: the slab form
+        assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.variant == 19 and p.workspace == 0
+        assert plan(api, dict(dec, m=5120, n=16, k=13824), workspace=ws, forced=K.ZLUDA_KERNEL_DECODE_W8A8, variant=6)[0] == 0   # under the 14336 cover
     st, p = plan(api, dict(dec, m=18944, n=32, k=3584))                       # under the 4096 cover, two token blocks
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.variant == 4
     st, p = plan(api, dict(dec, m=2048, n=17, k=2560), workspace=64 << 20)    # under the 3072 cover
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.variant == 13
-    st, p = plan(api, dict(dec, m=4096, n=16, k=11008))                       # under the 12288 cover
-    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.variant == 9
+    st, p = plan(api, dict(dec, m=4096, n=16, k=11008))                       # the slab form again
+    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.variant == 18
+    assert plan(api, dict(dec, m=4096, n=16, k=11008), forced=K.ZLUDA_KERNEL_DECODE_W8A8, variant=9)[0] == 0   # under the 12288 cover
     # no cover: K = 1536 lies between 1024 and three quarters of 2048, K = 20480 beyond the largest
     st, p = plan(api, dict(dec, m=8192, n=16, k=20480), workspace=64 << 20)
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_I8 and p.grid_z > 1 and p.grid_x * p.grid_z >= 128
@@ -205,8 +207,8 @@ def test_decode_k_between_the_stream_instantiations(api):
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_I8 and p.grid_z == 1
 
 
-def test_decode_slab_form_takes_one_token_block_under_4096(api):
-    """the slab form of the stream kernel: up to 16 tokens, 2048 < K <= 4096, int8 or e4m3, as long as 4 blocks of 16 rows
+def test_decode_slab_form_takes_one_token_block(api):
+    """the slab form of the stream kernel: up to 16 tokens, 2048 < K <= 16384, int8 or e4m3, as long as 4 blocks of 16 rows
     per CU hold the matrix; its grid is the fewest rounds of blocks shared out evenly"""
     dec = dict(I8, transa=1, d_type=K.CUDA_R_16BF, scale_type=K.CUDA_R_32F,
                pointer_mode=K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO,
@@ -218,15 +220,24 @@ def test_decode_slab_form_takes_one_token_block_under_4096(api):
                        (dict(F8, transa=1, m=14336, n=16, k=4096), 224), (dict(dec, m=4100, n=16, k=2064), 129)):
         st, p = plan(api, spec)
         assert st == 0 and p.kernel == DEC and p.variant == 16 and p.grid_x == grid and p.block == 256 and p.workspace == 0, (spec, p.variant, p.grid_x)
+    # beyond 4096: 8 waves x 2, 3, 4 units of 512 bytes, each shape from the next smaller cover up
+    for spec, variant, grid in ((dict(dec, m=5120, n=16, k=13824), 19, 160), (dict(dec, m=8192, n=16, k=8192), 17, 256),
+                                (dict(dec, m=4096, n=3, k=11008), 18, 256), (dict(dec, m=5120, n=16, k=5120), 17, 160),
+                                (dict(dec, m=2048, n=16, k=4112), 17, 128), (dict(F8, transa=1, m=4096, n=16, k=16384), 19, 256),
+                                (dict(dec, m=4096, n=16, k=12304), 19, 256)):
+        st, p = plan(api, spec)
+        assert st == 0 and p.kernel == DEC and p.variant == variant and p.grid_x == grid and p.block == 512, (spec, p.variant, p.grid_x)
     # tokens along M: the weights are operand B
     st, p = plan(api, dict(dec, transa=0, transb=1, order_a=1, order_b=1, order_c=1, order_d=1, m=16, n=4096, k=4096))
     assert st == 0 and p.kernel == DEC and p.variant == 16 and p.swapped == 1
     # outside its range: a second token block, K of at most half the cover or beyond it, more rows than 64 per CU
     for spec, variant in ((dict(dec, m=14336, n=17, k=4096), 4), (dict(dec, m=4096, n=16, k=2048), 7),
-                          (dict(dec, m=4096, n=16, k=4112), 14), (dict(dec, m=16400, n=16, k=4096), 4)):
+                          (dict(dec, m=16400, n=16, k=4096), 4)):
         st, p = plan(api, spec)
         assert st == 0 and p.kernel == DEC and p.variant == variant, (spec, p.variant)
         assert plan(api, spec, forced=DEC, variant=16)[0] == (0 if spec["m"] == 16400 else K.CUBLAS_STATUS_NOT_SUPPORTED)
+    st, p = plan(api, dict(dec, m=4096, n=16, k=16400))                           # K beyond the largest cover
+    assert st == 0 and not (p.kernel == DEC and p.variant >= 16)
     st, p = plan(api, dict(dec, m=16400, n=16, k=4096), forced=DEC, variant=16)   # forced: more workgroups than CUs
     assert st == 0 and p.grid_x == 257
     st, p = plan(api, dict(dec, m=14336, n=16, k=4096), cus=64)                   # a smaller device: too many rows
@@ -243,8 +254,9 @@ def test_fp8_decode_takes_the_streaming_kernel_under_a_cover_only(api):
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_F8
     st, p = plan(api, dict(f8, m=14336, n=33, k=8192))                      # 3 token blocks x 16 steps: too many fragments
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_F8
-    st, p = plan(api, dict(f8, m=4096, n=16, k=11008))                      # under the 12288 cover
-    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.variant == 9
+    st, p = plan(api, dict(f8, m=4096, n=16, k=11008))                      # one block of tokens: the slab form
+    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.variant == 18
+    assert plan(api, dict(f8, m=4096, n=16, k=11008), forced=K.ZLUDA_KERNEL_DECODE_W8A8, variant=9)[0] == 0   # under the 12288 cover
     st, p = plan(api, dict(f8, m=4096, n=16, k=20480))                      # no cover: no fp8 fallback variant
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_F8
     st, p = plan(api, dict(f8, m=4096, n=16, k=4096, b_type=K.CUDA_R_8F_E5M2))

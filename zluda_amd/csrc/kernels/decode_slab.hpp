@@ -31,24 +31,37 @@
 
 namespace zluda_amd {
 
-constexpr int kSlabWaves = 4;       // K slabs (waves) per workgroup
 constexpr int kSlabMaxBlocks = 4;   // 16-row blocks a workgroup can run
 
 // FAST != 0 as in decode_stream_kernel: every output leaves through the packed 8-byte store (1: no activation or
 // ReLU, 2: GELU; whatever code sits between the last weights and the store is exposed in full, so the path of
-// the plain epilogue is kept free of branches).  TAIL = K < 4096 (lanes past a wave's slab or past K fetch
-// nothing and read as zero).
+// the plain epilogue is kept free of branches).  TAIL: K is shorter than the NW * Q * UB bytes the instantiation
+// covers (lanes past a wave's slab or past K fetch nothing and read as zero).
+//
+// Two shapes of the same kernel:
+//   NW = 4, UB = 1024, Q = 1   K <= 4096: a wave's slab of a block is one unit of 16 rows x 1 KiB (one row per
+//                              DMA instruction); the activations pass through the second slot while the first
+//                              block is already on its way.
+//   NW = 8, UB = 512, Q = 2..4 K <= 16384: a slab is Q units of 16 rows x 512 bytes (two rows per instruction,
+//                              still four whole cache lines per row); the activations pass through both slots,
+//                              two units at a time, BEFORE the weights start: loading them in the MFMA layout
+//                              from global memory instead asks for 64-byte pieces of 16 * K bytes per workgroup,
+//                              which at K = 13824 and 20 rows per workgroup is 44 % of all it reads.
 constexpr int kSlabFactorLoads = 21;  // vector memory loads of the packed epilogue's factors, per lane
-template <int FAST, int KIND, bool TAIL>
-__global__ __launch_bounds__(kSlabWaves * 64) void decode_slab_kernel(DecodeParams prm) {
+template <int FAST, int KIND, bool TAIL, int NW = 4, int UB = 1024, int Q = 1>
+__global__ __launch_bounds__(NW * 64) void decode_slab_kernel(DecodeParams prm) {
   static_assert(KIND == KIND_I8 || KIND == KIND_F8, "int8 or fp8 (e4m3 x e4m3) operands");
+  static_assert((UB == 1024 || UB == 512) && Q >= 1 && Q <= 4 && (Q == 1 || TAIL), "see above; Q > 1 comes with the K checks");
   using acc_t = typename std::conditional<KIND == KIND_I8, v4i, v4f>::type;
-  constexpr int NW = kSlabWaves, MAXB = kSlabMaxBlocks;
-  constexpr int NFRAG = 16;            // 16-byte fragments per lane and block (1 KiB / 64 lanes)
-  constexpr int SLOT_V4 = 16 * 64;     // 16 rows x 1 KiB
+  constexpr int MAXB = kSlabMaxBlocks;
+  constexpr int NDMA = 16 * UB / 1024;  // DMA instructions per unit
+  constexpr int RPI = 1024 / UB;        // rows per instruction
+  constexpr int CPR = UB / 16;          // 16-byte chunks per row of a unit
+  constexpr int NFRAG = UB / 64;        // 16-byte fragments per lane and unit
+  constexpr int UNIT_V4 = 16 * CPR;
   static_assert(MAXB <= NW, "one wave per block runs the epilogue");
-  __shared__ v4i ring[NW][2][SLOT_V4];
-  __shared__ v4i red[NW][MAXB][64];
+  static_assert(MAXB * 64 <= 2 * UNIT_V4, "a wave's partial tiles fit into its own ring");
+  __shared__ v4i ring[NW][2][UNIT_V4];
 
   const GemmArgs &g = prm.g;
   const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
@@ -77,47 +90,87 @@ __global__ __launch_bounds__(kSlabWaves * 64) void decode_slab_kernel(DecodePara
   // bytes of LDS read as zero
   const __amdgpu_buffer_rsrc_t rsW = __builtin_amdgcn_make_buffer_rsrc((void *)Wg, 0, 0x80000000, 0x00020000);
   const __amdgpu_buffer_rsrc_t rsX = __builtin_amdgcn_make_buffer_rsrc((void *)Xg, 0, 0x80000000, 0x00020000);
-  const int kw = prm.spw * 64;          // bytes of K per wave (a multiple of 128, at most 1024)
+  const int kw = prm.spw * 64;          // bytes of K per wave (a multiple of 128, at most Q * UB)
   const int kwave = wave * kw;
-  // DMA instruction i of a block (row rho = i): this lane's chunk and its byte offset inside the row
-  int dma_off[16];
+  // DMA instruction i of a unit fills rows RPI * i .. of the slot linearly: the lane at position p of row rho
+  // fetches the chunk whose position is p, i.e. chunk (p & ~15) | ((p ^ rho) & 15) of the row's UB bytes.
+  // (UB = 512: the upper half of the wave takes the odd row; its row pitch goes into the vector offset.)
+  const int half = RPI == 2 ? lane >> 5 : 0;
+  int dma_off[NDMA];
 #pragma unroll
-  for (int i = 0; i < 16; i++) {
-    const int off = ((lane & 48) | ((lane ^ i) & 15)) << 4;
-    dma_off[i] = (!TAIL || (off < kw && kwave + off < K)) ? kwave + off : (int)0x80000000;
+  for (int i = 0; i < NDMA; i++) {
+    const int rho = RPI * i + half, pos = RPI == 2 ? lane & 31 : lane;
+    dma_off[i] = ((pos & ~15) | ((pos ^ rho) & 15)) << 4;
   }
-  auto issue_block = [&](int b, int slot) {
+  // vector offset of instruction i in unit q of the wave's slab, `pitch` = what the odd row adds
+  auto unit_voff = [&](int i, int q, int pitch) {
+    const int off = q * UB + dma_off[i];
+    const bool in = !TAIL || (off < kw && kwave + off < K);
+    return in ? kwave + off + pitch : (int)0x80000000;
+  };
+  auto issue_w = [&](int b, int q, int slot) {
     const int rb = row_base(b), re = row_end(b);
     v4i *dst = &ring[wave][slot][0];
 #pragma unroll
-    for (int i = 0; i < 16; i++) {
+    for (int i = 0; i < NDMA; i++) {
       // (rows past the end of a short block repeat its last row: in range, a cache hit, never used; the row
       // goes into the scalar offset, which leaves one scalar multiply per instruction and no vector work)
-      lds_dma16(rsW, dst + i * 64, dma_off[i], min(rb + i, re - 1) * ldw);
+      const int row = min(rb + RPI * i, re - 1);
+      lds_dma16(rsW, dst + i * 64, unit_voff(i, q, RPI == 2 && half && row + 1 < re ? ldw : 0), row * ldw);
     }
   };
-  // fragment f (0..15) of this lane: int8: K step f, 16 bytes at f*64 + g4*16; fp8: half (f & 1) of the 32
+  // (token rho = row of the unit; tokens past T repeat the last one and are never stored)
+  auto issue_x = [&](int q, int slot) {
+    v4i *dst = &ring[wave][slot][0];
+#pragma unroll
+    for (int i = 0; i < NDMA; i++) {
+      const int tok = min(RPI * i, T - 1);
+      lds_dma16(rsX, dst + i * 64, unit_voff(i, q, RPI == 2 && half && tok + 1 < T ? ldx : 0), tok * ldx);
+    }
+  };
+  // fragment f of this lane in a unit: int8: K step f, 16 bytes at f*64 + g4*16; fp8: half (f & 1) of the 32
   // bytes at (f/2)*128 + g4*32 of K step f/2
-  const uint32_t ring_base = lds_addr(&ring[wave][0][l16 * 64]);
+  const uint32_t ring_base = lds_addr(&ring[wave][0][l16 * CPR]);
   auto frag_addr = [&](int slot, int f) {
     const int c = KIND == KIND_I8 ? 4 * f + g4 : 8 * (f >> 1) + 2 * g4 + (f & 1);
-    return ring_base + slot * (SLOT_V4 * 16) + (((c & 48) | ((c ^ l16) & 15)) << 4);
+    return ring_base + slot * (UNIT_V4 * 16) + (((c & ~15) | ((c ^ l16) & 15)) << 4);
   };
+  // unit n of this wave = (block n / Q, unit n % Q of the slab), in slot n % 2; the wave runs nblk * Q of them
+  auto issue_unit = [&](int n, int slot) { issue_w(n / Q, n % Q, slot); };
 
-  // Activations into slot 1 (token rho = i; tokens past T repeat the last one and are never stored), the first
-  // weights behind them, and as soon as the activations are in registers the second block: nothing that needs
-  // more of the kernel arguments than pointers and sizes stands in front of the stream.
+  v4i xf[Q][NFRAG];
+  if constexpr (Q == 1) {
+    // Activations into slot 1, the first weights behind them, and as soon as the activations are in registers
+    // the second block: nothing that needs more of the kernel arguments than pointers and sizes stands in
+    // front of the stream.
+    issue_x(0, 1);
+    issue_unit(0, 0);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NDMA) : "memory");  // all but the youngest unit: the activations
 #pragma unroll
-  for (int i = 0; i < 16; i++) lds_dma16(rsX, &ring[wave][1][i * 64], dma_off[i], min(i, T - 1) * ldx);
-  issue_block(0, 0);
-  asm volatile("s_waitcnt vmcnt(16)" ::: "memory");  // all but the 16 youngest operations: the activations
-  v4i xf[NFRAG];
+    for (int f = 0; f < NFRAG; f++) xf[0][f] = lds_read16_unordered(frag_addr(1, f));
+    lds_values_ready(xf[0]);
+  } else {
+    // the activations of the whole slab, two units at a time through the two slots, then the first weights
 #pragma unroll
-  for (int f = 0; f < NFRAG; f++) xf[f] = lds_read16_unordered(frag_addr(1, f));
-  lds_values_ready(xf);
-  // (issued even when there is no second block -- then it fetches the first one again, never used -- so that
-  // the number of operations in flight is the same on every path)
-  issue_block(nblk > 1 ? 1 : 0, 1);
+    for (int q = 0; q < Q; q += 2) {
+      issue_x(q, 0);
+      if (q + 1 < Q) issue_x(q + 1, 1);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+      for (int f = 0; f < NFRAG; f++) xf[q][f] = lds_read16_unordered(frag_addr(0, f));
+      if (q + 1 < Q) {
+#pragma unroll
+        for (int f = 0; f < NFRAG; f++) xf[q + 1][f] = lds_read16_unordered(frag_addr(1, f));
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    }
+#pragma unroll
+    for (int q = 0; q < Q; q++) lds_values_ready(xf[q]);
+    issue_unit(0, 0);
+  }
+  // (the second unit is issued even when there is none -- then it fetches the first one again, never used -- so
+  // that the number of operations in flight is the same on every path)
+  issue_unit(nblk * Q > 1 ? 1 : 0, 1);
 
   // Who runs the epilogue: wave b takes block b, lane l the 4 rows (l/16)*4.. of token l%16, i.e. exactly the
   // accumulator registers lane l holds.
@@ -126,10 +179,10 @@ __global__ __launch_bounds__(kSlabWaves * 64) void decode_slab_kernel(DecodePara
   const int prow0 = row_base(has_pair ? wave : 0) + g4 * 4, pend = row_end(has_pair ? wave : 0);
   // Factor loads of the packed epilogue: every factor that lives in device memory -- alpha (scalar or vector),
   // the operand scales (scalar or per row / token), the bias (16 or 32 bits), the scale of D -- is read per
-  // lane here, behind the second block, and nothing waits for it before the last block does.  Exactly
+  // lane here, behind the second unit, and nothing waits for it before the last unit does.  Exactly
   // kSlabFactorLoads loads per lane, whatever the problem: a factor that is an immediate or absent reads a
   // dummy address instead, and the index passes through an empty asm so that equal addresses are not merged.
-  // The wait for the first block counts them.
+  // The wait for the first unit counts them.
   float f_al[4], f_sa[4], f_sb[4], f_sd = 1.0f;
   uint32_t f_b16[4], f_b32[4];
   const bool al_mem = g.alpha_mode != SCALAR_VALUE, al_vec = g.alpha_mode == VECTOR_DEV;
@@ -168,55 +221,61 @@ __global__ __launch_bounds__(kSlabWaves * 64) void decode_slab_kernel(DecodePara
 #pragma unroll
   for (int b = 0; b < MAXB; b++) {
     if (b < nblk) {
-      // Block b has landed when at most the next one is in flight -- and, for the first block, the factor loads
-      // issued behind the second.  The last block waits for everything, those loads included (they are as old
-      // as the second block): they are folded into one scale and one bias per row here, where the compiler's
-      // own wait for them (vmcnt(0), all it can prove) costs nothing.
-      if (b + 1 == nblk) {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        if (counted) {
 #pragma unroll
-          for (int v = 0; v < 4; v++) {
-            const float al = al_mem ? f_al[v] : g.alpha_val.f, sa = sa_mem ? f_sa[v] : 1.0f, sb = sb_mem ? f_sb[v] : 1.0f;
-            const float b16 = g.bias_type == CUDA_R_16F ? dec_f16((uint16_t)f_b16[v]) : dec_bf16((uint16_t)f_b16[v]);
-            f_al[v] = (al * sa) * sb;
-            f_sa[v] = bias32 ? bits2f(f_b32[v]) : bias16 ? b16 : 0.0f;
+      for (int q = 0; q < Q; q++) {
+        const int n = b * Q + q;  // (a compile-time number: both loops are unrolled)
+        // Unit n has landed when at most the next one is in flight -- and, for the first unit, the factor loads
+        // issued behind the second.  The last unit waits for everything, those loads included (they are as old
+        // as the second unit): they are folded into one scale and one bias per row here, where the compiler's
+        // own wait for them (vmcnt(0), all it can prove) costs nothing.
+        if (q == Q - 1 && b + 1 == nblk) {
+          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+          if (counted) {
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+              const float al = al_mem ? f_al[v] : g.alpha_val.f, sa = sa_mem ? f_sa[v] : 1.0f, sb = sb_mem ? f_sb[v] : 1.0f;
+              const float b16 = g.bias_type == CUDA_R_16F ? dec_f16((uint16_t)f_b16[v]) : dec_bf16((uint16_t)f_b16[v]);
+              f_al[v] = (al * sa) * sb;
+              f_sa[v] = bias32 ? bits2f(f_b32[v]) : bias16 ? b16 : 0.0f;
+            }
+            f_sd = g.d_scale ? f_sd : 1.0f;
           }
-          f_sd = g.d_scale ? f_sd : 1.0f;
+        } else if (n == 0 && counted) {
+          asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NDMA + kSlabFactorLoads) : "memory");
+        } else {
+          asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NDMA) : "memory");
         }
-      } else if (b == 0 && counted) {
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(16 + kSlabFactorLoads) : "memory");
-      } else {
-        asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
-      }
-      v4i w[NFRAG];
+        v4i w[NFRAG];
 #pragma unroll
-      for (int f = 0; f < NFRAG; f++) w[f] = lds_read16_unordered(frag_addr(b & 1, f));
-      lds_values_ready(w);  // in registers before the slot is refilled
-      if (b + 2 < nblk) issue_block(b + 2, b & 1);
-      if constexpr (KIND == KIND_I8) {
+        for (int f = 0; f < NFRAG; f++) w[f] = lds_read16_unordered(frag_addr(n & 1, f));
+        lds_values_ready(w);  // in registers before the slot is refilled
+        if ((n + 2) / Q < nblk) issue_unit(n + 2, n & 1);
+        if constexpr (KIND == KIND_I8) {
 #pragma unroll
-        for (int f = 0; f < NFRAG; f++) acc[b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[f], xf[f], acc[b], 0, 0, 0);
-      } else {
+          for (int f = 0; f < NFRAG; f++) acc[b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[f], xf[q][f], acc[b], 0, 0, 0);
+        } else {
 #pragma unroll
-        for (int f = 0; f < NFRAG; f += 2) {
-          const v8i wa = {w[f][0], w[f][1], w[f][2], w[f][3], w[f + 1][0], w[f + 1][1], w[f + 1][2], w[f + 1][3]};
-          const v8i xb = {xf[f][0], xf[f][1], xf[f][2], xf[f][3], xf[f + 1][0], xf[f + 1][1], xf[f + 1][2], xf[f + 1][3]};
-          acc[b] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa, xb, acc[b], 0, 0, 0, 0, 0, 0);
+          for (int f = 0; f < NFRAG; f += 2) {
+            const v4i x0 = xf[q][f], x1 = xf[q][f + 1];
+            const v8i wa = {w[f][0], w[f][1], w[f][2], w[f][3], w[f + 1][0], w[f + 1][1], w[f + 1][2], w[f + 1][3]};
+            const v8i xb = {x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+            acc[b] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa, xb, acc[b], 0, 0, 0, 0, 0, 0);
+          }
         }
       }
     }
   }
 
-  // the one meeting of the workgroup's waves: wave b sums the NW partial tiles of block b
+  // The one meeting of the workgroup's waves: wave b sums the NW partial tiles of block b.  A wave parks its
+  // tiles at the start of its own ring (everything it fetched has been consumed).
 #pragma unroll
-  for (int b = 0; b < MAXB; b++) red[wave][b][lane] = __builtin_bit_cast(v4i, acc[b]);
+  for (int b = 0; b < MAXB; b++) ring[wave][0][b * 64 + lane] = __builtin_bit_cast(v4i, acc[b]);
   lds_barrier();
   if (!has_pair) return;
   v4i part[NW];
-  const uint32_t red_base = lds_addr(&red[0][wave][lane]);
+  const uint32_t red_base = lds_addr(&ring[0][0][wave * 64 + lane]);
 #pragma unroll
-  for (int w2 = 0; w2 < NW; w2++) part[w2] = lds_read16_unordered(red_base + w2 * (MAXB * 64 * 16));
+  for (int w2 = 0; w2 < NW; w2++) part[w2] = lds_read16_unordered(red_base + w2 * (2 * UNIT_V4 * 16));
   lds_values_ready(part);
   acc_t s = __builtin_bit_cast(acc_t, part[0]);
 #pragma unroll

@@ -151,12 +151,12 @@ uint32_t launch_decode(const Lowered &l, const zluda_gemm_plan &plan, hipStream_
   const bool full = l.g.K == v.nw * v.steps * 64;
   const int nb = (T + 15) / 16;
   if (v.stream == 2) {
-    // slab kernel: one block of tokens, 4 slabs of at most 1 KiB of K, W and X through 2 GiB buffer windows,
-    // at most kSlabMaxBlocks blocks per workgroup: full_rounds round-robin blocks, then an even share (in
-    // quads of 4) of the rows that are left
+    // slab kernel: one block of tokens, nw slabs of K, W and X through 2 GiB buffer windows, at most
+    // kSlabMaxBlocks blocks per workgroup: full_rounds round-robin blocks, then an even share (in quads of 4)
+    // of the rows that are left
     const int64_t rows = plan.swapped ? l.g.N : l.g.M, ldw = plan.swapped ? l.g.b_sj : l.g.a_si;
     const int64_t ldx = plan.swapped ? l.g.a_si : l.g.b_sj;
-    if (nb != 1 || l.g.K > kSlabWaves * 1024 || (l.g.K & 15) || rows * ldw >= 0x7fffffffll ||
+    if (nb != 1 || l.g.K > v.nw * v.steps * 64 || (l.g.K & 15) || rows * ldw >= 0x7fffffffll ||
         (int64_t)(T - 1) * ldx + l.g.K >= 0x7fffffffll || plan.grid_x == 0)
       return CUBLAS_STATUS_NOT_SUPPORTED;
     const int64_t G = plan.grid_x;
@@ -165,7 +165,7 @@ uint32_t launch_decode(const Lowered &l, const zluda_gemm_plan &plan, hipStream_
     if (prm.full_rounds + (left > 0 ? 1 : 0) > kSlabMaxBlocks) return CUBLAS_STATUS_NOT_SUPPORTED;
     prm.rows_base = (int32_t)(quads / G);
     prm.rows_rem = (int32_t)(quads % G);
-    prm.spw = ((l.g.K + 511) / 512) * 2;  // a wave's slab: a quarter of K, rounded up to 128 bytes
+    prm.spw = ((l.g.K + v.nw * 128 - 1) / (v.nw * 128)) * 2;  // a wave's slab: K / nw, rounded up to 128 bytes
     return l.g.a_type == CUDA_R_8I ? launch_decode_slab_i8(prm, plan, s) : launch_decode_slab_f8(prm, plan, s);
   }
   if (v.stream) {

@@ -227,8 +227,9 @@ static bool decode_variant_ok(const Lowered &l, int variant) {
   const int64_t rows = swapped ? g.N : g.M, ldw = swapped ? g.b_sj : g.a_si;
   if (v.stream == 2) {
     const int64_t ldx = swapped ? g.a_si : g.b_sj;
-    const int cover = v.nw * v.steps * 64;
-    return nb == 1 && g.K <= cover && g.K * 2 > cover && (g.K & 15) == 0 && rows * ldw < 0x7fffffffll &&
+    // (the 4-wave shape serves K down to half of its 4096; an 8-wave shape the K above the next smaller cover)
+    const int cover = v.nw * v.steps * 64, below = v.nw == 4 ? cover / 2 : cover - 4096;
+    return nb == 1 && g.K <= cover && g.K > below && (g.K & 15) == 0 && rows * ldw < 0x7fffffffll &&
            (int64_t)(T - 1) * ldx + g.K < 0x7fffffffll;
   }
   // a stream instantiation covers nw * steps * 64 bytes of K and takes any K up to that (lanes past the end read

@@ -41,8 +41,9 @@ constexpr int kNumTrVariants = sizeof(kTrVariants) / sizeof(kTrVariants[0]);
 // stream == 0: weights loaded straight into registers, any K (grid-stride over 16-row blocks).
 // stream == 1: weights streamed through LDS in whole cache lines; covers K <= nw * steps * 64 (the planner
 // gives an instantiation the K values down to three quarters of its cover).
-// stream == 2: the slab form of the stream kernel (4 waves x 1 KiB of K, whole-KiB row segments, one reduction per
-// workgroup): one block of tokens, K down to half of its cover, at most 4 blocks of 16 rows per workgroup.
+// stream == 2: the slab form of the stream kernel (whole 512-byte or 1 KiB row segments, activations through LDS, one
+// reduction per workgroup): one block of tokens, at most 4 blocks of 16 rows per workgroup; 4 waves x 1 KiB for K down
+// to half of 4096, 8 waves x (steps / 8) units of 512 bytes each for the K between one cover and the next.
 struct DecodeVariant { int nw, steps, stream; };
 constexpr DecodeVariant kDecodeVariants[] = {
     {8, 8, 0},   // 0: 8 waves x 512 B of K per pass
@@ -62,6 +63,9 @@ constexpr DecodeVariant kDecodeVariants[] = {
     {4, 20, 1},  // 14: K = 5120
     {8, 32, 1},  // 15: K = 16384 (one block of 16 tokens: 32 fragments)
     {4, 16, 2},  // 16: slab form, 2048 < K <= 4096, up to 16 tokens, up to 64 rows per workgroup
+    {8, 16, 2},  // 17: slab form, 4096 < K <= 8192 (8 waves x 2 units of 512 bytes)
+    {8, 24, 2},  // 18: slab form, 8192 < K <= 12288
+    {8, 32, 2},  // 19: slab form, 12288 < K <= 16384
 };
 constexpr int kNumDecodeVariants = sizeof(kDecodeVariants) / sizeof(kDecodeVariants[0]);
 // Tokens come in blocks of 16; a wave keeps blocks x steps activation fragments (4 VGPRs each) in
