@@ -54,6 +54,12 @@ WORKLOADS = {
                          pointer_mode=K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO,
                          b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F,
                          epilogue=K.CUBLASLT_EPILOGUE_BIAS, bias_type=K.CUDA_R_32F)),
+    "decode_k13824": dict(name="W8A8 decode M=5120 N=16 K=13824 alpha-vec + per-token scale + fp32 bias -> bf16 (configuration 3's "
+                               "problem at a down-projection shape: few rows, long K)", kind="hbm", steps=200,
+                          spec=dict(I8, d_type=K.CUDA_R_16BF, scale_type=K.CUDA_R_32F, m=5120, n=16, k=13824,
+                                    pointer_mode=K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO,
+                                    b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F,
+                                    epilogue=K.CUBLASLT_EPILOGUE_BIAS, bias_type=K.CUDA_R_32F)),
     "c4": dict(name="fp8 e4m3 M=N=K=8192 per-tensor scales, bf16 bias + GELU -> bf16 (benchmark configuration 4)", kind="f8",
                steps=50,
                spec=dict(a_type=K.CUDA_R_8F_E4M3, b_type=K.CUDA_R_8F_E4M3, d_type=K.CUDA_R_16BF,
@@ -81,7 +87,8 @@ for _w in WORKLOADS.values():   # five equal batches
 # without a summary reports null.
 PROFILE_OF = {"c1": "gemm_mfma_tr_i8_c1_256", "c2": "gemm_mfma_pipe16_i8_c2_4096", "i8_4096_nt": "gemm_mfma_tr_i8_4096_nt",
               "i8_8192": "gemm_mfma_pipe16_i8_8192", "c3": "decode_slab_c3", "c4": "gemm_mfma_pipe16_f8_c4_8192",
-              "c5": "gemm_mfma_pipe_mxf4_c5_8192x4", "c5_b1": "gemm_mfma_pipe_mxf4_c5_8192_b1"}
+              "c5": "gemm_mfma_pipe_mxf4_c5_8192x4", "c5_b1": "gemm_mfma_pipe_mxf4_c5_8192_b1",
+              "decode_k13824": "decode_slab_k13824"}
 
 
 def measured_traffic(key):
@@ -123,12 +130,13 @@ class Buffers:
         dev = "cuda:0"
         g = torch.Generator(device=dev)
         g.manual_seed({"c2": 1, "c3": 2, "c4": 3, "c5": 4, "c5_b1": 4}.get(key, 5))
+        decode = WORKLOADS[key]["kind"] == "hbm"
         m, n, k, b = spec["m"], spec["n"], spec["k"], spec.get("batch", 1)
         self.keep = []
         self.bias = self.a_scale = self.b_scale = self.alpha_dev = None
         at = spec["a_type"]
         if at == K.CUDA_R_8I:
-            if key == "c3":   # round(N(0,32)) clipped to +-127
+            if decode:   # round(N(0,32)) clipped to +-127
                 mk = lambda r: torch.clamp(torch.round(torch.randn(r, k, device=dev, generator=g) * 32), -127, 127).to(torch.int8)
             else:             # uniform [-128, 127]
                 mk = lambda r: torch.randint(-128, 128, (r, k), device=dev, generator=g, dtype=torch.int8)
@@ -162,7 +170,7 @@ class Buffers:
             self.A, self.B, self.a_scale, self.b_scale = [a], bq, sa, sb
         dt = {K.CUDA_R_32I: torch.int32, K.CUDA_R_16BF: torch.bfloat16}[spec["d_type"]]
         self.D = torch.empty(b * m * n, device=dev, dtype=dt)
-        if key == "c3":
+        if decode:
             self.alpha_dev = torch.empty(m, device=dev).uniform_(0.001, 0.01, generator=g)
             self.b_scale = torch.empty(n, device=dev).uniform_(0.005, 0.02, generator=g)
             self.bias = torch.randn(m, device=dev, generator=g) * 0.02
@@ -313,12 +321,13 @@ def run_workload(torch, api, key, steps, warmup, with_hipblaslt):
     if key == "c4":
         nbytes += 8
     copies = 1
-    if key == "c3":
-        copies = 8   # 8 x 58.7 MB of weights > 256 MB Infinity Cache: every call streams from HBM
+    decode = w["kind"] == "hbm"
+    if decode:
+        copies = 8   # 8 x 58.7 MB (or more) of weights > 256 MB Infinity Cache: every call streams from HBM
     buf = Buffers(torch, key, spec, copies)
     call = MatmulCall(api, spec)
     call.set_pointers(bias=buf.bias.data_ptr() if buf.bias is not None else None,
-                      a_scale=buf.a_scale.data_ptr() if buf.a_scale is not None and key != "c3" else None,
+                      a_scale=buf.a_scale.data_ptr() if buf.a_scale is not None and not decode else None,
                       b_scale=buf.b_scale.data_ptr() if buf.b_scale is not None else None)
     int_scale = spec["scale_type"] == K.CUDA_R_32I
     one = C.c_int32(1) if int_scale else C.c_float(1.0)
@@ -403,9 +412,10 @@ def cpu_baseline(key, budget_s=12.0):
     from oracle.cases import Case
     spec = dict(WORKLOADS[key]["spec"])
     full_m = spec["m"]
-    rows = {"c1": full_m, "c2": full_m, "i8_4096_nt": full_m, "i8_8192": 2048, "c3": full_m, "c4": 256, "c5": 64, "c5_b1": 64}[key]
+    rows = {"c1": full_m, "c2": full_m, "i8_4096_nt": full_m, "i8_8192": 2048, "c3": full_m, "decode_k13824": full_m, "c4": 256, "c5": 64, "c5_b1": 64}[key]
     spec.update(m=rows, batch=1, alpha=1)
-    case = Case(spec, 1, int_dist="normal" if key == "c3" else "uniform")
+    decode = WORKLOADS[key]["kind"] == "hbm"
+    case = Case(spec, 1, int_dist="normal" if decode else "uniform")
     case.run_oracle()   # page in, spin up the OpenMP team
     reps, dt = 0, 0.0
     while dt < budget_s and reps < 1000:
@@ -414,8 +424,8 @@ def cpu_baseline(key, budget_s=12.0):
         dt += time.perf_counter() - t0
         reps += 1
     ops = 2 * rows * spec["n"] * spec["k"] * reps
-    unit = "GB/s" if key == "c3" else "TOPS"
-    val = (algorithmic(spec)[1] * reps / dt / 1e9) if key == "c3" else ops / dt / 1e12
+    unit = "GB/s" if decode else "TOPS"
+    val = (algorithmic(spec)[1] * reps / dt / 1e9) if decode else ops / dt / 1e12
     return {"value": val, "unit": unit, "cores": int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)),
             "kind": "port", "seconds": dt,
             "sample": "%d passes over %d of %d rows of D (full N=%d, K=%d, batch 1)%s, oracle/ref_gemm.c with OpenMP, "
@@ -459,7 +469,7 @@ def main():
     head = run_workload(torch, api, key, steps, args.warmup, not args.no_hipblaslt)
     also = {}
     if not args.only:
-        for other in ("c4", "i8_8192", "c3", "c5", "c5_b1", "c2", "c1", "i8_4096_nt"):
+        for other in ("c4", "i8_8192", "c3", "c5", "c5_b1", "c2", "c1", "i8_4096_nt", "decode_k13824"):
             if other == key:
                 continue
             try:

@@ -1,5 +1,5 @@
 // Skinny (<= 16 tokens) W8A8 decode GEMM, slab form of the LDS-streaming kernel (decode_stream.hpp) for
-// 2048 < K <= 4096: the same math and epilogue, a different road for the bytes.
+// 2048 < K <= 16384: the same math and epilogue, a different road for the bytes.
 //
 //   W : R rows x K int8 (or fp8 e4m3), K-contiguous (read exactly once)     X : T <= 16 rows x K, same type
 //   out(r, t) = sum_k W[r][k] * X[t][k]     int32 (fp32), then the fused float / integer epilogue
@@ -8,7 +8,8 @@
 // tokens (MI355X, 58.7 MB, a flat read of the same bytes takes 9.95 us; decode_stream_kernel 14.8 us):
 //   * One DMA instruction fetches ONE row x 1 KiB (64 lanes x 16 contiguous bytes) instead of 4 rows x 256
 //     bytes, a 16-row block of a wave's K slab is 16 instructions into a 16 KiB slot, two slots per wave.
-//     A workgroup is 4 waves, wave v owning K bytes [v*kw, (v+1)*kw) with kw <= 1024.
+//     A workgroup is 4 waves, wave v owning K bytes [v*kw, (v+1)*kw) with kw <= 1024.  (Beyond K = 4096: 8 waves,
+//     two rows x 512 bytes per instruction, a slab of up to four such units per block; see the template.)
 //   * The activations take the same road once (one token x 1 KiB per instruction into the second slot, whole
 //     cache lines) and are copied to registers before that slot joins the weight ring; loading them in the
 //     MFMA layout straight from global memory asks for 64-byte pieces and costs ~1 us more.
