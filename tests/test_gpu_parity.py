@@ -259,13 +259,33 @@ def test_decode_slab_variant_fp8(gpu_api, variant, k):
     check(gpu_api, dict(f8, m=332, n=13, k=k, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS, bias_type=K.CUDA_R_32F), 543, DEC, variant)
 
 
+@pytest.mark.parametrize("variant,k", [(20, 4096), (20, 3072), (20, 2064), (17, 8192), (17, 5120), (17, 4112)])
+def test_decode_slab_two_token_blocks(gpu_api, variant, k):
+    """17 .. 32 tokens on the 8-wave shapes of one or two units: ragged token counts, both epilogues, int8 and fp8,
+    tokens along M, several blocks per workgroup with a split remainder"""
+    DEC = K.ZLUDA_KERNEL_DECODE_W8A8
+    check(gpu_api, dict(DECODE, m=1000, n=32, k=k), 560, DEC, variant, int_dist="normal")
+    check(gpu_api, dict(DECODE, m=1000, n=17, k=k, bias_type=K.CUDA_R_16BF), 561, DEC, variant, int_dist="normal")
+    check_small_grid(gpu_api, dict(DECODE, m=1000, n=29, k=k, lda=k + 64), 562, variant, 17, int_dist="normal")
+    check_small_grid(gpu_api, dict(DECODE, m=1024, n=32, k=k, d_type=K.CUDA_R_16F), 563, variant, 16, int_dist="normal")
+    check(gpu_api, dict(I8, m=333, n=31, k=k, with_c=True), 564, DEC, variant)
+    check_small_grid(gpu_api, dict(I8, m=333, n=19, k=k, with_c=True, batch=2), 565, variant, 6)
+    check(gpu_api, dict(I8F, transa=0, transb=1, order_a=1, order_b=1, order_c=1, order_d=1, m=27, n=2048, k=k,
+                        epilogue=K.CUBLASLT_EPILOGUE_RELU_BIAS, bias_type=K.CUDA_R_16F, alpha_range=(0.001, 0.002)), 566, DEC, variant, int_dist="normal")
+    f8 = dict(F8, epilogue=K.CUBLASLT_EPILOGUE_BIAS, bias_type=K.CUDA_R_16BF, with_scalar_scales=True, scale_range=(0.05, 0.06))
+    check(gpu_api, dict(f8, m=1000, n=32, k=k), 567, DEC, variant)
+    check_small_grid(gpu_api, dict(f8, m=1000, n=21, k=k, lda=k + 64, d_type=K.CUDA_R_16F, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS), 568, variant, 17)
+    check(gpu_api, dict(F8, m=333, n=18, k=k, with_c=True, d_type=K.CUDA_R_32F, c_type=K.CUDA_R_32F), 569, DEC, variant)
+
+
 def test_decode_slab_is_refused_outside_its_range(gpu_api):
     """more than 16 tokens, K beyond the cover or under the next smaller one, more rows than 4 blocks per workgroup hold"""
     DEC = K.ZLUDA_KERNEL_DECODE_W8A8
     for variant, spec in ((16, dict(DECODE, m=512, n=17, k=4096)), (16, dict(DECODE, m=512, n=16, k=4112)),
                           (16, dict(DECODE, m=512, n=16, k=2048)), (17, dict(DECODE, m=512, n=16, k=4096)),
                           (17, dict(DECODE, m=512, n=16, k=8208)), (19, dict(DECODE, m=512, n=16, k=12288)),
-                          (19, dict(DECODE, m=512, n=17, k=16384))):
+                          (19, dict(DECODE, m=512, n=17, k=16384)), (20, dict(DECODE, m=512, n=16, k=4096)),
+                          (20, dict(DECODE, m=512, n=33, k=4096)), (17, dict(DECODE, m=512, n=33, k=8192))):
         st, _, _ = Case(spec, 550).run_gpu_plan(gpu_api, DEC, variant)
         assert st == K.CUBLAS_STATUS_NOT_SUPPORTED, (variant, spec, st)
     for variant, k in ((16, 4096), (18, 11008)):

@@ -193,8 +193,9 @@ def test_decode_k_between_the_stream_instantiations(api):
         assert plan(api, dict(dec, m=5120, n=16, k=13824), workspace=ws, forced=K.ZLUDA_KERNEL_DECODE_W8A8, variant=6)[0] == 0   # under the 14336 cover
     st, p = plan(api, dict(dec, m=18944, n=32, k=3584))                       # under the 4096 cover, two token blocks
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.variant == 4
-    st, p = plan(api, dict(dec, m=2048, n=17, k=2560), workspace=64 << 20)    # under the 3072 cover
-    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.variant == 13
+    st, p = plan(api, dict(dec, m=2048, n=16, k=2560), workspace=64 << 20, forced=K.ZLUDA_KERNEL_DECODE_W8A8, variant=13)   # under the 3072 cover
+    assert st == 0 and p.variant == 13
+    assert plan(api, dict(dec, m=2048, n=16, k=2560), forced=K.ZLUDA_KERNEL_DECODE_W8A8, variant=7)[0] == K.CUBLAS_STATUS_NOT_SUPPORTED   # 2048 does not cover it
     st, p = plan(api, dict(dec, m=4096, n=16, k=11008))                       # the slab form again
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.variant == 18
     assert plan(api, dict(dec, m=4096, n=16, k=11008), forced=K.ZLUDA_KERNEL_DECODE_W8A8, variant=9)[0] == 0   # under the 12288 cover
@@ -227,6 +228,12 @@ def test_decode_slab_form_takes_one_token_block(api):
                                 (dict(dec, m=4096, n=16, k=12304), 19, 256)):
         st, p = plan(api, spec)
         assert st == 0 and p.kernel == DEC and p.variant == variant and p.grid_x == grid and p.block == 512, (spec, p.variant, p.grid_x)
+    # 17 .. 32 tokens: the 8-wave shapes of one unit (up to two blocks of rows per CU) and of two units
+    for spec, variant, grid in ((dict(dec, m=4096, n=32, k=4096), 20, 256), (dict(dec, m=8192, n=17, k=3072), 20, 256),
+                                (dict(dec, m=8192, n=32, k=8192), 17, 256), (dict(F8, transa=1, m=5120, n=24, k=5120), 17, 160)):
+        st, p = plan(api, spec)
+        assert st == 0 and p.kernel == DEC and p.variant == variant and p.grid_x == grid and p.block == 512, (spec, p.variant, p.grid_x)
+    assert plan(api, dict(dec, m=8192, n=33, k=8192))[1].variant < 16 and plan(api, dict(dec, m=4096, n=17, k=12288))[1].variant < 16
     # tokens along M: the weights are operand B
     st, p = plan(api, dict(dec, transa=0, transb=1, order_a=1, order_b=1, order_c=1, order_d=1, m=16, n=4096, k=4096))
     assert st == 0 and p.kernel == DEC and p.variant == 16 and p.swapped == 1

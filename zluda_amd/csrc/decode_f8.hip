@@ -4,7 +4,7 @@ namespace zluda_amd {
 uint32_t launch_decode_stream_f8(const DecodeParams &prm, const zluda_gemm_plan &plan, int nb, hipStream_t s) {
   return launch_decode_stream_variant<KIND_F8>(prm, plan, nb, s);
 }
-uint32_t launch_decode_slab_f8(const DecodeParams &prm, const zluda_gemm_plan &plan, hipStream_t s) {
-  return launch_decode_slab<KIND_F8>(prm, plan, s);
+uint32_t launch_decode_slab_f8(const DecodeParams &prm, const zluda_gemm_plan &plan, int nb, hipStream_t s) {
+  return launch_decode_slab<KIND_F8>(prm, plan, nb, s);
 }
 } // namespace zluda_amd

@@ -70,7 +70,7 @@ inline uint32_t launch_decode_stream_variant(const DecodeParams &prm, const zlud
     ZLUDA_STREAM_CASE(13, 4, 12)
     ZLUDA_STREAM_CASE(14, 4, 20)
     ZLUDA_STREAM_CASE(15, 8, 32)
-    static_assert(kDecodeVariants[16].stream == 2 && kDecodeVariants[19].stream == 2, "variants 16 .. 19 are the slab kernel, launched by launch_decode_slab");
+    static_assert(kDecodeVariants[16].stream == 2 && kDecodeVariants[20].stream == 2, "variants 16 .. 20 are the slab kernel, launched by launch_decode_slab");
 #undef ZLUDA_STREAM_CASE
   default: return CUBLAS_STATUS_INVALID_VALUE;
   }
@@ -79,7 +79,7 @@ inline uint32_t launch_decode_stream_variant(const DecodeParams &prm, const zlud
 // the slab form of the stream kernel (kernels/decode_slab.hpp): up to 16 tokens; 4 waves x one 1 KiB unit for
 // K <= 4096 (steps == 16), 8 waves x steps / 8 units of 512 bytes for K <= 16384
 template <int KIND>
-inline uint32_t launch_decode_slab(const DecodeParams &prm, const zluda_gemm_plan &plan, hipStream_t s) {
+inline uint32_t launch_decode_slab(const DecodeParams &prm, const zluda_gemm_plan &plan, int nb, hipStream_t s) {
   const DecodeVariant &v = kDecodeVariants[plan.variant];
   dim3 grid(plan.grid_x, plan.grid_y, 1), block(v.nw * 64);
   // 0: element-wise epilogue, 1: packed store, 2: packed store behind a GELU
@@ -89,21 +89,24 @@ inline uint32_t launch_decode_slab(const DecodeParams &prm, const zluda_gemm_pla
   static_for_host<3>([&](auto fast_c) {
     constexpr int FAST = decltype(fast_c)::value;
     if (fast != FAST) return;
-    if (v.nw == 4 && v.steps == 16) {
+    if (v.nw == 4 && v.steps == 16 && nb == 1) {
       st = tail ? launch_kernel(decode_slab_kernel<FAST, KIND, true>, grid, block, s, prm)
                 : launch_kernel(decode_slab_kernel<FAST, KIND, false>, grid, block, s, prm);
-    } else if (v.nw == 8) {
+    } else if (v.nw == 8 && nb == 1) {
       static_for_host<3>([&](auto q_c) {
         constexpr int Q = decltype(q_c)::value + 2;
         if (v.steps == Q * 8) st = launch_kernel(decode_slab_kernel<FAST, KIND, true, 8, 512, Q>, grid, block, s, prm);
       });
+    } else if (v.nw == 8 && nb == 2) {  // two token blocks: one or two units per slab
+      if (v.steps == 8) st = launch_kernel(decode_slab_kernel<FAST, KIND, true, 8, 512, 1, 2>, grid, block, s, prm);
+      else if (v.steps == 16) st = launch_kernel(decode_slab_kernel<FAST, KIND, true, 8, 512, 2, 2>, grid, block, s, prm);
     }
   });
   return st;
 }
 
-uint32_t launch_decode_slab_i8(const DecodeParams &prm, const zluda_gemm_plan &plan, hipStream_t s);
-uint32_t launch_decode_slab_f8(const DecodeParams &prm, const zluda_gemm_plan &plan, hipStream_t s);
+uint32_t launch_decode_slab_i8(const DecodeParams &prm, const zluda_gemm_plan &plan, int nb, hipStream_t s);
+uint32_t launch_decode_slab_f8(const DecodeParams &prm, const zluda_gemm_plan &plan, int nb, hipStream_t s);
 uint32_t launch_decode_stream_i8(const DecodeParams &prm, const zluda_gemm_plan &plan, int nb, hipStream_t s);
 uint32_t launch_decode_stream_f8(const DecodeParams &prm, const zluda_gemm_plan &plan, int nb, hipStream_t s);
 

@@ -48,11 +48,14 @@ constexpr int kSlabMaxBlocks = 4;   // 16-row blocks a workgroup can run
 //                              two units at a time, BEFORE the weights start: loading them in the MFMA layout
 //                              from global memory instead asks for 64-byte pieces of 16 * K bytes per workgroup,
 //                              which at K = 13824 and 20 rows per workgroup is 44 % of all it reads.
+//   NW = 8, UB = 512, Q = 1..2, NB = 2   17..32 tokens, K <= 8192: a second block of 16 tokens doubles the
+//                              activation fragments and the accumulators; the 8 (block, token block) tiles of
+//                              the final reduction go one to each wave.
 constexpr int kSlabFactorLoads = 21;  // vector memory loads of the packed epilogue's factors, per lane
-template <int FAST, int KIND, bool TAIL, int NW = 4, int UB = 1024, int Q = 1>
+template <int FAST, int KIND, bool TAIL, int NW = 4, int UB = 1024, int Q = 1, int NB = 1>
 __global__ __launch_bounds__(NW * 64) void decode_slab_kernel(DecodeParams prm) {
   static_assert(KIND == KIND_I8 || KIND == KIND_F8, "int8 or fp8 (e4m3 x e4m3) operands");
-  static_assert((UB == 1024 || UB == 512) && Q >= 1 && Q <= 4 && (Q == 1 || TAIL), "see above; Q > 1 comes with the K checks");
+  static_assert((UB == 1024 || UB == 512) && Q >= 1 && Q * NB <= 4 && (Q * NB == 1 || TAIL), "see above; the shapes beyond the first come with the K checks");
   using acc_t = typename std::conditional<KIND == KIND_I8, v4i, v4f>::type;
   constexpr int MAXB = kSlabMaxBlocks;
   constexpr int NDMA = 16 * UB / 1024;  // DMA instructions per unit
@@ -60,8 +63,8 @@ __global__ __launch_bounds__(NW * 64) void decode_slab_kernel(DecodeParams prm) 
   constexpr int CPR = UB / 16;          // 16-byte chunks per row of a unit
   constexpr int NFRAG = UB / 64;        // 16-byte fragments per lane and unit
   constexpr int UNIT_V4 = 16 * CPR;
-  static_assert(MAXB <= NW, "one wave per block runs the epilogue");
-  static_assert(MAXB * 64 <= 2 * UNIT_V4, "a wave's partial tiles fit into its own ring");
+  static_assert(MAXB * NB <= NW, "one wave per (block, token block) runs the epilogue");
+  static_assert(MAXB * NB * 64 <= 2 * UNIT_V4, "a wave's partial tiles fit into its own ring");
   __shared__ v4i ring[NW][2][UNIT_V4];
 
   const GemmArgs &g = prm.g;
@@ -120,12 +123,12 @@ __global__ __launch_bounds__(NW * 64) void decode_slab_kernel(DecodeParams prm) 
       lds_dma16(rsW, dst + i * 64, unit_voff(i, q, RPI == 2 && half && row + 1 < re ? ldw : 0), row * ldw);
     }
   };
-  // (token rho = row of the unit; tokens past T repeat the last one and are never stored)
-  auto issue_x = [&](int q, int slot) {
+  // (token 16 * nbk + rho, rho = row of the unit; tokens past T repeat the last one and are never stored)
+  auto issue_x = [&](int nbk, int q, int slot) {
     v4i *dst = &ring[wave][slot][0];
 #pragma unroll
     for (int i = 0; i < NDMA; i++) {
-      const int tok = min(RPI * i, T - 1);
+      const int tok = min(16 * nbk + RPI * i, T - 1);
       lds_dma16(rsX, dst + i * 64, unit_voff(i, q, RPI == 2 && half && tok + 1 < T ? ldx : 0), tok * ldx);
     }
   };
@@ -139,45 +142,47 @@ __global__ __launch_bounds__(NW * 64) void decode_slab_kernel(DecodeParams prm) 
   // unit n of this wave = (block n / Q, unit n % Q of the slab), in slot n % 2; the wave runs nblk * Q of them
   auto issue_unit = [&](int n, int slot) { issue_w(n / Q, n % Q, slot); };
 
-  v4i xf[Q][NFRAG];
-  if constexpr (Q == 1) {
+  v4i xf[NB * Q][NFRAG];  // [token block * Q + unit]
+  if constexpr (NB * Q == 1) {
     // Activations into slot 1, the first weights behind them, and as soon as the activations are in registers
     // the second block: nothing that needs more of the kernel arguments than pointers and sizes stands in
     // front of the stream.
-    issue_x(0, 1);
+    issue_x(0, 0, 1);
     issue_unit(0, 0);
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NDMA) : "memory");  // all but the youngest unit: the activations
 #pragma unroll
     for (int f = 0; f < NFRAG; f++) xf[0][f] = lds_read16_unordered(frag_addr(1, f));
     lds_values_ready(xf[0]);
   } else {
-    // the activations of the whole slab, two units at a time through the two slots, then the first weights
+    // the activations of the whole slab (of every token block), two units at a time through the two slots, then
+    // the first weights
 #pragma unroll
-    for (int q = 0; q < Q; q += 2) {
-      issue_x(q, 0);
-      if (q + 1 < Q) issue_x(q + 1, 1);
+    for (int c = 0; c < NB * Q; c += 2) {
+      issue_x(c / Q, c % Q, 0);
+      if (c + 1 < NB * Q) issue_x((c + 1) / Q, (c + 1) % Q, 1);
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
-      for (int f = 0; f < NFRAG; f++) xf[q][f] = lds_read16_unordered(frag_addr(0, f));
-      if (q + 1 < Q) {
+      for (int f = 0; f < NFRAG; f++) xf[c][f] = lds_read16_unordered(frag_addr(0, f));
+      if (c + 1 < NB * Q) {
 #pragma unroll
-        for (int f = 0; f < NFRAG; f++) xf[q + 1][f] = lds_read16_unordered(frag_addr(1, f));
+        for (int f = 0; f < NFRAG; f++) xf[c + 1][f] = lds_read16_unordered(frag_addr(1, f));
       }
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     }
 #pragma unroll
-    for (int q = 0; q < Q; q++) lds_values_ready(xf[q]);
+    for (int c = 0; c < NB * Q; c++) lds_values_ready(xf[c]);
     issue_unit(0, 0);
   }
   // (the second unit is issued even when there is none -- then it fetches the first one again, never used -- so
   // that the number of operations in flight is the same on every path)
   issue_unit(nblk * Q > 1 ? 1 : 0, 1);
 
-  // Who runs the epilogue: wave b takes block b, lane l the 4 rows (l/16)*4.. of token l%16, i.e. exactly the
-  // accumulator registers lane l holds.
-  const bool has_pair = wave < nblk;
-  const int ptok = l16;
-  const int prow0 = row_base(has_pair ? wave : 0) + g4 * 4, pend = row_end(has_pair ? wave : 0);
+  // Who runs the epilogue: wave w takes block w % MAXB of token block w / MAXB, lane l the 4 rows (l/16)*4.. of
+  // token l%16 of that block, i.e. exactly the accumulator registers lane l holds.
+  const int pblk = wave % MAXB, pnb = wave / MAXB;
+  const bool has_pair = pblk < nblk && pnb < NB;
+  const int ptok = 16 * pnb + l16;
+  const int prow0 = row_base(has_pair ? pblk : 0) + g4 * 4, pend = row_end(has_pair ? pblk : 0);
   // Factor loads of the packed epilogue: every factor that lives in device memory -- alpha (scalar or vector),
   // the operand scales (scalar or per row / token), the bias (16 or 32 bits), the scale of D -- is read per
   // lane here, behind the second unit, and nothing waits for it before the last unit does.  Exactly
@@ -216,9 +221,11 @@ __global__ __launch_bounds__(NW * 64) void decode_slab_kernel(DecodeParams prm) 
   const bool relu = g.act == ACT_RELU, out_bf16 = g.d_type == CUDA_R_16BF;
   uint16_t *const Dq = (uint16_t *)g.D + g.d_sb * bt + (int64_t)ptok * (prm.swapped ? g.d_si : g.d_sj) + prow0;
 
-  acc_t acc[MAXB];
+  acc_t acc[MAXB][NB];
 #pragma unroll
-  for (int b = 0; b < MAXB; b++) acc[b] = acc_t{0, 0, 0, 0};
+  for (int b = 0; b < MAXB; b++)
+#pragma unroll
+    for (int nbk = 0; nbk < NB; nbk++) acc[b][nbk] = acc_t{0, 0, 0, 0};
 #pragma unroll
   for (int b = 0; b < MAXB; b++) {
     if (b < nblk) {
@@ -251,26 +258,33 @@ __global__ __launch_bounds__(NW * 64) void decode_slab_kernel(DecodeParams prm) 
         for (int f = 0; f < NFRAG; f++) w[f] = lds_read16_unordered(frag_addr(n & 1, f));
         lds_values_ready(w);  // in registers before the slot is refilled
         if ((n + 2) / Q < nblk) issue_unit(n + 2, n & 1);
-        if constexpr (KIND == KIND_I8) {
 #pragma unroll
-          for (int f = 0; f < NFRAG; f++) acc[b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[f], xf[q][f], acc[b], 0, 0, 0);
-        } else {
+        for (int nbk = 0; nbk < NB; nbk++) {
+          if constexpr (KIND == KIND_I8) {
 #pragma unroll
-          for (int f = 0; f < NFRAG; f += 2) {
-            const v4i x0 = xf[q][f], x1 = xf[q][f + 1];
-            const v8i wa = {w[f][0], w[f][1], w[f][2], w[f][3], w[f + 1][0], w[f + 1][1], w[f + 1][2], w[f + 1][3]};
-            const v8i xb = {x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
-            acc[b] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa, xb, acc[b], 0, 0, 0, 0, 0, 0);
+            for (int f = 0; f < NFRAG; f++)
+              acc[b][nbk] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[f], xf[nbk * Q + q][f], acc[b][nbk], 0, 0, 0);
+          } else {
+#pragma unroll
+            for (int f = 0; f < NFRAG; f += 2) {
+              const v4i x0 = xf[nbk * Q + q][f], x1 = xf[nbk * Q + q][f + 1];
+              const v8i wa = {w[f][0], w[f][1], w[f][2], w[f][3], w[f + 1][0], w[f + 1][1], w[f + 1][2], w[f + 1][3]};
+              const v8i xb = {x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+              acc[b][nbk] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa, xb, acc[b][nbk], 0, 0, 0, 0, 0, 0);
+            }
           }
         }
       }
     }
   }
 
-  // The one meeting of the workgroup's waves: wave b sums the NW partial tiles of block b.  A wave parks its
-  // tiles at the start of its own ring (everything it fetched has been consumed).
+  // The one meeting of the workgroup's waves: wave w sums the NW partial tiles of its (block, token block).  A
+  // wave parks its tiles at the start of its own ring (everything it fetched has been consumed), tile
+  // (b, nbk) at index nbk * MAXB + b, i.e. at the index of the wave that finishes it.
 #pragma unroll
-  for (int b = 0; b < MAXB; b++) ring[wave][0][b * 64 + lane] = __builtin_bit_cast(v4i, acc[b]);
+  for (int b = 0; b < MAXB; b++)
+#pragma unroll
+    for (int nbk = 0; nbk < NB; nbk++) ring[wave][0][(nbk * MAXB + b) * 64 + lane] = __builtin_bit_cast(v4i, acc[b][nbk]);
   lds_barrier();
   if (!has_pair) return;
   v4i part[NW];

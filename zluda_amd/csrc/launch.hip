@@ -21,8 +21,8 @@ namespace zluda_amd {
 uint32_t launch_decode_stream_i8(const DecodeParams &prm, const zluda_gemm_plan &plan, int nb, hipStream_t s) {
   return launch_decode_stream_variant<KIND_I8>(prm, plan, nb, s);
 }
-uint32_t launch_decode_slab_i8(const DecodeParams &prm, const zluda_gemm_plan &plan, hipStream_t s) {
-  return launch_decode_slab<KIND_I8>(prm, plan, s);
+uint32_t launch_decode_slab_i8(const DecodeParams &prm, const zluda_gemm_plan &plan, int nb, hipStream_t s) {
+  return launch_decode_slab<KIND_I8>(prm, plan, nb, s);
 }
 } // namespace zluda_amd
 
@@ -151,12 +151,12 @@ uint32_t launch_decode(const Lowered &l, const zluda_gemm_plan &plan, hipStream_
   const bool full = l.g.K == v.nw * v.steps * 64;
   const int nb = (T + 15) / 16;
   if (v.stream == 2) {
-    // slab kernel: one block of tokens, nw slabs of K, W and X through 2 GiB buffer windows, at most
+    // slab kernel: one block of tokens (two in the shapes of up to two units), nw slabs of K, W and X through 2 GiB buffer windows, at most
     // kSlabMaxBlocks blocks per workgroup: full_rounds round-robin blocks, then an even share (in quads of 4)
     // of the rows that are left
     const int64_t rows = plan.swapped ? l.g.N : l.g.M, ldw = plan.swapped ? l.g.b_sj : l.g.a_si;
     const int64_t ldx = plan.swapped ? l.g.a_si : l.g.b_sj;
-    if (nb != 1 || l.g.K > v.nw * v.steps * 64 || (l.g.K & 15) || rows * ldw >= 0x7fffffffll ||
+    if (nb > (v.nw == 8 && v.steps <= 16 ? 2 : 1) || l.g.K > v.nw * v.steps * 64 || (l.g.K & 15) || rows * ldw >= 0x7fffffffll ||
         (int64_t)(T - 1) * ldx + l.g.K >= 0x7fffffffll || plan.grid_x == 0)
       return CUBLAS_STATUS_NOT_SUPPORTED;
     const int64_t G = plan.grid_x;
@@ -166,7 +166,7 @@ uint32_t launch_decode(const Lowered &l, const zluda_gemm_plan &plan, hipStream_
     prm.rows_base = (int32_t)(quads / G);
     prm.rows_rem = (int32_t)(quads % G);
     prm.spw = ((l.g.K + v.nw * 128 - 1) / (v.nw * 128)) * 2;  // a wave's slab: K / nw, rounded up to 128 bytes
-    return l.g.a_type == CUDA_R_8I ? launch_decode_slab_i8(prm, plan, s) : launch_decode_slab_f8(prm, plan, s);
+    return l.g.a_type == CUDA_R_8I ? launch_decode_slab_i8(prm, plan, nb, s) : launch_decode_slab_f8(prm, plan, nb, s);
   }
   if (v.stream) {
     // the kernel addresses W through one 2 GiB buffer window and covers K <= nw * steps * 64

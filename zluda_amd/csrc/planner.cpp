@@ -228,8 +228,10 @@ static bool decode_variant_ok(const Lowered &l, int variant) {
   if (v.stream == 2) {
     const int64_t ldx = swapped ? g.a_si : g.b_sj;
     // (the 4-wave shape serves K down to half of its 4096; an 8-wave shape the K above the next smaller cover)
-    const int cover = v.nw * v.steps * 64, below = v.nw == 4 ? cover / 2 : cover - 4096;
-    return nb == 1 && g.K <= cover && g.K > below && (g.K & 15) == 0 && rows * ldw < 0x7fffffffll &&
+    const int cover = v.nw * v.steps * 64, below = cover == 4096 ? cover / 2 : cover - 4096;
+    // one block of tokens; two in the 8-wave shapes of one or two units (the one-unit shape exists for them alone)
+    const bool tokens_ok = v.nw == 4 ? nb == 1 : v.steps == 8 ? nb == 2 : v.steps == 16 ? nb <= 2 : nb == 1;
+    return tokens_ok && g.K <= cover && g.K > below && (g.K & 15) == 0 && rows * ldw < 0x7fffffffll &&
            (int64_t)(T - 1) * ldx + g.K < 0x7fffffffll;
   }
   // a stream instantiation covers nw * steps * 64 bytes of K and takes any K up to that (lanes past the end read
@@ -459,8 +461,14 @@ static int pick_decode_variant(const Lowered &l, uint32_t cus) {
   const int K = l.g.K;
   // the slab form where it applies and one workgroup per CU holds the rows (14336 x 16 x 4096 int8: 12.4 us
   // against 14.8 for the stream kernel proper)
+  // (two token blocks on one unit per slab, variant 20, only up to two blocks of rows per CU: 4096 x 32 x 4096
+  // 8.9 us against 10.0, but 14336 x 32 x 4096 18.1 against 16.7; with two units, variant 17, it wins
+  // throughout: 8192 x 32 x 8192 15.4 against 22.0)
+  const uint32_t rows = (uint32_t)std::max(l.g.M, l.g.N);
   for (int v = 0; v < kNumDecodeVariants; v++)
-    if (kDecodeVariants[v].stream == 2 && decode_variant_ok(l, v) && (uint32_t)std::max(l.g.M, l.g.N) <= 64 * cus) return v;
+    if (kDecodeVariants[v].stream == 2 && decode_variant_ok(l, v) && rows <= 64 * cus &&
+        !(kDecodeVariants[v].steps == 8 && rows > 32 * cus))
+      return v;
   // the stream instantiation with the least cover that takes K
   int best = -1;
   for (int v = 0; v < kNumDecodeVariants; v++)

@@ -42,8 +42,9 @@ constexpr int kNumTrVariants = sizeof(kTrVariants) / sizeof(kTrVariants[0]);
 // stream == 1: weights streamed through LDS in whole cache lines; covers K <= nw * steps * 64 (the planner
 // gives an instantiation the K values down to three quarters of its cover).
 // stream == 2: the slab form of the stream kernel (whole 512-byte or 1 KiB row segments, activations through LDS, one
-// reduction per workgroup): one block of tokens, at most 4 blocks of 16 rows per workgroup; 4 waves x 1 KiB for K down
-// to half of 4096, 8 waves x (steps / 8) units of 512 bytes each for the K between one cover and the next.
+// reduction per workgroup): at most 4 blocks of 16 rows per workgroup; 4 waves x 1 KiB for K down to half of 4096 and
+// up to 16 tokens, 8 waves x (steps / 8) units of 512 bytes each for the K between one cover and the next; the
+// 8-wave shapes of one or two units also take a second block of 16 tokens.
 struct DecodeVariant { int nw, steps, stream; };
 constexpr DecodeVariant kDecodeVariants[] = {
     {8, 8, 0},   // 0: 8 waves x 512 B of K per pass
@@ -66,6 +67,7 @@ constexpr DecodeVariant kDecodeVariants[] = {
     {8, 16, 2},  // 17: slab form, 4096 < K <= 8192 (8 waves x 2 units of 512 bytes)
     {8, 24, 2},  // 18: slab form, 8192 < K <= 12288
     {8, 32, 2},  // 19: slab form, 12288 < K <= 16384
+    {8, 8, 2},   // 20: slab form, 2048 < K <= 4096 for 17 .. 32 tokens (8 waves x 1 unit of 512 bytes, two token blocks)
 };
 constexpr int kNumDecodeVariants = sizeof(kDecodeVariants) / sizeof(kDecodeVariants[0]);
 // Tokens come in blocks of 16; a wave keeps blocks x steps activation fragments (4 VGPRs each) in
