@@ -50,6 +50,12 @@ typedef struct zluda_matmul_desc {
   const void *a_scale, *b_scale, *c_scale, *d_scale; /* device pointers or NULL (= 1) */
   int32_t a_scale_mode, b_scale_mode, c_scale_mode, d_scale_mode;
   int8_t fast_accum;
+  /* GELU_AUX / GELU_AUX_BIAS: the GELU input (the value in front of the activation) is also written here;
+   * DGELU / DGELU_BGRAD: it is read from here (cuda_types/src/cublaslt.rs:4182-4236).  A matrix of D's
+   * type, shape and order with its own leading dimension and batch stride (elements). */
+  void *epilogue_aux;
+  int64_t epilogue_aux_ld;
+  int64_t epilogue_aux_batch_stride;
 } zluda_matmul_desc;
 
 /* A fully specified matmul: what cublasLtMatmul receives (cuda_macros/src/cublaslt.rs:58-75). */

@@ -45,6 +45,7 @@ def lib():
         L.oracle_encode_f16.restype, L.oracle_encode_f16.argtypes = C.c_uint16, [C.c_float]
         L.oracle_decode_f16.restype, L.oracle_decode_f16.argtypes = C.c_float, [C.c_uint16]
         L.oracle_gelu.restype, L.oracle_gelu.argtypes = C.c_float, [C.c_float]
+        L.oracle_dgelu.restype, L.oracle_dgelu.argtypes = C.c_float, [C.c_float]
         for name in ("oracle_encode_e4m3_array", "oracle_encode_e5m2_array", "oracle_encode_bf16_array",
                      "oracle_decode_bf16_array", "oracle_encode_f16_array"):
             getattr(L, name).restype = None

@@ -180,7 +180,8 @@ class Case:
 
         # bias
         epi = s.get("epilogue", abi.CUBLASLT_EPILOGUE_DEFAULT)
-        if epi in (abi.CUBLASLT_EPILOGUE_BIAS, abi.CUBLASLT_EPILOGUE_RELU_BIAS, abi.CUBLASLT_EPILOGUE_GELU_BIAS):
+        if epi in (abi.CUBLASLT_EPILOGUE_BIAS, abi.CUBLASLT_EPILOGUE_RELU_BIAS, abi.CUBLASLT_EPILOGUE_GELU_BIAS,
+                   abi.CUBLASLT_EPILOGUE_GELU_AUX_BIAS):
             bt = s.get("bias_type", -1)
             if bt < 0:
                 bt = abi.CUDA_R_32F if s["d_type"] in (abi.CUDA_R_8I, abi.CUDA_R_32I, abi.CUDA_R_8F_E4M3,
@@ -190,16 +191,33 @@ class Case:
             self.bias = _encode(bvals, bt)
         # bias-gradient epilogues: the bias buffer is an output (M sums for BGRADA, N for BGRADB); it starts as a
         # canary, the oracle's result lands in self.bgrad_ref and the GPU's in self.bgrad_got
-        self.bgrad = {abi.CUBLASLT_EPILOGUE_BGRADA: 1, abi.CUBLASLT_EPILOGUE_BGRADB: 2}.get(epi, 0)
+        # (3: DGELU_BGRAD, the sums of D's rows)
+        self.bgrad = {abi.CUBLASLT_EPILOGUE_BGRADA: 1, abi.CUBLASLT_EPILOGUE_BGRADB: 2, abi.CUBLASLT_EPILOGUE_DGELU_BGRAD: 3}.get(epi, 0)
         if self.bgrad:
             bt = s.get("bias_type", -1)
             if bt < 0:
                 bt = abi.CUDA_R_32F if s["d_type"] in (abi.CUDA_R_8I, abi.CUDA_R_32I, abi.CUDA_R_8F_E4M3,
                                                        abi.CUDA_R_8F_E5M2) else s["d_type"]
             self.bgrad_type = bt
-            nb = (m if self.bgrad == 1 else n) + s.get("bias_batch_stride", 0) * (batch - 1)
+            nb = (n if self.bgrad == 2 else m) + s.get("bias_batch_stride", 0) * (batch - 1)
             self.bias = np.frombuffer(bytes([0xCD]) * (nb * (4 if bt == abi.CUDA_R_32F else 2)),
                                       dtype=np.float32 if bt == abi.CUDA_R_32F else np.uint16).copy()
+        # The aux matrix of GELU_AUX[_BIAS] (output: the GELU input, starts as a canary) and DGELU[_BGRAD] (input:
+        # random values): D's type and order, leading dimension spec["aux_ld"] (default: tight), batches
+        # spec["aux_batch_stride"] apart (default: tight).  self.aux_mode 1 = written, 2 = read.
+        self.aux = None
+        self.aux_mode = {abi.CUBLASLT_EPILOGUE_GELU_AUX: 1, abi.CUBLASLT_EPILOGUE_GELU_AUX_BIAS: 1,
+                         abi.CUBLASLT_EPILOGUE_DGELU: 2, abi.CUBLASLT_EPILOGUE_DGELU_BGRAD: 2}.get(epi, 0)
+        if self.aux_mode:
+            col = s.get("order_d", abi.CUBLASLT_ORDER_COL) == abi.CUBLASLT_ORDER_COL
+            lead, other = (m, n) if col else (n, m)
+            self.aux_ld = s.setdefault("aux_ld", lead)
+            self.aux_stride = s.setdefault("aux_batch_stride", self.aux_ld * other)
+            tot = self.aux_stride * (batch - 1) + self.aux_ld * other
+            if self.aux_mode == 1:
+                self.aux = np.frombuffer(bytes([0xCD]) * (tot * np.dtype(self.d_np).itemsize), dtype=self.d_np).copy()
+            else:
+                self.aux = _encode((rng.standard_normal(tot) * s.get("aux_std", 1.5)).astype(np.float32), s["d_type"])
 
     def new_d(self):
         """output storage pre-filled with a canary pattern"""
@@ -232,6 +250,8 @@ class Case:
         o.a_scale_mode, o.b_scale_mode = s.get("a_scale_mode", 0), s.get("b_scale_mode", 0)
         o.bias, o.a_scale, o.b_scale = ptrs.get("bias"), ptrs.get("a_scale"), ptrs.get("b_scale")
         o.c_scale, o.d_scale = ptrs.get("c_scale"), ptrs.get("d_scale")
+        o.epilogue_aux = ptrs.get("aux")
+        o.epilogue_aux_ld, o.epilogue_aux_batch_stride = s.get("aux_ld", 0), s.get("aux_batch_stride", 0)
         p.alpha, p.beta = ptrs["alpha"], ptrs["beta"]
         p.A, p.B, p.C, p.D = ptrs["A"], ptrs["B"], ptrs.get("C"), ptrs["D"]
         return p
@@ -242,9 +262,12 @@ class Case:
         bias = self.bias
         if self.bgrad:   # the oracle writes it: keep the canary for the GPU run
             bias = self.bgrad_ref = self.bias.copy()
+        aux = self.aux
+        if self.aux_mode == 1:   # the oracle writes it: keep the canary for the GPU run
+            aux = self.aux_ref = self.aux.copy()
         ptrs = {"A": hp(self.A), "B": hp(self.B), "C": hp(self.Cm), "D": hp(d), "alpha": hp(self.alpha),
                 "beta": hp(self.beta), "bias": hp(bias), "a_scale": hp(self.a_scale),
-                "b_scale": hp(self.b_scale), "c_scale": hp(self.c_scale), "d_scale": hp(self.d_scale)}
+                "b_scale": hp(self.b_scale), "c_scale": hp(self.c_scale), "d_scale": hp(self.d_scale), "aux": hp(aux)}
         p = self.problem(ptrs)
         st = oracle.gemm(p)
         assert st == 0, "oracle status %d" % st
@@ -268,7 +291,7 @@ class Case:
                                ("bias", self.bias, 0), ("a_scale", self.a_scale, 0),
                                ("b_scale", self.b_scale, 0), ("c_scale", self.c_scale, 0),
                                ("d_scale", self.d_scale, 0), ("alpha_dev", self.alpha, 0),
-                               ("beta_dev", self.beta, 0)):
+                               ("beta_dev", self.beta, 0), ("aux", self.aux, 0)):
             t, p = up(arr, off)
             keep.append(t)
             ptr[name] = p
@@ -315,7 +338,7 @@ class Case:
         self.last_workspace_needed = call.heuristic[0].workspaceSize if call.heuristic else None
         try:
             call.set_pointers(bias=ptr["bias"], a_scale=ptr["a_scale"], b_scale=ptr["b_scale"],
-                              c_scale=ptr["c_scale"], d_scale=ptr["d_scale"])
+                              c_scale=ptr["c_scale"], d_scale=ptr["d_scale"], aux=ptr["aux"])
             alpha, beta = self.scalars(ptr)
             stream = torch.cuda.current_stream().cuda_stream
             st = call.run(alpha, ptr["A"], ptr["B"], beta, ptr["C"], ptr["D"],
@@ -323,6 +346,8 @@ class Case:
             torch.cuda.synchronize()
             if self.bgrad:
                 self.bgrad_got = keep[3][:self.bias.nbytes].cpu().numpy().view(self.bias.dtype).copy()
+            if self.aux_mode == 1:
+                self.aux_got = keep[10][:self.aux.nbytes].cpu().numpy().view(self.aux.dtype).copy()
             return st, self.download(dt), call.kernel, call.variant
         finally:
             call.close()
@@ -375,16 +400,38 @@ class Case:
             rp.close()
 
     # ---- comparison -------------------------------------------------------------------------------
-    def compare_bgrad(self, got, ref, exact=False):
+    def compare_aux(self, got, ref, tol=1e-2):
+        """the aux matrix of GELU_AUX[_BIAS]: its padding keeps the canary, its elements (the GELU input) agree within
+        `tol` relative to max(|ref|, 1e-2 * rms)"""
+        s = self.spec
+        m, n = s["m"], s["n"]
+        col = s.get("order_d", abi.CUBLASLT_ORDER_COL) == abi.CUBLASLT_ORDER_COL
+        i, j = np.meshgrid(np.arange(m), np.arange(n), indexing="ij")
+        one = (j * self.aux_ld + i) if col else (i * self.aux_ld + j)
+        idx = np.concatenate([(one + b * self.aux_stride).ravel() for b in range(self.batch)])
+        mask = np.ones(got.size, bool)
+        mask[idx] = False
+        assert np.array_equal(got[mask], ref[mask]), "padding of the aux matrix was overwritten"
+        g, r = decode_storage(got[idx], s["d_type"]), decode_storage(ref[idx], s["d_type"])
+        assert np.isfinite(g).all() and np.isfinite(r).all()
+        rms = float(np.sqrt(np.mean(r * r)))
+        err = float(np.max(np.abs(g - r) / np.maximum(np.abs(r), 1e-2 * rms if rms > 0 else 1.0)))
+        print("aux matrix: max rel err %.3e" % err)
+        assert err <= tol, "aux matrix: max relative error %.3e > %.1e" % (err, tol)
+        return err
+
+    def compare_bgrad(self, got, ref, exact=False, floor_frac=1e-2):
         """bias gradients as stored (bias data type): bit-exact when `exact` (integer operands: the sums are
-        exact in int32 and convert the same way), else within 1e-2 of max(|ref|, 1e-2 * rms(ref)) -- the fp32
-        summation order of the GPU kernel is its own and the output may be a 16-bit float"""
+        exact in int32 and convert the same way), else within 1e-2 of max(|ref|, floor_frac * rms(ref)) -- the fp32
+        summation order of the GPU kernel is its own and the output may be a 16-bit float.  (DGELU_BGRAD sums
+        the elements of D as its two passes rounded them, hundreds of terms of either sign: callers pass
+        floor_frac=1, i.e. an absolute bound of 1 % of the rms of the sums.)"""
         g, r = decode_storage(got, self.bgrad_type), decode_storage(ref, self.bgrad_type)
         assert g.shape == r.shape
         if exact:
             np.testing.assert_array_equal(got, ref)
             return
-        floor = 1e-2 * float(np.sqrt(np.mean(r * r))) + 1e-30
+        floor = floor_frac * float(np.sqrt(np.mean(r * r))) + 1e-30
         err = np.abs(g - r) / np.maximum(np.abs(r), floor)
         print("bias gradient: max relative error %.3g" % float(err.max()), flush=True)
         assert err.max() <= 1e-2

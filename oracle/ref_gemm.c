@@ -19,6 +19,10 @@
  *                                                              cuda_types/src/cublaslt.rs:3813-3818
  *     OUTER_VEC_32F: A scale has M entries, B scale N entries  cuda_types/src/cublaslt.rs:3820-3826
  *     layout attributes (order, ld, batch count/stride)        cuda_types/src/cublaslt.rs:3981-4058
+ *     GELU_AUX[_BIAS]: as GELU[_BIAS]; the GELU input also goes to the aux matrix
+ *                                                              cuda_types/src/cublaslt.rs:4601-4619, 4182-4236
+ *     DGELU[_BGRAD]: D = gelu'(aux) * (alpha AB + beta C); _BGRAD: the bias buffer receives the gradient
+ *                                                              cuda_types/src/cublaslt.rs:4621-4660, 4151-4166
  * Number formats follow the OCP definitions (E4M3 finite-only, E5M2 IEEE-like, E2M1, UE8M0);
  * the E4M3/E5M2 encoders additionally follow ptx/lib/zluda_ptx_impl.cpp:659-672
  * (round-to-nearest-even, saturate to the largest finite value, |x| < 2^-10 resp. 2^-17 -> +-0).
@@ -32,10 +36,15 @@
  *   - e2m1 / ue8m0 decode: exhaustive against the closed-form OCP definition
  *   - float GEMMs: exact rational arithmetic on tiny shapes, numpy float64 otherwise
  *   - epilogue (alpha vector, outer scales, bias, relu/gelu): scalar formulas in numpy
+ *   - gelu': central differences of the GELU in float64, its values at 0 (1/2) and far out (0 and 1);
+ *     GELU_AUX: gelu(aux) reproduces D; DGELU_BGRAD: numpy row sums of D
  * PARITY UNPINNED (no fixture in the reference, no hipBLASLt run possible without a GPU):
  *   - which GELU hipBLASLt applies: the tanh form is restated here.  No CPU-side fixture pins it;
  *     on a GPU box tests/test_gpu_vs_hipblaslt.py tells the tanh and erf forms apart against
  *     hipBLASLt itself (it applies the tanh form)
+ *   - DGELU_BGRAD: that the gradient is the sum over D's columns, one value per row of D (the orientation of the
+ *     bias it is the gradient of), and that the aux matrix has D's order: the text cited above gives the lengths and
+ *     the leading dimension only; hipBLASLt offers none of the four aux epilogues for the 8-bit inputs of this path
  *   - the batch stride of the UE8M0 scale tensors for batch counts above 1 (restated as batches back to
  *     back, rows * K/32 bytes each): hipBLASLt takes MXFP4 at batch 1 only.  The layout inside a batch,
  *     plain [row][K/32] bytes for both operands, is pinned on a GPU box against hipBLASLt itself by the
@@ -257,6 +266,13 @@ float oracle_gelu(float x) {
   return 0.5f * x * (1.0f + tanhf(k0 * (x + k1 * x * x * x)));
 }
 
+/* its derivative: 0.5 (1 + tanh u) + 0.5 x (1 - tanh^2 u) u'(x),  u = k0 (x + k1 x^3) */
+float oracle_dgelu(float x) {
+  const double k0 = 0.7978845608028654, k1 = 0.044715, xd = x;
+  const double t = tanh(k0 * (xd + k1 * xd * xd * xd));
+  return (float)(0.5 * (1.0 + t) + 0.5 * xd * (1.0 - t * t) * k0 * (1.0 + 3.0 * k1 * xd * xd));
+}
+
 /* ------------------------------------------------------------------ element access ------- */
 
 static size_t type_bits(uint32_t t) {
@@ -354,15 +370,30 @@ uint32_t oracle_gemm(const zluda_gemm_problem *p) {
   const int beta_zero = pm == CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO;
 
   const uint32_t epi = op->epilogue;
+  /* GELU_AUX[_BIAS] (cuda_types/src/cublaslt.rs:4601-4619): as GELU[_BIAS], and the GELU input also goes to the aux
+   * matrix; DGELU[_BGRAD] (:4621-4660): D = gelu'(aux) * (alpha AB + beta C), _BGRAD: the sums of D's rows go to
+   * the bias buffer.  The aux matrix has D's type and order, leading dimension and batch stride from the
+   * descriptor (:4182-4236). */
+  const int gelu_aux = epi == CUBLASLT_EPILOGUE_GELU_AUX || epi == CUBLASLT_EPILOGUE_GELU_AUX_BIAS;
+  const int dgelu = epi == CUBLASLT_EPILOGUE_DGELU || epi == CUBLASLT_EPILOGUE_DGELU_BGRAD;
+  const int dgelu_bgrad = epi == CUBLASLT_EPILOGUE_DGELU_BGRAD;
   const int has_bias = epi == CUBLASLT_EPILOGUE_BIAS || epi == CUBLASLT_EPILOGUE_RELU_BIAS ||
-                       epi == CUBLASLT_EPILOGUE_GELU_BIAS;
+                       epi == CUBLASLT_EPILOGUE_GELU_BIAS || epi == CUBLASLT_EPILOGUE_GELU_AUX_BIAS;
   const int relu = epi == CUBLASLT_EPILOGUE_RELU || epi == CUBLASLT_EPILOGUE_RELU_BIAS;
-  const int gelu = epi == CUBLASLT_EPILOGUE_GELU || epi == CUBLASLT_EPILOGUE_GELU_BIAS;
+  const int gelu = epi == CUBLASLT_EPILOGUE_GELU || epi == CUBLASLT_EPILOGUE_GELU_BIAS || gelu_aux;
   /* BGRADA / BGRADB (cuda_types/src/cublaslt.rs:4636-4654): D as with DEFAULT; the bias buffer receives the
    * sums over K of op(A)'s rows (M values) / of op(B)'s columns (N values), in the bias data type */
   const int bgrad = epi == CUBLASLT_EPILOGUE_BGRADA ? 1 : epi == CUBLASLT_EPILOGUE_BGRADB ? 2 : 0;
-  if (!(epi == CUBLASLT_EPILOGUE_DEFAULT || has_bias || relu || gelu || bgrad))
+  if (!(epi == CUBLASLT_EPILOGUE_DEFAULT || has_bias || relu || gelu || bgrad || dgelu))
     return CUBLAS_STATUS_NOT_SUPPORTED;
+  if (gelu_aux || dgelu) {
+    const int64_t lead = p->d.order == CUBLASLT_ORDER_ROW ? N : M;
+    if (int_scale || !(p->d.type == CUDA_R_32F || p->d.type == CUDA_R_16F || p->d.type == CUDA_R_16BF))
+      return CUBLAS_STATUS_NOT_SUPPORTED;
+    if (!op->epilogue_aux || op->epilogue_aux_ld < lead) return CUBLAS_STATUS_INVALID_VALUE;
+    if (dgelu && op->d_scale) return CUBLAS_STATUS_NOT_SUPPORTED;
+    if (dgelu_bgrad && !op->bias) return CUBLAS_STATUS_INVALID_VALUE;
+  }
   if (bgrad && (a_blk || b_blk || op->a_scale || op->b_scale || !op->bias)) return CUBLAS_STATUS_NOT_SUPPORTED;
   uint32_t bias_type = op->bias_type >= 0 ? (uint32_t)op->bias_type
                        : (p->d.type == CUDA_R_8I || p->d.type == CUDA_R_32I ||
@@ -371,7 +402,11 @@ uint32_t oracle_gemm(const zluda_gemm_problem *p) {
                            : p->d.type;
 
   const int batch = p->d.batch_count > 0 ? p->d.batch_count : 1;
-  if (bgrad && batch > 1 && op->bias_batch_stride == 0) return CUBLAS_STATUS_NOT_SUPPORTED; /* aliased outputs */
+  if ((bgrad || dgelu_bgrad) && batch > 1 && op->bias_batch_stride == 0) return CUBLAS_STATUS_NOT_SUPPORTED; /* aliased outputs */
+  if (gelu_aux && batch > 1 && op->epilogue_aux_batch_stride == 0) return CUBLAS_STATUS_NOT_SUPPORTED;
+  zluda_matrix_layout auxl = p->d;   /* D's type and order with the aux matrix's own pitch */
+  auxl.ld = op->epilogue_aux_ld;
+  double *rowsum = dgelu_bgrad ? (double *)calloc((size_t)M, sizeof(double)) : NULL;
   const zluda_matrix_layout *cl = p->C ? &p->c : &p->d;
 
   /* dense K-contiguous copies of op(A) [M][K] and op(B) [N][K] for one batch */
@@ -426,6 +461,7 @@ uint32_t oracle_gemm(const zluda_gemm_problem *p) {
       }
     }
 
+    if (rowsum) memset(rowsum, 0, sizeof(double) * (size_t)M);
 #pragma omp parallel for schedule(dynamic, 1)
     for (int64_t j = 0; j < N; j++) {
       for (int64_t i = 0; i < M; i++) {
@@ -480,12 +516,25 @@ uint32_t oracle_gemm(const zluda_gemm_problem *p) {
         if (has_bias)
           x += load_as_float(op->bias, bias_type, i + op->bias_batch_stride * bt);
         if (relu) x = x > 0.0f ? x : 0.0f;
+        const int64_t auxidx = op->epilogue_aux_batch_stride * bt + elem_index(&auxl, i, j);
+        if (gelu_aux) store_from_float(op->epilogue_aux, p->d.type, auxidx, x);
         if (gelu) x = oracle_gelu(x);
+        if (dgelu) {
+          x *= oracle_dgelu(load_as_float(op->epilogue_aux, p->d.type, auxidx));
+          if (rowsum) {
+#pragma omp atomic
+            rowsum[i] += (double)x;
+          }
+        }
         x *= sd;
         store_from_float(p->D, p->d.type, didx, x);
       }
     }
+    if (rowsum)
+      for (int64_t i = 0; i < M; i++)
+        store_from_float((void *)op->bias, bias_type, i + op->bias_batch_stride * bt, (float)rowsum[i]);
   }
+  free(rowsum);
   free(fa); free(fb); free(ia); free(ib);
   return CUBLAS_STATUS_SUCCESS;
 }

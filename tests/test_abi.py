@@ -98,7 +98,10 @@ def test_matmul_desc_attributes(api):
     assert api.desc_set(d, D.CUBLASLT_MATMUL_DESC_EPILOGUE, C.c_uint32, D.CUBLASLT_EPILOGUE_BGRADA) == 0
     assert api.desc_set(d, D.CUBLASLT_MATMUL_DESC_EPILOGUE, C.c_uint32, D.CUBLASLT_EPILOGUE_BGRADB) == 0
     assert api.desc_set(d, D.CUBLASLT_MATMUL_DESC_EPILOGUE, C.c_uint32, D.CUBLASLT_EPILOGUE_GELU_BIAS) == 0
-    assert api.desc_set(d, D.CUBLASLT_MATMUL_DESC_EPILOGUE, C.c_uint32, D.CUBLASLT_EPILOGUE_DGELU) == NS
+    # every epilogue zluda_common/src/lib.rs:762-804 maps is taken; the ReLU bit-mask forms, which it does not map, are not
+    for e in (D.CUBLASLT_EPILOGUE_GELU_AUX, D.CUBLASLT_EPILOGUE_GELU_AUX_BIAS, D.CUBLASLT_EPILOGUE_DGELU, D.CUBLASLT_EPILOGUE_DGELU_BGRAD):
+        assert api.desc_set(d, D.CUBLASLT_MATMUL_DESC_EPILOGUE, C.c_uint32, e) == 0
+    assert api.desc_set(d, D.CUBLASLT_MATMUL_DESC_EPILOGUE, C.c_uint32, D.CUBLASLT_EPILOGUE_RELU_AUX) == NS
     assert api.desc_set(d, D.CUBLASLT_MATMUL_DESC_BIAS_DATA_TYPE, C.c_int32, D.CUDA_R_16BF) == 0
     assert api.desc_set(d, D.CUBLASLT_MATMUL_DESC_BIAS_POINTER, C.c_void_p, 0x1000) == 0
     # SCALE_TYPE: size check then type check (impl.rs:263-272)
@@ -115,7 +118,14 @@ def test_matmul_desc_attributes(api):
     assert api.desc_set(d, D.CUBLASLT_MATMUL_DESC_D_SCALE_MODE, C.c_int32, D.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F) == NS
     assert api.desc_set(d, D.CUBLASLT_MATMUL_DESC_ALPHA_VECTOR_BATCH_STRIDE, C.c_int64, 64) == 0
     assert api.desc_set(d, D.CUBLASLT_MATMUL_DESC_BIAS_BATCH_STRIDE, C.c_int64, 64) == 0
-    assert api.desc_set(d, D.CUBLASLT_MATMUL_DESC_EPILOGUE_AUX_POINTER, C.c_void_p, 1) == NS
+    # the aux matrix of the GELU_AUX / DGELU epilogues: pointer, leading dimension, batch stride; D's type only
+    assert api.desc_set(d, D.CUBLASLT_MATMUL_DESC_EPILOGUE_AUX_POINTER, C.c_void_p, 0x1000) == 0
+    assert api.desc_set(d, D.CUBLASLT_MATMUL_DESC_EPILOGUE_AUX_LD, C.c_int64, 4096) == 0
+    assert api.desc_set(d, D.CUBLASLT_MATMUL_DESC_EPILOGUE_AUX_BATCH_STRIDE, C.c_int64, 1 << 24) == 0
+    assert api.desc_set(d, D.CUBLASLT_MATMUL_DESC_EPILOGUE_AUX_LD, C.c_int32, 4096) == IV
+    assert api.desc_set(d, 22, C.c_int32, -1) == 0 and api.desc_set(d, 22, C.c_int32, D.CUDA_R_8F_E4M3) == NS   # EPILOGUE_AUX_DATA_TYPE
+    # everything else: NOT_SUPPORTED (impl.rs:302)
+    assert api.desc_set(d, 23, C.c_void_p, 1) == NS   # EPILOGUE_AUX_SCALE_POINTER
     assert api.cublasLtMatmulDescSetAttribute(d, D.CUBLASLT_MATMUL_DESC_TRANSA, None, 4) == IV
     # get: value, size query, wrong size
     v, w = C.c_int32(), C.c_size_t()

@@ -273,3 +273,64 @@ def test_bias_gradient_epilogues_against_numpy(which, typ, ta, tb, oa, ob):
         assert np.max(np.abs(got - want)) <= 1e-6 * max(1.0, np.max(np.abs(want)))
     # what lies between the batches' vectors stays untouched
     assert (case.bgrad_ref[rows:24].view(np.uint32) == 0xCDCDCDCD).all()
+
+
+def test_gelu_derivative_against_differences_and_limits():
+    """oracle_dgelu is the derivative of oracle's GELU: central differences of the float64 tanh form, 1/2 at 0, 0 and
+    1 far out, and gelu'(x) + gelu'(-x) = 1 (GELU(x) - GELU(-x) = x)"""
+    L = oracle.lib()
+    k0, k1 = 0.7978845608028654, 0.044715
+    gelu = lambda x: 0.5 * x * (1.0 + np.tanh(k0 * (x + k1 * x ** 3)))
+    for x in np.linspace(-6.0, 6.0, 241):
+        h = 1e-5
+        want = (gelu(x + h) - gelu(x - h)) / (2 * h)
+        got = L.oracle_dgelu(C.c_float(x))
+        assert abs(got - want) <= 2e-6, (x, got, want)
+        assert abs(L.oracle_dgelu(C.c_float(x)) + L.oracle_dgelu(C.c_float(-x)) - 1.0) <= 1e-6
+    assert L.oracle_dgelu(C.c_float(0.0)) == 0.5
+    assert abs(L.oracle_dgelu(C.c_float(-30.0))) <= 1e-7 and abs(L.oracle_dgelu(C.c_float(30.0)) - 1.0) <= 1e-7
+
+
+@pytest.mark.parametrize("dt", [abi.CUDA_R_32F, abi.CUDA_R_16BF])
+@pytest.mark.parametrize("od", [0, 1])
+def test_gelu_aux_and_dgelu_epilogues_against_numpy(dt, od):
+    """GELU_AUX_BIAS: the aux matrix holds alpha * op(A) op(B) + bias (the GELU input) at its own leading dimension and
+    batch stride, D its GELU; DGELU_BGRAD: D = (alpha * op(A) op(B) + beta * C) * gelu'(aux), the bias buffer the sums
+    of D's rows.  Both against numpy float64 from the layout definitions."""
+    k0, k1 = 0.7978845608028654, 0.044715
+    gelu = lambda x: 0.5 * x * (1.0 + np.tanh(k0 * (x + k1 * x ** 3)))
+    dgelu = lambda x: 0.5 * (1 + np.tanh(k0 * (x + k1 * x ** 3))) + 0.5 * x * (1 - np.tanh(k0 * (x + k1 * x ** 3)) ** 2) * k0 * (1 + 3 * k1 * x * x)
+    m, n, k, lda_aux = 13, 9, 40, 16
+    base = dict(a_type=abi.CUDA_R_16BF, b_type=abi.CUDA_R_16BF, d_type=dt, compute_type=abi.CUBLAS_COMPUTE_32F,
+                scale_type=abi.CUDA_R_32F, alpha=0.25, m=m, n=n, k=k, transa=1, batch=2, order_c=od, order_d=od,
+                aux_ld=lda_aux, aux_batch_stride=lda_aux * 16)
+    tol = 1e-4 if dt == abi.CUDA_R_32F else 2.0 ** -8   # (the oracle evaluates GELU in float32: 1 + tanh cancels for x << 0)
+
+    def logical(case, storage, ld, stride, b):
+        i, j = np.meshgrid(np.arange(m), np.arange(n), indexing="ij")
+        idx = (i * ld + j) if od else (j * ld + i)
+        return decode_storage(storage[idx + b * stride], dt).astype(np.float64)
+
+    fwd = Case(dict(base, epilogue=abi.CUBLASLT_EPILOGUE_GELU_AUX_BIAS, bias_type=abi.CUDA_R_32F), 91)
+    d = fwd.run_oracle()
+    _, ldd, sd = __import__("oracle.cases", fromlist=["_layout"])._layout(fwd.spec, "d", m, n)
+    for b in range(2):
+        A, B = op_matrices(fwd, b)
+        x = 0.25 * decode_storage(A, abi.CUDA_R_16BF).astype(np.float64) @ decode_storage(B, abi.CUDA_R_16BF).astype(np.float64)
+        x = x + fwd.bias.astype(np.float64)[:m, None]
+        aux = logical(fwd, fwd.aux_ref, lda_aux, lda_aux * 16, b)
+        assert np.max(np.abs(aux - x) / np.maximum(np.abs(x), 1e-3)) <= tol
+        got = logical(fwd, d, ldd, sd, b)
+        assert np.max(np.abs(got - gelu(x)) / np.maximum(np.abs(gelu(x)), 1e-2)) <= tol
+    bwd = Case(dict(base, epilogue=abi.CUBLASLT_EPILOGUE_DGELU_BGRAD, bias_type=abi.CUDA_R_32F, bias_batch_stride=16, with_c=True), 92)
+    d = bwd.run_oracle()
+    for b in range(2):
+        A, B = op_matrices(bwd, b)
+        y = 0.25 * decode_storage(A, abi.CUDA_R_16BF).astype(np.float64) @ decode_storage(B, abi.CUDA_R_16BF).astype(np.float64)
+        y = y + float(bwd.beta[0]) * logical(bwd, bwd.Cm, ldd, sd, b)
+        want = y * dgelu(logical(bwd, bwd.aux, lda_aux, lda_aux * 16, b))
+        got = logical(bwd, d, ldd, sd, b)
+        assert np.max(np.abs(got - want) / np.maximum(np.abs(want), 1e-2)) <= tol
+        sums = bwd.bgrad_ref[16 * b:16 * b + m].astype(np.float64)
+        assert np.max(np.abs(sums - want.sum(axis=1))) <= 1e-5 * max(1.0, np.max(np.abs(want.sum(axis=1)))) + (0 if dt == abi.CUDA_R_32F else 0)
+    assert (bwd.bgrad_ref[m:16].view(np.uint32) == 0xCDCDCDCD).all()

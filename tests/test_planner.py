@@ -306,5 +306,15 @@ def test_bias_gradient_epilogues_are_planned_like_the_plain_problem(api):
     assert st == K.CUBLAS_STATUS_NOT_SUPPORTED
     st, _ = plan(api, dict(bf, batch=2, bias_batch_stride=512, epilogue=K.CUBLASLT_EPILOGUE_BGRADA))
     assert st == 0
-    st, _ = plan(api, dict(F8, m=512, n=512, k=512, transa=1, epilogue=K.CUBLASLT_EPILOGUE_DGELU))
+    # GELU with its input kept, GELU's gradient: the plain problem's kernel (a second pass finishes D); the aux matrix needs
+    # a leading dimension that holds D's rows, D a float type of 16 or 32 bits
+    f8 = dict(F8, m=512, n=512, k=512, transa=1)
+    st0, p0 = plan(api, f8)
+    for epi in (K.CUBLASLT_EPILOGUE_GELU_AUX, K.CUBLASLT_EPILOGUE_GELU_AUX_BIAS, K.CUBLASLT_EPILOGUE_DGELU, K.CUBLASLT_EPILOGUE_DGELU_BGRAD):
+        st, p = plan(api, dict(f8, epilogue=epi, aux_ld=512))
+        assert st == 0 and (p.kernel, p.variant, p.grid_x, p.grid_y) == (p0.kernel, p0.variant, p0.grid_x, p0.grid_y)
+        assert plan(api, dict(f8, epilogue=epi))[0] == K.CUBLAS_STATUS_INVALID_VALUE
+        assert plan(api, dict(f8, epilogue=epi, aux_ld=504))[0] == K.CUBLAS_STATUS_INVALID_VALUE
+        assert plan(api, dict(f8, epilogue=epi, aux_ld=512, d_type=K.CUDA_R_8F_E4M3))[0] == K.CUBLAS_STATUS_NOT_SUPPORTED
+    st, _ = plan(api, dict(I8, m=512, n=512, k=512, transa=1, epilogue=K.CUBLASLT_EPILOGUE_GELU_AUX, aux_ld=512))   # int32 scale type
     assert st == K.CUBLAS_STATUS_NOT_SUPPORTED

@@ -67,6 +67,8 @@ CUBLASLT_MATMUL_DESC_EPILOGUE = 7
 CUBLASLT_MATMUL_DESC_BIAS_POINTER = 8
 CUBLASLT_MATMUL_DESC_BIAS_BATCH_STRIDE = 10
 CUBLASLT_MATMUL_DESC_EPILOGUE_AUX_POINTER = 11
+CUBLASLT_MATMUL_DESC_EPILOGUE_AUX_LD = 12
+CUBLASLT_MATMUL_DESC_EPILOGUE_AUX_BATCH_STRIDE = 13
 CUBLASLT_MATMUL_DESC_ALPHA_VECTOR_BATCH_STRIDE = 14
 CUBLASLT_MATMUL_DESC_SM_COUNT_TARGET = 15
 CUBLASLT_MATMUL_DESC_A_SCALE_POINTER = 17
@@ -105,7 +107,9 @@ CUBLASLT_EPILOGUE_GELU = 32
 CUBLASLT_EPILOGUE_GELU_BIAS = 36
 CUBLASLT_EPILOGUE_RELU_AUX = 130
 CUBLASLT_EPILOGUE_GELU_AUX = 160
+CUBLASLT_EPILOGUE_GELU_AUX_BIAS = 164
 CUBLASLT_EPILOGUE_DGELU = 192
+CUBLASLT_EPILOGUE_DGELU_BGRAD = 208
 CUBLASLT_EPILOGUE_BGRADA = 256
 CUBLASLT_EPILOGUE_BGRADB = 512
 
@@ -160,7 +164,8 @@ class zluda_matmul_desc(C.Structure):
                 ("bias_batch_stride", C.c_int64), ("alpha_vector_batch_stride", C.c_int64),
                 ("a_scale", C.c_void_p), ("b_scale", C.c_void_p), ("c_scale", C.c_void_p),
                 ("d_scale", C.c_void_p), ("a_scale_mode", C.c_int32), ("b_scale_mode", C.c_int32),
-                ("c_scale_mode", C.c_int32), ("d_scale_mode", C.c_int32), ("fast_accum", C.c_int8)]
+                ("c_scale_mode", C.c_int32), ("d_scale_mode", C.c_int32), ("fast_accum", C.c_int8),
+                ("epilogue_aux", C.c_void_p), ("epilogue_aux_ld", C.c_int64), ("epilogue_aux_batch_stride", C.c_int64)]
 
 
 class zluda_gemm_problem(C.Structure):

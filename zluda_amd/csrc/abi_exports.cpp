@@ -104,7 +104,9 @@ bool epilogue_supported(uint32_t e) {
   case CUBLASLT_EPILOGUE_DEFAULT: case CUBLASLT_EPILOGUE_RELU: case CUBLASLT_EPILOGUE_BIAS:
   case CUBLASLT_EPILOGUE_RELU_BIAS: case CUBLASLT_EPILOGUE_GELU: case CUBLASLT_EPILOGUE_GELU_BIAS:
   case CUBLASLT_EPILOGUE_BGRADA: case CUBLASLT_EPILOGUE_BGRADB:
-    return true;
+  case CUBLASLT_EPILOGUE_GELU_AUX: case CUBLASLT_EPILOGUE_GELU_AUX_BIAS:
+  case CUBLASLT_EPILOGUE_DGELU: case CUBLASLT_EPILOGUE_DGELU_BGRAD:
+    return true;  // (the set zluda_common/src/lib.rs:762-804 maps; the ReLU bit-mask forms are not in it)
   default: return false;
   }
 }
@@ -169,6 +171,17 @@ cublasStatus_t desc_attr(MatmulDescObj *o, uint32_t attr, bool set, const void *
   }
   case CUBLASLT_MATMUL_DESC_BIAS_POINTER: return access(set, d.bias, in, out, size, written);
   case CUBLASLT_MATMUL_DESC_BIAS_BATCH_STRIDE: return access(set, d.bias_batch_stride, in, out, size, written);
+  // (the reference maps these ids, zluda_common/src/lib.rs:664-674, but its set-attribute refuses them,
+  // zluda_blaslt/src/impl.rs:302: the GELU_AUX / DGELU epilogues it forwards cannot be used through it)
+  case CUBLASLT_MATMUL_DESC_EPILOGUE_AUX_POINTER: return access(set, d.epilogue_aux, in, out, size, written);
+  case CUBLASLT_MATMUL_DESC_EPILOGUE_AUX_LD: return access(set, d.epilogue_aux_ld, in, out, size, written);
+  case CUBLASLT_MATMUL_DESC_EPILOGUE_AUX_BATCH_STRIDE: return access(set, d.epilogue_aux_batch_stride, in, out, size, written);
+  case CUBLASLT_MATMUL_DESC_EPILOGUE_AUX_DATA_TYPE: {
+    int32_t v = -1;  // the aux matrix has D's type
+    cublasStatus_t st = access(set, v, in, out, size, written);
+    if (set && !st && v != -1) return CUBLAS_STATUS_NOT_SUPPORTED;
+    return st;
+  }
   case CUBLASLT_MATMUL_DESC_ALPHA_VECTOR_BATCH_STRIDE:
     return access(set, d.alpha_vector_batch_stride, in, out, size, written);
   case CUBLASLT_MATMUL_DESC_SM_COUNT_TARGET: return access(set, o->sm_count_target, in, out, size, written);

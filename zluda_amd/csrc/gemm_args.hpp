@@ -39,6 +39,12 @@ struct GemmArgs {
   // (2, N values) go to `bgrad` in bias_type, batches bias_sb apart; `bias` is NULL then
   void *bgrad;
   int32_t bgrad_src;
+  // GELU with its input kept (aux_mode 1: aux = x, D = gelu(x)) and its gradient (aux_mode 2: D = D * gelu'(aux),
+  // aux_bgrad: the row sums of that D go to `bgrad`).  Run as a second, element-wise pass behind the GEMM
+  // kernel; aux is a matrix of D's type and order, strides in elements.
+  void *aux;
+  int64_t aux_si, aux_sj, aux_sb;
+  int32_t aux_mode, aux_bgrad;
 };
 
 } // namespace zluda_amd

@@ -7,6 +7,7 @@
 
 #include "decode_launch.hpp"
 #include "launch_util.hpp"
+#include "kernels/aux_epilogue.hpp"
 #include "kernels/bgrad_reduce.hpp"
 #include "kernels/decode_w8a8.hpp"
 #include "kernels/gemm_generic.hpp"
@@ -234,6 +235,14 @@ uint32_t launch_planned(const zluda_gemm_problem *p, const zluda_gemm_plan *plan
   if (!family_supports(plan->kernel, l)) return CUBLAS_STATUS_INVALID_VALUE;
   if (ws_size < plan->workspace) return CUBLAS_STATUS_INVALID_VALUE;
   if (zluda_gemm_device_cu_count() == 0) return CUBLAS_STATUS_NOT_INITIALIZED;
+  // GELU_AUX: the GEMM kernel writes the GELU input where the caller wants it kept, unscaled; the second pass
+  // below reads it back and writes D.  (DGELU: the kernel writes D as usual and the second pass rewrites it.)
+  const GemmArgs whole = l.g;
+  if (whole.aux_mode == 1) {
+    l.g.D = whole.aux;
+    l.g.d_si = whole.aux_si; l.g.d_sj = whole.aux_sj; l.g.d_sb = whole.aux_sb;
+    l.g.d_scale = nullptr;
+  }
   switch (plan->kernel) {
   case ZLUDA_KERNEL_GENERIC: {
     dim3 grid(plan->grid_x, plan->grid_y, plan->grid_z);
@@ -248,6 +257,10 @@ uint32_t launch_planned(const zluda_gemm_problem *p, const zluda_gemm_plan *plan
   default: return CUBLAS_STATUS_NOT_SUPPORTED;
   }
   if (st == CUBLAS_STATUS_SUCCESS && l.g.bgrad_src) st = launch_bgrad(l.g, s);
+  if (st == CUBLAS_STATUS_SUCCESS && whole.aux_mode == 1)
+    st = launch_kernel(aux_gelu_kernel, dim3((uint32_t)(((int64_t)whole.M * whole.N + 255) / 256), whole.batch), dim3(256), s, whole);
+  if (st == CUBLAS_STATUS_SUCCESS && whole.aux_mode == 2)
+    st = launch_kernel(aux_dgelu_kernel, dim3((whole.M + (whole.d_si == 1 ? 63 : 3)) / (whole.d_si == 1 ? 64 : 4), whole.batch), dim3(256), s, whole);
   return st;
 }
 

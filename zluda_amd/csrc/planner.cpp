@@ -175,7 +175,34 @@ uint32_t lower_problem(const zluda_gemm_problem *p, bool dry, Lowered *out) {
   // the bias buffer is an output here: sums over K of op(A)'s rows / op(B)'s columns, D as with DEFAULT
   case CUBLASLT_EPILOGUE_BGRADA: g.act = ACT_NONE; g.bgrad_src = 1; break;
   case CUBLASLT_EPILOGUE_BGRADB: g.act = ACT_NONE; g.bgrad_src = 2; break;
+  // GELU with its input kept, and GELU's gradient: the GEMM kernel runs without the activation, a second
+  // element-wise pass (kernels/aux_epilogue.hpp) finishes D
+  case CUBLASLT_EPILOGUE_GELU_AUX: g.act = ACT_NONE; g.aux_mode = 1; break;
+  case CUBLASLT_EPILOGUE_GELU_AUX_BIAS: g.act = ACT_NONE; g.aux_mode = 1; has_bias = true; break;
+  case CUBLASLT_EPILOGUE_DGELU: g.act = ACT_NONE; g.aux_mode = 2; break;
+  case CUBLASLT_EPILOGUE_DGELU_BGRAD: g.act = ACT_NONE; g.aux_mode = 2; g.aux_bgrad = 1; break;
   default: return CUBLAS_STATUS_NOT_SUPPORTED;
+  }
+  if (g.aux_mode) {
+    // the aux matrix has D's type, shape and order (cuda_types/src/cublaslt.rs:4207-4236: its leading dimension
+    // is no less than D's rows); both passes go through D's type, which has to be a float type of 16 or 32 bits
+    if (g.int_scale || !(d.type == CUDA_R_32F || d.type == CUDA_R_16F || d.type == CUDA_R_16BF)) return CUBLAS_STATUS_NOT_SUPPORTED;
+    const int64_t lead = d.order == CUBLASLT_ORDER_COL ? M : N, other = d.order == CUBLASLT_ORDER_COL ? N : M;
+    if (op.epilogue_aux_ld < lead) return CUBLAS_STATUS_INVALID_VALUE;
+    if (g.batch > 1 && op.epilogue_aux_batch_stride < op.epilogue_aux_ld * other && op.epilogue_aux_batch_stride != 0)
+      return CUBLAS_STATUS_INVALID_VALUE;
+    if (g.batch > 1 && op.epilogue_aux_batch_stride == 0 && g.aux_mode == 1) return CUBLAS_STATUS_NOT_SUPPORTED;  // aliased outputs
+    if (g.aux_mode == 2 && g.d_scale) return CUBLAS_STATUS_NOT_SUPPORTED;  // (the scale would have to follow the gradient)
+    if (!dry && !op.epilogue_aux) return CUBLAS_STATUS_INVALID_VALUE;
+    g.aux = op.epilogue_aux;
+    g.aux_si = d.order == CUBLASLT_ORDER_COL ? 1 : op.epilogue_aux_ld;
+    g.aux_sj = d.order == CUBLASLT_ORDER_COL ? op.epilogue_aux_ld : 1;
+    g.aux_sb = op.epilogue_aux_batch_stride;
+    if (g.aux_bgrad) {
+      if (g.batch > 1 && op.bias_batch_stride == 0) return CUBLAS_STATUS_NOT_SUPPORTED;
+      if (!dry && !op.bias) return CUBLAS_STATUS_INVALID_VALUE;
+      g.bgrad = const_cast<void *>(op.bias);
+    }
   }
   if (g.bgrad_src) {
     // sums of the stored elements: defined here for unscaled operands only
@@ -186,7 +213,7 @@ uint32_t lower_problem(const zluda_gemm_problem *p, bool dry, Lowered *out) {
     if (!dry && !op.bias) return CUBLAS_STATUS_INVALID_VALUE;
     g.bgrad = const_cast<void *>(op.bias);
   }
-  if (has_bias || g.bgrad_src) {
+  if (has_bias || g.bgrad_src || g.aux_bgrad) {
     if (has_bias && !dry && !op.bias) return CUBLAS_STATUS_INVALID_VALUE;
     if (has_bias) g.bias = op.bias;
     g.bias_sb = op.bias_batch_stride;

@@ -184,6 +184,10 @@ class MatmulCall:
             api.check(api.desc_set(self.desc, D.CUBLASLT_MATMUL_DESC_B_SCALE_MODE, C.c_int32, s["b_scale_mode"]), "B_SCALE_MODE")
         if "bias_batch_stride" in s:
             api.check(api.desc_set(self.desc, D.CUBLASLT_MATMUL_DESC_BIAS_BATCH_STRIDE, C.c_int64, s["bias_batch_stride"]), "BIAS_BATCH_STRIDE")
+        if "aux_ld" in s:
+            api.check(api.desc_set(self.desc, D.CUBLASLT_MATMUL_DESC_EPILOGUE_AUX_LD, C.c_int64, s["aux_ld"]), "EPILOGUE_AUX_LD")
+        if "aux_batch_stride" in s:
+            api.check(api.desc_set(self.desc, D.CUBLASLT_MATMUL_DESC_EPILOGUE_AUX_BATCH_STRIDE, C.c_int64, s["aux_batch_stride"]), "EPILOGUE_AUX_BATCH_STRIDE")
         if "alpha_vector_batch_stride" in s:
             api.check(api.desc_set(self.desc, D.CUBLASLT_MATMUL_DESC_ALPHA_VECTOR_BATCH_STRIDE, C.c_int64,
                                    s["alpha_vector_batch_stride"]), "ALPHA_VECTOR_BATCH_STRIDE")
@@ -233,9 +237,10 @@ class MatmulCall:
     def variant(self):
         return int(self.algo.data[1] & 0xFFFFFFFF)
 
-    def set_pointers(self, bias=None, a_scale=None, b_scale=None, c_scale=None, d_scale=None):
+    def set_pointers(self, bias=None, a_scale=None, b_scale=None, c_scale=None, d_scale=None, aux=None):
         api, D = self.api, abi
         for attr, val in ((D.CUBLASLT_MATMUL_DESC_BIAS_POINTER, bias),
+                          (D.CUBLASLT_MATMUL_DESC_EPILOGUE_AUX_POINTER, aux),
                           (D.CUBLASLT_MATMUL_DESC_A_SCALE_POINTER, a_scale),
                           (D.CUBLASLT_MATMUL_DESC_B_SCALE_POINTER, b_scale),
                           (D.CUBLASLT_MATMUL_DESC_C_SCALE_POINTER, c_scale),
