@@ -384,7 +384,7 @@ class Case:
             if rp.why:
                 return None, rp.why
             if not rp.set_pointers(bias=ptr["bias"], a_scale=ptr["a_scale"], b_scale=ptr["b_scale"],
-                                   c_scale=ptr["c_scale"], d_scale=ptr["d_scale"]):
+                                   c_scale=ptr["c_scale"], d_scale=ptr["d_scale"], aux=ptr["aux"]):
                 return None, rp.why
             if not rp.find_algo():
                 return None, rp.why
@@ -395,6 +395,8 @@ class Case:
                 return None, "hipblasLtMatmul status %d" % st
             if self.bgrad:
                 self.bgrad_theirs = keep[3][:self.bias.nbytes].cpu().numpy().view(self.bias.dtype).copy()
+            if self.aux_mode == 1:
+                self.aux_theirs = keep[10][:self.aux.nbytes].cpu().numpy().view(self.aux.dtype).copy()
             return self.download(dt), ""
         finally:
             rp.close()

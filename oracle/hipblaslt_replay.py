@@ -21,6 +21,7 @@ L_BATCH_COUNT, L_STRIDE, L_TYPE, L_ORDER, L_ROWS, L_COLS, L_LD = 0, 1, 2, 3, 4, 
 # matmul desc attribute ids: ext/hipblaslt-sys/src/lib.rs:351-440 (+ 31/32 from the installed header)
 D_TRANSA, D_TRANSB, D_EPILOGUE, D_BIAS_POINTER, D_BIAS_DATA_TYPE = 0, 1, 2, 3, 4
 D_A_SCALE_POINTER, D_B_SCALE_POINTER, D_C_SCALE_POINTER, D_D_SCALE_POINTER = 5, 6, 7, 8
+D_AUX_POINTER, D_AUX_LD, D_AUX_BATCH_STRIDE = 10, 11, 12
 D_POINTER_MODE, D_A_SCALE_MODE, D_B_SCALE_MODE = 13, 31, 32
 P_MAX_WORKSPACE = 1
 
@@ -105,6 +106,9 @@ class Replay:
             if pm == abi.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO:
                 pm = abi.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_HOST   # hipBLASLt only has the BETA_HOST form
             bad |= dset(D_POINTER_MODE, C.c_int32, pm)
+        if "aux_ld" in s:
+            bad |= dset(D_AUX_LD, C.c_int64, s["aux_ld"])
+            bad |= dset(D_AUX_BATCH_STRIDE, C.c_int64, s.get("aux_batch_stride", 0))
         if "a_scale_mode" in s:
             bad |= dset(D_A_SCALE_MODE, C.c_int32, s["a_scale_mode"])
         if "b_scale_mode" in s:
@@ -148,8 +152,8 @@ class Replay:
         self.res = hipblasLtMatmulHeuristicResult_t()
         self._pointers_set = False
 
-    def set_pointers(self, bias=None, a_scale=None, b_scale=None, c_scale=None, d_scale=None):
-        for attr, val in ((D_BIAS_POINTER, bias), (D_A_SCALE_POINTER, a_scale), (D_B_SCALE_POINTER, b_scale),
+    def set_pointers(self, bias=None, a_scale=None, b_scale=None, c_scale=None, d_scale=None, aux=None):
+        for attr, val in ((D_BIAS_POINTER, bias), (D_AUX_POINTER, aux), (D_A_SCALE_POINTER, a_scale), (D_B_SCALE_POINTER, b_scale),
                           (D_C_SCALE_POINTER, c_scale), (D_D_SCALE_POINTER, d_scale)):
             if val is not None and self._dset(attr, C.c_void_p, val):
                 return False

@@ -44,7 +44,9 @@
  *     hipBLASLt itself (it applies the tanh form)
  *   - DGELU_BGRAD: that the gradient is the sum over D's columns, one value per row of D (the orientation of the
  *     bias it is the gradient of), and that the aux matrix has D's order: the text cited above gives the lengths and
- *     the leading dimension only; hipBLASLt offers none of the four aux epilogues for the 8-bit inputs of this path
+ *     the leading dimension only.  No CPU-side fixture pins it; on a GPU box tests/test_gpu_aux_epilogues.py
+ *     compares D, the aux matrix and the gradient with hipBLASLt itself for f16 operands (it offers these
+ *     epilogues for no other input type)
  *   - the batch stride of the UE8M0 scale tensors for batch counts above 1 (restated as batches back to
  *     back, rows * K/32 bytes each): hipBLASLt takes MXFP4 at batch 1 only.  The layout inside a batch,
  *     plain [row][K/32] bytes for both operands, is pinned on a GPU box against hipBLASLt itself by the

@@ -78,3 +78,24 @@ def test_aux_epilogues_refusals(gpu_api):
     case.spec["aux_ld"] = 64
     case.aux = None
     assert case.run_gpu_plan(gpu_api, K.ZLUDA_KERNEL_AUTO)[0] == K.CUBLAS_STATUS_INVALID_VALUE
+
+
+@pytest.mark.parametrize("epi", FWD + BWD)
+@pytest.mark.parametrize("ta,tb", [(1, 0), (0, 1)])
+def test_aux_epilogues_against_hipblaslt(gpu_api, epi, ta, tb, typ=K.CUDA_R_16F):
+    """the reference's backend on the same buffers (f16 operands: what the installed hipBLASLt offers these epilogues for;
+    it has no algorithm for bf16): the same D, the same aux matrix, the same bias gradient -- which pins the orientation of
+    the aux matrix and of the sums"""
+    spec = dict(BF, a_type=typ, b_type=typ, c_type=typ, d_type=typ, m=256, n=128, k=512, transa=ta, transb=tb, epilogue=epi,
+                aux_ld=264)
+    case = Case(spec, 960 + epi)
+    st, ours, _, _ = case.run_gpu(gpu_api)
+    assert st == 0
+    theirs, why = case.run_hipblaslt()
+    if theirs is None:
+        pytest.skip("hipBLASLt offers no algorithm here: " + why)
+    case.compare(ours, theirs, tol=1.6e-2, floor_frac=1e-2)
+    if case.aux_mode == 1:
+        case.compare_aux(case.aux_got, case.aux_theirs)
+    if case.bgrad:
+        case.compare_bgrad(case.bgrad_got, case.bgrad_theirs, floor_frac=1.0)
