@@ -1,7 +1,8 @@
 """cublasLtMatmul under HIP graph capture: the launch layer only enqueues kernels (no allocation, no
-memset, no synchronisation), so a serving loop can record its GEMMs once and replay them.  Three
+memset, no synchronisation), so a serving loop can record its GEMMs once and replay them.  Five
 calls of different kernel families -- including a split-K call, which is two kernels through the
-caller's workspace -- are captured into one graph; it is replayed several times with fresh operand
+caller's workspace, and a GELU_AUX_BIAS call, which is a GEMM kernel and an element-wise pass -- are
+captured into one graph; it is replayed several times with fresh operand
 contents between the replays, and every replay is checked against the CPU oracle."""
 import numpy as np
 import pytest
@@ -23,10 +24,17 @@ SPECS = [
           b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F, epilogue=K.CUBLASLT_EPILOGUE_BIAS,
           bias_type=K.CUDA_R_32F, alpha_range=(0.001, 0.01), scale_range=(0.005, 0.02), bias_std=0.02), 0,
      K.ZLUDA_KERNEL_DECODE_W8A8),
+    # 24 tokens, K = 8192: the 8-wave slab shape with two token blocks
+    (dict(I8, transa=1, c_type=K.CUDA_R_16BF, d_type=K.CUDA_R_16BF, scale_type=K.CUDA_R_32F, m=1000, n=24, k=8192,
+          epilogue=K.CUBLASLT_EPILOGUE_RELU_BIAS, alpha_range=(0.0005, 0.001)), 0, K.ZLUDA_KERNEL_DECODE_W8A8),
+    # GELU input kept: GEMM kernel into the aux matrix, then the element-wise pass into D
+    (dict(a_type=K.CUDA_R_8F_E4M3, b_type=K.CUDA_R_8F_E4M3, c_type=K.CUDA_R_16F, d_type=K.CUDA_R_16F, compute_type=K.CUBLAS_COMPUTE_32F,
+          scale_type=K.CUDA_R_32F, transa=1, m=384, n=264, k=512, epilogue=K.CUBLASLT_EPILOGUE_GELU_AUX_BIAS, aux_ld=400,
+          with_scalar_scales=True, scale_range=(0.05, 0.06)), 0, K.ZLUDA_KERNEL_MFMA_F8),
 ]
 
 
-def test_three_families_in_one_graph(gpu_api):
+def test_kernel_families_in_one_graph(gpu_api):
     import torch
     print("graph capture of", [s for s, _, _ in SPECS], flush=True)
     cases, calls, bufs = [], [], []
@@ -36,7 +44,7 @@ def test_three_families_in_one_graph(gpu_api):
         call = MatmulCall(gpu_api, case.spec, max_workspace=ws_bytes)
         assert call.kernel == want
         call.set_pointers(bias=ptr["bias"], a_scale=ptr["a_scale"], b_scale=ptr["b_scale"],
-                          c_scale=ptr["c_scale"], d_scale=ptr["d_scale"])
+                          c_scale=ptr["c_scale"], d_scale=ptr["d_scale"], aux=ptr["aux"])
         ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device="cuda:0")
         cases.append(case); calls.append(call); bufs.append((keep, ptr, dt, ws, ws_bytes))
 
@@ -70,6 +78,8 @@ def test_three_families_in_one_graph(gpu_api):
             torch.cuda.synchronize()
             for case, (keep, ptr, dt, ws, ws_bytes) in zip(cases, bufs):
                 case.compare(case.download(dt), case.run_oracle())
+                if case.aux_mode == 1:
+                    case.compare_aux(keep[10][:case.aux.nbytes].cpu().numpy().view(case.aux.dtype).copy(), case.aux_ref)
     finally:
         for call in calls:
             call.close()
