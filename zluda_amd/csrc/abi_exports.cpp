@@ -312,7 +312,7 @@ bool unpack_algo(const cublasLtMatmulAlgo_t *algo, uint32_t *kernel, int32_t *va
   if ((algo->data[0] >> 32) != ZLUDA_ALGO_MAGIC) return false;
   *kernel = (uint32_t)(algo->data[0] & 0xffffffffu);
   *variant = (int32_t)algo->data[1];
-  return *kernel >= ZLUDA_KERNEL_GENERIC && *kernel <= ZLUDA_KERNEL_MFMA_TR8;
+  return *kernel >= ZLUDA_KERNEL_GENERIC && *kernel <= ZLUDA_KERNEL_MFMA_H16;
 }
 
 // A/B forcing for measurements: ZLUDA_FORCE_KERNEL=<family>[:<variant>], read once per process (the
@@ -664,6 +664,8 @@ static int families_for_types(uint32_t computeType, uint32_t scaleType, uint32_t
   // 1024^3 A:T B:N admits every square-GEMM family; the decode family wants a skinny shape
   for (uint32_t k = ZLUDA_KERNEL_GENERIC; k <= ZLUDA_KERNEL_MFMA_MXF4; k++)
     if (zluda_gemm_plan_problem(&p, k, -1, 256, &plan) == CUBLAS_STATUS_SUCCESS) ids[count++] = (int)k;
+  if (zluda_gemm_plan_problem(&p, ZLUDA_KERNEL_MFMA_H16, -1, 256, &plan) == CUBLAS_STATUS_SUCCESS)
+    ids[count++] = ZLUDA_KERNEL_MFMA_H16;
   p.b.cols = p.c.cols = p.d.cols = 16;
   if (zluda_gemm_plan_problem(&p, ZLUDA_KERNEL_DECODE_W8A8, -1, 256, &plan) == CUBLAS_STATUS_SUCCESS)
     ids[count++] = ZLUDA_KERNEL_DECODE_W8A8;

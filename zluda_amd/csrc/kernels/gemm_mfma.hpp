@@ -5,6 +5,8 @@
 //   KIND_I8   : int8 x int8 -> int32         v_mfma_i32_32x32x32_i8
 //   KIND_F8   : e4m3/e5m2 -> fp32            v_mfma_f32_32x32x64_f8f6f4 (formats FP/FQ)
 //   KIND_MXF4 : e2m1 + UE8M0 per 32 -> fp32  v_mfma_scale_f32_32x32x64_f8f6f4 (cbsz=blgp=4)
+//   KIND_F16  : f16 x f16 -> fp32            v_mfma_f32_32x32x16_f16
+//   KIND_BF16 : bf16 x bf16 -> fp32          v_mfma_f32_32x32x16_bf16
 //
 // Naming inside the kernel: P is the operand whose row index runs along the unit-stride
 // dimension of D (it is fed as MFMA operand "B", so its index lands on lane%32 of the
@@ -28,7 +30,12 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
-enum { KIND_I8 = 0, KIND_F8 = 1, KIND_MXF4 = 2 };
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef __bf16 v8b __attribute__((ext_vector_type(8)));
+
+enum { KIND_I8 = 0, KIND_F8 = 1, KIND_MXF4 = 2, KIND_F16 = 3, KIND_BF16 = 4 };
+// 16-bit elements: 16 bytes (8 elements) of K per lane and MFMA, i.e. the byte geometry of int8
+constexpr bool kind_is_h16(int kind) { return kind == KIND_F16 || kind == KIND_BF16; }
 
 // depends on r mod 32 only, so rows 32 apart (the MFMA tiles of one wave) share a swizzle
 __device__ __forceinline__ int swz(int r) { return (r ^ ((r >> 3) & 3)) & 7; }

@@ -1,5 +1,5 @@
 // Software-pipelined MFMA GEMM for K-contiguous operands on gfx950: the production kernel of the
-// int8 / fp8 / MXFP4 families.
+// int8 / fp8 / MXFP4 / f16 / bf16 families.
 //
 // Same tiling, operand naming (P / Q) and epilogue as gemm_mfma.hpp; what differs is the K loop:
 //
@@ -66,7 +66,8 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
   static_assert((NSTAGE - 1) * NLOAD < 64, "vmcnt range");
   static_assert((NSTAGE * STAGE_V4 + 2 * CHUNK_V4) * 16 <= 160 * 1024, "LDS capacity");
   using acc_v = typename std::conditional<KIND == KIND_I8, v16i, v16f>::type;
-  using frag_v = typename std::conditional<KIND == KIND_I8, v4i, v8i>::type;
+  constexpr bool B16 = KIND == KIND_I8 || kind_is_h16(KIND);  // 16 bytes of K per lane and MFMA (else 32)
+  using frag_v = typename std::conditional<B16, v4i, v8i>::type;
   struct Frags { frag_v p[TP], q[TQ]; };
   struct Scales { int p[TP], q[TQ]; };  // MX scale dwords of one stage (one per MFMA tile row set)
 
@@ -91,7 +92,7 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
   const int p0 = tile_p * BP, q0 = tile_q * BQ;
 
   const int NP = prm.swapped ? g.N : g.M, NQ = prm.swapped ? g.M : g.N;
-  constexpr int ebits = KIND == KIND_MXF4 ? 4 : 8;
+  constexpr int ebits = KIND == KIND_MXF4 ? 4 : (kind_is_h16(KIND) ? 16 : 8);
   const int Kbytes = (int)((int64_t)g.K * ebits / 8);
   const uint8_t *Pg, *Qg;
   int ldp, ldq;
@@ -211,19 +212,19 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
         f.q[i] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
       }
     } else {
-      // int8: chunk ks*2+gsel (natural K order).  fp4: lane group gsel owns chunks gsel*KS .. +KS-1,
+      // int8, f16, bf16: chunk ks*2+gsel (natural K order).  fp4: lane group gsel owns chunks gsel*KS .. +KS-1,
       // so that its sub-steps use consecutive scale bytes
-      const int ch = (KIND == KIND_I8 ? ks * 2 + gsel : gsel * KS + ks) ^ fsw;
+      const int ch = (B16 ? ks * 2 + gsel : gsel * KS + ks) ^ fsw;
 #pragma unroll
       for (int i = 0; i < TP; i++) {
         const v4i lo = Pl[i * 32 * CPR + ch];
-        if constexpr (KIND == KIND_I8) f.p[i] = lo;
+        if constexpr (B16) f.p[i] = lo;
         else f.p[i] = v8i{lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
       }
 #pragma unroll
       for (int i = 0; i < TQ; i++) {
         const v4i lo = Ql[i * 32 * CPR + ch];
-        if constexpr (KIND == KIND_I8) f.q[i] = lo;
+        if constexpr (B16) f.q[i] = lo;
         else f.q[i] = v8i{lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
       }
     }
@@ -263,6 +264,12 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
           acc[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.q[a], f.p[b], acc[a][b], 0, 0, 0);
         else if constexpr (KIND == KIND_F8)
           acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.q[a], f.p[b], acc[a][b], FQ, FP, 0, 0, 0, 0);
+        else if constexpr (KIND == KIND_F16)
+          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, f.q[a]), __builtin_bit_cast(v8h, f.p[b]),
+                                                             acc[a][b], 0, 0, 0);
+        else if constexpr (KIND == KIND_BF16)
+          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8b, f.q[a]), __builtin_bit_cast(v8b, f.p[b]),
+                                                              acc[a][b], 0, 0, 0);
         else
           acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.q[a], f.p[b], acc[a][b], 4, 4, ks, sc.q[a],
                                                                        ks, sc.p[b]);

@@ -49,7 +49,7 @@ uint32_t launch_mfma(const Lowered &l, const zluda_gemm_plan &plan, void *ws, ui
     const uint64_t need = (uint64_t)plan.grid_z * l.g.batch * prm.tiles_p * v.bp * prm.tiles_q * v.bq * 4;
     if (!ws || (((uintptr_t)ws) & 15) || ws_size < need || plan.workspace != need) return CUBLAS_STATUS_INVALID_VALUE;
     const bool mx = plan.kernel == ZLUDA_KERNEL_MFMA_MXF4;
-    const int kbytes = mx ? l.g.K / 2 : l.g.K;
+    const int kbytes = mx ? l.g.K / 2 : (plan.kernel == ZLUDA_KERNEL_MFMA_H16 ? l.g.K * 2 : l.g.K);
     const int stages = (kbytes + v.bkb - 1) / v.bkb;
     prm.splits = (int32_t)plan.grid_z;
     prm.split_stages = (stages + prm.splits - 1) / prm.splits;
@@ -63,6 +63,7 @@ uint32_t launch_mfma(const Lowered &l, const zluda_gemm_plan &plan, void *ws, ui
   switch (plan.kernel) {
   case ZLUDA_KERNEL_MFMA_I8: st = launch_mfma_i8(prm, plan, s); break;
   case ZLUDA_KERNEL_MFMA_MXF4: st = launch_mfma_mxf4(prm, plan, s); break;
+  case ZLUDA_KERNEL_MFMA_H16: st = launch_mfma_h16(prm, plan, l.g.a_type == CUDA_R_16BF, s); break;
   case ZLUDA_KERNEL_MFMA_F8: {
     // MFMA operand "A" is Q, operand "B" is P (see gemm_mfma.hpp)
     const int fa = f8_fmt(l.g.a_type), fb = f8_fmt(l.g.b_type);
@@ -251,7 +252,9 @@ uint32_t launch_planned(const zluda_gemm_problem *p, const zluda_gemm_plan *plan
                  : launch_kernel(gemm_generic_kernel<false>, grid, dim3(256), s, l.g);
     break;
   }
-  case ZLUDA_KERNEL_MFMA_I8: case ZLUDA_KERNEL_MFMA_F8: case ZLUDA_KERNEL_MFMA_MXF4: st = launch_mfma(l, *plan, ws, ws_size, s); break;
+  case ZLUDA_KERNEL_MFMA_I8: case ZLUDA_KERNEL_MFMA_F8: case ZLUDA_KERNEL_MFMA_MXF4: case ZLUDA_KERNEL_MFMA_H16:
+    st = launch_mfma(l, *plan, ws, ws_size, s);
+    break;
   case ZLUDA_KERNEL_DECODE_W8A8: st = launch_decode(l, *plan, s); break;
   case ZLUDA_KERNEL_MFMA_TR8: st = launch_tr(l, *plan, ws, ws_size, s); break;
   default: return CUBLAS_STATUS_NOT_SUPPORTED;

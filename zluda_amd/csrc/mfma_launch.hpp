@@ -34,7 +34,7 @@ inline uint32_t launch_mfma_variant(const MfmaParams &prm, const zluda_gemm_plan
     static_assert(kMfmaVariants[V].bp == BP && kMfmaVariants[V].bq == BQ && kMfmaVariants[V].wp == WP &&   \
                   kMfmaVariants[V].wq == WQ && kMfmaVariants[V].bkb == 128 && kMfmaVariants[V].stages == 2 && \
                   kMfmaVariants[V].m16, "variant table mismatch");                                         \
-    if constexpr (KIND == KIND_MXF4) return CUBLAS_STATUS_INVALID_VALUE;                                   \
+    if constexpr (KIND != KIND_I8 && KIND != KIND_F8) return CUBLAS_STATUS_INVALID_VALUE;                                   \
     else return launch_kernel(gemm_mfma_pipe16_kernel<KIND, FQ, FP, BP, BQ, WP, WQ>, grid, dim3(WP * WQ * 64), s, prm);
     ZLUDA_MFMA16_CASE(8, 256, 256, 2, 4)
     ZLUDA_MFMA16_CASE(9, 192, 256, 2, 4)
@@ -48,5 +48,6 @@ inline uint32_t launch_mfma_variant(const MfmaParams &prm, const zluda_gemm_plan
 uint32_t launch_mfma_i8(const MfmaParams &prm, const zluda_gemm_plan &plan, hipStream_t s);
 uint32_t launch_mfma_f8(const MfmaParams &prm, const zluda_gemm_plan &plan, int fq, int fp, hipStream_t s);
 uint32_t launch_mfma_mxf4(const MfmaParams &prm, const zluda_gemm_plan &plan, hipStream_t s);
+uint32_t launch_mfma_h16(const MfmaParams &prm, const zluda_gemm_plan &plan, bool bf16, hipStream_t s);
 
 } // namespace zluda_amd

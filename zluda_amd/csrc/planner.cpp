@@ -291,6 +291,10 @@ bool family_supports(uint32_t kernel, const Lowered &l) {
     return fast_layout && l.span_ok && g.a_type == CUDA_R_4F_E2M1 && g.b_type == CUDA_R_4F_E2M1 &&
            g.a_scale_mode == SCALE_BLOCK32_UE8M0 && g.b_scale_mode == SCALE_BLOCK32_UE8M0 &&
            (g.K % 256) == 0 && ((((uintptr_t)g.a_scale) | ((uintptr_t)g.b_scale)) & 3) == 0 && d_fast;
+  case ZLUDA_KERNEL_MFMA_H16:
+    // f16 x f16 or bf16 x bf16 (lower_problem admits 16-bit operands of one type only)
+    return fast_layout && l.span_ok && (g.a_type == CUDA_R_16F || g.a_type == CUDA_R_16BF) && g.b_type == g.a_type &&
+           g.a_scale_mode != SCALE_BLOCK32_UE8M0 && g.b_scale_mode != SCALE_BLOCK32_UE8M0 && d_fast;
   case ZLUDA_KERNEL_MFMA_TR8: {
     // 8-bit operands, each with unit stride along K or along its row index; dword-aligned loads
     const bool types = (g.a_type == CUDA_R_8I && g.b_type == CUDA_R_8I) ||
@@ -340,7 +344,8 @@ static void fill_mfma_plan(const Lowered &l, int variant, uint32_t cus, uint64_t
   // kernel sums them and applies the epilogue.  Only if the caller's workspace holds the partial
   // tiles (padded to whole tiles).  (MXFP4 shares are whole scale chunks: the launcher rounds.)
   const uint64_t tiles = (uint64_t)plan->grid_x * plan->grid_y;
-  const uint32_t kt = ceil_div((uint32_t)((int64_t)g.K * (g.a_type == CUDA_R_4F_E2M1 ? 4 : 8) / 8), v.bkb);
+  const bool h16 = g.a_type == CUDA_R_16F || g.a_type == CUDA_R_16BF;
+  const uint32_t kt = ceil_div((uint32_t)((int64_t)g.K * (g.a_type == CUDA_R_4F_E2M1 ? 4 : (h16 ? 16 : 8)) / 8), v.bkb);
   // (below ~6 KiB of K per row the second kernel and the workspace traffic cost more than the idle CUs)
   const uint32_t kbytes = kt * v.bkb;
   // Skinny problems (<= 64 rows or columns) are memory bound: they split from 2 KiB of K per row on
@@ -384,7 +389,7 @@ static int pick_mfma_variant(const Lowered &l, uint32_t cus) {
     const MfmaVariant &t = kMfmaVariants[v];
     const uint64_t tiles = (uint64_t)ceil_div(np, t.bp) * ceil_div(nq, t.bq) * g.batch;
     if (t.m16) {
-      if (g.a_type == CUDA_R_4F_E2M1) continue;  // the 16x16 shapes serve int8 and fp8
+      if (g.a_type == CUDA_R_4F_E2M1 || g.a_type == CUDA_R_16F || g.a_type == CUDA_R_16BF) continue;  // the 16x16 shapes serve int8 and fp8
       // power bound or not: int8 gains from three quarters of the CUs busy on.  fp8 gains little and only on
       // long runs: the 192x256 tile from two full rounds on (6144^3: 190 us against 198), the 256x256 tile
       // from four (8192^3: 405 against 408; at two rounds, 8192x4096x4096, it loses 3 %)
@@ -517,7 +522,7 @@ extern "C" uint32_t zluda_gemm_variant_count(uint32_t kernel) {
   switch (kernel) {
   case ZLUDA_KERNEL_GENERIC: return 1;
   case ZLUDA_KERNEL_MFMA_I8: case ZLUDA_KERNEL_MFMA_F8: return kNumMfmaVariants;
-  case ZLUDA_KERNEL_MFMA_MXF4: return kNumMfmaVariants32;  // the 16x16-shape ones serve int8 and fp8
+  case ZLUDA_KERNEL_MFMA_MXF4: case ZLUDA_KERNEL_MFMA_H16: return kNumMfmaVariants32;  // the 16x16-shape ones serve int8 and fp8
   case ZLUDA_KERNEL_DECODE_W8A8: return kNumDecodeVariants;
   case ZLUDA_KERNEL_MFMA_TR8: return kNumTrVariants;
   default: return 0;
@@ -537,7 +542,8 @@ extern "C" uint32_t zluda_gemm_plan_problem(const zluda_gemm_problem *p, uint32_
   uint32_t kernel = forced_kernel;
   if (kernel == ZLUDA_KERNEL_AUTO) {
     static const uint32_t order[] = {ZLUDA_KERNEL_DECODE_W8A8, ZLUDA_KERNEL_MFMA_I8, ZLUDA_KERNEL_MFMA_F8,
-                                     ZLUDA_KERNEL_MFMA_MXF4, ZLUDA_KERNEL_MFMA_TR8, ZLUDA_KERNEL_GENERIC};
+                                     ZLUDA_KERNEL_MFMA_MXF4, ZLUDA_KERNEL_MFMA_H16, ZLUDA_KERNEL_MFMA_TR8,
+                                     ZLUDA_KERNEL_GENERIC};
     for (uint32_t k : order) {
       if (!family_supports(k, l)) continue;
       if (k == ZLUDA_KERNEL_DECODE_W8A8) {
@@ -571,9 +577,10 @@ extern "C" uint32_t zluda_gemm_plan_problem(const zluda_gemm_problem *p, uint32_
     plan->waves = (float)plan->grid_x * plan->grid_y * plan->grid_z / (float)(cu_count * 8);
     if (plan->grid_y > 65535) return CUBLAS_STATUS_NOT_SUPPORTED;
     break;
-  case ZLUDA_KERNEL_MFMA_I8: case ZLUDA_KERNEL_MFMA_F8: case ZLUDA_KERNEL_MFMA_MXF4: {
+  case ZLUDA_KERNEL_MFMA_I8: case ZLUDA_KERNEL_MFMA_F8: case ZLUDA_KERNEL_MFMA_MXF4: case ZLUDA_KERNEL_MFMA_H16: {
     int v = forced_variant >= 0 ? forced_variant : pick_mfma_variant(l, cu_count);
-    if (v >= kNumMfmaVariants || (kMfmaVariants[v].m16 && kernel == ZLUDA_KERNEL_MFMA_MXF4)) return CUBLAS_STATUS_INVALID_VALUE;
+    if (v >= kNumMfmaVariants || (kMfmaVariants[v].m16 && (kernel == ZLUDA_KERNEL_MFMA_MXF4 || kernel == ZLUDA_KERNEL_MFMA_H16)))
+      return CUBLAS_STATUS_INVALID_VALUE;
     fill_mfma_plan(l, v, cu_count, p->workspace_size, plan);
     break;
   }
