@@ -288,6 +288,10 @@ def test_algorithm_enumeration_and_configuration(api):
     f4 = (abi.CUBLAS_COMPUTE_32F, abi.CUDA_R_32F, abi.CUDA_R_4F_E2M1, abi.CUDA_R_4F_E2M1, abi.CUDA_R_16BF, abi.CUDA_R_16BF)
     assert api.cublasLtMatmulAlgoGetIds(h, *f4, 8, ids, C.byref(n)) == 0
     assert sorted(ids[:n.value]) == [abi.ZLUDA_KERNEL_GENERIC, abi.ZLUDA_KERNEL_MFMA_MXF4]
+    for t in (abi.CUDA_R_16BF, abi.CUDA_R_16F):
+        h16 = (abi.CUBLAS_COMPUTE_32F, abi.CUDA_R_32F, t, t, t, t)
+        assert api.cublasLtMatmulAlgoGetIds(h, *h16, 8, ids, C.byref(n)) == 0
+        assert sorted(ids[:n.value]) == [abi.ZLUDA_KERNEL_GENERIC, abi.ZLUDA_KERNEL_MFMA_H16, abi.ZLUDA_KERNEL_MFMA_TR16]
     # a combination nothing runs
     bad = (abi.CUBLAS_COMPUTE_32I, abi.CUDA_R_32I, abi.CUDA_R_32F, abi.CUDA_R_32F, abi.CUDA_R_32I, abi.CUDA_R_32I)
     assert api.cublasLtMatmulAlgoGetIds(h, *bad, 8, ids, C.byref(n)) == 0 and n.value == 0

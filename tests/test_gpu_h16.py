@@ -1,6 +1,6 @@
 """f16 x f16 and bf16 x bf16 problems (the 16-bit operand types cublasLtMatmul is mostly called with outside of quantized
 inference; the reference forwards them to hipBLASLt like everything else, zluda_blaslt/src/impl.rs:157-196) on the MFMA
-kernels: against the float64 oracle, and against hipBLASLt called the way the reference calls it."""
+kernels (K-contiguous operands on the pipelined kernel, every other layout on the transposing one): against the float64 oracle, and against hipBLASLt called the way the reference calls it."""
 import pytest
 
 from oracle.cases import Case
@@ -42,6 +42,44 @@ def test_k_contiguous_operands_run_on_the_16_bit_mfma_family(gpu_api, typ, shape
     for v in range(gpu_api.zluda_gemm_variant_count(K.ZLUDA_KERNEL_MFMA_H16)):
         st, got_v, kernel, variant = case.run_gpu(gpu_api, forced_kernel=K.ZLUDA_KERNEL_MFMA_H16, forced_variant=v)
         assert st == 0 and (kernel, variant) == (K.ZLUDA_KERNEL_MFMA_H16, v)
+        case.compare(got_v, ref, tol=1e-2)
+    if "order_d" in spec:
+        return  # (the installed hipBLASLt writes only part of a row-major D with a bias vector)
+    theirs, why = case.run_hipblaslt()
+    if theirs is None:
+        pytest.skip("hipBLASLt offers no algorithm here: " + why)
+    case.compare(got, theirs, tol=1e-2, floor_frac=1e-2)
+
+
+TR_SHAPES = [
+    dict(m=300, n=200, k=384, transa=0, transb=0),
+    dict(m=256, n=256, k=77, transa=0, transb=1),                                # odd K: neither operand has K pieces of 16 bytes
+    dict(m=513, n=130, k=1000, transa=1, transb=1, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS),
+    dict(m=150, n=90, k=4100, transa=0, transb=1, with_c=True),
+    dict(m=200, n=136, k=264, transa=0, transb=0, batch=3, d_type=K.CUDA_R_32F, c_type=K.CUDA_R_32F),
+    dict(m=320, n=200, k=256, transa=0, transb=0, order_d=1, order_c=1, epilogue=K.CUBLASLT_EPILOGUE_BIAS),
+    dict(m=300, n=200, k=392, transa=1, transb=0, lda=394, ldb=398),             # K-contiguous, pitches of 4-byte alignment only
+    dict(m=128, n=512, k=4096, transa=0, transb=0, ws=32 << 20),                 # few tiles, long K: split through the workspace
+]
+
+
+@pytest.mark.parametrize("typ", ["bf16", "f16"])
+@pytest.mark.parametrize("shape", range(len(TR_SHAPES)))
+def test_other_layouts_run_on_the_transposing_kernel(gpu_api, typ, shape):
+    """A:N, B:T, A:T B:T, row-major D and K-contiguous operands whose pitches are not multiples of 16 bytes"""
+    extra = dict(TR_SHAPES[shape])
+    ws = extra.pop("ws", 0)
+    spec = base(typ, **extra)
+    print("case", spec, flush=True)
+    case = Case(spec, 7900 + shape)
+    ref = case.run_oracle()
+    st, got, kernel, variant = case.run_gpu(gpu_api, workspace_bytes=ws)
+    assert st == 0 and kernel == K.ZLUDA_KERNEL_MFMA_TR16, (st, kernel)
+    assert (case.last_workspace_needed > 0) == (ws > 0)
+    case.compare(got, ref, tol=1e-2)
+    for v in range(gpu_api.zluda_gemm_variant_count(K.ZLUDA_KERNEL_MFMA_TR16)):
+        st, got_v, kernel, variant = case.run_gpu(gpu_api, forced_kernel=K.ZLUDA_KERNEL_MFMA_TR16, forced_variant=v, workspace_bytes=ws)
+        assert st == 0 and (kernel, variant) == (K.ZLUDA_KERNEL_MFMA_TR16, v)
         case.compare(got_v, ref, tol=1e-2)
     if "order_d" in spec:
         return  # (the installed hipBLASLt writes only part of a row-major D with a bias vector)

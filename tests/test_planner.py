@@ -59,9 +59,20 @@ def test_16_bit_operands_take_the_mfma_family_when_k_contiguous(api):
         # K in bytes decides the split: 4096 elements of 16 bits are 8 KiB per row
         st, p = plan(api, dict(H, m=512, n=256, k=4096, transa=1), workspace=64 << 20)
         assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_H16 and p.grid_z > 1
-        # pitches that are not multiples of 16 bytes leave the DMA kernel
+        # pitches that are not multiples of 16 bytes leave the DMA kernel for the transposing one (4-byte alignment) ...
         st, p = plan(api, dict(H, m=512, n=256, k=4096, transa=1, lda=4100))
-        assert st == 0 and p.kernel != K.ZLUDA_KERNEL_MFMA_H16
+        assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_TR16
+        # ... which is also what runs operands with unit stride along M or N
+        for ta, tb in ((0, 0), (0, 1), (1, 1)):
+            st, p = plan(api, dict(H, m=4096, n=4096, k=4096, transa=ta, transb=tb))
+            assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_TR16 and p.variant == 0 and p.grid_x == 256
+        # odd pitches (2-byte alignment) are left to the generic kernel
+        st, p = plan(api, dict(H, m=512, n=256, k=4096, transa=0, lda=513))
+        assert st == 0 and p.kernel == K.ZLUDA_KERNEL_GENERIC
+        assert api.zluda_gemm_variant_count(K.ZLUDA_KERNEL_MFMA_TR16) == 3
+        assert plan(api, dict(H, m=4096, n=4096, k=4096), forced=K.ZLUDA_KERNEL_MFMA_TR16, variant=3)[0] == K.CUBLAS_STATUS_INVALID_VALUE
+        assert plan(api, dict(H, m=4096, n=4096, k=4096), forced=K.ZLUDA_KERNEL_MFMA_TR8)[0] == K.CUBLAS_STATUS_NOT_SUPPORTED
+        assert plan(api, dict(I8, m=4096, n=4096, k=4096), forced=K.ZLUDA_KERNEL_MFMA_TR16)[0] == K.CUBLAS_STATUS_NOT_SUPPORTED
         # other operand types never reach it
         assert plan(api, dict(I8, m=512, n=256, k=4096, transa=1), forced=K.ZLUDA_KERNEL_MFMA_H16)[0] == K.CUBLAS_STATUS_NOT_SUPPORTED
 

@@ -312,7 +312,7 @@ bool unpack_algo(const cublasLtMatmulAlgo_t *algo, uint32_t *kernel, int32_t *va
   if ((algo->data[0] >> 32) != ZLUDA_ALGO_MAGIC) return false;
   *kernel = (uint32_t)(algo->data[0] & 0xffffffffu);
   *variant = (int32_t)algo->data[1];
-  return *kernel >= ZLUDA_KERNEL_GENERIC && *kernel <= ZLUDA_KERNEL_MFMA_H16;
+  return *kernel >= ZLUDA_KERNEL_GENERIC && *kernel <= ZLUDA_KERNEL_MFMA_TR16;
 }
 
 // A/B forcing for measurements: ZLUDA_FORCE_KERNEL=<family>[:<variant>], read once per process (the
@@ -674,6 +674,8 @@ static int families_for_types(uint32_t computeType, uint32_t scaleType, uint32_t
   p.op.transa = CUBLAS_OP_N;
   if (zluda_gemm_plan_problem(&p, ZLUDA_KERNEL_MFMA_TR8, -1, 256, &plan) == CUBLAS_STATUS_SUCCESS)
     ids[count++] = ZLUDA_KERNEL_MFMA_TR8;
+  if (zluda_gemm_plan_problem(&p, ZLUDA_KERNEL_MFMA_TR16, -1, 256, &plan) == CUBLAS_STATUS_SUCCESS)
+    ids[count++] = ZLUDA_KERNEL_MFMA_TR16;
   return count;
 }
 
@@ -739,7 +741,7 @@ cublasStatus_t cublasLtMatmulAlgoCapGetAttribute(const cublasLtMatmulAlgo_t *alg
   case 14 /* LD_NEGATIVE */: i32 = 0; return access(false, i32, nullptr, buf, sizeInBytes, sizeWritten);
   case 15 /* NUMERICAL_IMPL_FLAGS */: u64 = ~0ull; return access(false, u64, nullptr, buf, sizeInBytes, sizeWritten);
   case 16: case 17: /* MIN_ALIGNMENT_A/B_BYTES */
-    u32 = kernel == ZLUDA_KERNEL_GENERIC ? 1 : (kernel == ZLUDA_KERNEL_MFMA_TR8 ? 4 : 16);
+    u32 = kernel == ZLUDA_KERNEL_GENERIC ? 1 : (kernel == ZLUDA_KERNEL_MFMA_TR8 || kernel == ZLUDA_KERNEL_MFMA_TR16 ? 4 : 16);
     return access(false, u32, nullptr, buf, sizeInBytes, sizeWritten);
   case 18: case 19: /* MIN_ALIGNMENT_C/D_BYTES */ u32 = 1; return access(false, u32, nullptr, buf, sizeInBytes, sizeWritten);
   case 21 /* POINTER_ARRAY_BATCH_SUPPORT */: case 22 /* FLOATING_POINT_EMULATION_SUPPORT */:

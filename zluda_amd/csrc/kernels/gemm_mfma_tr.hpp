@@ -1,9 +1,9 @@
-// MFMA GEMM for 8-bit operands (int8, OCP fp8) of which at least one is NOT K-contiguous: a
-// column-major A without transpose (unit stride along M), a B with transpose (unit stride along N),
-// and their row-major counterparts.  v_mfma_i32_32x32x32_i8 / v_mfma_f32_32x32x64_f8f6f4 want 16 / 32
-// consecutive K bytes of one matrix row per lane, so such an operand is transposed on its way into
-// LDS; from there on the kernel is the K-contiguous one (same fragment layout, same epilogues:
-// gemm_mfma.hpp).
+// MFMA GEMM for 8-bit operands (int8, OCP fp8) and 16-bit operands (f16, bf16) of which at least one is
+// NOT K-contiguous: a column-major A without transpose (unit stride along M), a B with transpose (unit
+// stride along N), and their row-major counterparts.  v_mfma_i32_32x32x32_i8 / v_mfma_f32_32x32x16_f16 /
+// _bf16 / v_mfma_f32_32x32x64_f8f6f4 want 16 / 16 / 32 consecutive K bytes of one matrix row per lane, so
+// such an operand is transposed on its way into LDS; from there on the kernel is the K-contiguous one
+// (same fragment layout, same epilogues: gemm_mfma.hpp).
 //
 //   * WP x WQ waves (2 x 2, or 2 x 4 for the 256 x 256 tile), workgroup tile BP x BQ, 64 K bytes per
 //     stage, two LDS stages, one barrier per stage.  Every thread serves both operands, in groups of
@@ -18,6 +18,8 @@
 //     indices (IW = rows/16 bytes: dword, dwordx2, dwordx4), lanes of a wave run along the row index
 //     first so that an instruction reads whole 64..256-byte pieces of 4 K rows; 8 v_perm_b32 per 4 x 4 bytes
 //     turn the block into one dword of 4 consecutive K bytes per row, written with ds_write_b32.
+//     16-bit elements: 2 K rows x IW row indices per lane (2 IW bytes per K row: dwordx2, dwordx4 or two
+//     dwordx4), 2 v_perm_b32 per 2 x 2 elements, one dword of 2 consecutive K elements per row.
 //   * Operand with unit stride along K ("KC"): 16 bytes per lane, ds_write_b128.
 //   * LDS rows have a pitch of 80 bytes and are stored in permuted order, rho(i) = 16 r + ((g + s r) mod 16)
 //     for i = IW g + r, s = 16 / IW.  With that every ds_write_b32 instruction of the transposing path
@@ -55,28 +57,39 @@ __device__ __forceinline__ void transpose4x4(int x0, int x1, int x2, int x3, int
   out[3] = __builtin_amdgcn_perm(t23h, t01h, 0x07060302);
 }
 
+// 2 x 2 transpose of 16-bit elements: x[j] holds (row 0, row 1) of K index j; lo = K elements 0..1 of
+// row 0, hi = of row 1
+__device__ __forceinline__ void transpose2x2(int x0, int x1, int &lo, int &hi) {
+  lo = __builtin_amdgcn_perm(x1, x0, 0x05040100);  // x0.h0 x1.h0
+  hi = __builtin_amdgcn_perm(x1, x0, 0x07060302);  // x0.h1 x1.h1
+}
+
 // Global -> register -> LDS path of ROWS rows of a tile operand, served by 256 threads; KC: unit
-// stride along K.
-template <int ROWS, bool KC>
+// stride along K; ESZ: bytes per element.
+template <int ROWS, bool KC, int ESZ = 1>
 struct TrOperand {
-  static constexpr int IW = ROWS / 16;        // MC: row indices per lane (bytes per load)
-  static constexpr int NW = IW / 4;           // MC: dwords per load
+  static constexpr int IW = ROWS / 16;        // MC: row indices per lane
+  static constexpr int KR = 4 / ESZ;          // MC: K rows per lane (one dword of K per LDS row)
+  static constexpr int NW = IW * ESZ / 4;     // MC: dwords per K row and lane
   static constexpr int NCH = ROWS / 64;       // KC: 16-byte chunks per lane and stage
-  static constexpr int NREG = KC ? NCH * 4 : NW * 4;
+  static constexpr int NREG = KC ? NCH * 4 : NW * KR;
+  static constexpr int NLOADS = KC ? NCH : KR * (NW > 4 ? NW / 4 : 1);  // vector memory instructions per stage
+  static constexpr int NPERM = KC ? 0 : (ESZ == 1 ? NREG * 2 : NREG);   // v_perm_b32 per stage
+  static_assert(ESZ == 1 || ESZ == 2, "8- or 16-bit elements");
   static_assert(ROWS == 64 || ROWS == 128 || ROWS == 256, "64, 128 or 256 rows per group of 256 threads");
 
   __amdgpu_buffer_rsrc_t rs;
   int voff[KC ? NCH : 1];
   int kstep;     // byte offset of one stage
-  int kbytes;    // K
+  int kbytes;    // bytes of K per row
   int ld;        // MC: stride of one K row
   int tc;        // KC: byte offset of this lane's chunk in a stage
 
   // base: first byte of the operand (this batch); row0: first tile row; nrows: rows of the whole
-  // operand; ld_row / ld_k: byte strides (one of them is 1)
+  // operand; ld_row / ld_k: byte strides (one of them is ESZ); K: elements along K
   // t: index of the thread among the 256 that load this operand
   __device__ __forceinline__ void init(int t, const uint8_t *base, int row0, int nrows, int ld_row, int ld_k, int K) {
-    kbytes = K;
+    kbytes = K * ESZ;
     tc = (t & 3) * 16;
     if constexpr (KC) {
       rs = __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, 0x80000000, 0x00020000);
@@ -88,9 +101,9 @@ struct TrOperand {
       // the operand's extent, up to the end of its last dword (the range check is per dword; base
       // and ld_k are multiples of 4, so that dword lies in the same allocation granule): K rows past
       // the end read as zero
-      rs = __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, K > 0 ? (((K - 1) * ld_k + nrows + 3) & ~3) : 0, 0x00020000);
-      voff[0] = ((t >> 4) * 4) * ld_k + row0 + (t & 15) * IW;
-      kstep = 64 * ld_k;
+      rs = __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, K > 0 ? (((K - 1) * ld_k + nrows * ESZ + 3) & ~3) : 0, 0x00020000);
+      voff[0] = ((t >> 4) * KR) * ld_k + (row0 + (t & 15) * IW) * ESZ;
+      kstep = (64 / ESZ) * ld_k;
       ld = ld_k;
     }
   }
@@ -105,15 +118,18 @@ struct TrOperand {
       }
     } else {
 #pragma unroll
-      for (int j = 0; j < 4; j++) {
+      for (int j = 0; j < KR; j++) {
         if constexpr (NW == 1) {
           regs[j] = __builtin_amdgcn_raw_buffer_load_b32(rs, voff[0] + j * ld, kt * kstep, 0);
         } else if constexpr (NW == 2) {
           const v2i v = __builtin_bit_cast(v2i, __builtin_amdgcn_raw_buffer_load_b64(rs, voff[0] + j * ld, kt * kstep, 0));
           regs[j * 2] = v[0]; regs[j * 2 + 1] = v[1];
         } else {
-          const v4i v = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rs, voff[0] + j * ld, kt * kstep, 0));
-          regs[j * 4] = v[0]; regs[j * 4 + 1] = v[1]; regs[j * 4 + 2] = v[2]; regs[j * 4 + 3] = v[3];
+#pragma unroll
+          for (int h = 0; h < NW / 4; h++) {
+            const v4i v = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rs, voff[0] + j * ld + h * 16, kt * kstep, 0));
+            regs[j * NW + h * 4] = v[0]; regs[j * NW + h * 4 + 1] = v[1]; regs[j * NW + h * 4 + 2] = v[2]; regs[j * NW + h * 4 + 3] = v[3];
+          }
         }
       }
     }
@@ -130,10 +146,17 @@ struct TrOperand {
       const int g = t & 15, kb = t >> 4;
 #pragma unroll
       for (int c = 0; c < NW; c++) {
-        int out[4];
-        transpose4x4(regs[0 * NW + c], regs[1 * NW + c], regs[2 * NW + c], regs[3 * NW + c], out);
+        if constexpr (ESZ == 1) {
+          int out[4];
+          transpose4x4(regs[0 * NW + c], regs[1 * NW + c], regs[2 * NW + c], regs[3 * NW + c], out);
 #pragma unroll
-        for (int r = 0; r < 4; r++) d32[tr_rho<ROWS>(g, 4 * c + r) * 20 + kb] = out[r];
+          for (int r = 0; r < 4; r++) d32[tr_rho<ROWS>(g, 4 * c + r) * 20 + kb] = out[r];
+        } else {
+          int lo, hi;
+          transpose2x2(regs[c], regs[NW + c], lo, hi);
+          d32[tr_rho<ROWS>(g, 2 * c) * 20 + kb] = lo;
+          d32[tr_rho<ROWS>(g, 2 * c + 1) * 20 + kb] = hi;
+        }
       }
     }
   }
@@ -145,7 +168,9 @@ struct TrOperand {
 // chunk l/16), one MFMA per pair of fragments and stage.
 template <int KIND, int FQ, int FP, int BP, int BQ, int WP, int WQ, bool PKC, bool QKC, bool M16 = false>
 __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_tr_kernel(MfmaParams prm) {
-  static_assert(KIND == KIND_I8 || KIND == KIND_F8, "8-bit operands");
+  static_assert(KIND == KIND_I8 || KIND == KIND_F8 || kind_is_h16(KIND), "8- or 16-bit operands");
+  constexpr int ESZ = kind_is_h16(KIND) ? 2 : 1;
+  constexpr bool B16 = KIND != KIND_F8;  // 16 bytes of K per lane and MFMA (fp8: 32)
   static_assert(!M16 || KIND == KIND_I8, "the 16x16 form is instantiated for int8");
   constexpr int NT = WP * WQ * 64;
   static_assert(NT == 256 || NT == 512, "operand rows are dealt to groups of 256 threads");
@@ -154,7 +179,7 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_tr_kernel(MfmaParams pr
   constexpr int KS = KIND == KIND_F8 ? 1 : 2;  // MFMA sub-steps per 64-byte stage
   constexpr int STAGE_V4 = (BP + BQ) * 5;
   using acc_v = typename std::conditional<KIND == KIND_I8, v16i, v16f>::type;
-  using frag_v = typename std::conditional<KIND == KIND_I8, v4i, v8i>::type;
+  using frag_v = typename std::conditional<B16, v4i, v8i>::type;
 
   __shared__ v4i lds[2 * STAGE_V4];
 
@@ -175,29 +200,30 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_tr_kernel(MfmaParams pr
   const int p0 = tile_p * BP, q0 = tile_q * BQ;
   const int NP = prm.swapped ? g.N : g.M, NQ = prm.swapped ? g.M : g.N;
 
-  TrOperand<LP, PKC> P;
-  TrOperand<LQ, QKC> Q;
+  TrOperand<LP, PKC, ESZ> P;
+  TrOperand<LQ, QKC, ESZ> Q;
   const int tl = t & 255, grp = wave >> 2;
   const int lds_p = grp * LP * 5, lds_q = (BP + grp * LQ) * 5;  // this group's rows inside a stage
   // split-K (as in gemm_mfma_pipe_kernel): workgroup z of gridDim.z takes stages [z * split_stages, ...)
   // of K; the operands start k0 further along K and the rest of the kernel sees a shorter K
+  // (k0, Kl in elements; a stage is 64 bytes of K)
   int k0 = 0, Kl = g.K;
   if (prm.splits > 1) {
-    k0 = (int)blockIdx.z * prm.split_stages * 64;
-    Kl = max(0, min(g.K - k0, prm.split_stages * 64));
+    k0 = (int)blockIdx.z * prm.split_stages * (64 / ESZ);
+    Kl = max(0, min(g.K - k0, prm.split_stages * (64 / ESZ)));
   }
   {
-    const uint8_t *a = (const uint8_t *)g.A + g.a_sb * bt + (int64_t)k0 * g.a_sk;
-    const uint8_t *b = (const uint8_t *)g.B + g.b_sb * bt + (int64_t)k0 * g.b_sk;
+    const uint8_t *a = (const uint8_t *)g.A + (g.a_sb * bt + (int64_t)k0 * g.a_sk) * ESZ;
+    const uint8_t *b = (const uint8_t *)g.B + (g.b_sb * bt + (int64_t)k0 * g.b_sk) * ESZ;
     if (!prm.swapped) {
-      P.init(tl, a, p0 + grp * LP, NP, (int)g.a_si, (int)g.a_sk, Kl);
-      Q.init(tl, b, q0 + grp * LQ, NQ, (int)g.b_sj, (int)g.b_sk, Kl);
+      P.init(tl, a, p0 + grp * LP, NP, (int)g.a_si * ESZ, (int)g.a_sk * ESZ, Kl);
+      Q.init(tl, b, q0 + grp * LQ, NQ, (int)g.b_sj * ESZ, (int)g.b_sk * ESZ, Kl);
     } else {
-      P.init(tl, b, p0 + grp * LP, NP, (int)g.b_sj, (int)g.b_sk, Kl);
-      Q.init(tl, a, q0 + grp * LQ, NQ, (int)g.a_si, (int)g.a_sk, Kl);
+      P.init(tl, b, p0 + grp * LP, NP, (int)g.b_sj * ESZ, (int)g.b_sk * ESZ, Kl);
+      Q.init(tl, a, q0 + grp * LQ, NQ, (int)g.a_si * ESZ, (int)g.a_sk * ESZ, Kl);
     }
   }
-  const int KT = (Kl + 63) / 64;
+  const int KT = (Kl * ESZ + 63) / 64;
   const int KL = max(KT - 1, 0);  // last stage that holds data
   // K % 64 != 0: in the last stage a load instruction of an operand without unit K stride covers K rows
   // 16 * wave + j + 4 * {0..3}; when even the first of them is past the end every lane of the instruction
@@ -206,7 +232,7 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_tr_kernel(MfmaParams pr
   // front of the LDS stores, which consume the older stage's registers) could pass too early.  From the
   // first trip whose younger stage is that last stage (stage kt + 2 >= KL) the stores are therefore preceded
   // by a wait for everything.  With K % 64 == 0 no such instruction exists and nothing is added.
-  const int tail_from = (Kl & 63) ? KL - 2 : 0x7fffffff;
+  const int tail_from = ((Kl * ESZ) & 63) ? KL - 2 : 0x7fffffff;
 
   // LDS rows (in v4i units) of this lane's fragment rows
   int prow[TP], qrow[TQ];
@@ -276,7 +302,7 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_tr_kernel(MfmaParams pr
   // fragments of sub-step ks of the stage in `buf`
   struct Frags { frag_v p[TP], q[TQ]; };
   auto read_frags = [&](const v4i *buf, int ks, Frags &f) {
-    if constexpr (KIND == KIND_I8) {
+    if constexpr (B16) {
       const int ch = ks * 2 + gsel;
 #pragma unroll
       for (int b = 0; b < TP; b++) f.p[b] = buf[prow[b] + ch];
@@ -303,6 +329,12 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_tr_kernel(MfmaParams pr
       for (int b = 0; b < TP; b++) {
         if constexpr (KIND == KIND_I8)
           acc[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.q[a], f.p[b], acc[a][b], 0, 0, 0);
+        else if constexpr (KIND == KIND_F16)
+          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, f.q[a]), __builtin_bit_cast(v8h, f.p[b]),
+                                                             acc[a][b], 0, 0, 0);
+        else if constexpr (KIND == KIND_BF16)
+          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8b, f.q[a]), __builtin_bit_cast(v8b, f.p[b]),
+                                                              acc[a][b], 0, 0, 0);
         else
           acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.q[a], f.p[b], acc[a][b], FQ, FP, 0, 0, 0, 0);
       }
@@ -331,7 +363,7 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_tr_kernel(MfmaParams pr
       // write needs the eight permutes of its 4 x 4 block), the LDS writes come behind the later MFMAs
       constexpr int NM = TP * TQ, H = NM / 2 > 0 ? NM / 2 : 1;
       constexpr int NDR = KS == 2 ? (TP + TQ) : 0;
-      constexpr int NPERM = ((PKC ? 0 : P.NREG * 2) + (QKC ? 0 : Q.NREG * 2));
+      constexpr int NPERM = P.NPERM + Q.NPERM;
       constexpr int NDW = (PKC ? P.NCH : P.NREG) + (QKC ? Q.NCH : Q.NREG);
       static_for<NM>([&](auto i_c) {
         constexpr int i = decltype(i_c)::value;
@@ -360,7 +392,7 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_tr_kernel(MfmaParams pr
     if constexpr (KS == 2) {
       mfma_all(f1);
       constexpr int NM = TP * TQ, NDR = TP + TQ;
-      constexpr int NVM = (PKC ? P.NCH : 4) + (QKC ? Q.NCH : 4);
+      constexpr int NVM = P.NLOADS + Q.NLOADS;
       static_for<NM>([&](auto i_c) {
         constexpr int i = decltype(i_c)::value;
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
@@ -392,7 +424,7 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_tr_kernel(MfmaParams pr
     {
       constexpr int NM = HP16 * TQ16, H = NM / 2 > 0 ? NM / 2 : 1;
       constexpr int NDR = HP16;
-      constexpr int NPERM = ((PKC ? 0 : P.NREG * 2) + (QKC ? 0 : Q.NREG * 2));
+      constexpr int NPERM = P.NPERM + Q.NPERM;
       constexpr int NDW = (PKC ? P.NCH : P.NREG) + (QKC ? Q.NCH : Q.NREG);
       static_for<NM>([&](auto i_c) {
         constexpr int i = decltype(i_c)::value;
@@ -418,7 +450,7 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_tr_kernel(MfmaParams pr
     mfma16(H1{}, SC{});
     {
       constexpr int NM = HP16 * TQ16, NDR = HP16 + TQ16;
-      constexpr int NVM = (PKC ? P.NCH : 4) + (QKC ? Q.NCH : 4);
+      constexpr int NVM = P.NLOADS + Q.NLOADS;
       static_for<NM>([&](auto i_c) {
         constexpr int i = decltype(i_c)::value;
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);

@@ -1,4 +1,4 @@
-// Launchers of the transposing 8-bit MFMA kernel (kernels/gemm_mfma_tr.hpp); one translation unit per
+// Launchers of the transposing MFMA kernel (kernels/gemm_mfma_tr.hpp); one translation unit per
 // element kind so that the template instantiations compile in parallel.
 #pragma once
 #include <hip/hip_runtime.h>
@@ -50,5 +50,7 @@ uint32_t launch_tr_i8(const MfmaParams &prm, const zluda_gemm_plan &plan, bool p
 uint32_t launch_tr_f8(const MfmaParams &prm, const zluda_gemm_plan &plan, int fq, int fp, bool pkc, bool qkc, hipStream_t s);
 uint32_t launch_tr_f8_e5m2q(const MfmaParams &prm, const zluda_gemm_plan &plan, bool pkc, bool qkc, hipStream_t s);
 uint32_t launch_tr_f8_e5m2p(const MfmaParams &prm, const zluda_gemm_plan &plan, bool pkc, bool qkc, hipStream_t s);
+uint32_t launch_tr_f16(const MfmaParams &prm, const zluda_gemm_plan &plan, bool pkc, bool qkc, hipStream_t s);
+uint32_t launch_tr_bf16(const MfmaParams &prm, const zluda_gemm_plan &plan, bool pkc, bool qkc, hipStream_t s);
 
 } // namespace zluda_amd

@@ -295,18 +295,24 @@ bool family_supports(uint32_t kernel, const Lowered &l) {
     // f16 x f16 or bf16 x bf16 (lower_problem admits 16-bit operands of one type only)
     return fast_layout && l.span_ok && (g.a_type == CUDA_R_16F || g.a_type == CUDA_R_16BF) && g.b_type == g.a_type &&
            g.a_scale_mode != SCALE_BLOCK32_UE8M0 && g.b_scale_mode != SCALE_BLOCK32_UE8M0 && d_fast;
-  case ZLUDA_KERNEL_MFMA_TR8: {
-    // 8-bit operands, each with unit stride along K or along its row index; dword-aligned loads
-    const bool types = (g.a_type == CUDA_R_8I && g.b_type == CUDA_R_8I) ||
-                       (is_f8(g.a_type) && is_f8(g.b_type) && !(g.a_type == CUDA_R_8F_E5M2 && g.b_type == CUDA_R_8F_E5M2));
+  case ZLUDA_KERNEL_MFMA_TR8: case ZLUDA_KERNEL_MFMA_TR16: {
+    // 8-bit (TR8) or 16-bit (TR16) operands, each with unit stride along K or along its row index; dword-aligned loads
+    const bool h16 = g.a_type == CUDA_R_16F || g.a_type == CUDA_R_16BF;
+    const bool types = kernel == ZLUDA_KERNEL_MFMA_TR16
+                           ? (h16 && g.b_type == g.a_type)
+                           : ((g.a_type == CUDA_R_8I && g.b_type == CUDA_R_8I) ||
+                              (is_f8(g.a_type) && is_f8(g.b_type) && !(g.a_type == CUDA_R_8F_E5M2 && g.b_type == CUDA_R_8F_E5M2)));
+    const int64_t esz = h16 ? 2 : 1;
+    // (strides in bytes from here on)
     auto operand_ok = [&](const void *ptr, int64_t s_row, int64_t s_k, int64_t s_b, int rows) {
+      s_row *= esz; s_k *= esz; s_b *= esz;
       if ((((uintptr_t)ptr) & 3) || (g.batch > 1 && (s_b & 3))) return false;
-      const int64_t span = (int64_t)(rows - 1) * s_row + (int64_t)(g.K - 1) * s_k + 1;
+      const int64_t span = (int64_t)(rows - 1) * s_row + (int64_t)(g.K - 1) * s_k + esz;
       if (span >= 0x7fffffffll) return false;
-      if (s_k == 1) return (s_row & 3) == 0 && (g.K & 15) == 0;  // 16-byte pieces along K
+      if (s_k == esz) return (s_row & 3) == 0 && ((g.K * esz) & 15) == 0;  // 16-byte pieces along K
       // (offsets of K rows up to three stages past the end must stay below 2^32, where they are out
       // of range instead of wrapping into it)
-      return s_row == 1 && (s_k & 3) == 0 && (int64_t)(g.K + 256) * s_k < 0xffffffffll;
+      return s_row == esz && (s_k & 3) == 0 && (int64_t)(g.K + 256) * s_k < 0xffffffffll;
     };
     return types && d_fast && g.a_scale_mode != SCALE_BLOCK32_UE8M0 && g.b_scale_mode != SCALE_BLOCK32_UE8M0 &&
            operand_ok(g.A, g.a_si, g.a_sk, g.a_sb, g.M) && operand_ok(g.B, g.b_sj, g.b_sk, g.b_sb, g.N);
@@ -423,8 +429,9 @@ static void fill_tr_plan(const Lowered &l, int variant, uint32_t cus, uint64_t w
   const uint64_t tiles = (uint64_t)plan->grid_x * plan->grid_y;
   const uint64_t slots = (uint64_t)cus * std::min(per_cu, 4u);
   const bool skinny = std::min(g.M, g.N) <= 64;
-  if (tiles * 2 <= (skinny ? slots : (uint64_t)cus) && g.K >= 1024 && (uint64_t)ceil_div(np, v.bp) * v.bp <= (1u << 20)) {
-    uint32_t s = (uint32_t)std::min<uint64_t>({8, slots / tiles, (uint64_t)g.K / 512});
+  const uint64_t kbytes = (uint64_t)g.K * ((g.a_type == CUDA_R_16F || g.a_type == CUDA_R_16BF) ? 2 : 1);
+  if (tiles * 2 <= (skinny ? slots : (uint64_t)cus) && kbytes >= 1024 && (uint64_t)ceil_div(np, v.bp) * v.bp <= (1u << 20)) {
+    uint32_t s = (uint32_t)std::min<uint64_t>({8, slots / tiles, kbytes / 512});
     const uint64_t per_split = (uint64_t)g.batch * ceil_div(np, v.bp) * v.bp * ceil_div(nq, v.bq) * v.bq * 4;
     while (s > 1 && s * per_split > workspace_size) s--;
     if (s > 1) {
@@ -525,6 +532,7 @@ extern "C" uint32_t zluda_gemm_variant_count(uint32_t kernel) {
   case ZLUDA_KERNEL_MFMA_MXF4: case ZLUDA_KERNEL_MFMA_H16: return kNumMfmaVariants32;  // the 16x16-shape ones serve int8 and fp8
   case ZLUDA_KERNEL_DECODE_W8A8: return kNumDecodeVariants;
   case ZLUDA_KERNEL_MFMA_TR8: return kNumTrVariants;
+  case ZLUDA_KERNEL_MFMA_TR16: return kNumTrVariants - 1;  // the 16x16-shape one is an int8 instantiation
   default: return 0;
   }
 }
@@ -543,7 +551,7 @@ extern "C" uint32_t zluda_gemm_plan_problem(const zluda_gemm_problem *p, uint32_
   if (kernel == ZLUDA_KERNEL_AUTO) {
     static const uint32_t order[] = {ZLUDA_KERNEL_DECODE_W8A8, ZLUDA_KERNEL_MFMA_I8, ZLUDA_KERNEL_MFMA_F8,
                                      ZLUDA_KERNEL_MFMA_MXF4, ZLUDA_KERNEL_MFMA_H16, ZLUDA_KERNEL_MFMA_TR8,
-                                     ZLUDA_KERNEL_GENERIC};
+                                     ZLUDA_KERNEL_MFMA_TR16, ZLUDA_KERNEL_GENERIC};
     for (uint32_t k : order) {
       if (!family_supports(k, l)) continue;
       if (k == ZLUDA_KERNEL_DECODE_W8A8) {
@@ -584,7 +592,7 @@ extern "C" uint32_t zluda_gemm_plan_problem(const zluda_gemm_problem *p, uint32_
     fill_mfma_plan(l, v, cu_count, p->workspace_size, plan);
     break;
   }
-  case ZLUDA_KERNEL_MFMA_TR8: {
+  case ZLUDA_KERNEL_MFMA_TR8: case ZLUDA_KERNEL_MFMA_TR16: {
     int v = forced_variant >= 0 ? forced_variant : pick_tr_variant(l, cu_count);
     if (v >= kNumTrVariants || (kTrVariants[v].m16 && l.g.a_type != CUDA_R_8I)) return CUBLAS_STATUS_INVALID_VALUE;
     fill_tr_plan(l, v, cu_count, p->workspace_size, plan);
