@@ -35,7 +35,7 @@ from zluda_amd import abi, cublaslt  # noqa: E402
 from zluda_amd.cublaslt import MatmulCall  # noqa: E402
 
 K = abi
-PEAK = {"i8": 5000.0, "f8": 5000.0, "f4": 10100.0, "hbm": 8000.0}  # TOP/s, TFLOP/s, GB/s (MI355X datasheet)
+PEAK = {"i8": 5000.0, "f8": 5000.0, "f4": 10100.0, "bf16": 2500.0, "hbm": 8000.0}  # TOP/s, TFLOP/s, GB/s (MI355X datasheet)
 PEAK_CLOCK_MHZ = 2400.0   # the shader clock the datasheet's matrix peaks are quoted at
 
 I8 = dict(a_type=K.CUDA_R_8I, b_type=K.CUDA_R_8I, d_type=K.CUDA_R_32I, compute_type=K.CUBLAS_COMPUTE_32I,
@@ -76,6 +76,13 @@ WORKLOADS = {
                             compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F, transa=1, m=8192, n=8192, k=8192,
                             a_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_VEC32_UE8M0,
                             b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_VEC32_UE8M0)),
+    # not a benchmark configuration: the 16-bit operand type applications call cublasLtMatmul with most, on the same kernels
+    "bf16_8192": dict(name="bf16xbf16->bf16 M=N=K=8192 A:T B:N", kind="bf16", steps=25,
+                      spec=dict(a_type=K.CUDA_R_16BF, b_type=K.CUDA_R_16BF, d_type=K.CUDA_R_16BF,
+                                compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F, transa=1, m=8192, n=8192, k=8192)),
+    "bf16_8192_nn": dict(name="bf16xbf16->bf16 M=N=K=8192 A:N B:N (operand A transposed on its way into LDS)", kind="bf16", steps=25,
+                         spec=dict(a_type=K.CUDA_R_16BF, b_type=K.CUDA_R_16BF, d_type=K.CUDA_R_16BF,
+                                   compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F, transa=0, m=8192, n=8192, k=8192)),
 }
 for _w in WORKLOADS.values():   # five equal batches
     _w["steps"] = max(5, _w["steps"] // 5 * 5)
@@ -88,7 +95,7 @@ for _w in WORKLOADS.values():   # five equal batches
 PROFILE_OF = {"c1": "gemm_mfma_tr_i8_c1_256", "c2": "gemm_mfma_pipe16_i8_c2_4096", "i8_4096_nt": "gemm_mfma_tr_i8_4096_nt",
               "i8_8192": "gemm_mfma_pipe16_i8_8192", "c3": "decode_slab_c3", "c4": "gemm_mfma_pipe16_f8_c4_8192",
               "c5": "gemm_mfma_pipe_mxf4_c5_8192x4", "c5_b1": "gemm_mfma_pipe_mxf4_c5_8192_b1",
-              "decode_k13824": "decode_slab_k13824"}
+              "decode_k13824": "decode_slab_k13824", "bf16_8192": "gemm_mfma_pipe_bf16_8192", "bf16_8192_nn": "gemm_mfma_tr_bf16_8192_nn"}
 
 
 def measured_traffic(key):
@@ -142,6 +149,10 @@ class Buffers:
                 mk = lambda r: torch.randint(-128, 128, (r, k), device=dev, generator=g, dtype=torch.int8)
             self.A = [mk(m) for _ in range(copies)]
             self.B = mk(n)
+        elif at == K.CUDA_R_16BF:   # N(0,1); an operand that is not transposed is stored [K][rows]
+            mk = lambda r, t: torch.randn((r, k) if t else (k, r), device=dev, generator=g).to(torch.bfloat16)
+            self.A = [mk(m, spec.get("transa", 0))]
+            self.B = mk(n, not spec.get("transb", 0))
         elif at == K.CUDA_R_8F_E4M3:
             def mk(r):
                 x = torch.randn(r, k, device=dev, generator=g)
@@ -412,7 +423,8 @@ def cpu_baseline(key, budget_s=12.0):
     from oracle.cases import Case
     spec = dict(WORKLOADS[key]["spec"])
     full_m = spec["m"]
-    rows = {"c1": full_m, "c2": full_m, "i8_4096_nt": full_m, "i8_8192": 2048, "c3": full_m, "decode_k13824": full_m, "c4": 256, "c5": 64, "c5_b1": 64}[key]
+    rows = {"c1": full_m, "c2": full_m, "i8_4096_nt": full_m, "i8_8192": 2048, "c3": full_m, "decode_k13824": full_m, "c4": 256, "c5": 64, "c5_b1": 64,
+            "bf16_8192": 256, "bf16_8192_nn": 256}[key]
     spec.update(m=rows, batch=1, alpha=1)
     decode = WORKLOADS[key]["kind"] == "hbm"
     case = Case(spec, 1, int_dist="normal" if decode else "uniform")
@@ -469,7 +481,7 @@ def main():
     head = run_workload(torch, api, key, steps, args.warmup, not args.no_hipblaslt)
     also = {}
     if not args.only:
-        for other in ("c4", "i8_8192", "c3", "c5", "c5_b1", "c2", "c1", "i8_4096_nt", "decode_k13824"):
+        for other in ("c4", "i8_8192", "c3", "c5", "c5_b1", "c2", "c1", "i8_4096_nt", "decode_k13824", "bf16_8192", "bf16_8192_nn"):
             if other == key:
                 continue
             try:
@@ -482,7 +494,7 @@ def main():
         "metric": "cublasLtMatmul TOPS (int8/fp8/MXFP4, 8192^3) + decode GEMM HBM GB/s",
         "value": head["gbps"] if unit == "GB/s" else head["tops"], "unit": unit, "n_gpus": 1, "steps": steps,
         "warmup": head["warmup"], "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": {"i8": "int8", "hbm": "int8", "f8": "fp8_e4m3", "f4": "fp4_e2m1"}[WORKLOADS[key]["kind"]],
+        "vs_baseline": None, "dtype": {"i8": "int8", "hbm": "int8", "f8": "fp8_e4m3", "f4": "fp4_e2m1", "bf16": "bf16"}[WORKLOADS[key]["kind"]],
         "data": "synthetic", "config": {"workload": head["workload"], "kernel": head["kernel"]},
         "roofline": head["roofline"],
         "clock_mhz_observed": head["roofline"].get("clock_mhz_observed"),

@@ -669,7 +669,7 @@ static int families_for_types(uint32_t computeType, uint32_t scaleType, uint32_t
   p.b.cols = p.c.cols = p.d.cols = 16;
   if (zluda_gemm_plan_problem(&p, ZLUDA_KERNEL_DECODE_W8A8, -1, 256, &plan) == CUBLAS_STATUS_SUCCESS)
     ids[count++] = ZLUDA_KERNEL_DECODE_W8A8;
-  // the transposing 8-bit kernel is what runs the layouts with A or B not K-contiguous
+  // the transposing kernels are what runs the layouts with A or B not K-contiguous
   p.b.cols = p.c.cols = p.d.cols = n;
   p.op.transa = CUBLAS_OP_N;
   if (zluda_gemm_plan_problem(&p, ZLUDA_KERNEL_MFMA_TR8, -1, 256, &plan) == CUBLAS_STATUS_SUCCESS)
