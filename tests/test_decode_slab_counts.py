@@ -11,15 +11,16 @@ import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 KERNELS = os.path.join(ROOT, "zluda_amd", "csrc", "kernels")
+KINDS = ("KIND_I8", "KIND_F8", "KIND_F16", "KIND_BF16")
 
 
 @pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")
 def test_every_packed_instantiation_issues_exactly_the_counted_factor_loads(tmp_path):
     header = open(os.path.join(KERNELS, "decode_slab.hpp")).read()
     counted = int(re.search(r"constexpr int kSlabFactorLoads = (\d+);", header).group(1))
-    insts = ["%d, %s, %s" % (fast, kind, tail) for fast in (1, 2) for kind in ("KIND_I8", "KIND_F8") for tail in ("false", "true")]
-    insts += ["%d, %s, true, 8, 512, %d" % (fast, kind, q) for fast in (1, 2) for kind in ("KIND_I8", "KIND_F8") for q in (2, 3, 4)]
-    insts += ["%d, %s, true, 8, 512, %d, 2" % (fast, kind, q) for fast in (1, 2) for kind in ("KIND_I8", "KIND_F8") for q in (1, 2)]
+    insts = ["%d, %s, %s" % (fast, kind, tail) for fast in (1, 2) for kind in KINDS for tail in ("false", "true")]
+    insts += ["%d, %s, true, 8, 512, %d" % (fast, kind, q) for fast in (1, 2) for kind in KINDS for q in (2, 3, 4)]
+    insts += ["%d, %s, true, 8, 512, %d, 2" % (fast, kind, q) for fast in (1, 2) for kind in KINDS for q in (1, 2)]
     src = tmp_path / "slab_counts.hip"
     src.write_text('#include <hip/hip_runtime.h>\n#include "decode_slab.hpp"\nusing namespace zluda_amd;\n' + "".join(
         "template __global__ void zluda_amd::decode_slab_kernel<%s>(DecodeParams);\n" % i for i in insts))

@@ -89,6 +89,38 @@ def test_other_layouts_run_on_the_transposing_kernel(gpu_api, typ, shape):
     case.compare(got, theirs, tol=1e-2, floor_frac=1e-2)
 
 
+DECODE_SHAPES = [
+    (dict(m=1024, n=16, k=2048), 16),
+    (dict(m=1000, n=5, k=1536, lda=1600), 16),                                    # a K tail, ragged rows, padded pitch
+    (dict(m=2048, n=16, k=4096, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS), 17),
+    (dict(m=332, n=29, k=2048), 20),                                              # two token blocks
+    (dict(m=512, n=32, k=4096), 17),
+    (dict(m=1028, n=7, k=6144, epilogue=K.CUBLASLT_EPILOGUE_RELU_BIAS), 18),
+    (dict(m=640, n=12, k=7000, d_type=K.CUDA_R_32F, c_type=K.CUDA_R_32F), 19),    # element-wise epilogue
+    (dict(m=16, n=2048, k=4096), 17),                                             # tokens along M: the weights are B
+    (dict(m=900, n=16, k=4096, with_c=True), 17),
+    (dict(m=768, n=16, k=1280, batch=2), 16),
+]
+
+
+@pytest.mark.parametrize("typ", ["bf16", "f16"])
+@pytest.mark.parametrize("shape", range(len(DECODE_SHAPES)))
+def test_16_bit_weights_stream_through_the_slab_decode(gpu_api, typ, shape):
+    """few tokens, K-contiguous 16-bit weights of up to 16 KiB per row: the slab decode kernel with K counted in bytes"""
+    extra, variant = DECODE_SHAPES[shape]
+    spec = base(typ, **extra)
+    print("case", spec, flush=True)
+    case = Case(spec, 8000 + shape)
+    ref = case.run_oracle()
+    st, got, kernel, v = case.run_gpu(gpu_api)
+    assert st == 0 and (kernel, v) == (K.ZLUDA_KERNEL_DECODE_W8A8, variant), (st, kernel, v)
+    case.compare(got, ref, tol=1e-2)
+    theirs, why = case.run_hipblaslt()
+    if theirs is None:
+        pytest.skip("hipBLASLt offers no algorithm here: " + why)
+    case.compare(got, theirs, tol=1e-2, floor_frac=1e-2)
+
+
 @pytest.mark.parametrize("typ", ["bf16", "f16"])
 def test_16_bit_split_k_through_the_workspace(gpu_api, typ):
     spec = base(typ, m=512, n=256, k=8192, epilogue=K.CUBLASLT_EPILOGUE_BIAS)

@@ -77,6 +77,28 @@ def test_16_bit_operands_take_the_mfma_family_when_k_contiguous(api):
         assert plan(api, dict(I8, m=512, n=256, k=4096, transa=1), forced=K.ZLUDA_KERNEL_MFMA_H16)[0] == K.CUBLAS_STATUS_NOT_SUPPORTED
 
 
+def test_16_bit_weights_with_few_tokens_take_the_slab_decode(api):
+    """the slab form counts K in bytes: 2048 elements of 16 bits are the 4096 bytes of its first shape"""
+    for t in (K.CUDA_R_16BF, K.CUDA_R_16F):
+        H = dict(a_type=t, b_type=t, d_type=t, compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F, transa=1)
+        for k, variant in ((2048, 16), (1536, 16), (4096, 17), (6144, 18), (8192, 19)):
+            st, p = plan(api, dict(H, m=14336, n=16, k=k))
+            assert st == 0 and (p.kernel, p.variant) == (K.ZLUDA_KERNEL_DECODE_W8A8, variant), (k, p.kernel, p.variant)
+        st, p = plan(api, dict(H, m=4096, n=29, k=2048))
+        assert st == 0 and (p.kernel, p.variant) == (K.ZLUDA_KERNEL_DECODE_W8A8, 20)       # two token blocks
+        # K beyond 16 KiB per row, too many tokens, or no unit K stride: the MFMA tile kernels
+        assert plan(api, dict(H, m=4096, n=16, k=14336))[1].kernel == K.ZLUDA_KERNEL_MFMA_H16
+        assert plan(api, dict(H, m=14336, n=48, k=4096))[1].kernel == K.ZLUDA_KERNEL_MFMA_H16
+        assert plan(api, dict(H, m=14336, n=16, k=4096, transa=0))[1].kernel == K.ZLUDA_KERNEL_MFMA_TR16
+        # more than 64 rows per CU: tiles, unless K is long
+        assert plan(api, dict(H, m=28672, n=16, k=4096))[1].kernel == K.ZLUDA_KERNEL_MFMA_H16
+        st, p = plan(api, dict(H, m=28672, n=16, k=8192))
+        assert st == 0 and (p.kernel, p.variant, p.grid_x) == (K.ZLUDA_KERNEL_DECODE_W8A8, 19, 448)
+        # the other decode forms are 8-bit instantiations
+        for v in (0, 4, 5):
+            assert plan(api, dict(H, m=14336, n=16, k=2048), forced=K.ZLUDA_KERNEL_DECODE_W8A8, variant=v)[0] == K.CUBLAS_STATUS_NOT_SUPPORTED
+
+
 def test_small_problems_get_smaller_tiles(api):
     st, p = plan(api, dict(I8, m=1024, n=1024, k=1024, transa=1))
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_I8 and p.variant == 6 and p.grid_x == 256

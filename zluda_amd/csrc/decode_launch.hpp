@@ -84,7 +84,7 @@ inline uint32_t launch_decode_slab(const DecodeParams &prm, const zluda_gemm_pla
   dim3 grid(plan.grid_x, plan.grid_y, 1), block(v.nw * 64);
   // 0: element-wise epilogue, 1: packed store, 2: packed store behind a GELU
   const int fast = !decode_packed_output(prm.g, prm.swapped != 0) ? 0 : prm.g.act == ACT_GELU ? 2 : 1;
-  const bool tail = prm.g.K < v.nw * v.steps * 64;
+  const bool tail = prm.g.K * (kind_is_h16(KIND) ? 2 : 1) < v.nw * v.steps * 64;  // K bytes against the cover
   uint32_t st = CUBLAS_STATUS_NOT_SUPPORTED;
   static_for_host<3>([&](auto fast_c) {
     constexpr int FAST = decltype(fast_c)::value;
@@ -106,6 +106,7 @@ inline uint32_t launch_decode_slab(const DecodeParams &prm, const zluda_gemm_pla
 }
 
 uint32_t launch_decode_slab_i8(const DecodeParams &prm, const zluda_gemm_plan &plan, int nb, hipStream_t s);
+uint32_t launch_decode_slab_h16(const DecodeParams &prm, const zluda_gemm_plan &plan, int nb, bool bf16, hipStream_t s);
 uint32_t launch_decode_slab_f8(const DecodeParams &prm, const zluda_gemm_plan &plan, int nb, hipStream_t s);
 uint32_t launch_decode_stream_i8(const DecodeParams &prm, const zluda_gemm_plan &plan, int nb, hipStream_t s);
 uint32_t launch_decode_stream_f8(const DecodeParams &prm, const zluda_gemm_plan &plan, int nb, hipStream_t s);

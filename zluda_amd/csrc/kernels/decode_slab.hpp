@@ -3,6 +3,9 @@
 //
 //   W : R rows x K int8 (or fp8 e4m3), K-contiguous (read exactly once)     X : T <= 16 rows x K, same type
 //   out(r, t) = sum_k W[r][k] * X[t][k]     int32 (fp32), then the fused float / integer epilogue
+// The same kernel streams f16 / bf16 weights (KIND_F16 / KIND_BF16: v_mfma_f32_16x16x32_f16 / _bf16 take 16 bytes
+// of K per lane at the byte positions of the int8 instruction, so only the MFMA and the accumulator type
+// differ; every K below is then a count of BYTES, twice the element count).
 //
 // What differs from decode_stream_kernel, and what each point bought on a 14336 x 4096 int8 matrix with 16
 // tokens (MI355X, 58.7 MB, a flat read of the same bytes takes 9.95 us; decode_stream_kernel 14.8 us):
@@ -54,7 +57,9 @@ constexpr int kSlabMaxBlocks = 4;   // 16-row blocks a workgroup can run
 constexpr int kSlabFactorLoads = 21;  // vector memory loads of the packed epilogue's factors, per lane
 template <int FAST, int KIND, bool TAIL, int NW = 4, int UB = 1024, int Q = 1, int NB = 1>
 __global__ __launch_bounds__(NW * 64) void decode_slab_kernel(DecodeParams prm) {
-  static_assert(KIND == KIND_I8 || KIND == KIND_F8, "int8 or fp8 (e4m3 x e4m3) operands");
+  static_assert(KIND == KIND_I8 || KIND == KIND_F8 || kind_is_h16(KIND), "int8, fp8 (e4m3 x e4m3), f16 or bf16 operands");
+  constexpr int ESZ = kind_is_h16(KIND) ? 2 : 1;           // bytes per element
+  constexpr bool B16 = KIND != KIND_F8;                    // 16 bytes of K per lane and MFMA (fp8: 32)
   static_assert((UB == 1024 || UB == 512) && Q >= 1 && Q * NB <= 4 && (Q * NB == 1 || TAIL), "see above; the shapes beyond the first come with the K checks");
   using acc_t = typename std::conditional<KIND == KIND_I8, v4i, v4f>::type;
   constexpr int MAXB = kSlabMaxBlocks;
@@ -73,11 +78,11 @@ __global__ __launch_bounds__(NW * 64) void decode_slab_kernel(DecodeParams prm) 
   const int bt = blockIdx.y;
 
   const int R = prm.swapped ? g.N : g.M, T = prm.swapped ? g.M : g.N;
-  const uint8_t *Wg = (const uint8_t *)(prm.swapped ? g.B : g.A) + (prm.swapped ? g.b_sb : g.a_sb) * bt;
-  const uint8_t *Xg = (const uint8_t *)(prm.swapped ? g.A : g.B) + (prm.swapped ? g.a_sb : g.b_sb) * bt;
-  const int ldw = (int)(prm.swapped ? g.b_sj : g.a_si);
-  const int ldx = (int)(prm.swapped ? g.a_si : g.b_sj);
-  const int K = g.K;
+  const uint8_t *Wg = (const uint8_t *)(prm.swapped ? g.B : g.A) + (prm.swapped ? g.b_sb : g.a_sb) * bt * ESZ;
+  const uint8_t *Xg = (const uint8_t *)(prm.swapped ? g.A : g.B) + (prm.swapped ? g.a_sb : g.b_sb) * bt * ESZ;
+  const int ldw = (int)(prm.swapped ? g.b_sj : g.a_si) * ESZ;  // row pitches and K in bytes
+  const int ldx = (int)(prm.swapped ? g.a_si : g.b_sj) * ESZ;
+  const int K = g.K * ESZ;
 
   // Blocks of this workgroup: full_rounds round-robin blocks, then its share [rr0, rr1) (at most 16 rows, a
   // whole number of quads except at the very end of W) of the rows behind the last full round.  The split is
@@ -132,11 +137,11 @@ __global__ __launch_bounds__(NW * 64) void decode_slab_kernel(DecodeParams prm) 
       lds_dma16(rsX, dst + i * 64, unit_voff(i, q, RPI == 2 && half && tok + 1 < T ? ldx : 0), tok * ldx);
     }
   };
-  // fragment f of this lane in a unit: int8: K step f, 16 bytes at f*64 + g4*16; fp8: half (f & 1) of the 32
-  // bytes at (f/2)*128 + g4*32 of K step f/2
+  // fragment f of this lane in a unit: int8, f16, bf16: K step f, 16 bytes at f*64 + g4*16; fp8: half (f & 1) of
+  // the 32 bytes at (f/2)*128 + g4*32 of K step f/2
   const uint32_t ring_base = lds_addr(&ring[wave][0][l16 * CPR]);
   auto frag_addr = [&](int slot, int f) {
-    const int c = KIND == KIND_I8 ? 4 * f + g4 : 8 * (f >> 1) + 2 * g4 + (f & 1);
+    const int c = B16 ? 4 * f + g4 : 8 * (f >> 1) + 2 * g4 + (f & 1);
     return ring_base + slot * (UNIT_V4 * 16) + (((c & ~15) | ((c ^ l16) & 15)) << 4);
   };
   // unit n of this wave = (block n / Q, unit n % Q of the slab), in slot n % 2; the wave runs nblk * Q of them
@@ -264,6 +269,16 @@ __global__ __launch_bounds__(NW * 64) void decode_slab_kernel(DecodeParams prm) 
 #pragma unroll
             for (int f = 0; f < NFRAG; f++)
               acc[b][nbk] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[f], xf[nbk * Q + q][f], acc[b][nbk], 0, 0, 0);
+          } else if constexpr (KIND == KIND_F16) {
+#pragma unroll
+            for (int f = 0; f < NFRAG; f++)
+              acc[b][nbk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, w[f]), __builtin_bit_cast(v8h, xf[nbk * Q + q][f]),
+                                                                   acc[b][nbk], 0, 0, 0);
+          } else if constexpr (KIND == KIND_BF16) {
+#pragma unroll
+            for (int f = 0; f < NFRAG; f++)
+              acc[b][nbk] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8b, w[f]), __builtin_bit_cast(v8b, xf[nbk * Q + q][f]),
+                                                                    acc[b][nbk], 0, 0, 0);
           } else {
 #pragma unroll
             for (int f = 0; f < NFRAG; f += 2) {

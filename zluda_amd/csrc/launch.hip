@@ -156,14 +156,17 @@ uint32_t launch_decode(const Lowered &l, const zluda_gemm_plan &plan, hipStream_
   prm.nchunks = (prm.spw + v.steps - 1) / v.steps;
   const bool full = l.g.K == v.nw * v.steps * 64;
   const int nb = (T + 15) / 16;
+  const bool h16 = l.g.a_type == CUDA_R_16F || l.g.a_type == CUDA_R_16BF;
+  if (h16 && v.stream != 2) return CUBLAS_STATUS_NOT_SUPPORTED;  // 16-bit weights: the slab kernel only
   if (v.stream == 2) {
     // slab kernel: one block of tokens (two in the shapes of up to two units), nw slabs of K, W and X through 2 GiB buffer windows, at most
     // kSlabMaxBlocks blocks per workgroup: full_rounds round-robin blocks, then an even share (in quads of 4)
     // of the rows that are left
     const int64_t rows = plan.swapped ? l.g.N : l.g.M, ldw = plan.swapped ? l.g.b_sj : l.g.a_si;
     const int64_t ldx = plan.swapped ? l.g.a_si : l.g.b_sj;
-    if (nb > (v.nw == 8 && v.steps <= 16 ? 2 : 1) || l.g.K > v.nw * v.steps * 64 || (l.g.K & 15) || rows * ldw >= 0x7fffffffll ||
-        (int64_t)(T - 1) * ldx + l.g.K >= 0x7fffffffll || plan.grid_x == 0)
+    const int64_t esz = h16 ? 2 : 1, kb = l.g.K * esz;  // the kernel counts K and the pitches in bytes
+    if (nb > (v.nw == 8 && v.steps <= 16 ? 2 : 1) || kb > v.nw * v.steps * 64 || (kb & 15) || rows * ldw * esz >= 0x7fffffffll ||
+        ((int64_t)(T - 1) * ldx + l.g.K) * esz >= 0x7fffffffll || plan.grid_x == 0)
       return CUBLAS_STATUS_NOT_SUPPORTED;
     const int64_t G = plan.grid_x;
     prm.full_rounds = (int32_t)(rows / (16 * G));
@@ -171,7 +174,8 @@ uint32_t launch_decode(const Lowered &l, const zluda_gemm_plan &plan, hipStream_
     if (prm.full_rounds + (left > 0 ? 1 : 0) > kSlabMaxBlocks) return CUBLAS_STATUS_NOT_SUPPORTED;
     prm.rows_base = (int32_t)(quads / G);
     prm.rows_rem = (int32_t)(quads % G);
-    prm.spw = ((l.g.K + v.nw * 128 - 1) / (v.nw * 128)) * 2;  // a wave's slab: K / nw, rounded up to 128 bytes
+    prm.spw = (int32_t)((kb + v.nw * 128 - 1) / (v.nw * 128)) * 2;  // a wave's slab: K bytes / nw, rounded up to 128 bytes
+    if (h16) return launch_decode_slab_h16(prm, plan, nb, l.g.a_type == CUDA_R_16BF, s);
     return l.g.a_type == CUDA_R_8I ? launch_decode_slab_i8(prm, plan, nb, s) : launch_decode_slab_f8(prm, plan, nb, s);
   }
   if (v.stream) {

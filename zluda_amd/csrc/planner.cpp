@@ -248,6 +248,8 @@ static bool decode_variant_ok(const Lowered &l, int variant) {
   const GemmArgs &g = l.g;
   const DecodeVariant &v = kDecodeVariants[variant];
   const int T = std::min(g.M, g.N), nb = (T + 15) / 16;
+  const bool h16 = g.a_type == CUDA_R_16F || g.a_type == CUDA_R_16BF;
+  if (h16 && v.stream != 2) return false;  // 16-bit weights: the slab form only
   // the register-streaming kernel is int8 only; token blocks multiply its fragment registers
   if (!v.stream) return g.a_type == CUDA_R_8I && (nb == 1 || (nb == 2 && v.steps <= 8));
   const bool swapped = g.M < g.N;
@@ -258,8 +260,9 @@ static bool decode_variant_ok(const Lowered &l, int variant) {
     const int cover = v.nw * v.steps * 64, below = cover == 4096 ? cover / 2 : cover - 4096;
     // one block of tokens; two in the 8-wave shapes of one or two units (the one-unit shape exists for them alone)
     const bool tokens_ok = v.nw == 4 ? nb == 1 : v.steps == 8 ? nb == 2 : v.steps == 16 ? nb <= 2 : nb == 1;
-    return tokens_ok && g.K <= cover && g.K > below && (g.K & 15) == 0 && rows * ldw < 0x7fffffffll &&
-           (int64_t)(T - 1) * ldx + g.K < 0x7fffffffll;
+    const int64_t esz = h16 ? 2 : 1, kb = (int64_t)g.K * esz;  // covers are bytes of K
+    return tokens_ok && kb <= cover && kb > below && (kb & 15) == 0 && rows * ldw * esz < 0x7fffffffll &&
+           ((int64_t)(T - 1) * ldx + g.K) * esz < 0x7fffffffll;
   }
   // a stream instantiation covers nw * steps * 64 bytes of K and takes any K up to that (lanes past the end read
   // zero); more than a quarter of idle lanes is left to the smaller instantiations or to the MFMA tiles
@@ -318,8 +321,9 @@ bool family_supports(uint32_t kernel, const Lowered &l) {
            operand_ok(g.A, g.a_si, g.a_sk, g.a_sb, g.M) && operand_ok(g.B, g.b_sj, g.b_sk, g.b_sb, g.N);
   }
   case ZLUDA_KERNEL_DECODE_W8A8:
-    // int8, or e4m3 x e4m3 without block scales (the LDS-streaming variants only)
+    // int8, or e4m3 x e4m3 without block scales (the LDS-streaming variants only), or f16 / bf16 (the slab form only)
     return fast_layout && ((g.a_type == CUDA_R_8I && g.b_type == CUDA_R_8I) ||
+                           ((g.a_type == CUDA_R_16F || g.a_type == CUDA_R_16BF) && g.b_type == g.a_type) ||
                            (g.a_type == CUDA_R_8F_E4M3 && g.b_type == CUDA_R_8F_E4M3 &&
                             g.a_scale_mode != SCALE_BLOCK32_UE8M0 && g.b_scale_mode != SCALE_BLOCK32_UE8M0)) &&
            std::min(g.M, g.N) <= kDecodeMaxTokens && std::max(g.M, g.N) >= 64 && any_decode_variant_ok(l);
@@ -503,9 +507,12 @@ static int pick_decode_variant(const Lowered &l, uint32_t cus) {
   // (two token blocks on one unit per slab, variant 20, only up to two blocks of rows per CU: 4096 x 32 x 4096
   // 8.9 us against 10.0, but 14336 x 32 x 4096 18.1 against 16.7; with two units, variant 17, it wins
   // throughout: 8192 x 32 x 8192 15.4 against 22.0)
+  // (16-bit weights, which have no other streaming form, also beyond 64 rows per CU when K is long: bf16
+  // 28672 x 16 x 8192 in 1.75 rounds of workgroups 80 us against 99 on 128 x 64 MFMA tiles; at K = 4096 the two are level)
   const uint32_t rows = (uint32_t)std::max(l.g.M, l.g.N);
+  const bool h16_long = (l.g.a_type == CUDA_R_16F || l.g.a_type == CUDA_R_16BF) && K * 2 > 8192;
   for (int v = 0; v < kNumDecodeVariants; v++)
-    if (kDecodeVariants[v].stream == 2 && decode_variant_ok(l, v) && rows <= 64 * cus &&
+    if (kDecodeVariants[v].stream == 2 && decode_variant_ok(l, v) && (rows <= 64 * cus || h16_long) &&
         !(kDecodeVariants[v].steps == 8 && rows > 32 * cus))
       return v;
   // the stream instantiation with the least cover that takes K
@@ -555,6 +562,9 @@ extern "C" uint32_t zluda_gemm_plan_problem(const zluda_gemm_problem *p, uint32_
     for (uint32_t k : order) {
       if (!family_supports(k, l)) continue;
       if (k == ZLUDA_KERNEL_DECODE_W8A8) {
+        // (some variant takes the problem, but not necessarily the one the rules below pick for this chip: 16-bit
+        // weights have the slab form only, which is given at most 64 rows per CU)
+        if (!decode_variant_ok(l, pick_decode_variant(l, cu_count))) continue;
         const int tokens = std::min(l.g.M, l.g.N);
         const bool stream = kDecodeVariants[pick_decode_variant(l, cu_count)].stream;
         if (tokens > (stream ? kDecodeAutoMaxTokensStream : kDecodeAutoMaxTokens)) continue;
