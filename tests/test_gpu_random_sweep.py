@@ -15,7 +15,7 @@ from zluda_amd import abi as K, cublaslt
 pytestmark = pytest.mark.gpu
 BIG = True   # include shapes of several tiles of the large variants
 NVAR = {K.ZLUDA_KERNEL_MFMA_I8: 10, K.ZLUDA_KERNEL_MFMA_F8: 10, K.ZLUDA_KERNEL_MFMA_MXF4: 8, K.ZLUDA_KERNEL_MFMA_TR8: 4,
-        K.ZLUDA_KERNEL_DECODE_W8A8: 21}
+        K.ZLUDA_KERNEL_DECODE_W8A8: 21, K.ZLUDA_KERNEL_MFMA_H16: 8, K.ZLUDA_KERNEL_MFMA_TR16: 3}
 RNG = None
 
 
@@ -40,8 +40,8 @@ def dims():
     return int(RNG.integers(1, 400)), int(RNG.integers(1, 400)), int(RNG.integers(1, 700))
 
 
-def make():
-    fam = pick(["i8i", "i8f", "i8f", "f8", "f8", "mx", "fl"])
+def make(only=None):
+    fam = only or pick(["i8i", "i8f", "i8f", "f8", "f8", "mx", "fl"])
     m, n, k = dims()
     s = dict(m=m, n=n, k=k)
     s["transa"], s["transb"] = int(RNG.integers(2)), int(RNG.integers(2))
@@ -64,6 +64,10 @@ def make():
                  compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F, a_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_VEC32_UE8M0,
                  b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_VEC32_UE8M0)
         s.pop("order_a", None); s.pop("order_b", None)
+    elif fam == "h16":   # the 16-bit operand types at full size: their MFMA, transposing and decode kernels
+        t = pick([K.CUDA_R_16BF, K.CUDA_R_16F])
+        s.update(a_type=t, b_type=t, d_type=pick([t, t, K.CUDA_R_32F, K.CUDA_R_16BF]), compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F,
+                 alpha_range=(0.02, 0.05))
     else:
         t = pick([K.CUDA_R_16BF, K.CUDA_R_16F, K.CUDA_R_32F])
         s.update(a_type=t, b_type=t, d_type=pick([t, K.CUDA_R_32F]), compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F)
@@ -114,13 +118,16 @@ def make():
     return fam, s
 
 
-@pytest.mark.parametrize("chunk", range(6))
+@pytest.mark.parametrize("chunk", list(range(6)) + ["h16a", "h16b"])
 def test_random_problems_against_the_oracle(gpu_api, chunk):
     global RNG
+    only = None
+    if isinstance(chunk, str):   # the same draw restricted to f16 / bf16 operands
+        only, chunk = "h16", 6 + "ab".index(chunk[-1])
     RNG = np.random.default_rng(4200 + chunk)
     ran = 0
     for it in range(40):
-        fam, spec = make()
+        fam, spec = make(only)
         seed = 420000 + chunk * 1000 + it
         ws = pick([0, 0, 1 << 24])
         forced = pick([None, None, None, K.ZLUDA_KERNEL_GENERIC])
