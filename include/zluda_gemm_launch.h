@@ -79,7 +79,9 @@ enum {
   ZLUDA_KERNEL_DECODE_W8A8 = 5, /* skinny (<= 64 tokens) int8 / fp8 e4m3 streaming kernel, K split inside the workgroup */
   ZLUDA_KERNEL_MFMA_TR8 = 6,  /* int8 / fp8 MFMA with transposing loads: A or B not K-contiguous */
   ZLUDA_KERNEL_MFMA_H16 = 7,  /* v_mfma_f32_32x32x16_f16 / _bf16, K-contiguous A and B of one 16-bit type */
-  ZLUDA_KERNEL_MFMA_TR16 = 8  /* f16 / bf16 MFMA with transposing loads: A or B not K-contiguous */
+  ZLUDA_KERNEL_MFMA_TR16 = 8, /* f16 / bf16 MFMA with transposing loads: A or B not K-contiguous */
+  ZLUDA_KERNEL_MFMA_F32 = 9,  /* v_mfma_f32_32x32x2_f32, K-contiguous f32 A and B */
+  ZLUDA_KERNEL_MFMA_TR32 = 10 /* f32 MFMA with transposing loads: A or B not K-contiguous */
 };
 
 /* The 64-byte algo blob the application round-trips between the heuristic and cublasLtMatmul

@@ -292,6 +292,9 @@ def test_algorithm_enumeration_and_configuration(api):
         h16 = (abi.CUBLAS_COMPUTE_32F, abi.CUDA_R_32F, t, t, t, t)
         assert api.cublasLtMatmulAlgoGetIds(h, *h16, 8, ids, C.byref(n)) == 0
         assert sorted(ids[:n.value]) == [abi.ZLUDA_KERNEL_GENERIC, abi.ZLUDA_KERNEL_MFMA_H16, abi.ZLUDA_KERNEL_MFMA_TR16]
+    f32 = (abi.CUBLAS_COMPUTE_32F, abi.CUDA_R_32F, abi.CUDA_R_32F, abi.CUDA_R_32F, abi.CUDA_R_32F, abi.CUDA_R_32F)
+    assert api.cublasLtMatmulAlgoGetIds(h, *f32, 8, ids, C.byref(n)) == 0
+    assert sorted(ids[:n.value]) == [abi.ZLUDA_KERNEL_GENERIC, abi.ZLUDA_KERNEL_MFMA_F32, abi.ZLUDA_KERNEL_MFMA_TR32]
     # a combination nothing runs
     bad = (abi.CUBLAS_COMPUTE_32I, abi.CUDA_R_32I, abi.CUDA_R_32F, abi.CUDA_R_32F, abi.CUDA_R_32I, abi.CUDA_R_32I)
     assert api.cublasLtMatmulAlgoGetIds(h, *bad, 8, ids, C.byref(n)) == 0 and n.value == 0

@@ -37,7 +37,7 @@ def run(gpu_api, spec, seed, expect_kernel=None, **case_kw):
 
 
 @pytest.mark.parametrize("epi", FWD + BWD)
-@pytest.mark.parametrize("family", ["i8", "f8", "mx", "bf16", "bf16_kc", "f32", "decode", "tr"])
+@pytest.mark.parametrize("family", ["i8", "f8", "mx", "bf16", "bf16_kc", "f32", "f32_tr", "generic", "decode", "tr"])
 def test_aux_epilogues_through_every_kernel_family(gpu_api, epi, family):
     spec, kernel = {
         "i8": (dict(I8F, m=384, n=264, k=512), K.ZLUDA_KERNEL_MFMA_I8),
@@ -45,13 +45,16 @@ def test_aux_epilogues_through_every_kernel_family(gpu_api, epi, family):
         "mx": (dict(MX, m=256, n=128, k=512), K.ZLUDA_KERNEL_MFMA_MXF4),
         "bf16": (dict(BF, m=150, n=90, k=77, d_type=K.CUDA_R_32F), K.ZLUDA_KERNEL_MFMA_TR16),
         "bf16_kc": (dict(BF, m=150, n=90, k=200, transa=1, transb=0, d_type=K.CUDA_R_32F), K.ZLUDA_KERNEL_MFMA_H16),
-        "f32": (dict(BF, a_type=K.CUDA_R_32F, b_type=K.CUDA_R_32F, m=150, n=90, k=77, d_type=K.CUDA_R_32F), K.ZLUDA_KERNEL_GENERIC),
+        "f32": (dict(BF, a_type=K.CUDA_R_32F, b_type=K.CUDA_R_32F, m=150, n=90, k=200, transa=1, transb=0, d_type=K.CUDA_R_32F), K.ZLUDA_KERNEL_MFMA_F32),
+        "f32_tr": (dict(BF, a_type=K.CUDA_R_32F, b_type=K.CUDA_R_32F, m=150, n=90, k=77, d_type=K.CUDA_R_32F), K.ZLUDA_KERNEL_MFMA_TR32),
+        # (K-contiguous f32 rows whose length is not a multiple of 16 bytes: nothing but the generic kernel takes them)
+        "generic": (dict(BF, a_type=K.CUDA_R_32F, b_type=K.CUDA_R_32F, m=150, n=90, k=77, transa=1, transb=0, d_type=K.CUDA_R_32F), K.ZLUDA_KERNEL_GENERIC),
         "decode": (dict(I8F, m=1024, n=16, k=4096, alpha_range=(0.0002, 0.0004)), K.ZLUDA_KERNEL_DECODE_W8A8),
         "tr": (dict(I8F, transa=0, transb=1, m=256, n=320, k=256), K.ZLUDA_KERNEL_MFMA_TR8),
     }[family]
     spec = dict(spec, epilogue=epi)
     if epi in BWD:
-        spec["with_c"] = family in ("i8", "bf16", "f32")
+        spec["with_c"] = family in ("i8", "bf16", "f32", "generic")
     run(gpu_api, spec, 600 + epi, expect_kernel=kernel, int_dist="normal" if family == "decode" else "uniform")
 
 

@@ -26,7 +26,9 @@ CASES = [
     (dict(BF, m=96, n=80, k=200, transa=0, transb=1, bias_type=K.CUDA_R_32F), K.ZLUDA_KERNEL_MFMA_TR16, False),
     (dict(BF, m=96, n=80, k=200, transa=1, lda=201), K.ZLUDA_KERNEL_GENERIC, False),     # an odd pitch: 2-byte alignment only
     (dict(BF, a_type=K.CUDA_R_32F, b_type=K.CUDA_R_32F, m=96, n=80, k=200, transa=0, transb=1, bias_type=K.CUDA_R_32F),
-     K.ZLUDA_KERNEL_GENERIC, False),
+     K.ZLUDA_KERNEL_MFMA_TR32, False),
+    (dict(BF, a_type=K.CUDA_R_32F, b_type=K.CUDA_R_32F, m=96, n=80, k=200, transa=1, bias_type=K.CUDA_R_32F), K.ZLUDA_KERNEL_MFMA_F32, False),
+    (dict(BF, a_type=K.CUDA_R_32F, b_type=K.CUDA_R_32F, m=96, n=80, k=201, transa=1, bias_type=K.CUDA_R_32F), K.ZLUDA_KERNEL_GENERIC, False),
     (dict(I8F, m=512, n=384, k=1024, transa=1, bias_type=K.CUDA_R_32F), K.ZLUDA_KERNEL_MFMA_I8, True),
     (dict(I8F, m=320, n=256, k=768, transa=0, transb=1, bias_type=K.CUDA_R_32F), K.ZLUDA_KERNEL_MFMA_TR8, True),
     (dict(F8, m=1024, n=256, k=2048, transa=1), K.ZLUDA_KERNEL_MFMA_F8, False),

@@ -156,6 +156,30 @@ def test_last_real_stage_is_waited_for(gpu_api, variant):
         check(gpu_api, dict(F8, m=512, n=256, k=5 * bkb), 118 + rep, K.ZLUDA_KERNEL_MFMA_F8, variant)
 
 
+@pytest.mark.parametrize("variant", [3, 4, 5, 6])
+def test_mfma_mxf4_more_workgroups_than_cus(gpu_api, variant):
+    """grids of several rounds of workgroups per CU: a workgroup that follows another one on its CU sees other
+    memory timings than the first (the deeper LDS rings of the small tiles once counted their scale loads into the
+    waits for the data and multiplied blocks that had not landed)"""
+    for rep in range(3):
+        check(gpu_api, dict(MX, m=8000, n=256, k=2048, batch=3), 1160 + variant, K.ZLUDA_KERNEL_MFMA_MXF4, variant)
+    if variant == 5:   # the same through split-K shares (504 workgroups)
+        case = Case(dict(MX, m=1771, n=17, k=13824, batch=3, order_d=1), 1170)
+        ref = case.run_oracle()
+        for rep in range(3):
+            st, got, _, v = case.run_gpu(gpu_api, forced_kernel=K.ZLUDA_KERNEL_MFMA_MXF4, forced_variant=5, workspace_bytes=1 << 24)
+            assert st == 0 and v == 5
+            case.compare(got, ref)
+
+
+@pytest.mark.parametrize("family,kernel", [("i8", K.ZLUDA_KERNEL_MFMA_I8), ("f8", K.ZLUDA_KERNEL_MFMA_F8)])
+def test_small_tiles_on_grids_of_several_rounds(gpu_api, family, kernel):
+    """the 3- and 4-stage tile variants with more workgroups than CUs and a K tail"""
+    base = I8 if family == "i8" else F8
+    for variant in (4, 5, 6):
+        check(gpu_api, dict(base, m=8000, n=200, k=400 if family == "i8" else 272, batch=3), 1180 + variant, kernel, variant)
+
+
 def test_mxf4_generic_agrees(gpu_api):
     check(gpu_api, dict(MX, m=96, n=80, k=384), 70, K.ZLUDA_KERNEL_GENERIC)
 

@@ -77,6 +77,24 @@ def test_16_bit_operands_take_the_mfma_family_when_k_contiguous(api):
         assert plan(api, dict(I8, m=512, n=256, k=4096, transa=1), forced=K.ZLUDA_KERNEL_MFMA_H16)[0] == K.CUBLAS_STATUS_NOT_SUPPORTED
 
 
+def test_f32_operands_take_their_mfma_families(api):
+    F = dict(a_type=K.CUDA_R_32F, b_type=K.CUDA_R_32F, d_type=K.CUDA_R_32F, compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F)
+    st, p = plan(api, dict(F, m=8192, n=8192, k=8192, transa=1))
+    assert st == 0 and (p.kernel, p.variant, p.grid_x, p.block) == (K.ZLUDA_KERNEL_MFMA_F32, 0, 1024, 512)
+    for ta, tb in ((0, 0), (0, 1), (1, 1)):
+        st, p = plan(api, dict(F, m=4096, n=4096, k=4096, transa=ta, transb=tb))
+        assert st == 0 and (p.kernel, p.variant) == (K.ZLUDA_KERNEL_MFMA_TR32, 0)
+    # K-contiguous rows of 4-byte alignment only: the transposing kernel, if they are whole 16-byte pieces long
+    assert plan(api, dict(F, m=512, n=256, k=4096, transa=1, lda=4097))[1].kernel == K.ZLUDA_KERNEL_MFMA_TR32
+    assert plan(api, dict(F, m=512, n=256, k=4097, transa=1))[1].kernel == K.ZLUDA_KERNEL_GENERIC
+    # any K when neither operand is K-contiguous
+    assert plan(api, dict(F, m=512, n=256, k=4097, transa=0, transb=1))[1].kernel == K.ZLUDA_KERNEL_MFMA_TR32
+    assert api.zluda_gemm_variant_count(K.ZLUDA_KERNEL_MFMA_F32) == 8 and api.zluda_gemm_variant_count(K.ZLUDA_KERNEL_MFMA_TR32) == 3
+    # a skinny f32 problem is not a decode problem
+    assert plan(api, dict(F, m=14336, n=16, k=2048, transa=1))[1].kernel == K.ZLUDA_KERNEL_MFMA_F32
+    assert plan(api, dict(F, m=4096, n=4096, k=4096, transa=1), forced=K.ZLUDA_KERNEL_MFMA_H16)[0] == K.CUBLAS_STATUS_NOT_SUPPORTED
+
+
 def test_16_bit_weights_with_few_tokens_take_the_slab_decode(api):
     """the slab form counts K in bytes: 2048 elements of 16 bits are the 4096 bytes of its first shape"""
     for t in (K.CUDA_R_16BF, K.CUDA_R_16F):

@@ -138,6 +138,8 @@ ZLUDA_KERNEL_DECODE_W8A8 = 5
 ZLUDA_KERNEL_MFMA_TR8 = 6
 ZLUDA_KERNEL_MFMA_H16 = 7
 ZLUDA_KERNEL_MFMA_TR16 = 8
+ZLUDA_KERNEL_MFMA_F32 = 9
+ZLUDA_KERNEL_MFMA_TR32 = 10
 ZLUDA_ALGO_MAGIC = 0x5A4C4441
 
 TYPE_BITS = {CUDA_R_32F: 32, CUDA_R_32I: 32, CUDA_R_16F: 16, CUDA_R_16BF: 16, CUDA_R_8I: 8,

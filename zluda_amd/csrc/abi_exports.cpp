@@ -312,7 +312,7 @@ bool unpack_algo(const cublasLtMatmulAlgo_t *algo, uint32_t *kernel, int32_t *va
   if ((algo->data[0] >> 32) != ZLUDA_ALGO_MAGIC) return false;
   *kernel = (uint32_t)(algo->data[0] & 0xffffffffu);
   *variant = (int32_t)algo->data[1];
-  return *kernel >= ZLUDA_KERNEL_GENERIC && *kernel <= ZLUDA_KERNEL_MFMA_TR16;
+  return *kernel >= ZLUDA_KERNEL_GENERIC && *kernel <= ZLUDA_KERNEL_MFMA_TR32;
 }
 
 // A/B forcing for measurements: ZLUDA_FORCE_KERNEL=<family>[:<variant>], read once per process (the
@@ -666,6 +666,8 @@ static int families_for_types(uint32_t computeType, uint32_t scaleType, uint32_t
     if (zluda_gemm_plan_problem(&p, k, -1, 256, &plan) == CUBLAS_STATUS_SUCCESS) ids[count++] = (int)k;
   if (zluda_gemm_plan_problem(&p, ZLUDA_KERNEL_MFMA_H16, -1, 256, &plan) == CUBLAS_STATUS_SUCCESS)
     ids[count++] = ZLUDA_KERNEL_MFMA_H16;
+  if (zluda_gemm_plan_problem(&p, ZLUDA_KERNEL_MFMA_F32, -1, 256, &plan) == CUBLAS_STATUS_SUCCESS)
+    ids[count++] = ZLUDA_KERNEL_MFMA_F32;
   p.b.cols = p.c.cols = p.d.cols = 16;
   if (zluda_gemm_plan_problem(&p, ZLUDA_KERNEL_DECODE_W8A8, -1, 256, &plan) == CUBLAS_STATUS_SUCCESS)
     ids[count++] = ZLUDA_KERNEL_DECODE_W8A8;
@@ -676,6 +678,8 @@ static int families_for_types(uint32_t computeType, uint32_t scaleType, uint32_t
     ids[count++] = ZLUDA_KERNEL_MFMA_TR8;
   if (zluda_gemm_plan_problem(&p, ZLUDA_KERNEL_MFMA_TR16, -1, 256, &plan) == CUBLAS_STATUS_SUCCESS)
     ids[count++] = ZLUDA_KERNEL_MFMA_TR16;
+  if (zluda_gemm_plan_problem(&p, ZLUDA_KERNEL_MFMA_TR32, -1, 256, &plan) == CUBLAS_STATUS_SUCCESS)
+    ids[count++] = ZLUDA_KERNEL_MFMA_TR32;
   return count;
 }
 
@@ -741,7 +745,7 @@ cublasStatus_t cublasLtMatmulAlgoCapGetAttribute(const cublasLtMatmulAlgo_t *alg
   case 14 /* LD_NEGATIVE */: i32 = 0; return access(false, i32, nullptr, buf, sizeInBytes, sizeWritten);
   case 15 /* NUMERICAL_IMPL_FLAGS */: u64 = ~0ull; return access(false, u64, nullptr, buf, sizeInBytes, sizeWritten);
   case 16: case 17: /* MIN_ALIGNMENT_A/B_BYTES */
-    u32 = kernel == ZLUDA_KERNEL_GENERIC ? 1 : (kernel == ZLUDA_KERNEL_MFMA_TR8 || kernel == ZLUDA_KERNEL_MFMA_TR16 ? 4 : 16);
+    u32 = kernel == ZLUDA_KERNEL_GENERIC ? 1 : (kernel == ZLUDA_KERNEL_MFMA_TR8 || kernel == ZLUDA_KERNEL_MFMA_TR16 || kernel == ZLUDA_KERNEL_MFMA_TR32 ? 4 : 16);
     return access(false, u32, nullptr, buf, sizeInBytes, sizeWritten);
   case 18: case 19: /* MIN_ALIGNMENT_C/D_BYTES */ u32 = 1; return access(false, u32, nullptr, buf, sizeInBytes, sizeWritten);
   case 21 /* POINTER_ARRAY_BATCH_SUPPORT */: case 22 /* FLOATING_POINT_EMULATION_SUPPORT */:

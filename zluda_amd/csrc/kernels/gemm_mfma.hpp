@@ -7,6 +7,7 @@
 //   KIND_MXF4 : e2m1 + UE8M0 per 32 -> fp32  v_mfma_scale_f32_32x32x64_f8f6f4 (cbsz=blgp=4)
 //   KIND_F16  : f16 x f16 -> fp32            v_mfma_f32_32x32x16_f16
 //   KIND_BF16 : bf16 x bf16 -> fp32          v_mfma_f32_32x32x16_bf16
+//   KIND_F32  : f32 x f32 -> fp32            v_mfma_f32_32x32x2_f32 (four per 16 bytes of K and lane)
 //
 // Naming inside the kernel: P is the operand whose row index runs along the unit-stride
 // dimension of D (it is fed as MFMA operand "B", so its index lands on lane%32 of the
@@ -33,9 +34,13 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef __bf16 v8b __attribute__((ext_vector_type(8)));
 
-enum { KIND_I8 = 0, KIND_F8 = 1, KIND_MXF4 = 2, KIND_F16 = 3, KIND_BF16 = 4 };
+enum { KIND_I8 = 0, KIND_F8 = 1, KIND_MXF4 = 2, KIND_F16 = 3, KIND_BF16 = 4, KIND_F32 = 5 };
 // 16-bit elements: 16 bytes (8 elements) of K per lane and MFMA, i.e. the byte geometry of int8
 constexpr bool kind_is_h16(int kind) { return kind == KIND_F16 || kind == KIND_BF16; }
+// bytes per element of the kinds whose elements are whole bytes
+constexpr int kind_esz(int kind) { return kind_is_h16(kind) ? 2 : (kind == KIND_F32 ? 4 : 1); }
+// f32: a lane's 16 bytes are four K elements, one v_mfma_f32_32x32x2_f32 each; element e of lane group g of the
+// 32-byte step s is K index 8 s + 4 g + e for both operands, which is all the instruction asks of a K order
 
 // depends on r mod 32 only, so rows 32 apart (the MFMA tiles of one wave) share a swizzle
 __device__ __forceinline__ int swz(int r) { return (r ^ ((r >> 3) & 3)) & 7; }

@@ -1,5 +1,5 @@
 // Software-pipelined MFMA GEMM for K-contiguous operands on gfx950: the production kernel of the
-// int8 / fp8 / MXFP4 / f16 / bf16 families.
+// int8 / fp8 / MXFP4 / f16 / bf16 / f32 families.
 //
 // Same tiling, operand naming (P / Q) and epilogue as gemm_mfma.hpp; what differs is the K loop:
 //
@@ -54,7 +54,13 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
   constexpr int LS = MX ? (SPARTS + NWV * (CH - NSTAGE) - 1) / (NWV * (CH - NSTAGE)) : 0;
   constexpr int PRO_S = MX ? (SPARTS + NWV - 1) / NWV : 0;  // per wave, for the first chunk
   constexpr int CHUNK_V4 = MX ? (BP + BQ) * 2 : 0;
-  constexpr int NLOAD = LP + LQ + LS;          // vmcnt units per stage
+  constexpr int NLOAD = LP + LQ + LS;          // vector memory instructions per stage
+  // The counted waits only count the DATA instructions of the younger stages: the scale instructions of a stage
+  // are issued in front of its data, so a wait that also covers them costs nothing, and it does not depend on when
+  // the surplus ones (which read one cache line over and over) are counted as done -- seen on MI355X: with the
+  // scale instructions counted, workgroups that follow another one on their CU multiplied 1 KiB blocks of the last
+  // operand rows of a stage before they had landed.
+  constexpr int NDATA = LP + LQ;
   constexpr int WTP = BP / WP, WTQ = BQ / WQ;
   constexpr int TP = WTP / 32, TQ = WTQ / 32;
   constexpr int KS = BKB_ / (KIND == KIND_F8 ? 64 : 32);  // MFMA sub-steps per stage
@@ -66,7 +72,8 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
   static_assert((NSTAGE - 1) * NLOAD < 64, "vmcnt range");
   static_assert((NSTAGE * STAGE_V4 + 2 * CHUNK_V4) * 16 <= 160 * 1024, "LDS capacity");
   using acc_v = typename std::conditional<KIND == KIND_I8, v16i, v16f>::type;
-  constexpr bool B16 = KIND == KIND_I8 || kind_is_h16(KIND);  // 16 bytes of K per lane and MFMA (else 32)
+  constexpr bool B16 = KIND == KIND_I8 || kind_is_h16(KIND) || KIND == KIND_F32;  // 16 bytes of K per lane and sub-step (else 32)
+  constexpr int MPS = KIND == KIND_F32 ? 4 : 1;  // MFMAs per fragment pair and sub-step
   using frag_v = typename std::conditional<B16, v4i, v8i>::type;
   struct Frags { frag_v p[TP], q[TQ]; };
   struct Scales { int p[TP], q[TQ]; };  // MX scale dwords of one stage (one per MFMA tile row set)
@@ -92,7 +99,7 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
   const int p0 = tile_p * BP, q0 = tile_q * BQ;
 
   const int NP = prm.swapped ? g.N : g.M, NQ = prm.swapped ? g.M : g.N;
-  constexpr int ebits = KIND == KIND_MXF4 ? 4 : (kind_is_h16(KIND) ? 16 : 8);
+  constexpr int ebits = KIND == KIND_MXF4 ? 4 : 8 * kind_esz(KIND);
   const int Kbytes = (int)((int64_t)g.K * ebits / 8);
   const uint8_t *Pg, *Qg;
   int ldp, ldq;
@@ -256,6 +263,16 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
   auto mfma_all = [&](const Frags &f, const Scales &sc, auto ks_c) {
     constexpr int ks = decltype(ks_c)::value;
     (void)sc;
+    if constexpr (KIND == KIND_F32) {
+      // element by element: TP * TQ independent MFMAs between two that feed the same accumulator
+#pragma unroll
+      for (int e = 0; e < 4; e++)
+#pragma unroll
+        for (int a = 0; a < TQ; a++)
+#pragma unroll
+          for (int b = 0; b < TP; b++)
+            acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(bits2f((uint32_t)f.q[a][e]), bits2f((uint32_t)f.p[b][e]), acc[a][b], 0, 0, 0);
+    } else {
 #pragma unroll
     for (int a = 0; a < TQ; a++)
 #pragma unroll
@@ -274,6 +291,7 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
           acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.q[a], f.p[b], acc[a][b], 4, 4, ks, sc.q[a],
                                                                        ks, sc.p[b]);
       }
+    }
   };
 
   // ---- prologue: stages 0 .. NSTAGE-1 in flight, stage 0 landed -----------------------------------
@@ -287,7 +305,7 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
     for (int i = 0; i < LS; i++) issue_scale_part(0, SPARTS, s * STAGE_V4);  // surplus: one line, overwritten by the data
     issue_stage(s, s * STAGE_V4);
   }
-  wait_vmcnt_barrier<(NSTAGE - 1) * NLOAD>();
+  wait_vmcnt_barrier<(NSTAGE - 1) * NDATA>();
 
   Frags fa, fb;
   Scales sc_cur, sc_nxt;
@@ -314,7 +332,7 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
         // left with the fragment reads and the refill
         if constexpr (s == 0) load_scales(kt + 1, sc_nxt);
       } else {
-        wait_vmcnt_barrier<(NSTAGE - 2) * NLOAD>();
+        wait_vmcnt_barrier<(NSTAGE - 2) * NDATA>();
         // reads first: the compiler cannot prove that the DMA (an LDS write) and these reads hit
         // different slots, so whatever comes second in the source stays second in the schedule
         load_frags(so_next, std::integral_constant<int, 0>{}, nxt);
@@ -328,7 +346,7 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
       // first half of them and the LDS DMA of the refill behind the second half.  Without the
       // pattern the scheduler either sinks every ds_read to its first use (the wave then stalls on
       // it) or keeps the loads in one block in front of the MFMAs (the matrix pipe idles meanwhile).
-      constexpr int NM = TP * TQ, NDS = (TP + TQ) * (KIND == KIND_F8 ? 2 : 1) + (KIND == KIND_MXF4 && (KS == 1 ? last : s == 0) ? TP + TQ : 0);
+      constexpr int NM = TP * TQ * MPS, NDS = (TP + TQ) * (KIND == KIND_F8 ? 2 : 1) + (KIND == KIND_MXF4 && (KS == 1 ? last : s == 0) ? TP + TQ : 0);
       constexpr int NVM = last ? NLOAD : 0, H1 = NM / 2 > 0 ? NM / 2 : 1, H2 = NM - H1 > 0 ? NM - H1 : 1;
       static_for<NM>([&](auto i_c) {
         constexpr int i = decltype(i_c)::value;

@@ -1,4 +1,4 @@
-// MFMA GEMM for 8-bit operands (int8, OCP fp8) and 16-bit operands (f16, bf16) of which at least one is
+// MFMA GEMM for 8-bit operands (int8, OCP fp8), 16-bit operands (f16, bf16) and f32 operands of which at least one is
 // NOT K-contiguous: a column-major A without transpose (unit stride along M), a B with transpose (unit
 // stride along N), and their row-major counterparts.  v_mfma_i32_32x32x32_i8 / v_mfma_f32_32x32x16_f16 /
 // _bf16 / v_mfma_f32_32x32x64_f8f6f4 want 16 / 16 / 32 consecutive K bytes of one matrix row per lane, so
@@ -20,6 +20,7 @@
 //     turn the block into one dword of 4 consecutive K bytes per row, written with ds_write_b32.
 //     16-bit elements: 2 K rows x IW row indices per lane (2 IW bytes per K row: dwordx2, dwordx4 or two
 //     dwordx4), 2 v_perm_b32 per 2 x 2 elements, one dword of 2 consecutive K elements per row.
+//     f32: 1 K row x IW row indices per lane; every loaded dword is already one LDS dword (no permute).
 //   * Operand with unit stride along K ("KC"): 16 bytes per lane, ds_write_b128.
 //   * LDS rows have a pitch of 80 bytes and are stored in permuted order, rho(i) = 16 r + ((g + s r) mod 16)
 //     for i = IW g + r, s = 16 / IW.  With that every ds_write_b32 instruction of the transposing path
@@ -74,8 +75,8 @@ struct TrOperand {
   static constexpr int NCH = ROWS / 64;       // KC: 16-byte chunks per lane and stage
   static constexpr int NREG = KC ? NCH * 4 : NW * KR;
   static constexpr int NLOADS = KC ? NCH : KR * (NW > 4 ? NW / 4 : 1);  // vector memory instructions per stage
-  static constexpr int NPERM = KC ? 0 : (ESZ == 1 ? NREG * 2 : NREG);   // v_perm_b32 per stage
-  static_assert(ESZ == 1 || ESZ == 2, "8- or 16-bit elements");
+  static constexpr int NPERM = KC ? 0 : (ESZ == 1 ? NREG * 2 : ESZ == 2 ? NREG : 0);   // v_perm_b32 per stage
+  static_assert(ESZ == 1 || ESZ == 2 || ESZ == 4, "8-, 16- or 32-bit elements");
   static_assert(ROWS == 64 || ROWS == 128 || ROWS == 256, "64, 128 or 256 rows per group of 256 threads");
 
   __amdgpu_buffer_rsrc_t rs;
@@ -151,11 +152,13 @@ struct TrOperand {
           transpose4x4(regs[0 * NW + c], regs[1 * NW + c], regs[2 * NW + c], regs[3 * NW + c], out);
 #pragma unroll
           for (int r = 0; r < 4; r++) d32[tr_rho<ROWS>(g, 4 * c + r) * 20 + kb] = out[r];
-        } else {
+        } else if constexpr (ESZ == 2) {
           int lo, hi;
           transpose2x2(regs[c], regs[NW + c], lo, hi);
           d32[tr_rho<ROWS>(g, 2 * c) * 20 + kb] = lo;
           d32[tr_rho<ROWS>(g, 2 * c + 1) * 20 + kb] = hi;
+        } else {
+          d32[tr_rho<ROWS>(g, c) * 20 + kb] = regs[c];
         }
       }
     }
@@ -168,8 +171,9 @@ struct TrOperand {
 // chunk l/16), one MFMA per pair of fragments and stage.
 template <int KIND, int FQ, int FP, int BP, int BQ, int WP, int WQ, bool PKC, bool QKC, bool M16 = false>
 __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_tr_kernel(MfmaParams prm) {
-  static_assert(KIND == KIND_I8 || KIND == KIND_F8 || kind_is_h16(KIND), "8- or 16-bit operands");
-  constexpr int ESZ = kind_is_h16(KIND) ? 2 : 1;
+  static_assert(KIND == KIND_I8 || KIND == KIND_F8 || kind_is_h16(KIND) || KIND == KIND_F32, "8-, 16- or 32-bit operands");
+  constexpr int ESZ = kind_esz(KIND);
+  constexpr int MPS = KIND == KIND_F32 ? 4 : 1;  // MFMAs per fragment pair and sub-step
   constexpr bool B16 = KIND != KIND_F8;  // 16 bytes of K per lane and MFMA (fp8: 32)
   static_assert(!M16 || KIND == KIND_I8, "the 16x16 form is instantiated for int8");
   constexpr int NT = WP * WQ * 64;
@@ -323,6 +327,15 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_tr_kernel(MfmaParams pr
     }
   };
   auto mfma_all = [&](const Frags &f) {
+    if constexpr (KIND == KIND_F32) {
+#pragma unroll
+      for (int e = 0; e < 4; e++)
+#pragma unroll
+        for (int a = 0; a < TQ; a++)
+#pragma unroll
+          for (int b = 0; b < TP; b++)
+            acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(bits2f((uint32_t)f.q[a][e]), bits2f((uint32_t)f.p[b][e]), acc[a][b], 0, 0, 0);
+    } else {
 #pragma unroll
     for (int a = 0; a < TQ; a++)
 #pragma unroll
@@ -338,6 +351,7 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_tr_kernel(MfmaParams pr
         else
           acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.q[a], f.p[b], acc[a][b], FQ, FP, 0, 0, 0, 0);
       }
+    }
   };
 
   // One stage (kt), entered with: stage kt complete in `cur`, its sub-step-0 fragments in `f0`, stage
@@ -361,7 +375,7 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_tr_kernel(MfmaParams pr
     {
       // the fragment reads of sub-step 1 go out with the first MFMAs, the byte permutes follow (an LDS
       // write needs the eight permutes of its 4 x 4 block), the LDS writes come behind the later MFMAs
-      constexpr int NM = TP * TQ, H = NM / 2 > 0 ? NM / 2 : 1;
+      constexpr int NM = TP * TQ * MPS, H = NM / 2 > 0 ? NM / 2 : 1;
       constexpr int NDR = KS == 2 ? (TP + TQ) : 0;
       constexpr int NPERM = P.NPERM + Q.NPERM;
       constexpr int NDW = (PKC ? P.NCH : P.NREG) + (QKC ? Q.NCH : Q.NREG);
@@ -391,7 +405,7 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_tr_kernel(MfmaParams pr
     read_frags(nxt, 0, f0);
     if constexpr (KS == 2) {
       mfma_all(f1);
-      constexpr int NM = TP * TQ, NDR = TP + TQ;
+      constexpr int NM = TP * TQ * MPS, NDR = TP + TQ;
       constexpr int NVM = P.NLOADS + Q.NLOADS;
       static_for<NM>([&](auto i_c) {
         constexpr int i = decltype(i_c)::value;

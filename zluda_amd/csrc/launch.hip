@@ -49,7 +49,7 @@ uint32_t launch_mfma(const Lowered &l, const zluda_gemm_plan &plan, void *ws, ui
     const uint64_t need = (uint64_t)plan.grid_z * l.g.batch * prm.tiles_p * v.bp * prm.tiles_q * v.bq * 4;
     if (!ws || (((uintptr_t)ws) & 15) || ws_size < need || plan.workspace != need) return CUBLAS_STATUS_INVALID_VALUE;
     const bool mx = plan.kernel == ZLUDA_KERNEL_MFMA_MXF4;
-    const int kbytes = mx ? l.g.K / 2 : (plan.kernel == ZLUDA_KERNEL_MFMA_H16 ? l.g.K * 2 : l.g.K);
+    const int kbytes = mx ? l.g.K / 2 : (plan.kernel == ZLUDA_KERNEL_MFMA_H16 ? l.g.K * 2 : plan.kernel == ZLUDA_KERNEL_MFMA_F32 ? l.g.K * 4 : l.g.K);
     const int stages = (kbytes + v.bkb - 1) / v.bkb;
     prm.splits = (int32_t)plan.grid_z;
     prm.split_stages = (stages + prm.splits - 1) / prm.splits;
@@ -64,6 +64,7 @@ uint32_t launch_mfma(const Lowered &l, const zluda_gemm_plan &plan, void *ws, ui
   case ZLUDA_KERNEL_MFMA_I8: st = launch_mfma_i8(prm, plan, s); break;
   case ZLUDA_KERNEL_MFMA_MXF4: st = launch_mfma_mxf4(prm, plan, s); break;
   case ZLUDA_KERNEL_MFMA_H16: st = launch_mfma_h16(prm, plan, l.g.a_type == CUDA_R_16BF, s); break;
+  case ZLUDA_KERNEL_MFMA_F32: st = launch_mfma_f32(prm, plan, s); break;
   case ZLUDA_KERNEL_MFMA_F8: {
     // MFMA operand "A" is Q, operand "B" is P (see gemm_mfma.hpp)
     const int fa = f8_fmt(l.g.a_type), fb = f8_fmt(l.g.b_type);
@@ -100,7 +101,7 @@ uint32_t launch_tr(const Lowered &l, const zluda_gemm_plan &plan, void *ws, uint
     // split-K: partial tiles go through the caller's workspace (64 K bytes per stage)
     const uint64_t need = (uint64_t)plan.grid_z * l.g.batch * prm.tiles_p * v.bp * prm.tiles_q * v.bq * 4;
     if (!ws || (((uintptr_t)ws) & 15) || ws_size < need || plan.workspace != need) return CUBLAS_STATUS_INVALID_VALUE;
-    const int stages = (l.g.K * (plan.kernel == ZLUDA_KERNEL_MFMA_TR16 ? 2 : 1) + 63) / 64;
+    const int stages = (l.g.K * (plan.kernel == ZLUDA_KERNEL_MFMA_TR16 ? 2 : plan.kernel == ZLUDA_KERNEL_MFMA_TR32 ? 4 : 1) + 63) / 64;
     prm.splits = (int32_t)plan.grid_z;
     prm.split_stages = (stages + prm.splits - 1) / prm.splits;
     prm.ws = ws;
@@ -114,6 +115,8 @@ uint32_t launch_tr(const Lowered &l, const zluda_gemm_plan &plan, void *ws, uint
     st = launch_tr_f16(prm, plan, pkc, qkc, s);
   } else if (l.g.a_type == CUDA_R_16BF) {
     st = launch_tr_bf16(prm, plan, pkc, qkc, s);
+  } else if (l.g.a_type == CUDA_R_32F) {
+    st = launch_tr_f32(prm, plan, pkc, qkc, s);
   } else {
     const int fa = f8_fmt(l.g.a_type), fb = f8_fmt(l.g.b_type);
     st = launch_tr_f8(prm, plan, plan.swapped ? fa : fb, plan.swapped ? fb : fa, pkc, qkc, s);
@@ -261,10 +264,11 @@ uint32_t launch_planned(const zluda_gemm_problem *p, const zluda_gemm_plan *plan
     break;
   }
   case ZLUDA_KERNEL_MFMA_I8: case ZLUDA_KERNEL_MFMA_F8: case ZLUDA_KERNEL_MFMA_MXF4: case ZLUDA_KERNEL_MFMA_H16:
+  case ZLUDA_KERNEL_MFMA_F32:
     st = launch_mfma(l, *plan, ws, ws_size, s);
     break;
   case ZLUDA_KERNEL_DECODE_W8A8: st = launch_decode(l, *plan, s); break;
-  case ZLUDA_KERNEL_MFMA_TR8: case ZLUDA_KERNEL_MFMA_TR16: st = launch_tr(l, *plan, ws, ws_size, s); break;
+  case ZLUDA_KERNEL_MFMA_TR8: case ZLUDA_KERNEL_MFMA_TR16: case ZLUDA_KERNEL_MFMA_TR32: st = launch_tr(l, *plan, ws, ws_size, s); break;
   default: return CUBLAS_STATUS_NOT_SUPPORTED;
   }
   if (st == CUBLAS_STATUS_SUCCESS && l.g.bgrad_src) st = launch_bgrad(l.g, s);

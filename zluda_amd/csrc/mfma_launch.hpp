@@ -49,5 +49,6 @@ uint32_t launch_mfma_i8(const MfmaParams &prm, const zluda_gemm_plan &plan, hipS
 uint32_t launch_mfma_f8(const MfmaParams &prm, const zluda_gemm_plan &plan, int fq, int fp, hipStream_t s);
 uint32_t launch_mfma_mxf4(const MfmaParams &prm, const zluda_gemm_plan &plan, hipStream_t s);
 uint32_t launch_mfma_h16(const MfmaParams &prm, const zluda_gemm_plan &plan, bool bf16, hipStream_t s);
+uint32_t launch_mfma_f32(const MfmaParams &prm, const zluda_gemm_plan &plan, hipStream_t s);
 
 } // namespace zluda_amd

@@ -52,5 +52,6 @@ uint32_t launch_tr_f8_e5m2q(const MfmaParams &prm, const zluda_gemm_plan &plan, 
 uint32_t launch_tr_f8_e5m2p(const MfmaParams &prm, const zluda_gemm_plan &plan, bool pkc, bool qkc, hipStream_t s);
 uint32_t launch_tr_f16(const MfmaParams &prm, const zluda_gemm_plan &plan, bool pkc, bool qkc, hipStream_t s);
 uint32_t launch_tr_bf16(const MfmaParams &prm, const zluda_gemm_plan &plan, bool pkc, bool qkc, hipStream_t s);
+uint32_t launch_tr_f32(const MfmaParams &prm, const zluda_gemm_plan &plan, bool pkc, bool qkc, hipStream_t s);
 
 } // namespace zluda_amd

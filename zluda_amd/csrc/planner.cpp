@@ -298,14 +298,17 @@ bool family_supports(uint32_t kernel, const Lowered &l) {
     // f16 x f16 or bf16 x bf16 (lower_problem admits 16-bit operands of one type only)
     return fast_layout && l.span_ok && (g.a_type == CUDA_R_16F || g.a_type == CUDA_R_16BF) && g.b_type == g.a_type &&
            g.a_scale_mode != SCALE_BLOCK32_UE8M0 && g.b_scale_mode != SCALE_BLOCK32_UE8M0 && d_fast;
-  case ZLUDA_KERNEL_MFMA_TR8: case ZLUDA_KERNEL_MFMA_TR16: {
-    // 8-bit (TR8) or 16-bit (TR16) operands, each with unit stride along K or along its row index; dword-aligned loads
-    const bool h16 = g.a_type == CUDA_R_16F || g.a_type == CUDA_R_16BF;
-    const bool types = kernel == ZLUDA_KERNEL_MFMA_TR16
+  case ZLUDA_KERNEL_MFMA_F32:
+    return fast_layout && l.span_ok && g.a_type == CUDA_R_32F && g.b_type == CUDA_R_32F && d_fast;
+  case ZLUDA_KERNEL_MFMA_TR8: case ZLUDA_KERNEL_MFMA_TR16: case ZLUDA_KERNEL_MFMA_TR32: {
+    // 8-bit (TR8), 16-bit (TR16) or f32 (TR32) operands, each with unit stride along K or along its row index; dword-aligned loads
+    const bool h16 = g.a_type == CUDA_R_16F || g.a_type == CUDA_R_16BF, f32 = g.a_type == CUDA_R_32F;
+    const bool types = kernel == ZLUDA_KERNEL_MFMA_TR32 ? (f32 && g.b_type == CUDA_R_32F)
+                       : kernel == ZLUDA_KERNEL_MFMA_TR16
                            ? (h16 && g.b_type == g.a_type)
                            : ((g.a_type == CUDA_R_8I && g.b_type == CUDA_R_8I) ||
                               (is_f8(g.a_type) && is_f8(g.b_type) && !(g.a_type == CUDA_R_8F_E5M2 && g.b_type == CUDA_R_8F_E5M2)));
-    const int64_t esz = h16 ? 2 : 1;
+    const int64_t esz = f32 ? 4 : h16 ? 2 : 1;
     // (strides in bytes from here on)
     auto operand_ok = [&](const void *ptr, int64_t s_row, int64_t s_k, int64_t s_b, int rows) {
       s_row *= esz; s_k *= esz; s_b *= esz;
@@ -354,8 +357,7 @@ static void fill_mfma_plan(const Lowered &l, int variant, uint32_t cus, uint64_t
   // kernel sums them and applies the epilogue.  Only if the caller's workspace holds the partial
   // tiles (padded to whole tiles).  (MXFP4 shares are whole scale chunks: the launcher rounds.)
   const uint64_t tiles = (uint64_t)plan->grid_x * plan->grid_y;
-  const bool h16 = g.a_type == CUDA_R_16F || g.a_type == CUDA_R_16BF;
-  const uint32_t kt = ceil_div((uint32_t)((int64_t)g.K * (g.a_type == CUDA_R_4F_E2M1 ? 4 : (h16 ? 16 : 8)) / 8), v.bkb);
+  const uint32_t kt = ceil_div((uint32_t)((int64_t)g.K * type_bits(g.a_type) / 8), v.bkb);
   // (below ~6 KiB of K per row the second kernel and the workspace traffic cost more than the idle CUs)
   const uint32_t kbytes = kt * v.bkb;
   // Skinny problems (<= 64 rows or columns) are memory bound: they split from 2 KiB of K per row on
@@ -399,7 +401,7 @@ static int pick_mfma_variant(const Lowered &l, uint32_t cus) {
     const MfmaVariant &t = kMfmaVariants[v];
     const uint64_t tiles = (uint64_t)ceil_div(np, t.bp) * ceil_div(nq, t.bq) * g.batch;
     if (t.m16) {
-      if (g.a_type == CUDA_R_4F_E2M1 || g.a_type == CUDA_R_16F || g.a_type == CUDA_R_16BF) continue;  // the 16x16 shapes serve int8 and fp8
+      if (type_bits(g.a_type) != 8) continue;  // the 16x16 shapes serve int8 and fp8
       // power bound or not: int8 gains from three quarters of the CUs busy on.  fp8 gains little and only on
       // long runs: the 192x256 tile from two full rounds on (6144^3: 190 us against 198), the 256x256 tile
       // from four (8192^3: 405 against 408; at two rounds, 8192x4096x4096, it loses 3 %)
@@ -433,7 +435,7 @@ static void fill_tr_plan(const Lowered &l, int variant, uint32_t cus, uint64_t w
   const uint64_t tiles = (uint64_t)plan->grid_x * plan->grid_y;
   const uint64_t slots = (uint64_t)cus * std::min(per_cu, 4u);
   const bool skinny = std::min(g.M, g.N) <= 64;
-  const uint64_t kbytes = (uint64_t)g.K * ((g.a_type == CUDA_R_16F || g.a_type == CUDA_R_16BF) ? 2 : 1);
+  const uint64_t kbytes = (uint64_t)g.K * type_bits(g.a_type) / 8;
   if (tiles * 2 <= (skinny ? slots : (uint64_t)cus) && kbytes >= 1024 && (uint64_t)ceil_div(np, v.bp) * v.bp <= (1u << 20)) {
     uint32_t s = (uint32_t)std::min<uint64_t>({8, slots / tiles, kbytes / 512});
     const uint64_t per_split = (uint64_t)g.batch * ceil_div(np, v.bp) * v.bp * ceil_div(nq, v.bq) * v.bq * 4;
@@ -536,10 +538,10 @@ extern "C" uint32_t zluda_gemm_variant_count(uint32_t kernel) {
   switch (kernel) {
   case ZLUDA_KERNEL_GENERIC: return 1;
   case ZLUDA_KERNEL_MFMA_I8: case ZLUDA_KERNEL_MFMA_F8: return kNumMfmaVariants;
-  case ZLUDA_KERNEL_MFMA_MXF4: case ZLUDA_KERNEL_MFMA_H16: return kNumMfmaVariants32;  // the 16x16-shape ones serve int8 and fp8
+  case ZLUDA_KERNEL_MFMA_MXF4: case ZLUDA_KERNEL_MFMA_H16: case ZLUDA_KERNEL_MFMA_F32: return kNumMfmaVariants32;  // the 16x16-shape ones serve int8 and fp8
   case ZLUDA_KERNEL_DECODE_W8A8: return kNumDecodeVariants;
   case ZLUDA_KERNEL_MFMA_TR8: return kNumTrVariants;
-  case ZLUDA_KERNEL_MFMA_TR16: return kNumTrVariants - 1;  // the 16x16-shape one is an int8 instantiation
+  case ZLUDA_KERNEL_MFMA_TR16: case ZLUDA_KERNEL_MFMA_TR32: return kNumTrVariants - 1;  // the 16x16-shape one is an int8 instantiation
   default: return 0;
   }
 }
@@ -558,7 +560,7 @@ extern "C" uint32_t zluda_gemm_plan_problem(const zluda_gemm_problem *p, uint32_
   if (kernel == ZLUDA_KERNEL_AUTO) {
     static const uint32_t order[] = {ZLUDA_KERNEL_DECODE_W8A8, ZLUDA_KERNEL_MFMA_I8, ZLUDA_KERNEL_MFMA_F8,
                                      ZLUDA_KERNEL_MFMA_MXF4, ZLUDA_KERNEL_MFMA_H16, ZLUDA_KERNEL_MFMA_TR8,
-                                     ZLUDA_KERNEL_MFMA_TR16, ZLUDA_KERNEL_GENERIC};
+                                     ZLUDA_KERNEL_MFMA_TR16, ZLUDA_KERNEL_MFMA_F32, ZLUDA_KERNEL_MFMA_TR32, ZLUDA_KERNEL_GENERIC};
     for (uint32_t k : order) {
       if (!family_supports(k, l)) continue;
       if (k == ZLUDA_KERNEL_DECODE_W8A8) {
@@ -595,14 +597,15 @@ extern "C" uint32_t zluda_gemm_plan_problem(const zluda_gemm_problem *p, uint32_
     plan->waves = (float)plan->grid_x * plan->grid_y * plan->grid_z / (float)(cu_count * 8);
     if (plan->grid_y > 65535) return CUBLAS_STATUS_NOT_SUPPORTED;
     break;
-  case ZLUDA_KERNEL_MFMA_I8: case ZLUDA_KERNEL_MFMA_F8: case ZLUDA_KERNEL_MFMA_MXF4: case ZLUDA_KERNEL_MFMA_H16: {
+  case ZLUDA_KERNEL_MFMA_I8: case ZLUDA_KERNEL_MFMA_F8: case ZLUDA_KERNEL_MFMA_MXF4: case ZLUDA_KERNEL_MFMA_H16:
+  case ZLUDA_KERNEL_MFMA_F32: {
     int v = forced_variant >= 0 ? forced_variant : pick_mfma_variant(l, cu_count);
-    if (v >= kNumMfmaVariants || (kMfmaVariants[v].m16 && (kernel == ZLUDA_KERNEL_MFMA_MXF4 || kernel == ZLUDA_KERNEL_MFMA_H16)))
+    if (v >= kNumMfmaVariants || (kMfmaVariants[v].m16 && kernel != ZLUDA_KERNEL_MFMA_I8 && kernel != ZLUDA_KERNEL_MFMA_F8))
       return CUBLAS_STATUS_INVALID_VALUE;
     fill_mfma_plan(l, v, cu_count, p->workspace_size, plan);
     break;
   }
-  case ZLUDA_KERNEL_MFMA_TR8: case ZLUDA_KERNEL_MFMA_TR16: {
+  case ZLUDA_KERNEL_MFMA_TR8: case ZLUDA_KERNEL_MFMA_TR16: case ZLUDA_KERNEL_MFMA_TR32: {
     int v = forced_variant >= 0 ? forced_variant : pick_tr_variant(l, cu_count);
     if (v >= kNumTrVariants || (kTrVariants[v].m16 && l.g.a_type != CUDA_R_8I)) return CUBLAS_STATUS_INVALID_VALUE;
     fill_tr_plan(l, v, cu_count, p->workspace_size, plan);
