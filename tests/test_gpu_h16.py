@@ -121,6 +121,16 @@ def test_16_bit_weights_stream_through_the_slab_decode(gpu_api, typ, shape):
     case.compare(got, theirs, tol=1e-2, floor_frac=1e-2)
 
 
+def test_16_bit_slab_decode_on_more_workgroups_than_cus(gpu_api):
+    """long K keeps the slab form beyond 64 rows per CU: 320 workgroups, the later ones following another on their CU"""
+    case = Case(base("bf16", m=20480, n=16, k=8192), 8050)
+    ref = case.run_oracle()
+    for rep in range(2):
+        st, got, kernel, v = case.run_gpu(gpu_api)
+        assert st == 0 and (kernel, v) == (K.ZLUDA_KERNEL_DECODE_W8A8, 19)
+        case.compare(got, ref, tol=1e-2)
+
+
 @pytest.mark.parametrize("typ", ["bf16", "f16"])
 def test_16_bit_split_k_through_the_workspace(gpu_api, typ):
     spec = base(typ, m=512, n=256, k=8192, epilogue=K.CUBLASLT_EPILOGUE_BIAS)
