@@ -1,7 +1,7 @@
 """Seeded random sweep on the GPU: problems drawn over every family of the library (int8 with integer and with
 float scaling, fp8 in its three operand mixes, MXFP4, 16/32-bit floats), transposes, orders, padded and
 unaligned leading dimensions, batches, pointer modes, scale modes, every epilogue incl. the bias gradients,
-decode-like and split-K-like shapes, with and without a workspace -- each through the planner's choice and
+decode-like and split-K-like shapes, grids of several rounds of workgroups, with and without a workspace -- each through the planner's choice and
 then through up to three other tile variants of the family it chose, all against the CPU oracle.  The draw
 is deterministic (fixed seed), so a failure names a case that can be rerun."""
 import json
@@ -37,6 +37,8 @@ def dims():
         return pick([256, 320, 512, 640]), pick([256, 384, 512]), pick([256, 512, 768, 1024])
     if r < 0.75 and BIG:
         return int(RNG.integers(200, 1500)), int(RNG.integers(200, 1500)), int(RNG.integers(64, 1200))
+    if r < 0.81 and BIG:   # more workgroups than CUs for most tile shapes: later workgroups follow another one on their CU
+        return int(RNG.integers(2000, 5000)), int(RNG.integers(1500, 4500)), int(RNG.integers(32, 420))
     return int(RNG.integers(1, 400)), int(RNG.integers(1, 400)), int(RNG.integers(1, 700))
 
 
