@@ -50,12 +50,11 @@ def test_16_bit_operands_take_the_mfma_family_when_k_contiguous(api):
     for t in (K.CUDA_R_16BF, K.CUDA_R_16F):
         H = dict(a_type=t, b_type=t, d_type=t, compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F)
         st, p = plan(api, dict(H, m=8192, n=8192, k=8192, transa=1))
-        assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_H16 and p.variant == 0 and p.grid_x == 1024 and p.block == 512
+        assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_H16 and p.variant == 8 and p.grid_x == 1024 and p.block == 512   # on the 16x16 MFMA shape
         st, p = plan(api, dict(H, m=2048, n=2048, k=2048, transa=1))
         assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_H16 and p.variant in (3, 4) and p.grid_x == 256
-        # the 16x16 MFMA shapes are int8 / fp8 instantiations
-        assert plan(api, dict(H, m=8192, n=8192, k=8192, transa=1), forced=K.ZLUDA_KERNEL_MFMA_H16, variant=8)[0] == K.CUBLAS_STATUS_INVALID_VALUE
-        assert api.zluda_gemm_variant_count(K.ZLUDA_KERNEL_MFMA_H16) == 8
+        assert plan(api, dict(H, m=6144, n=6144, k=6144, transa=1))[1].variant == 9
+        assert api.zluda_gemm_variant_count(K.ZLUDA_KERNEL_MFMA_H16) == 10
         # K in bytes decides the split: 4096 elements of 16 bits are 8 KiB per row
         st, p = plan(api, dict(H, m=512, n=256, k=4096, transa=1), workspace=64 << 20)
         assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_H16 and p.grid_z > 1

@@ -230,7 +230,8 @@ __device__ __forceinline__ void mfma16_store_tile(const MfmaParams &prm, AccV (&
 // ---- the kernel ----------------------------------------------------------------------------------------
 template <int KIND, int FQ, int FP, int BP, int BQ, int WP, int WQ>
 __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe16_kernel(MfmaParams prm) {
-  static_assert(KIND == KIND_I8 || KIND == KIND_F8, "int8 and fp8 operands");
+  static_assert(KIND == KIND_I8 || KIND == KIND_F8 || kind_is_h16(KIND), "int8, fp8, f16 and bf16 operands");
+  constexpr int ESZ = kind_esz(KIND);          // f16 / bf16: the byte geometry of int8 (v_mfma_f32_16x16x32_*: 16 bytes of K per lane)
   constexpr int NT = WP * WQ * 64, NWV = NT / 64;
   constexpr int BKB = 128, CPR = 8, RPW = 8;
   constexpr int RPP = NWV * RPW;               // rows filled per DMA pass of the workgroup
@@ -245,7 +246,7 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe16_kernel(MfmaParam
   static_assert(WTP % 32 == 0 && WTQ % 32 == 0, "wave tiles start on multiples of 32 rows (fragment swizzle)");
   static_assert(NSTAGE * STAGE_V4 * 16 <= 160 * 1024, "LDS capacity");
   using acc_v = typename std::conditional<KIND == KIND_I8, v4i, v4f>::type;
-  using frag_v = typename std::conditional<KIND == KIND_I8, v4i, v8i>::type;
+  using frag_v = typename std::conditional<KIND != KIND_F8, v4i, v8i>::type;
   struct Frag { frag_v k[KS]; };
 
   __shared__ v4i lds[NSTAGE * STAGE_V4];
@@ -267,15 +268,15 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe16_kernel(MfmaParam
   const int p0 = tile_p * BP, q0 = tile_q * BQ;
 
   const int NP = prm.swapped ? g.N : g.M, NQ = prm.swapped ? g.M : g.N;
-  const int Kbytes = g.K;
+  const int Kbytes = g.K * ESZ;
   const uint8_t *Pg, *Qg;
   int ldp, ldq;
   if (!prm.swapped) {
-    Pg = (const uint8_t *)g.A + g.a_sb * bt; ldp = (int)g.a_si;
-    Qg = (const uint8_t *)g.B + g.b_sb * bt; ldq = (int)g.b_sj;
+    Pg = (const uint8_t *)g.A + g.a_sb * bt * ESZ; ldp = (int)g.a_si * ESZ;
+    Qg = (const uint8_t *)g.B + g.b_sb * bt * ESZ; ldq = (int)g.b_sj * ESZ;
   } else {
-    Pg = (const uint8_t *)g.B + g.b_sb * bt; ldp = (int)g.b_sj;
-    Qg = (const uint8_t *)g.A + g.a_sb * bt; ldq = (int)g.a_si;
+    Pg = (const uint8_t *)g.B + g.b_sb * bt * ESZ; ldp = (int)g.b_sj * ESZ;
+    Qg = (const uint8_t *)g.A + g.a_sb * bt * ESZ; ldq = (int)g.a_si * ESZ;
   }
   // split-K: this workgroup's share of the stages starts k0 bytes into every row
   int Kbytes_local = Kbytes, k0 = 0;
@@ -384,6 +385,10 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe16_kernel(MfmaParam
           const int i = x / HQ, j = x % HQ;
           acc_v &c = acc[ph * HP + i][qh * HQ + j];
           if constexpr (KIND == KIND_I8) c = __builtin_amdgcn_mfma_i32_16x16x64_i8(pf[ph][i].k[ks], qf[qh][j].k[ks], c, 0, 0, 0);
+          else if constexpr (KIND == KIND_F16)
+            c = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, pf[ph][i].k[ks]), __builtin_bit_cast(v8h, qf[qh][j].k[ks]), c, 0, 0, 0);
+          else if constexpr (KIND == KIND_BF16)
+            c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8b, pf[ph][i].k[ks]), __builtin_bit_cast(v8b, qf[qh][j].k[ks]), c, 0, 0, 0);
           else c = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(pf[ph][i].k[ks], qf[qh][j].k[ks], c, FP, FQ, 0, 0, 0, 0);
         }
   };

@@ -30,11 +30,11 @@ inline uint32_t launch_mfma_variant(const MfmaParams &prm, const zluda_gemm_plan
     ZLUDA_MFMA_CASE(6, 64, 64, 2, 2, 128, 3)
     ZLUDA_MFMA_CASE(7, 192, 256, 2, 4, 128, 2)
 #define ZLUDA_MFMA16_CASE(V, BP, BQ, WP, WQ)                                                                \
-  case V:  /* the 16x16 MFMA shapes: int8 and fp8 only */                                                  \
+  case V:  /* the 16x16 MFMA shapes: int8, fp8, f16, bf16 */                                               \
     static_assert(kMfmaVariants[V].bp == BP && kMfmaVariants[V].bq == BQ && kMfmaVariants[V].wp == WP &&   \
                   kMfmaVariants[V].wq == WQ && kMfmaVariants[V].bkb == 128 && kMfmaVariants[V].stages == 2 && \
                   kMfmaVariants[V].m16, "variant table mismatch");                                         \
-    if constexpr (KIND != KIND_I8 && KIND != KIND_F8) return CUBLAS_STATUS_INVALID_VALUE;                                   \
+    if constexpr (KIND != KIND_I8 && KIND != KIND_F8 && !kind_is_h16(KIND)) return CUBLAS_STATUS_INVALID_VALUE;                                   \
     else return launch_kernel(gemm_mfma_pipe16_kernel<KIND, FQ, FP, BP, BQ, WP, WQ>, grid, dim3(WP * WQ * 64), s, prm);
     ZLUDA_MFMA16_CASE(8, 256, 256, 2, 4)
     ZLUDA_MFMA16_CASE(9, 192, 256, 2, 4)

@@ -401,11 +401,13 @@ static int pick_mfma_variant(const Lowered &l, uint32_t cus) {
     const MfmaVariant &t = kMfmaVariants[v];
     const uint64_t tiles = (uint64_t)ceil_div(np, t.bp) * ceil_div(nq, t.bq) * g.batch;
     if (t.m16) {
-      if (type_bits(g.a_type) != 8) continue;  // the 16x16 shapes serve int8 and fp8
+      const bool h16 = g.a_type == CUDA_R_16F || g.a_type == CUDA_R_16BF;
+      if (type_bits(g.a_type) != 8 && !h16) continue;  // the 16x16 shapes serve int8, fp8, f16 and bf16
       // power bound or not: int8 gains from three quarters of the CUs busy on.  fp8 gains little and only on
       // long runs: the 192x256 tile from two full rounds on (6144^3: 190 us against 198), the 256x256 tile
       // from four (8192^3: 405 against 408; at two rounds, 8192x4096x4096, it loses 3 %)
-      const uint64_t need = g.a_type == CUDA_R_8I ? ((uint64_t)cus * 3 + 3) / 4 : (uint64_t)cus * (t.bp == 256 ? 4 : 2);
+      // (f16 / bf16 as int8: bf16 8192^3 776 us against 840, 4096^3 102 against 108, 6144^3 336 against 360)
+      const uint64_t need = (g.a_type == CUDA_R_8I || h16) ? ((uint64_t)cus * 3 + 3) / 4 : (uint64_t)cus * (t.bp == 256 ? 4 : 2);
       if (tiles < need) continue;
     }
     const uint64_t rounds = (tiles + cus - 1) / cus;
@@ -537,8 +539,8 @@ using namespace zluda_amd;
 extern "C" uint32_t zluda_gemm_variant_count(uint32_t kernel) {
   switch (kernel) {
   case ZLUDA_KERNEL_GENERIC: return 1;
-  case ZLUDA_KERNEL_MFMA_I8: case ZLUDA_KERNEL_MFMA_F8: return kNumMfmaVariants;
-  case ZLUDA_KERNEL_MFMA_MXF4: case ZLUDA_KERNEL_MFMA_H16: case ZLUDA_KERNEL_MFMA_F32: return kNumMfmaVariants32;  // the 16x16-shape ones serve int8 and fp8
+  case ZLUDA_KERNEL_MFMA_I8: case ZLUDA_KERNEL_MFMA_F8: case ZLUDA_KERNEL_MFMA_H16: return kNumMfmaVariants;
+  case ZLUDA_KERNEL_MFMA_MXF4: case ZLUDA_KERNEL_MFMA_F32: return kNumMfmaVariants32;  // the 16x16-shape ones serve int8 and fp8
   case ZLUDA_KERNEL_DECODE_W8A8: return kNumDecodeVariants;
   case ZLUDA_KERNEL_MFMA_TR8: return kNumTrVariants;
   case ZLUDA_KERNEL_MFMA_TR16: case ZLUDA_KERNEL_MFMA_TR32: return kNumTrVariants - 1;  // the 16x16-shape one is an int8 instantiation
@@ -600,7 +602,8 @@ extern "C" uint32_t zluda_gemm_plan_problem(const zluda_gemm_problem *p, uint32_
   case ZLUDA_KERNEL_MFMA_I8: case ZLUDA_KERNEL_MFMA_F8: case ZLUDA_KERNEL_MFMA_MXF4: case ZLUDA_KERNEL_MFMA_H16:
   case ZLUDA_KERNEL_MFMA_F32: {
     int v = forced_variant >= 0 ? forced_variant : pick_mfma_variant(l, cu_count);
-    if (v >= kNumMfmaVariants || (kMfmaVariants[v].m16 && kernel != ZLUDA_KERNEL_MFMA_I8 && kernel != ZLUDA_KERNEL_MFMA_F8))
+    if (v >= kNumMfmaVariants || (kMfmaVariants[v].m16 && kernel != ZLUDA_KERNEL_MFMA_I8 && kernel != ZLUDA_KERNEL_MFMA_F8 &&
+                                  kernel != ZLUDA_KERNEL_MFMA_H16))
       return CUBLAS_STATUS_INVALID_VALUE;
     fill_mfma_plan(l, v, cu_count, p->workspace_size, plan);
     break;

@@ -8,7 +8,7 @@ namespace zluda_amd {
 
 // MFMA tile configurations (index = plan.variant for the MFMA families): workgroup tile bp x bq,
 // wp x wq waves, `bkb` bytes of K per LDS stage, `stages` LDS stages
-struct MfmaVariant { int bp, bq, wp, wq, bkb, stages, m16; };  // m16: the 16x16 MFMA shapes (gemm_mfma_pipe16.hpp; int8 and fp8)
+struct MfmaVariant { int bp, bq, wp, wq, bkb, stages, m16; };  // m16: the 16x16 MFMA shapes (gemm_mfma_pipe16.hpp; not MXFP4, not f32)
 constexpr MfmaVariant kMfmaVariants[] = {
     {256, 256, 2, 4, 128, 2, 0},  // 0: 8 waves, 128x64 per wave
     {256, 256, 2, 2, 128, 2, 0},  // 1: 4 waves, 128x128 per wave
@@ -18,7 +18,7 @@ constexpr MfmaVariant kMfmaVariants[] = {
     {128, 64, 2, 2, 128, 3, 0},   // 5: 4 waves, 64x32 per wave: skinny problems
     {64, 64, 2, 2, 128, 3, 0},    // 6: 4 waves, 32x32 per wave: problems of a few hundred tiles at most
     {192, 256, 2, 4, 128, 2, 0},  // 7: 8 waves, 96x64 per wave: extents that 256 divides badly (3072, 6144, ...)
-    // the same tiles on v_mfma_*_16x16x* (int8 and fp8): less energy per multiply-add, and GEMMs that keep the
+    // the same tiles on v_mfma_*_16x16x* (int8, fp8, f16, bf16): less energy per multiply-add, and GEMMs that keep the
     // chip busy are power bound
     {256, 256, 2, 4, 128, 2, 1},  // 8: variant 0's
     {192, 256, 2, 4, 128, 2, 1},  // 9: variant 7's
