@@ -165,7 +165,7 @@ struct TrOperand {
   }
 };
 
-// M16 (int8 only): the MFMAs are v_mfma_i32_16x16x64_i8 with P as operand "A" and the epilogues of
+// M16 (int8, f16, bf16): the MFMAs are v_mfma_i32_16x16x64_i8 / v_mfma_f32_16x16x32_f16 / _bf16 with P as operand "A" and the epilogues of
 // gemm_mfma_pipe16.hpp -- the shape that needs less energy per multiply-add, for problems that keep the whole
 // chip busy (see there).  A fragment is then 16 rows x the 64 K bytes of a stage (lane l: row l%16, 16-byte
 // chunk l/16), one MFMA per pair of fragments and stage.
@@ -175,7 +175,8 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_tr_kernel(MfmaParams pr
   constexpr int ESZ = kind_esz(KIND);
   constexpr int MPS = KIND == KIND_F32 ? 4 : 1;  // MFMAs per fragment pair and sub-step
   constexpr bool B16 = KIND != KIND_F8;  // 16 bytes of K per lane and MFMA (fp8: 32)
-  static_assert(!M16 || KIND == KIND_I8, "the 16x16 form is instantiated for int8");
+  static_assert(!M16 || KIND == KIND_I8 || kind_is_h16(KIND), "the 16x16 form is instantiated for int8, f16 and bf16");
+  using acc16_v = typename std::conditional<KIND == KIND_I8, v4i, v4f>::type;
   constexpr int NT = WP * WQ * 64;
   static_assert(NT == 256 || NT == 512, "operand rows are dealt to groups of 256 threads");
   constexpr int LP = BP * 256 / NT, LQ = BQ * 256 / NT;  // rows of P / Q one group loads
@@ -262,7 +263,7 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_tr_kernel(MfmaParams pr
   }
   // ---- the 16x16 form ------------------------------------------------------------------------------
   constexpr int TP16 = WTP / 16, TQ16 = WTQ / 16, HP16 = TP16 / 2;
-  v4i acc16[M16 ? TP16 : 1][M16 ? TQ16 : 1];
+  acc16_v acc16[M16 ? TP16 : 1][M16 ? TQ16 : 1];
   int prow16[M16 ? TP16 : 1], qrow16[M16 ? TQ16 : 1];  // this lane's 16-byte piece of each fragment (v4i units)
   if constexpr (M16) {
     const int r16 = lane & 15, g4 = lane >> 4;
@@ -279,7 +280,7 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_tr_kernel(MfmaParams pr
 #pragma unroll
     for (int b = 0; b < TP16; b++)
 #pragma unroll
-      for (int a = 0; a < TQ16; a++) acc16[b][a] = v4i{0, 0, 0, 0};
+      for (int a = 0; a < TQ16; a++) acc16[b][a] = acc16_v{0, 0, 0, 0};
   }
   // fragment registers: both halves of P (the second is read while the first is multiplied) and the Q
   // fragments of two stages (the next stage's arrive while this stage's are still in use)
@@ -300,7 +301,15 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_tr_kernel(MfmaParams pr
     for (int i = 0; i < HP16; i++)
 #pragma unroll
       for (int a = 0; a < TQ16; a++)
-        acc16[h * HP16 + i][a] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fp16[h][i], fq16[sidx][a], acc16[h * HP16 + i][a], 0, 0, 0);
+      {
+        acc16_v &c = acc16[h * HP16 + i][a];
+        if constexpr (KIND == KIND_F16)
+          c = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, fp16[h][i]), __builtin_bit_cast(v8h, fq16[sidx][a]), c, 0, 0, 0);
+        else if constexpr (KIND == KIND_BF16)
+          c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8b, fp16[h][i]), __builtin_bit_cast(v8b, fq16[sidx][a]), c, 0, 0, 0);
+        else if constexpr (KIND == KIND_I8)
+          c = __builtin_amdgcn_mfma_i32_16x16x64_i8(fp16[h][i], fq16[sidx][a], c, 0, 0, 0);
+      }
   };
 
   // fragments of sub-step ks of the stage in `buf`

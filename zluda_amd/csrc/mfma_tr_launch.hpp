@@ -28,10 +28,10 @@ inline uint32_t launch_tr_variant(const MfmaParams &prm, const zluda_gemm_plan &
     ZLUDA_TR_CASE(0, 256, 256, 2, 4)
     ZLUDA_TR_CASE(1, 128, 128, 2, 2)
     ZLUDA_TR_CASE(2, 64, 64, 2, 2)
-  case 3:  // variant 0's tile on the 16x16 MFMA shape (int8)
+  case 3:  // variant 0's tile on the 16x16 MFMA shape (int8, f16, bf16)
     static_assert(kTrVariants[3].bp == 256 && kTrVariants[3].bq == 256 && kTrVariants[3].wp == 2 && kTrVariants[3].wq == 4 &&
                   kTrVariants[3].m16, "variant table mismatch");
-    if constexpr (KIND == KIND_I8) {
+    if constexpr (KIND == KIND_I8 || kind_is_h16(KIND)) {
 #define ZLUDA_TR16_MODE(PK, QK)                                                                                  \
   if (pkc == PK && qkc == QK)                                                                                    \
     return launch_kernel(gemm_mfma_tr_kernel<KIND, FQ, FP, 256, 256, 2, 4, PK, QK, true>, grid, dim3(512), s, prm);

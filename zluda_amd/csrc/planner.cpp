@@ -467,8 +467,9 @@ static int pick_tr_variant(const Lowered &l, uint32_t cus) {
     const TrVariant &t = kTrVariants[v];
     const TrCost &c = kTrCost[v];
     const uint64_t tiles = (uint64_t)ceil_div(np, t.bp) * ceil_div(nq, t.bq) * g.batch;
-    // the 16x16 shape: int8 only, and only where the chip is full enough to sit at its power cap
-    if (t.m16 && (g.a_type != CUDA_R_8I || tiles * 4 < (uint64_t)cus * 3)) continue;
+    // the 16x16 shape: int8, f16 and bf16, and only where the chip is full enough to sit at its power cap
+    const bool m16_type = g.a_type == CUDA_R_8I || g.a_type == CUDA_R_16F || g.a_type == CUDA_R_16BF;
+    if (t.m16 && (!m16_type || tiles * 4 < (uint64_t)cus * 3)) continue;
     const uint64_t slots = (uint64_t)cus * c.per_cu;
     const uint64_t full = tiles / slots, rem = tiles % slots;
     double cost = (double)full * (c.base + c.slope * c.per_cu);
@@ -542,8 +543,8 @@ extern "C" uint32_t zluda_gemm_variant_count(uint32_t kernel) {
   case ZLUDA_KERNEL_MFMA_I8: case ZLUDA_KERNEL_MFMA_F8: case ZLUDA_KERNEL_MFMA_H16: return kNumMfmaVariants;
   case ZLUDA_KERNEL_MFMA_MXF4: case ZLUDA_KERNEL_MFMA_F32: return kNumMfmaVariants32;  // the 16x16-shape ones serve int8 and fp8
   case ZLUDA_KERNEL_DECODE_W8A8: return kNumDecodeVariants;
-  case ZLUDA_KERNEL_MFMA_TR8: return kNumTrVariants;
-  case ZLUDA_KERNEL_MFMA_TR16: case ZLUDA_KERNEL_MFMA_TR32: return kNumTrVariants - 1;  // the 16x16-shape one is an int8 instantiation
+  case ZLUDA_KERNEL_MFMA_TR8: case ZLUDA_KERNEL_MFMA_TR16: return kNumTrVariants;
+  case ZLUDA_KERNEL_MFMA_TR32: return kNumTrVariants - 1;  // the 16x16-shape one is not instantiated for f32
   default: return 0;
   }
 }
@@ -610,7 +611,8 @@ extern "C" uint32_t zluda_gemm_plan_problem(const zluda_gemm_problem *p, uint32_
   }
   case ZLUDA_KERNEL_MFMA_TR8: case ZLUDA_KERNEL_MFMA_TR16: case ZLUDA_KERNEL_MFMA_TR32: {
     int v = forced_variant >= 0 ? forced_variant : pick_tr_variant(l, cu_count);
-    if (v >= kNumTrVariants || (kTrVariants[v].m16 && l.g.a_type != CUDA_R_8I)) return CUBLAS_STATUS_INVALID_VALUE;
+    if (v >= kNumTrVariants || (kTrVariants[v].m16 && l.g.a_type != CUDA_R_8I && l.g.a_type != CUDA_R_16F && l.g.a_type != CUDA_R_16BF))
+      return CUBLAS_STATUS_INVALID_VALUE;
     fill_tr_plan(l, v, cu_count, p->workspace_size, plan);
     break;
   }

@@ -28,12 +28,12 @@ constexpr int kNumMfmaVariants = sizeof(kMfmaVariants) / sizeof(kMfmaVariants[0]
 
 // tile configurations of the transposing 8-bit MFMA kernel (index = plan.variant for
 // ZLUDA_KERNEL_MFMA_TR8): workgroup tile bp x bq, wp x wq waves, always 64 K bytes per stage
-struct TrVariant { int bp, bq, wp, wq, m16; };  // m16: int8 on v_mfma_i32_16x16x64_i8 (as the variants 8 .. above)
+struct TrVariant { int bp, bq, wp, wq, m16; };  // m16: int8 / f16 / bf16 on the 16x16 MFMA shapes (as the variants 8 .. above)
 constexpr TrVariant kTrVariants[] = {
     {256, 256, 2, 4, 0},  // 0: 8 waves, 128x64 per wave, one workgroup per CU
     {128, 128, 2, 2, 0},  // 1: 4 waves, 64x64 per wave, two workgroups per CU
     {64, 64, 2, 2, 0},    // 2: 4 waves, 32x32 per wave, four or more per CU: small and skinny problems
-    {256, 256, 2, 4, 1},  // 3: variant 0 on the 16x16 MFMA shape, int8 only: grids that fill the chip
+    {256, 256, 2, 4, 1},  // 3: variant 0 on the 16x16 MFMA shape, int8 / f16 / bf16: grids that fill the chip
 };
 constexpr int kNumTrVariants = sizeof(kTrVariants) / sizeof(kTrVariants[0]);
 
