@@ -54,7 +54,7 @@ def test_16_bit_operands_take_the_mfma_family_when_k_contiguous(api):
         st, p = plan(api, dict(H, m=2048, n=2048, k=2048, transa=1))
         assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_H16 and p.variant in (3, 4) and p.grid_x == 256
         assert plan(api, dict(H, m=6144, n=6144, k=6144, transa=1))[1].variant == 9
-        assert api.zluda_gemm_variant_count(K.ZLUDA_KERNEL_MFMA_H16) == 10
+        assert api.zluda_gemm_variant_count(K.ZLUDA_KERNEL_MFMA_H16) == 11
         # K in bytes decides the split: 4096 elements of 16 bits are 8 KiB per row
         st, p = plan(api, dict(H, m=512, n=256, k=4096, transa=1), workspace=64 << 20)
         assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_H16 and p.grid_z > 1
@@ -116,6 +116,19 @@ def test_16_bit_weights_with_few_tokens_take_the_slab_decode(api):
             assert plan(api, dict(H, m=14336, n=16, k=2048), forced=K.ZLUDA_KERNEL_DECODE_W8A8, variant=v)[0] == K.CUBLAS_STATUS_NOT_SUPPORTED
 
 
+def test_skinny_problems_of_one_workgroup_per_cu_get_the_deep_ring(api):
+    st, p = plan(api, dict(I8, m=14336, n=64, k=4096, transa=1))
+    assert st == 0 and (p.kernel, p.variant, p.grid_x, p.grid_z) == (K.ZLUDA_KERNEL_MFMA_I8, 10, 224, 1)
+    st, p = plan(api, dict(I8, m=14336, n=64, k=4096, transa=1), cus=128)            # two workgroups per CU: the 3-stage ring, several per CU
+    assert st == 0 and p.variant != 10
+    st, p = plan(api, dict(I8, m=4096, n=64, k=4096, transa=1), workspace=64 << 20)  # split along K instead
+    assert st == 0 and p.variant == 6 and p.grid_z > 1
+    st, p = plan(api, dict(I8, m=4096, n=64, k=1024, transa=1))                      # a short K never fills the ring
+    assert st == 0 and p.variant == 6
+    st, p = plan(api, dict(MX, m=14336, n=64, k=8192, transa=1))                     # MXFP4 scale chunks span 4 stages
+    assert st == 0 and p.variant != 10
+
+
 def test_small_problems_get_smaller_tiles(api):
     st, p = plan(api, dict(I8, m=1024, n=1024, k=1024, transa=1))
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_I8 and p.variant == 6 and p.grid_x == 256
@@ -144,7 +157,7 @@ def test_extents_that_256_divides_badly_get_the_192_row_tile(api):
     st, p = plan(api, dict(MX, m=8192, n=8192, k=8192, transa=1))      # MXFP4 has no 16x16-shape variant
     assert st == 0 and p.variant == 0
     assert plan(api, dict(MX, m=8192, n=8192, k=8192, transa=1), forced=K.ZLUDA_KERNEL_MFMA_MXF4, variant=8)[0] == K.CUBLAS_STATUS_INVALID_VALUE
-    assert api.zluda_gemm_variant_count(K.ZLUDA_KERNEL_MFMA_I8) == 10 and api.zluda_gemm_variant_count(K.ZLUDA_KERNEL_MFMA_MXF4) == 8
+    assert api.zluda_gemm_variant_count(K.ZLUDA_KERNEL_MFMA_I8) == 11 and api.zluda_gemm_variant_count(K.ZLUDA_KERNEL_MFMA_MXF4) == 8
 
 
 def test_row_major_output_swaps_operands(api):
@@ -219,10 +232,11 @@ def test_fp4_must_be_k_contiguous(api):
 def test_forced_variants(api):
     spec = dict(I8, m=4096, n=4096, k=4096, transa=1)
     for v, (grid, block) in enumerate([(256, 512), (256, 256), (512, 256), (1024, 256), (1024, 256), (2048, 256), (4096, 256),
-                                       (352, 512), (256, 512), (352, 512)]):
+                                       (352, 512), (256, 512), (352, 512), (4096, 256)]):
         st, p = plan(api, spec, forced=K.ZLUDA_KERNEL_MFMA_I8, variant=v)
         assert st == 0 and p.variant == v and p.grid_x == grid and p.block == block
-    assert plan(api, spec, forced=K.ZLUDA_KERNEL_MFMA_I8, variant=10)[0] == K.CUBLAS_STATUS_INVALID_VALUE
+    assert plan(api, spec, forced=K.ZLUDA_KERNEL_MFMA_I8, variant=11)[0] == K.CUBLAS_STATUS_INVALID_VALUE
+    assert plan(api, dict(MX, m=4096, n=4096, k=4096, transa=1), forced=K.ZLUDA_KERNEL_MFMA_MXF4, variant=10)[0] == K.CUBLAS_STATUS_INVALID_VALUE
     assert plan(api, spec, forced=K.ZLUDA_KERNEL_MFMA_F8)[0] == K.CUBLAS_STATUS_NOT_SUPPORTED
 
 
@@ -325,8 +339,10 @@ def test_fp8_decode_takes_the_streaming_kernel_under_a_cover_only(api):
     f8 = dict(F8, transa=1)
     st, p = plan(api, dict(f8, m=14336, n=17, k=4096))
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.variant == 4 and p.grid_x == 256
-    st, p = plan(api, dict(f8, m=14336, n=48, k=4096))                      # up to 48 tokens while the variant applies
+    st, p = plan(api, dict(f8, m=8192, n=48, k=4096))                       # up to 48 tokens while the variant applies ...
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8
+    st, p = plan(api, dict(f8, m=14336, n=48, k=4096))                      # ... and the rows are at most 32 per CU
+    assert st == 0 and (p.kernel, p.variant, p.grid_x) == (K.ZLUDA_KERNEL_MFMA_F8, 10, 224)   # 64x64 tiles on the 6-stage ring
     st, p = plan(api, dict(f8, m=14336, n=49, k=4096))                      # beyond: MFMA tiles
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_F8
     st, p = plan(api, dict(f8, m=14336, n=33, k=8192))                      # 3 token blocks x 16 steps: too many fragments

@@ -39,6 +39,11 @@ inline uint32_t launch_mfma_variant(const MfmaParams &prm, const zluda_gemm_plan
     ZLUDA_MFMA16_CASE(8, 256, 256, 2, 4)
     ZLUDA_MFMA16_CASE(9, 192, 256, 2, 4)
 #undef ZLUDA_MFMA16_CASE
+  case 10:
+    static_assert(kMfmaVariants[10].bp == 64 && kMfmaVariants[10].bq == 64 && kMfmaVariants[10].wp == 2 && kMfmaVariants[10].wq == 2 &&
+                  kMfmaVariants[10].bkb == 128 && kMfmaVariants[10].stages == 6 && !kMfmaVariants[10].m16, "variant table mismatch");
+    if constexpr (KIND == KIND_MXF4) return CUBLAS_STATUS_INVALID_VALUE;
+    else return launch_kernel(gemm_mfma_pipe_kernel<KIND, FQ, FP, 64, 64, 2, 2, 128, 6>, grid, dim3(256), s, prm);
   default: return CUBLAS_STATUS_INVALID_VALUE;
   }
 #undef ZLUDA_MFMA_CASE

@@ -22,6 +22,9 @@ constexpr MfmaVariant kMfmaVariants[] = {
     // chip busy are power bound
     {256, 256, 2, 4, 128, 2, 1},  // 8: variant 0's
     {192, 256, 2, 4, 128, 2, 1},  // 9: variant 7's
+    // skinny, memory-bound problems of at most one workgroup per CU: variant 6's tile with a ring of 6 stages, i.e. 80 KiB
+    // instead of 32 KiB of operand rows in flight per CU (not MXFP4: its scale chunks span 4 stages)
+    {64, 64, 2, 2, 128, 6, 0},    // 10
 };
 constexpr int kNumMfmaVariants32 = 8;  // the first ones, on the 32x32 shapes: what MXFP4 has
 constexpr int kNumMfmaVariants = sizeof(kMfmaVariants) / sizeof(kMfmaVariants[0]);
