@@ -76,7 +76,8 @@ enum {
   ZLUDA_KERNEL_MFMA_I8 = 2,   /* v_mfma_i32_32x32x32_i8, K-contiguous A and B */
   ZLUDA_KERNEL_MFMA_F8 = 3,   /* v_mfma_f32_32x32x64_f8f6f4 (e4m3/e5m2) */
   ZLUDA_KERNEL_MFMA_MXF4 = 4, /* v_mfma_scale_f32_32x32x64_f8f6f4, E2M1 + UE8M0/32 */
-  ZLUDA_KERNEL_DECODE_W8A8 = 5, /* skinny (<= 64 tokens) int8 / fp8 e4m3 streaming kernel, K split inside the workgroup */
+  ZLUDA_KERNEL_DECODE_W8A8 = 5, /* skinny (<= 64 tokens) int8 / fp8 e4m3 streaming kernel, K split inside the workgroup
+                                   (its slab form also streams f16 / bf16 weights) */
   ZLUDA_KERNEL_MFMA_TR8 = 6,  /* int8 / fp8 MFMA with transposing loads: A or B not K-contiguous */
   ZLUDA_KERNEL_MFMA_H16 = 7,  /* v_mfma_f32_32x32x16_f16 / _bf16, K-contiguous A and B of one 16-bit type */
   ZLUDA_KERNEL_MFMA_TR16 = 8, /* f16 / bf16 MFMA with transposing loads: A or B not K-contiguous */
