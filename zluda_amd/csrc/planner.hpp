@@ -80,7 +80,8 @@ constexpr int kDecodeMaxTokens = 64;      // what the family can run
 constexpr int kDecodeAutoMaxTokens = 32;  // what the planner gives it whatever the variant ...
 constexpr int kDecodeAutoMaxTokensStream = 48;  // ... and when the LDS-streaming variant applies: 3 token blocks still beat
                                                 // 64-wide MFMA tiles (6144x48x4096 fp8: 13 us against 16), 4 blocks do not
-                                                // (14336x56x4096: 21 us against 19)
+                                                // (14336x56x4096: 21 us against 19); three blocks only up to 32 rows per CU
+                                                // (planner.cpp: beyond, the 6-stage 64 x 64 tiles are as fast or faster)
 
 struct Lowered {
   GemmArgs g;
