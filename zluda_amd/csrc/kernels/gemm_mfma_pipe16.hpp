@@ -57,7 +57,11 @@ __device__ __forceinline__ void mfma16_store_raw(__amdgpu_buffer_rsrc_t rs, int 
 // 16-byte stores).  The activation and the 16-bit format are workgroup-uniform branches per 16 x 16 tile
 // (one instantiation serves them all: the 64 tiles of a wave are unrolled, so every further template
 // argument multiplies a large body).
-template <int KIND, int WP, int WQ, int TP, int TQ, bool WIDE, class AccV>
+// FENCE: the scheduler may not move instructions from one row of 16 x 16 tiles to the next (a wave that holds more
+// than the accumulators across the epilogue has no registers for what the scheduler would otherwise hoist).
+// ACT_T / BF16_T >= 0 fix the activation / the 16-bit format at compile time (no branch per tile: a wave that has its
+// SIMD to itself cannot hide them behind another wave's work).
+template <int KIND, int WP, int WQ, int TP, int TQ, bool WIDE, bool FENCE = false, int ACT_T = -1, int BF16_T = -1, class AccV>
 __device__ __forceinline__ void mfma16_store_f(const MfmaParams &prm, AccV (&acc)[TP][TQ], int p0, int q0, int NP, int NQ, int bt) {
   constexpr int WTP = TP * 16, WTQ = TQ * 16;
   constexpr int ESZ = WIDE ? 4 : 2;
@@ -66,6 +70,8 @@ __device__ __forceinline__ void mfma16_store_f(const MfmaParams &prm, AccV (&acc
   const int wp = wave % WP, wq = wave / WP;
   Epilogue ep(g, bt);
   const bool swp = prm.swapped != 0;
+  const int act = ACT_T >= 0 ? ACT_T : g.act;
+  const bool to_bf16 = BF16_T >= 0 ? BF16_T != 0 : g.d_type == CUDA_R_16BF;
   const int d_sq = (int)(swp ? g.d_si : g.d_sj);  // < 2^22 (checked by the dispatcher)
   const int pc = p0 + wp * WTP, qc = q0 + wq * WTQ;
   const int64_t corner = (int64_t)qc * d_sq + pc;
@@ -119,10 +125,10 @@ __device__ __forceinline__ void mfma16_store_f(const MfmaParams &prm, AccV (&acc
         const float accf = KIND == KIND_I8 ? (float)to_bits(acc[a][b][e]) : bits2f((uint32_t)to_bits(acc[a][b][e]));
         x[e] = (swp ? qs[b] * ps[e] : ps[e] * qs[b]) * accf + (swp ? qb[b] : pb[e]);
       }
-      if (g.act == ACT_GELU) {
+      if (act == ACT_GELU) {
 #pragma unroll
         for (int e = 0; e < 4; e++) x[e] = gelu_tanh(x[e]);
-      } else if (g.act == ACT_RELU) {
+      } else if (act == ACT_RELU) {
 #pragma unroll
         for (int e = 0; e < 4; e++) x[e] = x[e] > 0.0f ? x[e] : 0.0f;
       }
@@ -134,11 +140,12 @@ __device__ __forceinline__ void mfma16_store_f(const MfmaParams &prm, AccV (&acc
         buffer_store_b128_guarded(pk, rs, voff, soff);
       } else {
         v2i pk;
-        if (g.d_type == CUDA_R_16BF) { pk[0] = (int)pack_bf16x2(x[0], x[1]); pk[1] = (int)pack_bf16x2(x[2], x[3]); }
+        if (to_bf16) { pk[0] = (int)pack_bf16x2(x[0], x[1]); pk[1] = (int)pack_bf16x2(x[2], x[3]); }
         else { pk[0] = (int)pack_f16x2(x[0], x[1]); pk[1] = (int)pack_f16x2(x[2], x[3]); }
         __builtin_amdgcn_raw_buffer_store_b64(pk, rs, voff, soff, 0);
       }
     }
+    if constexpr (FENCE) __builtin_amdgcn_sched_barrier(0);
   }
 }
 

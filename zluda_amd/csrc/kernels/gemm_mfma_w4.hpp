@@ -1,0 +1,516 @@
+// Persistent MFMA GEMM for K-contiguous int8 / fp8 operands on gfx950: four waves, one per SIMD, each with a
+// 128 x 128 share of a 256 x 256 workgroup tile, on the 16x16 instruction shapes
+//   int8 : v_mfma_i32_16x16x64_i8            fp8 : v_mfma_f32_16x16x128_f8f6f4
+// for problems whose tiles fill the chip several times over.
+//
+// Against gemm_mfma_pipe16.hpp (eight waves of 128 x 64), same LDS ring, DMA, swizzle and fragment layout:
+//   * A 128 x 128 wave tile multiplies every fragment it reads from LDS with eight others instead of four or
+//     eight: 32 ds_read_b128 per wave and stage, 128 per workgroup instead of 192.
+//   * The 64 accumulator tiles of a wave (256 registers) live in the AGPRs, which leaves the 256 architectural
+//     VGPRs to the fragments.  The MFMAs are inline assembly with the accumulator as a tied "+a" operand: given
+//     the builtin, the register allocator picks different registers for the result and the addend of most
+//     MFMAs at this pressure and fills the loop with v_accvgpr moves and spills.  For the same reason the
+//     epilogues fetch the accumulators with explicit v_accvgpr_read (left to itself the allocator parks most of
+//     them in scratch memory right behind their last MFMA).
+//   * Inline assembly is opaque to the scheduler, so the order of the loop is the order of the source: every
+//     sub-step is written out as MFMA, the LDS reads and DMA instructions that follow it, MFMA, ...
+//   * A wave that has its SIMD to itself has nobody to issue MFMAs while it waits, so what it waits for matters
+//     more than how many instructions it issues.  Measured on MI355X (cycles per 16x16x128 MFMA of a lone wave):
+//     MFMAs alone 32; with one vector memory instruction behind every MFMA 64, behind every second one 40 -- the
+//     CU's address unit takes one 1 KiB instruction per 16 clocks for all four SIMDs, and a wave that queues them
+//     faster stalls at issue.  The 16 DMA instructions of a stage are therefore spread over the two sub-steps
+//     that follow the barrier, one behind every second MFMA (all 16 in the first of them: 7 % slower at 8192^3).
+//   * One workgroup per CU walks a list of tiles (workgroup w takes tiles w, w + G, w + 2G, ... of the XCD-aware
+//     order of the other kernels; G = grid size), and the stream of K stages runs on across tile boundaries:
+//     the DMA is two stages ahead whatever tile they belong to.  The epilogue of a tile (straight from the
+//     accumulators, no LDS) runs between two stages with the next tile's first two stages in flight, so neither
+//     the fill latency of a tile's first stages nor the wait for a new workgroup is paid per tile.
+//   * Every wait for the DMA is vmcnt(0) (a stage is requested one stage time before it is read and nothing
+//     younger is in flight at that point), so no assumption about the order in which loads retire is made.
+//
+// Hazards the compiler cannot see through the assembly are covered by hand: s_nop between the accumulator
+// initialisation and the first MFMA, and between the last MFMA of a tile and the first read of its results.
+#pragma once
+#include "gemm_mfma_pipe16.hpp"
+
+namespace zluda_amd {
+
+// the fast epilogue an instantiation carries; everything else a problem may ask for (and every tile that is not
+// complete along P) takes the element-wise path through LDS
+enum { W4_EPI_I32 = 0, W4_EPI_BF16 = 1, W4_EPI_BF16_GELU = 2 };
+
+// one accumulator element, AGPR -> VGPR
+template <class T>
+__device__ __forceinline__ int w4_acc_read(const T &elem) {
+  int raw = 0;
+#if defined(__HIP_DEVICE_COMPILE__)  // (the register constraints mean something else to the host pass)
+  asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(raw) : "a"(elem));
+#endif
+  return raw;
+}
+
+// Float epilogue of the four-wave kernel: D bf16 / f16 = act((scale_p * scale_q) * acc + bias) * scale_d straight from the
+// accumulators (layout of gemm_mfma_pipe16.hpp: lane l holds P = 16a + 4 (l / 16) + e, Q = 16b + l % 16) on tiles complete
+// along P, for problems in which nothing varies along Q (no per-column scale vector; for a row-major D no per-row vector
+// or bias).  A wave that has its SIMD to itself cannot hide branches or dependent chains behind another wave, so everything
+// that depends on the problem's modes is decided once, up front, into per-lane factors, and the 64 tiles are straight-line
+// code: one FMA per element, then the activation (ACT fixed at compile time) with D's scale folded into it.
+template <int KIND, int ACT, bool BF16, int WTP, int WTQ, int TP, int TQ, class AccV>
+__device__ __forceinline__ void w4_store_f16(const MfmaParams &prm, AccV (&acc)[TP][TQ], int p0, int q0, int NP, int NQ, int bt,
+                                             int wp, int wq) {
+  const GemmArgs &g = prm.g;
+  const int lane = threadIdx.x & 63;
+  Epilogue ep(g, bt);
+  const bool swp = prm.swapped != 0;
+  const int d_sq = (int)(swp ? g.d_si : g.d_sj);  // < 2^22 (checked before this path is taken)
+  const int pc = p0 + wp * WTP, qc = q0 + wq * WTQ;
+  const int64_t corner = (int64_t)qc * d_sq + pc;
+  char *Dw = (char *)g.D + (g.d_sb * bt + corner) * 2;
+  const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)Dw, 0, tile_window_bytes(d_sq, NP, NQ, corner, 2), 0x00020000);
+  const int voff = ((lane & 15) * d_sq + 4 * (lane >> 4)) * 2;
+  const int prow = pc + 4 * (lane >> 4);  // first of the lane's four P indices in tile row 0
+  // the one factor along Q (uniform) and D's scale: without an activation both fold into the P factors
+  const float q_u = swp ? ep.row_scale(0) : ep.col_scale(0);
+  const float fold = ACT == ACT_NONE ? q_u * ep.sd : q_u;
+  const float inv_sd = 1.0f / ep.sd;
+  float ps[TP][4], pb[TP][4];
+  const bool p_vec = swp ? ep.sb_v != nullptr : (ep.alpha_v != nullptr || ep.sa_v != nullptr);
+  if (p_vec) {
+#pragma unroll
+    for (int a = 0; a < TP; a++)
+#pragma unroll
+      for (int e = 0; e < 4; e++) ps[a][e] = (swp ? ep.col_scale(prow + a * 16 + e) : ep.row_scale(prow + a * 16 + e)) * fold;
+  } else {
+    const float u = (swp ? ep.col_scale(0) : ep.row_scale(0)) * fold;
+#pragma unroll
+    for (int a = 0; a < TP; a++)
+#pragma unroll
+      for (int e = 0; e < 4; e++) ps[a][e] = u;
+  }
+  if (!swp && g.bias != nullptr) {
+    const float bfold = ACT == ACT_NONE ? ep.sd : 1.0f;
+#pragma unroll
+    for (int a = 0; a < TP; a++)
+#pragma unroll
+      for (int e = 0; e < 4; e++) pb[a][e] = ep.bias_at(prow + a * 16 + e) * bfold;
+  } else {
+#pragma unroll
+    for (int a = 0; a < TP; a++)
+#pragma unroll
+      for (int e = 0; e < 4; e++) pb[a][e] = 0.0f;
+  }
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int a = 0; a < TP; a++) {
+    // The row's accumulators first, by explicit reads (left to itself the register allocator parks most accumulators
+    // in scratch memory between their last MFMA and this point instead of leaving them in the AGPRs); then TQ * 4
+    // independent chains for the scheduler to interleave.
+    int raw[TQ][4];
+#pragma unroll
+    for (int b = 0; b < TQ; b++)
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        raw[b][e] = w4_acc_read(acc[a][b][e]);
+      }
+    // written stage by stage over the whole row, which is the order the scheduler then keeps: every instruction
+    // has TQ * 4 - 1 independent ones between itself and its consumer
+    float x[TQ][4], z[TQ][4];
+#pragma unroll
+    for (int b = 0; b < TQ; b++)
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        const float accf = KIND == KIND_I8 ? (float)raw[b][e] : bits2f((uint32_t)raw[b][e]);
+        x[b][e] = __builtin_fmaf(accf, ps[a][e], pb[a][e]);
+      }
+    if constexpr (ACT == ACT_GELU) {
+      // x * sigmoid(2u) * sd (gelu_tanh of numeric.hpp) with sd folded into the reciprocal: x / ((1 + e) / sd)
+      const float c0 = -2.0f * 0.7978845608028654f * 1.4426950408889634f, c1 = 0.044715f * c0;
+#pragma unroll
+      for (int b = 0; b < TQ; b++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) z[b][e] = x[b][e] * x[b][e];
+#pragma unroll
+      for (int b = 0; b < TQ; b++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) z[b][e] = __builtin_fmaf(z[b][e], c1, c0);
+#pragma unroll
+      for (int b = 0; b < TQ; b++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) z[b][e] = x[b][e] * z[b][e];
+#pragma unroll
+      for (int b = 0; b < TQ; b++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) z[b][e] = __builtin_amdgcn_exp2f(z[b][e]);
+#pragma unroll
+      for (int b = 0; b < TQ; b++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) z[b][e] = __builtin_fmaf(z[b][e], inv_sd, inv_sd);
+#pragma unroll
+      for (int b = 0; b < TQ; b++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) z[b][e] = __builtin_amdgcn_rcpf(z[b][e]);
+#pragma unroll
+      for (int b = 0; b < TQ; b++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) x[b][e] = x[b][e] * z[b][e];
+    } else if constexpr (ACT == ACT_RELU) {
+#pragma unroll
+      for (int b = 0; b < TQ; b++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) x[b][e] = (x[b][e] > 0.0f ? x[b][e] : 0.0f) * ep.sd;
+    }
+#pragma unroll
+    for (int b = 0; b < TQ; b++) {
+      v2i pk;
+      if constexpr (BF16) { pk[0] = (int)pack_bf16x2(x[b][0], x[b][1]); pk[1] = (int)pack_bf16x2(x[b][2], x[b][3]); }
+      else { pk[0] = (int)pack_f16x2(x[b][0], x[b][1]); pk[1] = (int)pack_f16x2(x[b][2], x[b][3]); }
+      __builtin_amdgcn_raw_buffer_store_b64(pk, rs, voff, (b * 16 * d_sq + a * 16) * 2, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);  // one tile row at a time: what the scheduler hoists across rows costs registers
+  }
+}
+
+// Integer epilogue of the four-wave kernel: D int32 = alpha * acc (beta == 0, scalar alpha) on tiles complete along P
+// with 16-byte aligned columns: 16 bytes per lane straight from the accumulators.
+template <int WTP, int WTQ, int TP, int TQ, class AccV>
+__device__ __forceinline__ void w4_store_i32(const MfmaParams &prm, AccV (&acc)[TP][TQ], int p0, int q0, int NP, int NQ, int bt,
+                                             int wp, int wq) {
+  const GemmArgs &g = prm.g;
+  const int lane = threadIdx.x & 63;
+  const int ialpha = g.alpha_mode == SCALAR_VALUE ? g.alpha_val.i : *(const int32_t *)g.alpha_ptr;
+  const int64_t d_sq = prm.swapped ? g.d_si : g.d_sj;
+  const int pc = p0 + wp * WTP, qc = q0 + wq * WTQ;
+  const int64_t corner = (int64_t)qc * d_sq + pc;
+  int32_t *Dw = (int32_t *)g.D + g.d_sb * bt + corner;
+  const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)Dw, 0, tile_window_bytes(d_sq, NP, NQ, corner, 4), 0x00020000);
+  const int pitch = (int)d_sq;
+  const int voff = ((lane & 15) * pitch + 4 * (lane >> 4)) * 4;
+#pragma unroll
+  for (int a = 0; a < TP; a++) {
+    v4i v[TQ];
+#pragma unroll
+    for (int b = 0; b < TQ; b++)
+#pragma unroll
+      for (int e = 0; e < 4; e++) v[b][e] = w4_acc_read(acc[a][b][e]);
+#pragma unroll
+    for (int b = 0; b < TQ; b++) {
+      if (ialpha != 1) v[b] *= ialpha;
+      buffer_store_b128_guarded(v[b], rs, voff, (b * 16 * pitch + a * 16) * 4);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
+// Everything else (tiles that are partial along P, C reads, other output types, vectors along Q, unaligned D): element by
+// element through the scalar epilogue, one row of 16 x 16 tiles at a time staged in the wave's share of LDS.  Correct for
+// whatever the planner admits; not fast.  The caller guarantees that no wave still needs the LDS tiles.
+template <int KIND, int WTP, int WTQ, int TP, int TQ, class AccV>
+__device__ __forceinline__ void w4_store_general(const MfmaParams &prm, AccV (&acc)[TP][TQ], int *lds_words, int p0, int q0, int NP,
+                                                 int NQ, int bt, int wp, int wq) {
+  const GemmArgs &g = prm.g;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  int *stage = lds_words + wave * (WTQ * 16);  // [Q index of the wave tile][16 P indices of the row]
+  Epilogue ep(g, bt);
+  const bool swp = prm.swapped != 0;
+#pragma unroll
+  for (int a = 0; a < TP; a++) {
+#pragma unroll
+    for (int b = 0; b < TQ; b++) {
+      v4i v;
+#pragma unroll
+      for (int e = 0; e < 4; e++) v[e] = w4_acc_read(acc[a][b][e]);
+      *(v4i *)&stage[(b * 16 + (lane & 15)) * 16 + 4 * (lane >> 4)] = v;
+    }
+    // (LDS executes the writes and reads of one wave in program order: no barrier for wave-private rows)
+#pragma unroll 1
+    for (int e = lane; e < WTQ * 16; e += 64) {
+      const int ql = e / 16, pl = e % 16;
+      const int pi = p0 + wp * WTP + a * 16 + pl, qi = q0 + wq * WTQ + ql;
+      if (pi >= NP || qi >= NQ) continue;
+      const int raw = stage[ql * 16 + pl];
+      const int i = swp ? qi : pi, j = swp ? pi : qi;
+      if (g.int_scale) ep.store_int(i, j, raw);
+      else ep.store_f(i, j, KIND == KIND_I8 ? (float)raw : bits2f((uint32_t)raw));
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
+// whether the instantiation's fast epilogue serves the problem (on tiles complete along P)
+template <int KIND, int EPI>
+__device__ __forceinline__ bool w4_fast_epilogue_ok(const MfmaParams &prm) {
+  const GemmArgs &g = prm.g;
+  const int64_t d_sq = prm.swapped ? g.d_si : g.d_sj;
+  const int dbytes = EPI == W4_EPI_I32 ? 4 : 2;
+  const bool aligned = (((uintptr_t)g.D) & 15) == 0 && ((d_sq * dbytes) & 15) == 0 && ((g.d_sb * dbytes) & 15) == 0 &&
+                       d_sq < (1 << 22);
+  if (!aligned) return false;
+  if constexpr (EPI == W4_EPI_I32) {
+    return KIND == KIND_I8 && g.int_scale && g.d_type == CUDA_R_32I && g.alpha_mode != VECTOR_DEV && g.beta_mode == SCALAR_VALUE &&
+           g.beta_val.i == 0;
+  } else {
+    // vectors that run along Q (a per-column scale; for a row-major D the per-row ones and the bias) are not served
+    const bool q_vec = prm.swapped ? (g.alpha_mode == VECTOR_DEV || g.a_scale_mode == SCALE_OUTER_VEC || g.bias != nullptr)
+                                   : g.b_scale_mode == SCALE_OUTER_VEC;
+    return !g.int_scale && g.beta_mode == SCALAR_VALUE && g.beta_val.f == 0.0f && g.d_type == CUDA_R_16BF && !q_vec &&
+           g.act == (EPI == W4_EPI_BF16_GELU ? ACT_GELU : ACT_NONE);
+  }
+}
+
+template <int KIND, int FQ, int FP, int EPI>
+__global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
+  static_assert(KIND == KIND_I8 || KIND == KIND_F8, "int8 and fp8 operands");
+  constexpr int BP = 256, BQ = 256, WP = 2, WQ = 2;
+  constexpr int NWV = 4;
+  constexpr int BKB = 128, CPR = 8, RPW = 8;
+  constexpr int RPP = NWV * RPW;               // rows filled per DMA pass of the workgroup
+  constexpr int LP = BP / RPP, LQ = BQ / RPP;  // DMA instructions per thread, stage and operand
+  constexpr int NLOAD = LP + LQ;
+  constexpr int WTP = BP / WP, WTQ = BQ / WQ, TP = WTP / 16, TQ = WTQ / 16;
+  constexpr int HP = TP / 2, HQ = TQ / 2;      // fragments per half of the wave tile
+  constexpr int KS = KIND == KIND_F8 ? 1 : 2;  // MFMAs per fragment pair (K halves of the 128-byte stage)
+  constexpr int STAGE_V4 = (BP + BQ) * CPR;    // one slot in 16-byte words: P rows, then Q rows
+  constexpr int NM = HP * HQ * KS;             // MFMAs per sub-step
+  constexpr int NRD = 2 * HP;                  // ds_read_b128 per sub-step (HP == HQ)
+  static_assert(HP == HQ, "square wave tile");
+  using acc_v = typename std::conditional<KIND == KIND_I8, v4i, v4f>::type;
+  using frag_v = typename std::conditional<KIND != KIND_F8, v4i, v8i>::type;
+  struct Frag { frag_v k[KS]; };
+
+  __shared__ v4i lds[2 * STAGE_V4];
+
+  const GemmArgs &g = prm.g;
+  const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int wp = wave % WP, wq = wave / WP;
+  const int r16 = lane & 15, g4 = lane >> 4;
+
+  const int NP = prm.swapped ? g.N : g.M, NQ = prm.swapped ? g.M : g.N;
+  const int Kbytes = g.K;
+  const int KT2 = (Kbytes + 2 * BKB - 1) / (2 * BKB) * 2;  // stages per tile, an even number: a last odd one multiplies zeros
+  const int total = prm.tiles_p * prm.tiles_q;
+  const int ntiles = total * g.batch;
+  const int G = (int)gridDim.x;
+  const int my_tiles = (ntiles - (int)blockIdx.x + G - 1) / G;  // >= 1: the grid never exceeds the tile count
+  const int ldp = (int)(prm.swapped ? g.b_sj : g.a_si), ldq = (int)(prm.swapped ? g.a_si : g.b_sj);
+
+  // n-th tile of this workgroup -> tile corner and batch (the order of gemm_mfma_pipe_kernel: the 8 XCDs take
+  // turns at workgroup ids, so ids are spread over 8 contiguous ranges of the tile order, which walks groups
+  // of group_p tiles along P; G is a multiple of 8 whenever total is)
+  auto tile_coords = [&](int n, int &p0, int &q0, int &bt) __attribute__((always_inline)) {
+    const int idx = (int)blockIdx.x + n * G;
+    bt = idx / total;
+    int w = idx - bt * total;
+    if ((total & 7) == 0) w = (w & 7) * (total >> 3) + (w >> 3);
+    const int group = prm.group_p * prm.tiles_q;
+    const int gid = w / group, first_p = gid * prm.group_p;
+    const int gsz = min(prm.tiles_p - first_p, prm.group_p);
+    p0 = (first_p + (w % group) % gsz) * BP;
+    q0 = ((w % group) / gsz) * BQ;
+  };
+
+  // ---- the DMA side: two stages ahead of the MFMAs, across tile boundaries ----------------------------------
+  // one wave instruction fills 8 rows x 128 bytes; lane l -> row l / 8, slot l % 8, global chunk slot ^ swizzle(row)
+  const int dr = lane / CPR, dslot = lane % CPR;
+  const int drow = wave * RPW + dr;  // passes advance by RPP = 32 rows: same swizzle
+  const int dcg = dslot ^ swz(drow);
+  const int lane_k_left = Kbytes - dcg * 16;  // a stage that starts at or beyond this many K bytes is past the end for this lane
+  int d_live = -1;         // 0 once the list is exhausted: the loads that remain read one cache line nobody uses
+  int voffP[LP], voffQ[LQ];
+  __amdgpu_buffer_rsrc_t rsP, rsQ;
+  auto dma_tile = [&](int n) __attribute__((always_inline)) {
+    int p0, q0, bt;
+    tile_coords(n, p0, q0, bt);
+    const uint8_t *Pg = prm.swapped ? (const uint8_t *)g.B + g.b_sb * bt : (const uint8_t *)g.A + g.a_sb * bt;
+    const uint8_t *Qg = prm.swapped ? (const uint8_t *)g.A + g.a_sb * bt : (const uint8_t *)g.B + g.b_sb * bt;
+    // 2 GiB raw buffer windows: an offset with bit 31 set is out of range and reads as zero
+    rsP = __builtin_amdgcn_make_buffer_rsrc((void *)Pg, 0, 0x80000000, 0x00020000);
+    rsQ = __builtin_amdgcn_make_buffer_rsrc((void *)Qg, 0, 0x80000000, 0x00020000);
+#pragma unroll
+    for (int i = 0; i < LP; i++) voffP[i] = min(p0 + drow + RPP * i, NP - 1) * ldp + dcg * 16;
+#pragma unroll
+    for (int i = 0; i < LQ; i++) voffQ[i] = min(q0 + drow + RPP * i, NQ - 1) * ldq + dcg * 16;
+  };
+  // instructions [I0, I1) of the NLOAD that bring stage dk of the DMA side's tile into the slot at `so`.  Lanes
+  // past the end of K (the tail of the last stage, the whole padding stage of an odd stage count) are out of
+  // range: zeros, no traffic.
+  auto issue_part = [&](int dk, int so, auto i0_c, auto i1_c) __attribute__((always_inline)) {
+    constexpr int I0 = decltype(i0_c)::value, I1 = decltype(i1_c)::value;
+    const int soff = (dk * BKB) & d_live;
+    const int oob = soff < lane_k_left ? 0 : (int)0x80000000;
+    v4i *base = &lds[so];
+    static_for<I1 - I0>([&](auto k_c) {
+      constexpr int k = I0 + decltype(k_c)::value;
+      if constexpr (k < LP) lds_dma16(rsP, base + (wave * RPW + RPP * k) * CPR, (voffP[k] | oob) & d_live, soff);
+      else lds_dma16(rsQ, base + (BP + wave * RPW + RPP * (k - LP)) * CPR, (voffQ[k - LP] | oob) & d_live, soff);
+    });
+  };
+
+  // ---- fragment addressing (as gemm_mfma_pipe16_kernel) -------------------------------------------------------
+  int fragP[2][2], fragQ[2][2];  // [tile parity][first / second 16-byte piece of the lane], 16-byte words inside a slot
+#pragma unroll
+  for (int par = 0; par < 2; par++)
+#pragma unroll
+    for (int kk = 0; kk < 2; kk++) {
+      const int row = par * 16 + r16;
+      const int ch = (KIND == KIND_F8 ? 2 * g4 + kk : 4 * kk + g4) ^ swz(row);
+      fragP[par][kk] = (wp * WTP + row) * CPR + ch;
+      fragQ[par][kk] = (BP + wq * WTQ + row) * CPR + ch;
+    }
+  Frag pf[2][HP], qf[2][HQ];  // [half of the wave tile][fragment]
+  // ds_read_b128 number r (0 .. NRD-1) of half h of P / of Q from the slot at `so`
+  auto read_piece = [&](int so, const int (&fr)[2][2], Frag (&dst)[HP], auto h_c, auto r_c) {
+    constexpr int h = decltype(h_c)::value, r = decltype(r_c)::value;
+    constexpr int i = r / 2, kk = r % 2, tile = h * HP + i;
+    const v4i x = lds[so + (tile >> 1) * 32 * CPR + fr[tile & 1][kk]];
+    if constexpr (KIND == KIND_F8) {
+#pragma unroll
+      for (int e = 0; e < 4; e++) dst[i].k[0][4 * kk + e] = x[e];
+    } else {
+      dst[i].k[kk] = x;
+    }
+  };
+
+  acc_v acc[TP][TQ];
+  auto zero_acc = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int a = 0; a < TP; a++)
+#pragma unroll
+      for (int b = 0; b < TQ; b++)
+#pragma unroll
+        for (int v = 0; v < 4; v++) acc[a][b][v] = 0;
+    // (the pins keep the zeros in the AGPRs the MFMAs use; the s_nop covers VALU write -> MFMA read of SrcC)
+#if defined(__HIP_DEVICE_COMPILE__)
+#pragma unroll
+    for (int a = 0; a < TP; a++)
+#pragma unroll
+      for (int b = 0; b < TQ; b++) asm volatile("" : "+a"(acc[a][b]));
+    asm volatile("s_nop 4" ::: "memory");
+#endif
+  };
+  // MFMA number x of the sub-step (P half ph, Q half qh): K half x / (HP * HQ), tile pair (i, j) with i the
+  // slower index, so that the fragments a sub-step reads first are the ones the next sub-step multiplies first
+  auto mfma_one = [&](auto ph_c, auto qh_c, auto x_c) __attribute__((always_inline)) {
+    constexpr int ph = decltype(ph_c)::value, qh = decltype(qh_c)::value, x = decltype(x_c)::value;
+    constexpr int ks = x / (HP * HQ), i = (x % (HP * HQ)) / HQ, j = x % HQ;
+    acc_v &c = acc[ph * HP + i][qh * HQ + j];
+    const frag_v &pa = pf[ph][i].k[ks], &qb = qf[qh][j].k[ks];  // (named here: asm operands alone do not capture)
+#if defined(__HIP_DEVICE_COMPILE__)  // (the register constraints mean something else to the host pass)
+    if constexpr (KIND == KIND_I8) {
+      asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(c) : "v"(pa), "v"(qb));
+    } else if constexpr (FP == 0 && FQ == 0) {
+      asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(c) : "v"(pa), "v"(qb));
+    } else if constexpr (FP == 1 && FQ == 0) {
+      asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 cbsz:1" : "+a"(c) : "v"(pa), "v"(qb));
+    } else if constexpr (FP == 0 && FQ == 1) {
+      asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 blgp:1" : "+a"(c) : "v"(pa), "v"(qb));
+    } else {
+      asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 cbsz:1 blgp:1" : "+a"(c) : "v"(pa), "v"(qb));
+    }
+#endif
+  };
+
+  // One sub-step: its NM MFMAs in order; behind each of the first NRD of them one fragment read (`rd(r)`), and the
+  // NLOAD DMA instructions spread evenly behind all of them when the sub-step refills a slot.
+  auto substep = [&](auto ph_c, auto qh_c, auto &&rd, auto l0_c, auto l1_c, int dma_dk, int dma_so) __attribute__((always_inline)) {
+    constexpr int L0 = decltype(l0_c)::value, L1 = decltype(l1_c)::value;  // DMA instructions [L0, L1) of the stage ride along
+    static_assert(NM >= NRD && NM >= L1 - L0, "room for the reads and the DMA of a sub-step");
+    static_for<NM>([&](auto x_c) {
+      constexpr int x = decltype(x_c)::value;
+      mfma_one(ph_c, qh_c, x_c);
+      if constexpr (x < NRD) rd(x_c);
+      if constexpr (L1 > L0) {
+        // spread evenly: a wave that has its SIMD to itself and queues vector memory instructions faster than the CU's
+        // address unit takes them (one 1 KiB instruction per 16 clocks, for all four SIMDs) keeps its next MFMA waiting
+        constexpr int D0 = L0 + (L1 - L0) * x / NM, D1 = L0 + (L1 - L0) * (x + 1) / NM;
+        if constexpr (D1 > D0) issue_part(dma_dk, dma_so, std::integral_constant<int, D0>{}, std::integral_constant<int, D1>{});
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  };
+
+  using P0 = std::integral_constant<int, 0>;
+  using P1 = std::integral_constant<int, 1>;
+  // One stage of the stream; ODD = parity of its number = its slot (a tile has an even number of stages, so the
+  // parity inside a tile is the parity in the stream).  On entry P half 0 and Q half ODD are in registers; it
+  // leaves P half 0 and Q half 1 - ODD of the next stage there, and refills its slot with stage dk of the DMA
+  // side's tile.
+  //   (P0, QA) reads QB | (P0, QB) reads P1 | barrier | (P1, QB) reads P0', refills the slot | (P1, QA) reads QB'
+  auto do_stage = [&](auto odd_c, int dk) __attribute__((always_inline)) {
+    constexpr int ODD = decltype(odd_c)::value;
+    constexpr int so = ODD * STAGE_V4, so_next = (1 - ODD) * STAGE_V4;
+    using QA = std::integral_constant<int, ODD>;
+    using QB = std::integral_constant<int, 1 - ODD>;
+    using Z = std::integral_constant<int, 0>;
+    using LS = std::integral_constant<int, NLOAD / 2>;
+    using LN = std::integral_constant<int, NLOAD>;
+    substep(P0{}, QA{}, [&](auto r_c) { read_piece(so, fragQ, qf[1 - ODD], QB{}, r_c); }, Z{}, Z{}, 0, 0);
+    substep(P0{}, QB{}, [&](auto r_c) { read_piece(so, fragP, pf[1], P1{}, r_c); }, Z{}, Z{}, 0, 0);
+    // every fragment of the stage has been requested: wait for them and for this wave's share of the next stage,
+    // meet the other waves; then this slot is free and the other one readable
+    wait_vmcnt_barrier<0>();
+    substep(P1{}, QB{}, [&](auto r_c) { read_piece(so_next, fragP, pf[0], P0{}, r_c); }, Z{}, LS{}, dk, so);
+    substep(P1{}, QA{}, [&](auto r_c) { read_piece(so_next, fragQ, qf[1 - ODD], QB{}, r_c); }, LS{}, LN{}, dk, so);
+  };
+  // two stages, which refill their slots with stages dk and dk + 1 of the DMA side's tile
+  auto do_pair = [&](int dk) __attribute__((always_inline)) {
+    do_stage(std::integral_constant<int, 0>{}, dk);
+    do_stage(std::integral_constant<int, 1>{}, dk + 1);
+  };
+  // the fragments a tile's first stage expects in registers (P half 0, Q half 0), from slot 0
+  auto first_frags = [&]() __attribute__((always_inline)) {
+    static_for<NRD>([&](auto r_c) { read_piece(0, fragP, pf[0], P0{}, r_c); });
+    static_for<NRD>([&](auto r_c) { read_piece(0, fragQ, qf[0], P0{}, r_c); });
+  };
+  // (re)starts the stream at tile n: its first two stages requested and landed, its first fragments in registers
+  auto prime = [&](int n) __attribute__((always_inline)) {
+    d_live = -1;
+    dma_tile(n);
+    issue_part(0, 0, std::integral_constant<int, 0>{}, std::integral_constant<int, NLOAD>{});
+    issue_part(1, STAGE_V4, std::integral_constant<int, 0>{}, std::integral_constant<int, NLOAD>{});
+    wait_vmcnt_barrier<0>();
+    first_frags();
+  };
+
+  const bool fast = w4_fast_epilogue_ok<KIND, EPI>(prm);
+  // epilogue of the tile at (p0, q0, bt); returns false when it needed the LDS (the stream must be primed again)
+  auto epilogue = [&](int p0, int q0, int bt) __attribute__((always_inline)) -> bool {
+    // MFMA write -> read of the accumulators: the wait states the compiler would insert if it could see the MFMAs.
+    // Nothing that reads an accumulator may be scheduled in front of them (every MFMA is followed by a scheduling
+    // barrier, and so are they).
+    asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    if (fast && p0 + BP <= NP) {
+      if constexpr (EPI == W4_EPI_I32) w4_store_i32<WTP, WTQ>(prm, acc, p0, q0, NP, NQ, bt, wp, wq);
+      else w4_store_f16<KIND, EPI == W4_EPI_BF16_GELU ? ACT_GELU : ACT_NONE, true, WTP, WTQ>(prm, acc, p0, q0, NP, NQ, bt, wp, wq);
+      return true;
+    }
+    // the element-wise epilogue stages the accumulators in LDS: let the stages in flight land first
+    wait_vmcnt_barrier<0>();
+    w4_store_general<KIND, WTP, WTQ>(prm, acc, (int *)&lds[0], p0, q0, NP, NQ, bt, wp, wq);
+    __syncthreads();
+    return false;
+  };
+
+  // ---- the stream -------------------------------------------------------------------------------------------------
+  prime(0);
+  for (int n = 0; n < my_tiles; n++) {
+    int p0, q0, bt;
+    tile_coords(n, p0, q0, bt);
+    zero_acc();
+    for (int kt = 2; kt < KT2; kt += 2) do_pair(kt);
+    // the last two stages of the tile fetch the first two of the next one
+    if (n + 1 < my_tiles) dma_tile(n + 1);
+    else d_live = 0;
+    do_pair(0);
+    const bool kept = epilogue(p0, q0, bt);
+    // The first fragments of the next tile are fetched again behind the epilogue (its first stage landed before the
+    // last barrier): holding them across it would take 64 of the registers the epilogue needs.
+    if (n + 1 < my_tiles) {
+      if (kept) first_frags();
+      else prime(n + 1);
+    }
+  }
+  __builtin_amdgcn_s_waitcnt(0);  // the loads past the end of the list have landed before the wave ends
+}
+
+} // namespace zluda_amd
