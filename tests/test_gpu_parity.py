@@ -38,7 +38,7 @@ def check(gpu_api, spec, seed, kernel=None, variant=-1, expect_kernel=None, tol=
 
 
 # ---- int8 -> int32 MFMA, every tile variant --------------------------------
-@pytest.mark.parametrize("variant", range(11))
+@pytest.mark.parametrize("variant", range(12))
 @pytest.mark.parametrize("m,n,k", [(256, 256, 128), (300, 200, 144), (512, 384, 1024)])
 def test_mfma_i8_variants(gpu_api, variant, m, n, k):
     check(gpu_api, dict(I8, m=m, n=n, k=k, lda=k + 16 if k == 144 else k), 10 + variant, K.ZLUDA_KERNEL_MFMA_I8, variant)
@@ -46,7 +46,7 @@ def test_mfma_i8_variants(gpu_api, variant, m, n, k):
 
 def test_mfma_i8_alpha_beta_batch_and_padding(gpu_api):
     spec = dict(I8, m=200, n=136, k=272, batch=3, with_c=True, ldd=208, ldc=204, lda=288, stride_d=208 * 136 + 48)
-    for variant in (0, 1, 4, 6, 8, 9, 10):
+    for variant in (0, 1, 4, 6, 8, 9, 10, 11):
         check(gpu_api, spec, 3, K.ZLUDA_KERNEL_MFMA_I8, variant)
     # device scalars
     check(gpu_api, dict(spec, pointer_mode=K.CUBLASLT_POINTER_MODE_DEVICE), 4, K.ZLUDA_KERNEL_MFMA_I8, 1)
@@ -57,10 +57,11 @@ def test_mfma_i8_row_major_output_swaps(gpu_api):
     check(gpu_api, spec, 5, K.ZLUDA_KERNEL_MFMA_I8, 1)
     check(gpu_api, spec, 5, K.ZLUDA_KERNEL_MFMA_I8, 4)
     check(gpu_api, spec, 5, K.ZLUDA_KERNEL_MFMA_I8, 8)
+    check(gpu_api, spec, 5, K.ZLUDA_KERNEL_MFMA_I8, 11)
 
 
 # full tiles take the register-direct / vectorised epilogues; cover each of them per tile shape
-@pytest.mark.parametrize("variant", range(11))
+@pytest.mark.parametrize("variant", range(12))
 def test_mfma_full_tile_epilogues(gpu_api, variant):
     full = dict(m=512, n=256, k=384)
     check(gpu_api, dict(I8, **full, alpha=1), 110, K.ZLUDA_KERNEL_MFMA_I8, variant)
@@ -82,7 +83,7 @@ def test_mfma_full_tile_epilogues(gpu_api, variant):
         check(gpu_api, dict(MX, m=512, n=256, k=1024), 116, K.ZLUDA_KERNEL_MFMA_MXF4, variant)
 
 
-@pytest.mark.parametrize("variant", range(11))
+@pytest.mark.parametrize("variant", range(12))
 def test_mfma_ragged_token_count_keeps_the_fast_epilogues(gpu_api, variant):
     """M a multiple of every tile height, N ragged (tokens): the stores of the columns past the end fall
     outside the buffer window; padding, the next batch and the canary behind D must stay untouched"""
@@ -102,7 +103,7 @@ def test_mfma_ragged_token_count_keeps_the_fast_epilogues(gpu_api, variant):
           K.ZLUDA_KERNEL_MFMA_F8, variant)
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8, 9])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 11])
 def test_mfma_i8_float_epilogue(gpu_api, variant):
     spec = dict(I8F, m=260, n=140, k=512, epilogue=K.CUBLASLT_EPILOGUE_RELU_BIAS, bias_type=K.CUDA_R_32F,
                 pointer_mode=K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_HOST, with_c=True,
@@ -117,7 +118,7 @@ def test_mfma_i8_float_epilogue(gpu_api, variant):
 
 
 # ---- fp8 -------------------------------------------------------------------------------------------
-@pytest.mark.parametrize("variant", range(11))
+@pytest.mark.parametrize("variant", range(12))
 def test_mfma_f8_variants(gpu_api, variant):
     check(gpu_api, dict(F8, m=256, n=256, k=256), 20 + variant, K.ZLUDA_KERNEL_MFMA_F8, variant)
     check(gpu_api, dict(F8, m=320, n=272, k=400, lda=416, ldb=400, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS,

@@ -32,7 +32,7 @@ def test_baseline_configs_pick_the_intended_kernels(api):
     st, p = plan(api, dict(I8, m=256, n=256, k=256, transa=0, transb=1))            # config 1: A:N B:T
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_TR8 and p.variant == 2 and p.grid_x == 16 and p.block == 256
     st, p = plan(api, dict(I8, m=4096, n=4096, k=4096, transa=1))                   # config 2
-    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_I8 and p.variant == 8 and p.grid_x == 256 and p.block == 512   # 256x256 on the 16x16 MFMA shapes
+    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_I8 and p.variant == 11 and p.grid_x == 256 and p.block == 256   # 256x256, four waves, one workgroup per CU
     st, p = plan(api, dict(I8, m=14336, n=16, k=4096, transa=1, d_type=K.CUDA_R_16BF, scale_type=K.CUDA_R_32F,
                            pointer_mode=K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO,
                            b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F,
@@ -40,7 +40,7 @@ def test_baseline_configs_pick_the_intended_kernels(api):
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_DECODE_W8A8 and p.swapped == 0 and p.block == 256
     assert p.variant == 16 and p.grid_x == 224     # streamed through LDS in slabs: 896 blocks of 16 rows, 4 per workgroup
     st, p = plan(api, dict(F8, m=8192, n=8192, k=8192, transa=1, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS))  # config 4
-    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_F8 and p.grid_x == 1024
+    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_F8 and p.variant == 11 and p.grid_x == 256 and p.grid_y == 1   # 1024 tiles, 4 per workgroup
     st, p = plan(api, dict(MX, m=8192, n=8192, k=8192, transa=1, batch=4))          # config 5
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_MXF4 and p.grid_x == 1024 and p.grid_y == 4
     assert p.workspace == 0
@@ -147,17 +147,54 @@ def test_extents_that_256_divides_badly_get_the_192_row_tile(api):
     st, p = plan(api, dict(I8, m=2048, n=2048, k=2048, transa=1, batch=2))   # 128 tiles of 256x256: half of the chip idles
     assert st == 0 and not (p.variant in (8, 9))
     st, p = plan(api, dict(I8, m=8192, n=8192, k=8192, transa=1))
-    assert st == 0 and p.variant == 8
+    assert st == 0 and p.variant == 11
     st, p = plan(api, dict(F8, m=14336, n=4096, k=4096, transa=1))   # 5 rounds of 192x256 lose to 4 of 256x256
-    assert st == 0 and p.variant == 0                                # (fp8 takes the 16x16-shape 256x256 tile from four full rounds on)
+    assert st == 0 and p.variant == 11
     st, p = plan(api, dict(F8, m=8192, n=8192, k=8192, transa=1))
-    assert st == 0 and p.variant == 8
+    assert st == 0 and p.variant == 11
     st, p = plan(api, dict(F8, m=8192, n=4096, k=4096, transa=1))
-    assert st == 0 and p.variant == 0
+    assert st == 0 and p.variant == 11
     st, p = plan(api, dict(MX, m=8192, n=8192, k=8192, transa=1))      # MXFP4 has no 16x16-shape variant
     assert st == 0 and p.variant == 0
     assert plan(api, dict(MX, m=8192, n=8192, k=8192, transa=1), forced=K.ZLUDA_KERNEL_MFMA_MXF4, variant=8)[0] == K.CUBLAS_STATUS_INVALID_VALUE
-    assert api.zluda_gemm_variant_count(K.ZLUDA_KERNEL_MFMA_I8) == 11 and api.zluda_gemm_variant_count(K.ZLUDA_KERNEL_MFMA_MXF4) == 8
+    assert api.zluda_gemm_variant_count(K.ZLUDA_KERNEL_MFMA_I8) == 12 and api.zluda_gemm_variant_count(K.ZLUDA_KERNEL_MFMA_MXF4) == 8
+
+
+def test_the_four_wave_kernel_is_chosen_for_what_its_epilogues_serve(api):
+    """variant 11: one workgroup per CU walks the 256 x 256 tiles of all batches; int8 -> int32 and e4m3 x e4m3 -> bf16 with
+    nothing that varies along the index across D's unit stride, no activation or GELU, from one round of tiles and 2 KiB of K"""
+    big = dict(m=8192, n=8192, k=8192, transa=1)
+    assert plan(api, dict(F8, **big))[1].variant == 11
+    assert plan(api, dict(F8, **big, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS))[1].variant == 11
+    assert plan(api, dict(F8, **big, epilogue=K.CUBLASLT_EPILOGUE_BIAS, pointer_mode=K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO))[1].variant == 11
+    # what it has no epilogue for stays on the eight-wave kernel with the same tile
+    assert plan(api, dict(F8, **big, epilogue=K.CUBLASLT_EPILOGUE_RELU))[1].variant == 8
+    assert plan(api, dict(F8, **big, d_type=K.CUDA_R_16F))[1].variant == 8
+    assert plan(api, dict(F8, **big, d_type=K.CUDA_R_32F))[1].variant == 8
+    assert plan(api, dict(F8, **big, b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F))[1].variant == 8
+    assert plan(api, dict(F8, **big, order_c=1, order_d=1, epilogue=K.CUBLASLT_EPILOGUE_BIAS))[1].variant == 8     # the bias runs along Q
+    assert plan(api, dict(F8, **big, order_c=1, order_d=1))[1].variant == 11
+    assert plan(api, dict(F8, **big, a_type=K.CUDA_R_8F_E5M2))[1].variant == 8
+    assert plan(api, dict(F8, **big, pointer_mode=K.CUBLASLT_POINTER_MODE_DEVICE))[1].variant == 8                 # beta unknown until it runs
+    assert plan(api, dict(F8, **big, ldd=8196))[1].variant == 8                                                    # columns of D not 16-byte aligned
+    assert plan(api, dict(I8, **big, d_type=K.CUDA_R_16BF, scale_type=K.CUDA_R_32F))[1].variant == 8
+    # grids: one workgroup per CU at most, all batches in one list
+    st, p = plan(api, dict(F8, m=4096, n=4096, k=4096, transa=1, batch=3))
+    assert st == 0 and p.variant == 11 and p.grid_x == 256 and p.grid_y == 1 and p.grid_z == 1 and p.workspace == 0 and p.waves == 3.0
+    st, p = plan(api, dict(F8, **big), cus=304)
+    assert st == 0 and p.variant == 11 and p.grid_x == 304
+    st, p = plan(api, dict(F8, **big), cus=300)     # a multiple of 8, so that a workgroup's tiles stay with one XCD
+    assert st == 0 and p.grid_x == 296
+    st, p = plan(api, dict(I8, m=4096, n=3072, k=4096, transa=1), forced=K.ZLUDA_KERNEL_MFMA_I8, variant=11)
+    assert st == 0 and p.grid_x == 192
+    # too few tiles or a short K: other variants
+    assert plan(api, dict(F8, m=4096, n=2048, k=4096, transa=1))[1].variant != 11
+    assert plan(api, dict(F8, m=16384, n=8192, k=1024, transa=1))[1].variant != 11
+    # never with a workspace split, never for other operand types
+    assert plan(api, dict(I8, m=1024, n=256, k=8192, transa=1), forced=K.ZLUDA_KERNEL_MFMA_I8, variant=11, workspace=64 << 20)[1].grid_z == 1
+    assert plan(api, dict(F8, **big, a_type=K.CUDA_R_8F_E5M2), forced=K.ZLUDA_KERNEL_MFMA_F8, variant=11)[0] == K.CUBLAS_STATUS_NOT_SUPPORTED
+    bf = dict(a_type=K.CUDA_R_16BF, b_type=K.CUDA_R_16BF, d_type=K.CUDA_R_16BF, compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F)
+    assert plan(api, dict(bf, **big), forced=K.ZLUDA_KERNEL_MFMA_H16, variant=11)[0] == K.CUBLAS_STATUS_INVALID_VALUE
 
 
 def test_row_major_output_swaps_operands(api):
@@ -232,10 +269,10 @@ def test_fp4_must_be_k_contiguous(api):
 def test_forced_variants(api):
     spec = dict(I8, m=4096, n=4096, k=4096, transa=1)
     for v, (grid, block) in enumerate([(256, 512), (256, 256), (512, 256), (1024, 256), (1024, 256), (2048, 256), (4096, 256),
-                                       (352, 512), (256, 512), (352, 512), (4096, 256)]):
+                                       (352, 512), (256, 512), (352, 512), (4096, 256), (256, 256)]):
         st, p = plan(api, spec, forced=K.ZLUDA_KERNEL_MFMA_I8, variant=v)
         assert st == 0 and p.variant == v and p.grid_x == grid and p.block == block
-    assert plan(api, spec, forced=K.ZLUDA_KERNEL_MFMA_I8, variant=11)[0] == K.CUBLAS_STATUS_INVALID_VALUE
+    assert plan(api, spec, forced=K.ZLUDA_KERNEL_MFMA_I8, variant=12)[0] == K.CUBLAS_STATUS_INVALID_VALUE
     assert plan(api, dict(MX, m=4096, n=4096, k=4096, transa=1), forced=K.ZLUDA_KERNEL_MFMA_MXF4, variant=10)[0] == K.CUBLAS_STATUS_INVALID_VALUE
     assert plan(api, spec, forced=K.ZLUDA_KERNEL_MFMA_F8)[0] == K.CUBLAS_STATUS_NOT_SUPPORTED
 

@@ -394,6 +394,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
     constexpr int ks = x / (HP * HQ), i = (x % (HP * HQ)) / HQ, j = x % HQ;
     acc_v &c = acc[ph * HP + i][qh * HQ + j];
     const frag_v &pa = pf[ph][i].k[ks], &qb = qf[qh][j].k[ks];  // (named here: asm operands alone do not capture)
+    (void)c; (void)pa; (void)qb;
 #if defined(__HIP_DEVICE_COMPILE__)  // (the register constraints mean something else to the host pass)
     if constexpr (KIND == KIND_I8) {
       asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(c) : "v"(pa), "v"(qb));

@@ -32,11 +32,35 @@ namespace {
 inline int f8_fmt(uint32_t t) { return t == CUDA_R_8F_E5M2 ? 1 : 0; }
 
 // `ws` / `ws_size`: the scratch that holds split-K partial tiles (the caller's workspace, or the library's own)
-uint32_t launch_mfma(const Lowered &l, const zluda_gemm_plan &plan, void *ws, uint64_t ws_size, hipStream_t s) {
+uint32_t launch_mfma(const Lowered &l, const zluda_gemm_plan &plan_in, void *ws, uint64_t ws_size, hipStream_t s) {
   MfmaParams prm;
   prm.g = l.g;
+  if (plan_in.variant >= (uint32_t)kNumMfmaVariants) return CUBLAS_STATUS_INVALID_VALUE;
+  zluda_gemm_plan plan = plan_in;
+  if (kMfmaVariants[plan.variant].w4) {
+    // The four-wave kernel carries three epilogues.  What the call turns out to ask for beyond them (a beta that is not
+    // zero, a D that is not 16-byte aligned: known only now) runs on the eight-wave kernel with the same tile, which
+    // needs no workspace either.
+    const uint32_t cus = zluda_gemm_device_cu_count();
+    const int epi = w4_epilogue_class(l, false);
+    const int np = plan.swapped ? l.g.N : l.g.M, nq = plan.swapped ? l.g.M : l.g.N;
+    const uint64_t all = (uint64_t)((np + 255) / 256) * ((nq + 255) / 256) * l.g.batch;
+    if (epi != W4_CLASS_NONE) {
+      const uint32_t slots = cus >= 8 ? cus / 8 * 8 : cus;
+      if (plan.grid_x == 0 || plan.grid_x > all || plan.grid_x > slots || plan.grid_y != 1 || plan.grid_z > 1) return CUBLAS_STATUS_INVALID_VALUE;
+      prm.swapped = plan.swapped;
+      prm.tiles_p = (np + 255) / 256; prm.tiles_q = (nq + 255) / 256;
+      prm.group_p = 8;
+      prm.splits = 1; prm.split_stages = 0; prm.ws = nullptr;
+      return plan.kernel == ZLUDA_KERNEL_MFMA_I8 ? launch_mfma_w4_i8(prm, epi, plan.grid_x, s)
+                                                 : launch_mfma_w4_f8(prm, epi, plan.grid_x, s);
+    }
+    plan.variant = 8;
+    plan.grid_x = (uint32_t)(all / l.g.batch); plan.grid_y = l.g.batch; plan.grid_z = 1;
+    plan.block = 512;
+    plan.workspace = 0;
+  }
   prm.swapped = plan.swapped;
-  if (plan.variant >= (uint32_t)kNumMfmaVariants) return CUBLAS_STATUS_INVALID_VALUE;
   const MfmaVariant &v = kMfmaVariants[plan.variant];
   const int np = plan.swapped ? l.g.N : l.g.M, nq = plan.swapped ? l.g.M : l.g.N;
   prm.tiles_p = (np + v.bp - 1) / v.bp;

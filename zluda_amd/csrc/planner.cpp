@@ -226,6 +226,7 @@ uint32_t lower_problem(const zluda_gemm_problem *p, bool dry, Lowered *out) {
   }
 
   out->g = g;
+  out->has_bias = has_bias;
   out->a_kcontig = g.a_sk == 1;
   out->b_kcontig = g.b_sk == 1;
   auto al16 = [](const void *ptr, int64_t pitch_elems, int64_t bstride, int bits, bool batched) {
@@ -336,6 +337,30 @@ bool family_supports(uint32_t kernel, const Lowered &l) {
 
 static uint32_t ceil_div(uint32_t a, uint32_t b) { return (a + b - 1) / b; }
 
+int w4_epilogue_class(const Lowered &l, bool dry) {
+  const GemmArgs &g = l.g;
+  if (g.aux_mode || g.beta_mode != SCALAR_VALUE) return W4_CLASS_NONE;
+  const bool swapped = g.d_si != 1;
+  const int64_t d_sq = swapped ? g.d_si : g.d_sj;
+  const int dbytes = g.d_type == CUDA_R_32I ? 4 : 2;
+  if (((d_sq * dbytes) & 15) || (g.batch > 1 && ((g.d_sb * dbytes) & 15)) || d_sq >= (1 << 22) || (((uintptr_t)g.D) & 15))
+    return W4_CLASS_NONE;
+  if (g.a_type == CUDA_R_8I && g.b_type == CUDA_R_8I) {
+    if (!g.int_scale || g.d_type != CUDA_R_32I || g.alpha_mode == VECTOR_DEV || (!dry && g.beta_val.i != 0)) return W4_CLASS_NONE;
+    return W4_CLASS_I32;
+  }
+  if (g.a_type == CUDA_R_8F_E4M3 && g.b_type == CUDA_R_8F_E4M3 && g.a_scale_mode != SCALE_BLOCK32_UE8M0 &&
+      g.b_scale_mode != SCALE_BLOCK32_UE8M0) {
+    if (g.d_type != CUDA_R_16BF || (g.act != ACT_NONE && g.act != ACT_GELU) || (!dry && g.beta_val.f != 0.0f)) return W4_CLASS_NONE;
+    // nothing may vary along Q, the index that does not run along D's unit stride
+    const bool q_vec = swapped ? (g.alpha_mode == VECTOR_DEV || g.a_scale_mode == SCALE_OUTER_VEC || l.has_bias)
+                               : g.b_scale_mode == SCALE_OUTER_VEC;
+    if (q_vec) return W4_CLASS_NONE;
+    return g.act == ACT_GELU ? W4_CLASS_BF16_GELU : W4_CLASS_BF16;
+  }
+  return W4_CLASS_NONE;
+}
+
 static void fill_mfma_plan(const Lowered &l, int variant, uint32_t cus, uint64_t workspace_size,
                            zluda_gemm_plan *plan) {
   const GemmArgs &g = l.g;
@@ -347,6 +372,17 @@ static void fill_mfma_plan(const Lowered &l, int variant, uint32_t cus, uint64_t
   plan->swapped = swapped;
   plan->grid_x = tp * tq; plan->grid_y = g.batch; plan->grid_z = 1;
   plan->block = v.wp * v.wq * 64;
+  if (v.w4) {
+    // one workgroup per CU (a multiple of 8 of them, so that a workgroup's tiles stay on one XCD's share of the tile
+    // order) walks the tiles of all batches; never split along K
+    const uint64_t all = (uint64_t)tp * tq * g.batch;
+    const uint32_t slots = cus >= 8 ? cus / 8 * 8 : cus;
+    plan->grid_x = (uint32_t)std::min<uint64_t>(all, slots);
+    plan->grid_y = 1;
+    plan->waves = (float)all / (float)cus;
+    plan->workspace = 0;
+    return;
+  }
   // data stages, plus two chunks of 32 scale bytes per tile row for MXFP4
   const uint32_t lds = (uint32_t)v.stages * (v.bp + v.bq) * v.bkb + (l.g.a_type == CUDA_R_4F_E2M1 ? 64u * (v.bp + v.bq) : 0u);
   const uint32_t per_cu = std::max(1u, std::min(160u * 1024u / lds, 2048u / plan->block));
@@ -387,7 +423,7 @@ static void fill_mfma_plan(const Lowered &l, int variant, uint32_t cus, uint64_t
 // 27.5), so they are only chosen for grids that fill the chip; the same tiles at 256x128 and 128x128 measured
 // no better than the 32x32 ones anywhere and are not instantiated.
 static const float kMfmaVariantEfficiency[kNumMfmaVariants] = {1.00f, 0.95f, 0.80f, 0.70f, 0.72f, 0.55f, 0.40f, 0.85f,
-                                                               1.05f, 0.89f, 0.40f};
+                                                               1.05f, 0.89f, 0.40f, 1.10f};
 
 static int pick_mfma_variant(const Lowered &l, uint32_t cus) {
   const GemmArgs &g = l.g;
@@ -401,7 +437,14 @@ static int pick_mfma_variant(const Lowered &l, uint32_t cus) {
     const MfmaVariant &t = kMfmaVariants[v];
     const uint64_t tiles = (uint64_t)ceil_div(np, t.bp) * ceil_div(nq, t.bq) * g.batch;
     if (t.stages > 4) continue;  // the deep ring: see below
-    if (t.m16) {
+    if (t.w4) {
+      // The four-wave kernel, for the problems its epilogues serve: level with the best other variant from one round of
+      // tiles on, 4-7 % ahead from four (8192^3: int8 410 us against 429, fp8 360 against 389; 8192 x 4096 x 4096 fp8
+      // 103 against 109; 4096^3 int8 59.4 against 59.5), but not on a short K, where the per-tile work around the loop
+      // shows (16384 x 8192 x 1024 fp8: 167 us against 153 for variant 0)
+      if (w4_epilogue_class(l, true) == W4_CLASS_NONE || g.K < 2048) continue;
+      if (tiles < (g.a_type == CUDA_R_8I ? ((uint64_t)cus * 3 + 3) / 4 : (uint64_t)cus)) continue;
+    } else if (t.m16) {
       const bool h16 = g.a_type == CUDA_R_16F || g.a_type == CUDA_R_16BF;
       if (type_bits(g.a_type) != 8 && !h16) continue;  // the 16x16 shapes serve int8, fp8, f16 and bf16
       // power bound or not: int8 gains from three quarters of the CUs busy on.  fp8 gains little and only on
@@ -541,7 +584,8 @@ using namespace zluda_amd;
 extern "C" uint32_t zluda_gemm_variant_count(uint32_t kernel) {
   switch (kernel) {
   case ZLUDA_KERNEL_GENERIC: return 1;
-  case ZLUDA_KERNEL_MFMA_I8: case ZLUDA_KERNEL_MFMA_F8: case ZLUDA_KERNEL_MFMA_H16: return kNumMfmaVariants;
+  case ZLUDA_KERNEL_MFMA_I8: case ZLUDA_KERNEL_MFMA_F8: return kNumMfmaVariants;
+  case ZLUDA_KERNEL_MFMA_H16: return kNumMfmaVariantsH16;
   case ZLUDA_KERNEL_MFMA_MXF4: case ZLUDA_KERNEL_MFMA_F32: return kNumMfmaVariants32;  // the 16x16-shape ones serve int8 and fp8
   case ZLUDA_KERNEL_DECODE_W8A8: return kNumDecodeVariants;
   case ZLUDA_KERNEL_MFMA_TR8: case ZLUDA_KERNEL_MFMA_TR16: return kNumTrVariants;
@@ -608,8 +652,11 @@ extern "C" uint32_t zluda_gemm_plan_problem(const zluda_gemm_problem *p, uint32_
   case ZLUDA_KERNEL_MFMA_F32: {
     int v = forced_variant >= 0 ? forced_variant : pick_mfma_variant(l, cu_count);
     if (v >= kNumMfmaVariants || (v >= kNumMfmaVariants32 && kernel != ZLUDA_KERNEL_MFMA_I8 && kernel != ZLUDA_KERNEL_MFMA_F8 &&
-                                  kernel != ZLUDA_KERNEL_MFMA_H16))
+                                  kernel != ZLUDA_KERNEL_MFMA_H16) || (v >= kNumMfmaVariantsH16 && kernel == ZLUDA_KERNEL_MFMA_H16))
       return CUBLAS_STATUS_INVALID_VALUE;
+    // the four-wave kernel exists for int8 and for e4m3 x e4m3 without block scales
+    if (kMfmaVariants[v].w4 && !(l.g.a_type == CUDA_R_8I || (l.g.a_type == CUDA_R_8F_E4M3 && l.g.b_type == CUDA_R_8F_E4M3)))
+      return CUBLAS_STATUS_NOT_SUPPORTED;
     fill_mfma_plan(l, v, cu_count, p->workspace_size, plan);
     // Skinny problems that end up with at most one 64 x 64 workgroup per CU and are not split along K are bound
     // by what a CU keeps in flight: the 6-stage ring of variant 10 (80 KiB instead of 32) takes 8-17 % less time

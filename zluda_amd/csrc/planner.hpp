@@ -8,25 +8,30 @@ namespace zluda_amd {
 
 // MFMA tile configurations (index = plan.variant for the MFMA families): workgroup tile bp x bq,
 // wp x wq waves, `bkb` bytes of K per LDS stage, `stages` LDS stages
-struct MfmaVariant { int bp, bq, wp, wq, bkb, stages, m16; };  // m16: the 16x16 MFMA shapes (gemm_mfma_pipe16.hpp; not MXFP4, not f32)
+struct MfmaVariant { int bp, bq, wp, wq, bkb, stages, m16, w4; };  // m16: the 16x16 MFMA shapes (gemm_mfma_pipe16.hpp; not MXFP4, not f32)
+                                                                // w4: the persistent four-wave kernel (gemm_mfma_w4.hpp; int8 and e4m3 x e4m3)
 constexpr MfmaVariant kMfmaVariants[] = {
-    {256, 256, 2, 4, 128, 2, 0},  // 0: 8 waves, 128x64 per wave
-    {256, 256, 2, 2, 128, 2, 0},  // 1: 4 waves, 128x128 per wave
-    {256, 128, 2, 2, 128, 2, 0},  // 2: 4 waves, 128x64 per wave
-    {128, 128, 2, 2, 128, 2, 0},  // 3: 4 waves, 64x64 per wave, two workgroups per CU
-    {128, 128, 2, 2, 64, 4, 0},   // 4: same tile, half-line stages, deeper ring (short K)
-    {128, 64, 2, 2, 128, 3, 0},   // 5: 4 waves, 64x32 per wave: skinny problems
-    {64, 64, 2, 2, 128, 3, 0},    // 6: 4 waves, 32x32 per wave: problems of a few hundred tiles at most
-    {192, 256, 2, 4, 128, 2, 0},  // 7: 8 waves, 96x64 per wave: extents that 256 divides badly (3072, 6144, ...)
+    {256, 256, 2, 4, 128, 2, 0, 0},  // 0: 8 waves, 128x64 per wave
+    {256, 256, 2, 2, 128, 2, 0, 0},  // 1: 4 waves, 128x128 per wave
+    {256, 128, 2, 2, 128, 2, 0, 0},  // 2: 4 waves, 128x64 per wave
+    {128, 128, 2, 2, 128, 2, 0, 0},  // 3: 4 waves, 64x64 per wave, two workgroups per CU
+    {128, 128, 2, 2, 64, 4, 0, 0},   // 4: same tile, half-line stages, deeper ring (short K)
+    {128, 64, 2, 2, 128, 3, 0, 0},   // 5: 4 waves, 64x32 per wave: skinny problems
+    {64, 64, 2, 2, 128, 3, 0, 0},    // 6: 4 waves, 32x32 per wave: problems of a few hundred tiles at most
+    {192, 256, 2, 4, 128, 2, 0, 0},  // 7: 8 waves, 96x64 per wave: extents that 256 divides badly (3072, 6144, ...)
     // the same tiles on v_mfma_*_16x16x* (int8, fp8, f16, bf16): less energy per multiply-add, and GEMMs that keep the
     // chip busy are power bound
-    {256, 256, 2, 4, 128, 2, 1},  // 8: variant 0's
-    {192, 256, 2, 4, 128, 2, 1},  // 9: variant 7's
+    {256, 256, 2, 4, 128, 2, 1, 0},  // 8: variant 0's
+    {192, 256, 2, 4, 128, 2, 1, 0},  // 9: variant 7's
     // skinny, memory-bound problems of at most one workgroup per CU: variant 6's tile with a ring of 6 stages, i.e. 80 KiB
     // instead of 32 KiB of operand rows in flight per CU (not MXFP4: its scale chunks span 4 stages)
-    {64, 64, 2, 2, 128, 6, 0},    // 10
+    {64, 64, 2, 2, 128, 6, 0, 0},    // 10
+    // variant 8's tile with four waves of 128 x 128, one workgroup per CU walking a list of tiles (int8 and e4m3 x e4m3 with
+    // the epilogues of kW4Epilogues below; no split along K): 4-6 % less time than variant 8 on grids of several rounds
+    {256, 256, 2, 2, 128, 2, 1, 1},  // 11
 };
 constexpr int kNumMfmaVariants32 = 8;  // the first ones, on the 32x32 shapes: what MXFP4 has
+constexpr int kNumMfmaVariantsH16 = 11;  // f16 / bf16: everything but the four-wave kernel
 constexpr int kNumMfmaVariants = sizeof(kMfmaVariants) / sizeof(kMfmaVariants[0]);
 
 // tile configurations of the transposing 8-bit MFMA kernel (index = plan.variant for
@@ -83,8 +88,13 @@ constexpr int kDecodeAutoMaxTokensStream = 48;  // ... and when the LDS-streamin
                                                 // (14336x56x4096: 21 us against 19); three blocks only up to 32 rows per CU
                                                 // (planner.cpp: beyond, the 6-stage 64 x 64 tiles are as fast or faster)
 
+// the fast epilogues the four-wave kernel is instantiated with (gemm_mfma_w4.hpp: W4_EPI_*); what else a problem asks for
+// runs on variant 8
+enum { W4_CLASS_NONE = -1, W4_CLASS_I32 = 0, W4_CLASS_BF16 = 1, W4_CLASS_BF16_GELU = 2 };
+
 struct Lowered {
   GemmArgs g;
+  bool has_bias;              // the epilogue adds a bias vector (its pointer may still be NULL when planning)
   bool a_kcontig, b_kcontig;  // unit K stride
   bool aligned16;             // A, B, their row pitches and batch strides are 16-byte aligned
   bool span_ok;               // one batch of A and of B each spans < 2 GiB
@@ -93,6 +103,10 @@ struct Lowered {
 // Validates `p` and fills `out`.  With dry=true (heuristic time) data pointers and host scalars are
 // not dereferenced and NULL data pointers are allowed.
 uint32_t lower_problem(const zluda_gemm_problem *p, bool dry, Lowered *out);
+
+// the fast epilogue of the four-wave kernel that serves the problem, or W4_CLASS_NONE; `dry`: planning (beta and the
+// pointers are not known yet and are taken to be zero / aligned)
+int w4_epilogue_class(const Lowered &l, bool dry);
 
 // which kernel families can run the lowered problem
 bool family_supports(uint32_t kernel, const Lowered &l);
