@@ -8,15 +8,21 @@ on.  The other benchmark configurations, the 8192^3 int8 case and configuration 
 ride along under "also", each with its own roofline figures and, when the installed hipBLASLt has a
 solution, the time of the reference's hipBLASLt-forwarded path on the same buffers.
 
-Timing: W warm-up calls (default: half a second's worth, so that the power management has settled), then
-exactly K calls between two synchronisations (wall clock -> `value`); HIP
+Timing: first an untimed stretch of calls of `--settle` seconds (default 0.5: the power management needs a few
+hundred milliseconds of load to settle, and what a burst shows before that is up to 15 % off what a running job
+sees), then W warm-up calls, then exactly K calls between two synchronisations (wall clock -> `value`); HIP
 events on the launch stream split the K calls into five batches, and `roofline.kernel_ms` is the median
 batch.  A one-wave probe kernel on a second stream samples the shader cycle counter against the real-time
 counter during one more (untimed) batch: `clock_mhz_observed`, and `frac_at_observed_clock` = the
 roofline fraction against the datasheet peak scaled to that clock (the peak assumes 2400 MHz).
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c2|c3|c4|c5|c5_b1|i8_8192|i8_4096_nt] [--only]
-                  [--no-cpu] [--no-hipblaslt] [--copy-probe] [--sustained SECONDS]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--settle SECONDS] [--workload c1|c2|c3|c4|c5|c5_b1|i8_8192|...] [--only]
+                  [--also LIST] [--no-cpu] [--no-hipblaslt] [--copy-probe] [--sustained SECONDS] [--full]
+
+The line the script prints stays under 8 KB: the headline's figures, then under "also" one compact entry per other
+workload in the order the metric names them (decode, int8 8192^3, MXFP4, ...).  `roofline.vs_hipblaslt` is the
+headline's rate over the hipBLASLt-forwarded path's on the same buffers, `roofline.decode_c3` the decode half of the
+metric.  --full prints every workload's whole record instead (for profiles/ and notes).
 """
 import argparse
 import ctypes as C
@@ -192,28 +198,33 @@ class Buffers:
 NBATCH = 5
 
 
-AUTO_WARMUP_SECONDS = 0.5
+SETTLE_SECONDS = 0.5   # --settle: untimed stretch of calls in front of every measurement
+DEFAULT_WARMUP = 10
 
 
-def time_calls(torch, fn, steps, warmup):
-    """`warmup` untimed calls, then exactly `steps` calls between two synchronisations.  warmup < 0: as many
-    calls as take AUTO_WARMUP_SECONDS (at least 10) -- the power management needs a few hundred milliseconds
-    of load to settle, and a burst measured before that is up to 15 % slower than what a long-running job sees.
+def settle(torch, fn, seconds):
+    """Back-to-back calls for `seconds` (no timing): under matrix load the part reaches its power cap after a few hundred
+    milliseconds, and only then does a short measurement show what a long-running job sees.  Returns the calls made."""
+    if seconds <= 0:
+        return 0
+    t0, n, chunk = time.perf_counter(), 0, 8
+    while time.perf_counter() - t0 < seconds:
+        for i in range(chunk):
+            fn(n + i)
+        n += chunk
+        torch.cuda.synchronize()   # bounds the queue: the stretch ends when the clock says so, not thousands of calls later
+        chunk = min(chunk * 2, 256)
+    return n
+
+
+def time_calls(torch, fn, steps, warmup, settle_s=None):
+    """An untimed settle stretch, `warmup` untimed calls, then exactly `steps` calls between two synchronisations.
     Returns (wall seconds for the `steps` calls, median over NBATCH equal batches of the seconds per call by HIP
-    events on the launch stream, [seconds per call of each batch], warm-up calls made)."""
+    events on the launch stream, [seconds per call of each batch], warm-up calls made, settle calls made)."""
+    settled = settle(torch, fn, SETTLE_SECONDS if settle_s is None else settle_s)
     if warmup < 0:
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for i in range(10):
-            fn(i)
-        e1.record()
-        e1.synchronize()
-        per = max(e0.elapsed_time(e1) * 1e-3 / 10, 1e-6)
-        warmup = 10 + min(int(AUTO_WARMUP_SECONDS / per), 100000)
-        first = 10
-    else:
-        first = 0
-    for i in range(first, warmup):
+        warmup = DEFAULT_WARMUP
+    for i in range(warmup):
         fn(i)
     torch.cuda.synchronize()
     nb = NBATCH if steps % NBATCH == 0 else 1
@@ -228,7 +239,7 @@ def time_calls(torch, fn, steps, warmup):
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     batches = sorted(ev[b].elapsed_time(ev[b + 1]) * 1e-3 / per for b in range(nb))
-    return wall, batches[len(batches) // 2], batches, warmup
+    return wall, batches[len(batches) // 2], batches, warmup, settled
 
 
 _probe = None
@@ -352,14 +363,15 @@ def run_workload(torch, api, key, steps, warmup, with_hipblaslt):
         st = call.run(alpha, a_ptrs[i % copies], bp, zero, None, dp, None, 0, stream)
         if st:
             raise RuntimeError("cublasLtMatmul status %d on workload %s" % (st, key))
-    wall, per_call, batches, warmed = time_calls(torch, ours, steps, warmup)
+    wall, per_call, batches, warmed, settled = time_calls(torch, ours, steps, warmup)
     bound = "hbm" if w["kind"] == "hbm" else "mfma"
     achieved = (nbytes / per_call / 1e9) if bound == "hbm" else (ops / per_call / 1e12)
     peak = PEAK[w["kind"]]
     traffic, traffic_file = measured_traffic(key)
     clock = observed_clock_mhz(torch, ours, max(steps // NBATCH, 4), per_call)
     res = {
-        "workload": w["name"], "steps": steps, "warmup": warmed, "ms_per_step": wall / steps * 1e3,
+        "workload": w["name"], "steps": steps, "warmup": warmed, "settle_s": SETTLE_SECONDS, "settle_calls": settled,
+        "ms_per_step": wall / steps * 1e3,
         "tops": ops / (wall / steps) / 1e12, "gbps": nbytes / (wall / steps) / 1e9,
         "kernel": {"family": call.kernel, "variant": call.variant},
         "roofline": {"bound": bound, "achieved": achieved, "peak": peak, "unit": "GB/s" if bound == "hbm" else "TFLOP/s",
@@ -404,7 +416,7 @@ def time_hipblaslt(torch, spec, buf, alpha, zero, a_ptrs, copies, steps, warmup,
             st = rp.run(alpha, a_ptrs[i % copies], bp, zero, None, dp, stream)
             if st:
                 raise RuntimeError("hipblasLtMatmul status %d" % st)
-        wall, per_call, _, _ = time_calls(torch, theirs, steps, warmup)
+        wall, per_call, _, _, _ = time_calls(torch, theirs, steps, warmup)
         clock = observed_clock_mhz(torch, theirs, max(steps // NBATCH, 4), per_call)
         sus = sustained(torch, theirs, SUSTAIN_SECONDS) if SUSTAIN_SECONDS > 0 else None
         rp.close()
@@ -445,14 +457,47 @@ def cpu_baseline(key, budget_s=12.0):
                                               "; rate of the slab, extrapolated to the whole problem" if rows < full_m else "", dt)}
 
 
+ALSO_DEFAULT = ("c3", "i8_8192", "c5", "c5_b1", "c2", "c1", "i8_4096_nt", "decode_k13824")   # the order the metric names them in
+ALSO_KEYS = {"c3": "decode_c3"}
+
+
+def compact(res):
+    """one workload's record cut down to what the line has room for"""
+    r = res["roofline"]
+    out = {"ms": round(r["kernel_ms"], 5), "frac": round(r["frac"], 4), "kernel": "%d/%d" % (res["kernel"]["family"], res["kernel"]["variant"])}
+    if r["bound"] == "hbm":
+        out["gbps"] = round(r["achieved"], 1)
+        if "flat_read_gbps" in r:
+            out["flat_read_gbps"] = round(r["flat_read_gbps"], 1)
+    else:
+        out["tops"] = round(r["achieved"], 1)
+    if r.get("traffic"):
+        out["traffic"] = r["traffic"]
+    h = res.get("hipblaslt_forwarded")
+    if h is not None:
+        if h.get("available"):
+            out["hipblaslt_ms"] = round(h["kernel_ms"], 5)
+            out["vs_hipblaslt"] = round(h["kernel_ms"] / r["kernel_ms"], 3)
+        else:
+            out["hipblaslt"] = (h.get("why") or "unavailable")[:60]
+    if res.get("sustained"):
+        out["sustained_us"] = round(res["sustained"]["us_per_call"], 1)
+    return out
+
+
 def main():
+    global SUSTAIN_SECONDS, SETTLE_SECONDS
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=0)
-    ap.add_argument("--warmup", type=int, default=-1,
-                    help="untimed calls before the timed ones; default: as many as take %.1f s (at least 10)" % AUTO_WARMUP_SECONDS)
+    ap.add_argument("--warmup", type=int, default=-1, help="untimed calls between the settle stretch and the timed calls (default %d)" % DEFAULT_WARMUP)
+    ap.add_argument("--settle", type=float, default=SETTLE_SECONDS, metavar="SECONDS",
+                    help="untimed stretch of calls in front of every measurement, whatever --warmup says: the power "
+                         "management needs a few hundred milliseconds of load to settle (0 = off)")
     ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS))
     ap.add_argument("--only", action="store_true", help="skip the other workloads")
+    ap.add_argument("--also", default=",".join(ALSO_DEFAULT), help="the other workloads to run, in order (default: %(default)s)")
+    ap.add_argument("--full", action="store_true", help="whole records for every workload instead of the compact line")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-hipblaslt", action="store_true")
     ap.add_argument("--sustained", type=float, default=0.0, metavar="SECONDS",
@@ -468,8 +513,8 @@ def main():
         sys.exit("bench.py needs a HIP device; there is no CPU path to benchmark")
     api = cublaslt.load()
     torch.cuda.init()
-    global SUSTAIN_SECONDS
     SUSTAIN_SECONDS = args.sustained
+    SETTLE_SECONDS = max(args.settle, 0.0)
     key = args.workload
     steps = args.steps or WORKLOADS[key]["steps"]
     if args.copy_probe:
@@ -481,8 +526,8 @@ def main():
     head = run_workload(torch, api, key, steps, args.warmup, not args.no_hipblaslt)
     also = {}
     if not args.only:
-        for other in ("c4", "i8_8192", "c3", "c5", "c5_b1", "c2", "c1", "i8_4096_nt", "decode_k13824", "bf16_8192", "bf16_8192_nn"):
-            if other == key:
+        for other in [o for o in args.also.split(",") if o]:
+            if other == key or other not in WORKLOADS:
                 continue
             try:
                 also[other] = run_workload(torch, api, other, WORKLOADS[other]["steps"], args.warmup, not args.no_hipblaslt)
@@ -490,21 +535,36 @@ def main():
                 also[other] = {"error": "%s: %s" % (type(e).__name__, e)}
             torch.cuda.empty_cache()
     unit = "GB/s" if WORKLOADS[key]["kind"] == "hbm" else "TOPS"
+    roof = dict(head["roofline"])
+    if not args.full:
+        roof.pop("kernel_ms_batches", None)
+    hb = head.get("hipblaslt_forwarded") or {}
+    if hb.get("available"):
+        # the reference's forwarded path on the same buffers, same timing: its rate and ours over it
+        roof["hipblaslt_tops" if unit == "TOPS" else "hipblaslt_gbps"] = hb["tops"] if unit == "TOPS" else hb["gbps"]
+        roof["vs_hipblaslt"] = hb["kernel_ms"] / head["roofline"]["kernel_ms"]
+    elif hb:
+        roof["hipblaslt"] = (hb.get("why") or "unavailable")[:80]
+    c3 = also.get("c3")
+    if c3 and "roofline" in c3:   # the decode half of the metric, where the driver keeps it
+        r3 = c3["roofline"]
+        roof["decode_c3"] = {"gbps": r3["achieved"], "frac": r3["frac"], "kernel_ms": r3["kernel_ms"], "peak": r3["peak"],
+                             "flat_read_gbps": r3.get("flat_read_gbps")}
     line = {
         "metric": "cublasLtMatmul TOPS (int8/fp8/MXFP4, 8192^3) + decode GEMM HBM GB/s",
         "value": head["gbps"] if unit == "GB/s" else head["tops"], "unit": unit, "n_gpus": 1, "steps": steps,
         "warmup": head["warmup"], "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": {"i8": "int8", "hbm": "int8", "f8": "fp8_e4m3", "f4": "fp4_e2m1", "bf16": "bf16"}[WORKLOADS[key]["kind"]],
         "data": "synthetic", "config": {"workload": head["workload"], "kernel": head["kernel"]},
-        "roofline": head["roofline"],
-        "clock_mhz_observed": head["roofline"].get("clock_mhz_observed"),
-        "frac_at_observed_clock": head["roofline"].get("frac_at_observed_clock"),
+        "settle_s": head["settle_s"],
+        "roofline": roof,
         "cpu_baseline": None if args.no_cpu else cpu_baseline(key),
         "sustained": head.get("sustained"),
-        "hipblaslt_forwarded": head.get("hipblaslt_forwarded"),
         "device": torch.cuda.get_device_name(0), "cu_count": api.zluda_gemm_device_cu_count(),
-        "also": also,
+        "also": also if args.full else {k: (v if "error" in v else compact(v)) for k, v in also.items()},
     }
+    if args.full:
+        line["hipblaslt_forwarded"] = head.get("hipblaslt_forwarded")
     print(json.dumps(line))
 
 

@@ -56,6 +56,7 @@ typedef struct zluda_matmul_desc {
   void *epilogue_aux;
   int64_t epilogue_aux_ld;
   int64_t epilogue_aux_batch_stride;
+  int32_t epilogue_aux_type; /* cudaDataType or -1 (= D's type, the only one served: anything else is NOT_SUPPORTED) */
 } zluda_matmul_desc;
 
 /* A fully specified matmul: what cublasLtMatmul receives (cuda_macros/src/cublaslt.rs:58-75). */
@@ -118,7 +119,9 @@ uint32_t zluda_gemm_launch(const zluda_gemm_problem *p, const zluda_gemm_plan *p
  * library runs on holds its own copy until the process ends); `p->workspace` is ignored.  Plan with
  * p->workspace_size = ZLUDA_GEMM_STATIC_SCRATCH_BYTES so that zluda_gemm_plan_problem sizes the split for it;
  * a plan that needs more returns CUBLAS_STATUS_ALLOC_FAILED (3) and launches nothing.  The call allocates and
- * frees nothing (the first call on a device looks up the array's address).  All calls on one device share that
+ * frees nothing.  The first call on a device looks up the array's address, which it will not do while `stream` is
+ * being captured (CUBLAS_STATUS_NOT_SUPPORTED): make one call on the device outside the capture first; from then on
+ * calls may be captured.  All calls on one device -- replays of a captured graph included -- share that
  * device's array: calls that may overlap on one device (two streams, two threads) race on it and must be
  * serialised by the caller; nothing in it needs clearing between calls. */
 #define ZLUDA_GEMM_STATIC_SCRATCH_BYTES (32u << 20)

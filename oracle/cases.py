@@ -252,6 +252,7 @@ class Case:
         o.c_scale, o.d_scale = ptrs.get("c_scale"), ptrs.get("d_scale")
         o.epilogue_aux = ptrs.get("aux")
         o.epilogue_aux_ld, o.epilogue_aux_batch_stride = s.get("aux_ld", 0), s.get("aux_batch_stride", 0)
+        o.epilogue_aux_type = s.get("aux_type", -1)
         p.alpha, p.beta = ptrs["alpha"], ptrs["beta"]
         p.A, p.B, p.C, p.D = ptrs["A"], ptrs["B"], ptrs.get("C"), ptrs["D"]
         return p

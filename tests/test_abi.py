@@ -123,7 +123,8 @@ def test_matmul_desc_attributes(api):
     assert api.desc_set(d, D.CUBLASLT_MATMUL_DESC_EPILOGUE_AUX_LD, C.c_int64, 4096) == 0
     assert api.desc_set(d, D.CUBLASLT_MATMUL_DESC_EPILOGUE_AUX_BATCH_STRIDE, C.c_int64, 1 << 24) == 0
     assert api.desc_set(d, D.CUBLASLT_MATMUL_DESC_EPILOGUE_AUX_LD, C.c_int32, 4096) == IV
-    assert api.desc_set(d, 22, C.c_int32, -1) == 0 and api.desc_set(d, 22, C.c_int32, D.CUDA_R_8F_E4M3) == NS   # EPILOGUE_AUX_DATA_TYPE
+    # EPILOGUE_AUX_DATA_TYPE: kept in the descriptor (a type other than D's is refused when the problem is planned)
+    assert api.desc_set(d, 22, C.c_int32, D.CUDA_R_16BF) == 0 and api.desc_set(d, 22, C.c_int32, -1) == 0
     # everything else: NOT_SUPPORTED (impl.rs:302)
     assert api.desc_set(d, 23, C.c_void_p, 1) == NS   # EPILOGUE_AUX_SCALE_POINTER
     assert api.cublasLtMatmulDescSetAttribute(d, D.CUBLASLT_MATMUL_DESC_TRANSA, None, 4) == IV

@@ -40,3 +40,16 @@ def test_every_packed_instantiation_issues_exactly_the_counted_factor_loads(tmp_
                 found[name], name = n, None
     assert len(found) == len(insts), sorted(found)
     assert all(v == counted for v in found.values()), (counted, found)
+
+
+@pytest.mark.skipif(shutil.which("g++") is None, reason="needs g++")
+def test_no_issued_dma_instruction_is_wholly_out_of_range(tmp_path):
+    """The counted waits of the slab kernel assume that loads retire in the order they were issued, which an instruction
+    whose 64 lanes are all out of range does not do.  tests/host_c/slab_addr_check.cpp runs the kernel's own addressing
+    functions (kernels/decode_slab_addr.hpp) on the host over every shape and K the launcher gives the kernel: every
+    instruction has a lane in range, and the lanes in range fetch each K byte of each row exactly once."""
+    exe = tmp_path / "slab_addr_check"
+    subprocess.run(["g++", "-O2", "-std=c++17", os.path.join(ROOT, "tests", "host_c", "slab_addr_check.cpp"), "-o", str(exe)], check=True)
+    res = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert res.returncode == 0, res.stdout
+    assert int(res.stdout.split()[0]) > 300

@@ -87,6 +87,20 @@ def test_fp8_scaled_bias_gelu_within_tolerance_of_hipblaslt(gpu_api):
     print("max relative difference to hipBLASLt %.3e" % err)
 
 
+def test_config4_fp8_8192_within_tolerance_of_hipblaslt(gpu_api):
+    """benchmark configuration 4 at its own size and with its own recipe (x ~ N(0,1), q = e4m3(x * 448 / max|x|), per-tensor
+    scales max|x| / 448, bf16 bias ~ N(0, 0.02), GELU, bf16 D), element by element against hipBLASLt called the way the
+    reference forwards it.  Both sides use the fp8 MFMA, so the strict floor applies."""
+    spec = dict(F8, m=8192, n=8192, k=8192, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS, bias_type=K.CUDA_R_16BF,
+                f8_amax_quant=True, bias_std=0.02)
+    case, ours, theirs, why, kern = both(gpu_api, spec, 3)
+    assert kern == K.ZLUDA_KERNEL_MFMA_F8
+    if theirs is None:
+        pytest.skip("hipBLASLt offers no algorithm here: " + why)
+    err = case.compare(ours, theirs, tol=1e-2, floor_frac=1e-2)
+    print("max relative difference to hipBLASLt at 8192^3 %.3e" % err)
+
+
 def test_decode_config3_decomposed_through_hipblaslt(gpu_api):
     """benchmark configuration 3 at full size.  hipBLASLt has no int8 -> bf16 algorithm with an alpha vector, so
     the reference's backend pins the integer part: its int8 -> int32 GEMM of the same operands, followed on

@@ -439,5 +439,9 @@ def test_bias_gradient_epilogues_are_planned_like_the_plain_problem(api):
         assert plan(api, dict(f8, epilogue=epi))[0] == K.CUBLAS_STATUS_INVALID_VALUE
         assert plan(api, dict(f8, epilogue=epi, aux_ld=504))[0] == K.CUBLAS_STATUS_INVALID_VALUE
         assert plan(api, dict(f8, epilogue=epi, aux_ld=512, d_type=K.CUDA_R_8F_E4M3))[0] == K.CUBLAS_STATUS_NOT_SUPPORTED
+        # the aux matrix has D's type: naming that type is the same as leaving the default, any other type is not served
+        assert plan(api, dict(f8, epilogue=epi, aux_ld=512, aux_type=K.CUDA_R_16BF))[0] == 0
+        assert plan(api, dict(f8, epilogue=epi, aux_ld=512, aux_type=K.CUDA_R_16F))[0] == K.CUBLAS_STATUS_NOT_SUPPORTED
+        assert plan(api, dict(f8, epilogue=epi, aux_ld=512, aux_type=K.CUDA_R_8F_E4M3))[0] == K.CUBLAS_STATUS_NOT_SUPPORTED
     st, _ = plan(api, dict(I8, m=512, n=512, k=512, transa=1, epilogue=K.CUBLASLT_EPILOGUE_GELU_AUX, aux_ld=512))   # int32 scale type
     assert st == K.CUBLAS_STATUS_NOT_SUPPORTED

@@ -81,3 +81,47 @@ def test_noalloc_rejects_a_plan_beyond_the_scratch(gpu_api):
     torch.cuda.synchronize()
     assert st == K.CUBLAS_STATUS_ALLOC_FAILED
     assert bool((dt[case._guard:case._guard + 64] == 0xCD).all()), "nothing may have been launched"
+
+
+def test_noalloc_under_graph_capture_after_a_warm_up_call(gpu_api):
+    """the entry point is for callers that record their GEMMs into a HIP graph: after one call outside the capture
+    (which looks up the scratch array) a split-K call is captured and replayed three times with fresh operands in
+    between, every replay against the workspace entry point's result for the same operands"""
+    import torch
+    spec = dict(I8, m=256, n=256, k=16384)
+    case = Case(spec, 710)
+    keep, ptr, dt = case.upload()
+    ptrs = dict(ptr)
+    ptrs["alpha"], ptrs["beta"] = case.alpha.ctypes.data, case.beta.ctypes.data
+    p = case.problem(ptrs)
+    p.workspace_size = SCRATCH
+    plan = abi.zluda_gemm_plan()
+    assert gpu_api.zluda_gemm_plan_problem(C.byref(p), K.ZLUDA_KERNEL_MFMA_I8, -1, gpu_api.zluda_gemm_device_cu_count(), C.byref(plan)) == 0
+    assert plan.grid_z > 1
+    p.workspace = None
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        assert gpu_api.zluda_gemm_launch_noalloc(C.byref(p), C.byref(plan), side.cuda_stream) == 0   # the warm-up call
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            assert gpu_api.zluda_gemm_launch_noalloc(C.byref(p), C.byref(plan), torch.cuda.current_stream().cuda_stream) == 0
+    ws = torch.empty(plan.workspace, dtype=torch.uint8, device="cuda:0")
+    for replay in range(3):
+        fresh = Case(spec, 720 + replay)
+        case.A = fresh.A
+        raw = np.frombuffer(case.A.tobytes(), dtype=np.uint8)
+        keep[0][:raw.size] = torch.from_numpy(raw.copy()).to("cuda:0")
+        canary = np.frombuffer(case.new_d().tobytes(), dtype=np.uint8)
+        dt[:canary.size] = torch.from_numpy(canary.copy()).to("cuda:0")
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = case.download(dt)
+        dt[:canary.size] = torch.from_numpy(canary.copy()).to("cuda:0")
+        p.workspace, p.workspace_size = ws.data_ptr(), plan.workspace
+        assert gpu_api.zluda_gemm_launch(C.byref(p), C.byref(plan), torch.cuda.current_stream().cuda_stream) == 0
+        torch.cuda.synchronize()
+        p.workspace, p.workspace_size = None, SCRATCH
+        assert np.array_equal(got, case.download(dt)), "replay %d" % replay
+        case.compare(got, case.run_oracle())

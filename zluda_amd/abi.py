@@ -169,7 +169,8 @@ class zluda_matmul_desc(C.Structure):
                 ("a_scale", C.c_void_p), ("b_scale", C.c_void_p), ("c_scale", C.c_void_p),
                 ("d_scale", C.c_void_p), ("a_scale_mode", C.c_int32), ("b_scale_mode", C.c_int32),
                 ("c_scale_mode", C.c_int32), ("d_scale_mode", C.c_int32), ("fast_accum", C.c_int8),
-                ("epilogue_aux", C.c_void_p), ("epilogue_aux_ld", C.c_int64), ("epilogue_aux_batch_stride", C.c_int64)]
+                ("epilogue_aux", C.c_void_p), ("epilogue_aux_ld", C.c_int64), ("epilogue_aux_batch_stride", C.c_int64),
+                ("epilogue_aux_type", C.c_int32)]
 
 
 class zluda_gemm_problem(C.Structure):

@@ -176,12 +176,9 @@ cublasStatus_t desc_attr(MatmulDescObj *o, uint32_t attr, bool set, const void *
   case CUBLASLT_MATMUL_DESC_EPILOGUE_AUX_POINTER: return access(set, d.epilogue_aux, in, out, size, written);
   case CUBLASLT_MATMUL_DESC_EPILOGUE_AUX_LD: return access(set, d.epilogue_aux_ld, in, out, size, written);
   case CUBLASLT_MATMUL_DESC_EPILOGUE_AUX_BATCH_STRIDE: return access(set, d.epilogue_aux_batch_stride, in, out, size, written);
-  case CUBLASLT_MATMUL_DESC_EPILOGUE_AUX_DATA_TYPE: {
-    int32_t v = -1;  // the aux matrix has D's type
-    cublasStatus_t st = access(set, v, in, out, size, written);
-    if (set && !st && v != -1) return CUBLAS_STATUS_NOT_SUPPORTED;
-    return st;
-  }
+  // -1 or D's own type (what frameworks that set it pass for 16-bit outputs); which of the two it is can only be told
+  // once D's layout is known, so the value is kept and the problem refused when it is lowered (planner.cpp)
+  case CUBLASLT_MATMUL_DESC_EPILOGUE_AUX_DATA_TYPE: return access(set, d.epilogue_aux_type, in, out, size, written);
   case CUBLASLT_MATMUL_DESC_ALPHA_VECTOR_BATCH_STRIDE:
     return access(set, d.alpha_vector_batch_stride, in, out, size, written);
   case CUBLASLT_MATMUL_DESC_SM_COUNT_TARGET: return access(set, o->sm_count_target, in, out, size, written);
@@ -279,6 +276,7 @@ void init_desc(MatmulDescObj *o, cublasComputeType_t computeType, cudaDataType_t
   o->d.transa = o->d.transb = CUBLAS_OP_N;
   o->d.epilogue = CUBLASLT_EPILOGUE_DEFAULT;
   o->d.bias_type = -1;
+  o->d.epilogue_aux_type = -1;
 }
 void init_pref(PrefObj *o) {
   memset(o, 0, sizeof(*o));
@@ -651,7 +649,7 @@ static int families_for_types(uint32_t computeType, uint32_t scaleType, uint32_t
                               uint32_t D, int *ids) {
   zluda_gemm_problem p;
   memset(&p, 0, sizeof(p));
-  p.op.compute_type = computeType; p.op.scale_type = scaleType; p.op.bias_type = -1;
+  p.op.compute_type = computeType; p.op.scale_type = scaleType; p.op.bias_type = -1; p.op.epilogue_aux_type = -1;
   p.op.transa = CUBLAS_OP_T; p.op.transb = CUBLAS_OP_N; p.op.epilogue = CUBLASLT_EPILOGUE_DEFAULT;
   const uint64_t n = 1024;
   p.a = {A, CUBLASLT_ORDER_COL, n, n, (int64_t)n, 1, (int64_t)(n * n)};

@@ -31,6 +31,7 @@
 // (c & 48) | ((c ^ rho) & 15) of the row's KiB: the DMA of a row lands linearly (lane l fetches the chunk whose
 // position is l) and the 16-rows-same-chunk fragment reads hit 16 different bank groups.
 #pragma once
+#include "decode_slab_addr.hpp"
 #include "decode_stream.hpp"
 
 namespace zluda_amd {
@@ -107,16 +108,12 @@ __global__ __launch_bounds__(NW * 64) void decode_slab_kernel(DecodeParams prm) 
   const int half = RPI == 2 ? lane >> 5 : 0;
   int dma_off[NDMA];
 #pragma unroll
-  for (int i = 0; i < NDMA; i++) {
-    const int rho = RPI * i + half, pos = RPI == 2 ? lane & 31 : lane;
-    dma_off[i] = ((pos & ~15) | ((pos ^ rho) & 15)) << 4;
-  }
-  // vector offset of instruction i in unit q of the wave's slab, `pitch` = what the odd row adds
-  auto unit_voff = [&](int i, int q, int pitch) {
-    const int off = q * UB + dma_off[i];
-    const bool in = !TAIL || (off < kw && kwave + off < K);
-    return in ? kwave + off + pitch : (int)0x80000000;
-  };
+  for (int i = 0; i < NDMA; i++) dma_off[i] = slab_dma_offset(UB, lane, i);
+  // vector offset of instruction i in unit q of the wave's slab, `pitch` = what the odd row adds.  A unit that holds
+  // no byte of K (decode_slab_addr.hpp) is fetched as real loads and its MFMAs are skipped: no instruction the kernel
+  // issues has all of its lanes out of range, which the counted waits below depend on.
+  auto unit_voff = [&](int i, int q, int pitch) { return slab_unit_voff(TAIL, UB, dma_off[i], q, kw, kwave, K, pitch); };
+  auto unit_empty = [&](int q) { return slab_unit_empty(TAIL, UB, q, kw, kwave, K); };  // (wave-uniform)
   auto issue_w = [&](int b, int q, int slot) {
     const int rb = row_base(b), re = row_end(b);
     v4i *dst = &ring[wave][slot][0];
@@ -263,6 +260,7 @@ __global__ __launch_bounds__(NW * 64) void decode_slab_kernel(DecodeParams prm) 
         for (int f = 0; f < NFRAG; f++) w[f] = lds_read16_unordered(frag_addr(n & 1, f));
         lds_values_ready(w);  // in registers before the slot is refilled
         if ((n + 2) / Q < nblk) issue_unit(n + 2, n & 1);
+        if (unit_empty(q)) continue;  // (fetched for the count only)
 #pragma unroll
         for (int nbk = 0; nbk < NB; nbk++) {
           if constexpr (KIND == KIND_I8) {

@@ -1,0 +1,45 @@
+// Addressing of the slab decode kernel's DMA instructions (decode_slab.hpp), in plain C++ so that the same
+// functions run in the kernel and in a host-side check of what the kernel issues.
+//
+// A wave's slab of a 16-row block is Q units of 16 rows x UB bytes of K; DMA instruction i of a unit fills rows
+// RPI * i .. RPI * i + RPI - 1 of the slot linearly (RPI = 1024 / UB rows of UB bytes each): the lane at position p
+// of row rho fetches the chunk whose position is p, i.e. chunk (p & ~15) | ((p ^ rho) & 15) of the row's UB bytes.
+#pragma once
+
+#if defined(__HIPCC__)
+#define ZLUDA_SLAB_FN __host__ __device__ inline
+#else
+#define ZLUDA_SLAB_FN inline
+#endif
+
+namespace zluda_amd {
+
+constexpr int kSlabOutOfRange = (int)0x80000000;  // a vector offset with bit 31 set: the lane fetches nothing, its LDS bytes read as zero
+
+// byte offset inside the unit's UB bytes of K that lane `lane` of instruction `i` fetches
+ZLUDA_SLAB_FN int slab_dma_offset(int ub, int lane, int i) {
+  const int rpi = 1024 / ub;
+  const int half = rpi == 2 ? lane >> 5 : 0;
+  const int rho = rpi * i + half, pos = rpi == 2 ? lane & 31 : lane;
+  return ((pos & ~15) | ((pos ^ rho) & 15)) << 4;
+}
+
+// Unit q of a wave's slab holds no byte of K: the wave's share kw of K ends before it, or K itself does (kwave = first
+// K byte of the wave).  Such a unit is fetched all the same -- the number of operations in flight is what the counted
+// waits rely on -- but as real loads of bytes nobody multiplies: an instruction whose lanes are ALL out of range
+// completes without a memory round trip and can retire ahead of older loads, which would let a counted wait pass
+// while an older unit is still in flight.
+ZLUDA_SLAB_FN bool slab_unit_empty(bool tail, int ub, int q, int kw, int kwave, int K) {
+  return tail && (q * ub >= kw || kwave + q * ub >= K);
+}
+
+// vector offset (bytes from the row's start) of lane `lane` of instruction `i` in unit `q`; `dma_off` =
+// slab_dma_offset(ub, lane, i), `pitch` = what the odd row of a two-row instruction adds
+ZLUDA_SLAB_FN int slab_unit_voff(bool tail, int ub, int dma_off, int q, int kw, int kwave, int K, int pitch) {
+  if (slab_unit_empty(tail, ub, q, kw, kwave, K)) return dma_off;  // the row's first bytes: in range, a cache hit, never multiplied
+  const int off = q * ub + dma_off;
+  const bool in = !tail || (off < kw && kwave + off < K);
+  return in ? kwave + off + pitch : kSlabOutOfRange;
+}
+
+} // namespace zluda_amd

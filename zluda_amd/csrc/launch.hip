@@ -330,6 +330,7 @@ extern "C" uint32_t zluda_gemm_strided_batched_ex(uint32_t transa, uint32_t tran
   p.op.transa = transa; p.op.transb = transb;
   p.op.epilogue = CUBLASLT_EPILOGUE_DEFAULT;
   p.op.bias_type = -1;
+  p.op.epilogue_aux_type = -1;
   const bool ta = transa != CUBLAS_OP_N, tb = transb != CUBLAS_OP_N;
   p.a = {a_type, CUBLASLT_ORDER_COL, (uint64_t)(ta ? k : m), (uint64_t)(ta ? m : k), lda, batch_count, stride_a};
   p.b = {b_type, CUBLASLT_ORDER_COL, (uint64_t)(tb ? n : k), (uint64_t)(tb ? k : n), ldb, batch_count, stride_b};

@@ -24,6 +24,11 @@ extern "C" uint32_t zluda_gemm_launch_noalloc(const zluda_gemm_problem *p, const
   static std::atomic<void *> scratch_of[64];  // zero-initialised; racing first calls store the same value
   void *ws = scratch_of[dev].load(std::memory_order_acquire);
   if (!ws) {
+    // The look-up may load the code object, which is not something to do in the middle of a stream capture: a caller that
+    // captures warms the entry point up with one call outside the capture first (any plan, even one that needs no scratch).
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing((hipStream_t)stream, &cap) != hipSuccess) return CUBLAS_STATUS_NOT_INITIALIZED;
+    if (cap != hipStreamCaptureStatusNone) return CUBLAS_STATUS_NOT_SUPPORTED;
     void *ptr = nullptr;
     if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return CUBLAS_STATUS_NOT_INITIALIZED;
     scratch_of[dev].store(ptr, std::memory_order_release);

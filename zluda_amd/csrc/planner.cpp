@@ -187,6 +187,7 @@ uint32_t lower_problem(const zluda_gemm_problem *p, bool dry, Lowered *out) {
     // the aux matrix has D's type, shape and order (cuda_types/src/cublaslt.rs:4207-4236: its leading dimension
     // is no less than D's rows); both passes go through D's type, which has to be a float type of 16 or 32 bits
     if (g.int_scale || !(d.type == CUDA_R_32F || d.type == CUDA_R_16F || d.type == CUDA_R_16BF)) return CUBLAS_STATUS_NOT_SUPPORTED;
+    if (op.epilogue_aux_type != -1 && (uint32_t)op.epilogue_aux_type != d.type) return CUBLAS_STATUS_NOT_SUPPORTED;
     const int64_t lead = d.order == CUBLASLT_ORDER_COL ? M : N, other = d.order == CUBLASLT_ORDER_COL ? N : M;
     if (op.epilogue_aux_ld < lead) return CUBLAS_STATUS_INVALID_VALUE;
     if (g.batch > 1 && op.epilogue_aux_batch_stride < op.epilogue_aux_ld * other && op.epilogue_aux_batch_stride != 0)

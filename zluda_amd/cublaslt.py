@@ -184,6 +184,8 @@ class MatmulCall:
             api.check(api.desc_set(self.desc, D.CUBLASLT_MATMUL_DESC_B_SCALE_MODE, C.c_int32, s["b_scale_mode"]), "B_SCALE_MODE")
         if "bias_batch_stride" in s:
             api.check(api.desc_set(self.desc, D.CUBLASLT_MATMUL_DESC_BIAS_BATCH_STRIDE, C.c_int64, s["bias_batch_stride"]), "BIAS_BATCH_STRIDE")
+        if "aux_type" in s:
+            api.check(api.desc_set(self.desc, D.CUBLASLT_MATMUL_DESC_EPILOGUE_AUX_DATA_TYPE, C.c_int32, s["aux_type"]), "EPILOGUE_AUX_DATA_TYPE")
         if "aux_ld" in s:
             api.check(api.desc_set(self.desc, D.CUBLASLT_MATMUL_DESC_EPILOGUE_AUX_LD, C.c_int64, s["aux_ld"]), "EPILOGUE_AUX_LD")
         if "aux_batch_stride" in s:
