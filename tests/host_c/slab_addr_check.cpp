@@ -27,7 +27,7 @@ static void check(int nw, int ub, int Q, int K) {
         int in_range = 0;
         for (int lane = 0; lane < 64; lane++) {
           const int off = slab_dma_offset(ub, lane, i);
-          const int v = slab_unit_voff(tail, ub, off, q, kw, kwave, K, 0);
+          const int v = slab_unit_voff(tail, ub, lane, off, q, kw, kwave, K, 0);
           if (v == kSlabOutOfRange) continue;
           in_range++;
           if (v < 0 || v + 16 > K) { printf("nw %d ub %d Q %d K %d wave %d unit %d instruction %d lane %d: offset %d outside the row\n", nw, ub, Q, K, wave, q, i, lane, v); exit(1); }

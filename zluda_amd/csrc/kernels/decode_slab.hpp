@@ -112,7 +112,7 @@ __global__ __launch_bounds__(NW * 64) void decode_slab_kernel(DecodeParams prm) 
   // vector offset of instruction i in unit q of the wave's slab, `pitch` = what the odd row adds.  A unit that holds
   // no byte of K (decode_slab_addr.hpp) is fetched as real loads and its MFMAs are skipped: no instruction the kernel
   // issues has all of its lanes out of range, which the counted waits below depend on.
-  auto unit_voff = [&](int i, int q, int pitch) { return slab_unit_voff(TAIL, UB, dma_off[i], q, kw, kwave, K, pitch); };
+  auto unit_voff = [&](int i, int q, int pitch) { return slab_unit_voff(TAIL, UB, lane, dma_off[i], q, kw, kwave, K, pitch); };
   auto unit_empty = [&](int q) { return slab_unit_empty(TAIL, UB, q, kw, kwave, K); };  // (wave-uniform)
   auto issue_w = [&](int b, int q, int slot) {
     const int rb = row_base(b), re = row_end(b);
@@ -174,6 +174,18 @@ __global__ __launch_bounds__(NW * 64) void decode_slab_kernel(DecodeParams prm) 
 #pragma unroll
     for (int c = 0; c < NB * Q; c++) lds_values_ready(xf[c]);
     issue_unit(0, 0);
+  }
+  // Activation fragments of a unit that holds no byte of K: zero, so that the 16 stray bytes per instruction that the
+  // unit's weight loads bring multiply to nothing without a branch around the MFMAs.
+  // int8: exact.  e4m3 has no infinity, and a NaN among the stray weights is one the row's own product holds too.
+  if constexpr (TAIL && !kind_is_h16(KIND)) {
+#pragma unroll
+    for (int c = 0; c < NB * Q; c++) {
+      if (unit_empty(c % Q)) {
+#pragma unroll
+        for (int f = 0; f < NFRAG; f++) xf[c][f] = v4i{0, 0, 0, 0};
+      }
+    }
   }
   // (the second unit is issued even when there is none -- then it fetches the first one again, never used -- so
   // that the number of operations in flight is the same on every path)
@@ -260,7 +272,11 @@ __global__ __launch_bounds__(NW * 64) void decode_slab_kernel(DecodeParams prm) 
         for (int f = 0; f < NFRAG; f++) w[f] = lds_read16_unordered(frag_addr(n & 1, f));
         lds_values_ready(w);  // in registers before the slot is refilled
         if ((n + 2) / Q < nblk) issue_unit(n + 2, n & 1);
-        if (unit_empty(q)) continue;  // (fetched for the count only)
+        // (a unit that holds no byte of K was fetched for the count only: for 8-bit operands its activation fragments
+        // are zero -- see above --, 16-bit ones, whose stray weights may be infinite, skip its MFMAs)
+        if constexpr (kind_is_h16(KIND)) {
+          if (unit_empty(q)) continue;
+        }
 #pragma unroll
         for (int nbk = 0; nbk < NB; nbk++) {
           if constexpr (KIND == KIND_I8) {

@@ -7,7 +7,7 @@
 #pragma once
 
 #if defined(__HIPCC__)
-#define ZLUDA_SLAB_FN __host__ __device__ inline
+#define ZLUDA_SLAB_FN __host__ __device__ __forceinline__
 #else
 #define ZLUDA_SLAB_FN inline
 #endif
@@ -26,17 +26,18 @@ ZLUDA_SLAB_FN int slab_dma_offset(int ub, int lane, int i) {
 
 // Unit q of a wave's slab holds no byte of K: the wave's share kw of K ends before it, or K itself does (kwave = first
 // K byte of the wave).  Such a unit is fetched all the same -- the number of operations in flight is what the counted
-// waits rely on -- but as real loads of bytes nobody multiplies: an instruction whose lanes are ALL out of range
-// completes without a memory round trip and can retire ahead of older loads, which would let a counted wait pass
-// while an older unit is still in flight.
+// waits rely on -- with ONE lane of every instruction in range (16 bytes nobody multiplies): an instruction whose
+// lanes are ALL out of range completes without a memory round trip and can retire ahead of older loads, which would
+// let a counted wait pass while an older unit is still in flight.  (All 64 lanes in range measured 25 % slower at
+// 5120 x 16 x 13824, where one unit in 32 is empty.)
 ZLUDA_SLAB_FN bool slab_unit_empty(bool tail, int ub, int q, int kw, int kwave, int K) {
   return tail && (q * ub >= kw || kwave + q * ub >= K);
 }
 
-// vector offset (bytes from the row's start) of lane `lane` of instruction `i` in unit `q`; `dma_off` =
+// vector offset (bytes from the row's start) of lane `lane` of an instruction of unit `q`; `dma_off` =
 // slab_dma_offset(ub, lane, i), `pitch` = what the odd row of a two-row instruction adds
-ZLUDA_SLAB_FN int slab_unit_voff(bool tail, int ub, int dma_off, int q, int kw, int kwave, int K, int pitch) {
-  if (slab_unit_empty(tail, ub, q, kw, kwave, K)) return dma_off;  // the row's first bytes: in range, a cache hit, never multiplied
+ZLUDA_SLAB_FN int slab_unit_voff(bool tail, int ub, int lane, int dma_off, int q, int kw, int kwave, int K, int pitch) {
+  if (slab_unit_empty(tail, ub, q, kw, kwave, K)) return lane == 0 ? dma_off : kSlabOutOfRange;  // (lane 0: 16 bytes of the row's start)
   const int off = q * ub + dma_off;
   const bool in = !tail || (off < kw && kwave + off < K);
   return in ? kwave + off + pitch : kSlabOutOfRange;
