@@ -40,6 +40,8 @@ namespace zluda_amd {
 enum { W4_EPI_I32 = 0, W4_EPI_BF16 = 1, W4_EPI_BF16_GELU = 2 };
 
 // one accumulator element, AGPR -> VGPR
+typedef unsigned v2u __attribute__((ext_vector_type(2)));
+
 template <class T>
 __device__ __forceinline__ int w4_acc_read(const T &elem) {
   int raw = 0;
@@ -67,106 +69,169 @@ __device__ __forceinline__ void w4_store_f16(const MfmaParams &prm, AccV (&acc)[
   const int64_t corner = (int64_t)qc * d_sq + pc;
   char *Dw = (char *)g.D + (g.d_sb * bt + corner) * 2;
   const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)Dw, 0, tile_window_bytes(d_sq, NP, NQ, corner, 2), 0x00020000);
-  const int voff = ((lane & 15) * d_sq + 4 * (lane >> 4)) * 2;
   const int prow = pc + 4 * (lane >> 4);  // first of the lane's four P indices in tile row 0
   // the one factor along Q (uniform) and D's scale: without an activation both fold into the P factors
   const float q_u = swp ? ep.row_scale(0) : ep.col_scale(0);
   const float fold = ACT == ACT_NONE ? q_u * ep.sd : q_u;
   const float inv_sd = 1.0f / ep.sd;
+  // The factors along P (a lane's four consecutive indices of each of the TP tile rows), every mode decided once and
+  // every vector fetched 16 (or 8) bytes at a time where its alignment allows.
   float ps[TP][4], pb[TP][4];
-  const bool p_vec = swp ? ep.sb_v != nullptr : (ep.alpha_v != nullptr || ep.sa_v != nullptr);
-  if (p_vec) {
+  const float *vec1 = swp ? ep.sb_v : ep.alpha_v, *vec2 = swp ? nullptr : ep.sa_v;  // per-P scale vectors (or null)
+  const float uni = (swp ? ep.sb_s : ep.alpha_s * ep.sa_s) * fold;                   // (a scalar beside a vector is 1)
+  auto load4 = [&](const float *v, int a, float (&out)[4]) __attribute__((always_inline)) {
+    const float *q = v + prow + a * 16;
+    if ((((uintptr_t)v) & 15) == 0) {
+      const v4f t = *(const v4f *)q;
 #pragma unroll
-    for (int a = 0; a < TP; a++)
+      for (int e = 0; e < 4; e++) out[e] = t[e];
+    } else {
 #pragma unroll
-      for (int e = 0; e < 4; e++) ps[a][e] = (swp ? ep.col_scale(prow + a * 16 + e) : ep.row_scale(prow + a * 16 + e)) * fold;
-  } else {
-    const float u = (swp ? ep.col_scale(0) : ep.row_scale(0)) * fold;
+      for (int e = 0; e < 4; e++) out[e] = q[e];
+    }
+  };
 #pragma unroll
-    for (int a = 0; a < TP; a++)
+  for (int a = 0; a < TP; a++)
 #pragma unroll
-      for (int e = 0; e < 4; e++) ps[a][e] = u;
+    for (int e = 0; e < 4; e++) ps[a][e] = uni;
+  if (vec1 != nullptr) {
+#pragma unroll
+    for (int a = 0; a < TP; a++) {
+      float t[4];
+      load4(vec1, a, t);
+#pragma unroll
+      for (int e = 0; e < 4; e++) ps[a][e] *= t[e];
+    }
   }
+  if (vec2 != nullptr) {
+#pragma unroll
+    for (int a = 0; a < TP; a++) {
+      float t[4];
+      load4(vec2, a, t);
+#pragma unroll
+      for (int e = 0; e < 4; e++) ps[a][e] *= t[e];
+    }
+  }
+#pragma unroll
+  for (int a = 0; a < TP; a++)
+#pragma unroll
+    for (int e = 0; e < 4; e++) pb[a][e] = 0.0f;
   if (!swp && g.bias != nullptr) {
     const float bfold = ACT == ACT_NONE ? ep.sd : 1.0f;
+    if (g.bias_type == CUDA_R_32F) {
+      const float *bv = (const float *)g.bias + g.bias_sb * bt;
 #pragma unroll
-    for (int a = 0; a < TP; a++)
+      for (int a = 0; a < TP; a++) {
+        float t[4];
+        load4(bv, a, t);
 #pragma unroll
-      for (int e = 0; e < 4; e++) pb[a][e] = ep.bias_at(prow + a * 16 + e) * bfold;
-  } else {
+        for (int e = 0; e < 4; e++) pb[a][e] = t[e] * bfold;
+      }
+    } else {
+      const uint16_t *bv = (const uint16_t *)g.bias + g.bias_sb * bt;
+      const bool wide = (((uintptr_t)bv) & 7) == 0, is_bf16 = g.bias_type == CUDA_R_16BF;
 #pragma unroll
-    for (int a = 0; a < TP; a++)
+      for (int a = 0; a < TP; a++) {
+        const uint16_t *q = bv + prow + a * 16;
+        uint32_t h[4];
+        if (wide) {
+          const v2i t = *(const v2i *)q;
+          h[0] = (uint32_t)t[0] & 0xffffu; h[1] = (uint32_t)t[0] >> 16; h[2] = (uint32_t)t[1] & 0xffffu; h[3] = (uint32_t)t[1] >> 16;
+        } else {
 #pragma unroll
-      for (int e = 0; e < 4; e++) pb[a][e] = 0.0f;
+          for (int e = 0; e < 4; e++) h[e] = q[e];
+        }
+#pragma unroll
+        for (int e = 0; e < 4; e++) pb[a][e] = (is_bf16 ? dec_bf16((uint16_t)h[e]) : dec_f16((uint16_t)h[e])) * bfold;
+      }
+    }
   }
   __builtin_amdgcn_sched_barrier(0);
+  // One column of 16 x 16 tiles (TP tiles, 16 Q indices) at a time.  Lane l = 16 g + c holds rows 4g .. 4g + 3 of column c of
+  // each tile: two packed dwords.  Tiles a and a + 1 trade halves between the lane groups g and g ^ 1 (v_permlane16_swap:
+  // the odd groups' registers of the first operand against the even groups' of the second), after which a lane of an even
+  // group holds rows 4g .. 4g + 7 of tile a and a lane of an odd group rows 4(g-1) .. 4(g-1) + 7 of tile a + 1: 16 bytes per
+  // lane, and a store instruction writes 64 contiguous bytes of each of 16 columns instead of 32.
+  static_assert(TP % 2 == 0, "tiles along P are stored in pairs");
+  const int grp = lane >> 4;
+  const int voff16 = ((lane & 15) * d_sq + ((grp & 1) ? 4 * grp + 12 : 4 * grp)) * 2;
 #pragma unroll
-  for (int a = 0; a < TP; a++) {
-    // The row's accumulators first, by explicit reads (left to itself the register allocator parks most accumulators
-    // in scratch memory between their last MFMA and this point instead of leaving them in the AGPRs); then TQ * 4
-    // independent chains for the scheduler to interleave.
-    int raw[TQ][4];
+  for (int b = 0; b < TQ; b++) {
+    // The column's accumulators first, by explicit reads (left to itself the register allocator parks most accumulators
+    // in scratch memory between their last MFMA and this point instead of leaving them in the AGPRs); then TP * 4
+    // independent chains, written stage by stage over the whole column, which is the order the scheduler then keeps:
+    // every instruction has TP * 4 - 1 independent ones between itself and its consumer.
+    int raw[TP][4];
 #pragma unroll
-    for (int b = 0; b < TQ; b++)
+    for (int a = 0; a < TP; a++)
+#pragma unroll
+      for (int e = 0; e < 4; e++) raw[a][e] = w4_acc_read(acc[a][b][e]);
+    float x[TP][4], z[TP][4];
+#pragma unroll
+    for (int a = 0; a < TP; a++)
 #pragma unroll
       for (int e = 0; e < 4; e++) {
-        raw[b][e] = w4_acc_read(acc[a][b][e]);
-      }
-    // written stage by stage over the whole row, which is the order the scheduler then keeps: every instruction
-    // has TQ * 4 - 1 independent ones between itself and its consumer
-    float x[TQ][4], z[TQ][4];
-#pragma unroll
-    for (int b = 0; b < TQ; b++)
-#pragma unroll
-      for (int e = 0; e < 4; e++) {
-        const float accf = KIND == KIND_I8 ? (float)raw[b][e] : bits2f((uint32_t)raw[b][e]);
-        x[b][e] = __builtin_fmaf(accf, ps[a][e], pb[a][e]);
+        const float accf = KIND == KIND_I8 ? (float)raw[a][e] : bits2f((uint32_t)raw[a][e]);
+        x[a][e] = __builtin_fmaf(accf, ps[a][e], pb[a][e]);
       }
     if constexpr (ACT == ACT_GELU) {
       // x * sigmoid(2u) * sd (gelu_tanh of numeric.hpp) with sd folded into the reciprocal: x / ((1 + e) / sd)
       const float c0 = -2.0f * 0.7978845608028654f * 1.4426950408889634f, c1 = 0.044715f * c0;
 #pragma unroll
-      for (int b = 0; b < TQ; b++)
+      for (int a = 0; a < TP; a++)
 #pragma unroll
-        for (int e = 0; e < 4; e++) z[b][e] = x[b][e] * x[b][e];
+        for (int e = 0; e < 4; e++) z[a][e] = x[a][e] * x[a][e];
 #pragma unroll
-      for (int b = 0; b < TQ; b++)
+      for (int a = 0; a < TP; a++)
 #pragma unroll
-        for (int e = 0; e < 4; e++) z[b][e] = __builtin_fmaf(z[b][e], c1, c0);
+        for (int e = 0; e < 4; e++) z[a][e] = __builtin_fmaf(z[a][e], c1, c0);
 #pragma unroll
-      for (int b = 0; b < TQ; b++)
+      for (int a = 0; a < TP; a++)
 #pragma unroll
-        for (int e = 0; e < 4; e++) z[b][e] = x[b][e] * z[b][e];
+        for (int e = 0; e < 4; e++) z[a][e] = x[a][e] * z[a][e];
 #pragma unroll
-      for (int b = 0; b < TQ; b++)
+      for (int a = 0; a < TP; a++)
 #pragma unroll
-        for (int e = 0; e < 4; e++) z[b][e] = __builtin_amdgcn_exp2f(z[b][e]);
+        for (int e = 0; e < 4; e++) z[a][e] = __builtin_amdgcn_exp2f(z[a][e]);
 #pragma unroll
-      for (int b = 0; b < TQ; b++)
+      for (int a = 0; a < TP; a++)
 #pragma unroll
-        for (int e = 0; e < 4; e++) z[b][e] = __builtin_fmaf(z[b][e], inv_sd, inv_sd);
+        for (int e = 0; e < 4; e++) z[a][e] = __builtin_fmaf(z[a][e], inv_sd, inv_sd);
 #pragma unroll
-      for (int b = 0; b < TQ; b++)
+      for (int a = 0; a < TP; a++)
 #pragma unroll
-        for (int e = 0; e < 4; e++) z[b][e] = __builtin_amdgcn_rcpf(z[b][e]);
+        for (int e = 0; e < 4; e++) z[a][e] = __builtin_amdgcn_rcpf(z[a][e]);
 #pragma unroll
-      for (int b = 0; b < TQ; b++)
+      for (int a = 0; a < TP; a++)
 #pragma unroll
-        for (int e = 0; e < 4; e++) x[b][e] = x[b][e] * z[b][e];
+        for (int e = 0; e < 4; e++) x[a][e] = x[a][e] * z[a][e];
     } else if constexpr (ACT == ACT_RELU) {
 #pragma unroll
-      for (int b = 0; b < TQ; b++)
+      for (int a = 0; a < TP; a++)
 #pragma unroll
-        for (int e = 0; e < 4; e++) x[b][e] = (x[b][e] > 0.0f ? x[b][e] : 0.0f) * ep.sd;
+        for (int e = 0; e < 4; e++) x[a][e] = (x[a][e] > 0.0f ? x[a][e] : 0.0f) * ep.sd;
     }
 #pragma unroll
-    for (int b = 0; b < TQ; b++) {
-      v2i pk;
-      if constexpr (BF16) { pk[0] = (int)pack_bf16x2(x[b][0], x[b][1]); pk[1] = (int)pack_bf16x2(x[b][2], x[b][3]); }
-      else { pk[0] = (int)pack_f16x2(x[b][0], x[b][1]); pk[1] = (int)pack_f16x2(x[b][2], x[b][3]); }
-      __builtin_amdgcn_raw_buffer_store_b64(pk, rs, voff, (b * 16 * d_sq + a * 16) * 2, 0);
+    for (int a = 0; a < TP; a += 2) {
+      uint32_t lo[2], hi[2];  // tile a, tile a + 1
+      if constexpr (BF16) {
+        lo[0] = pack_bf16x2(x[a][0], x[a][1]); lo[1] = pack_bf16x2(x[a][2], x[a][3]);
+        hi[0] = pack_bf16x2(x[a + 1][0], x[a + 1][1]); hi[1] = pack_bf16x2(x[a + 1][2], x[a + 1][3]);
+      } else {
+        lo[0] = pack_f16x2(x[a][0], x[a][1]); lo[1] = pack_f16x2(x[a][2], x[a][3]);
+        hi[0] = pack_f16x2(x[a + 1][0], x[a + 1][1]); hi[1] = pack_f16x2(x[a + 1][2], x[a + 1][3]);
+      }
+      v4i pk;
+#if defined(__HIP_DEVICE_COMPILE__)
+      const v2u s0 = __builtin_amdgcn_permlane16_swap(lo[0], hi[0], false, false);
+      const v2u s1 = __builtin_amdgcn_permlane16_swap(lo[1], hi[1], false, false);
+      pk = v4i{(int)s0[0], (int)s1[0], (int)s0[1], (int)s1[1]};
+#else
+      pk = v4i{(int)lo[0], (int)lo[1], (int)hi[0], (int)hi[1]};
+#endif
+      buffer_store_b128_guarded(pk, rs, voff16, (b * 16 * d_sq + a * 16) * 2);
     }
-    __builtin_amdgcn_sched_barrier(0);  // one tile row at a time: what the scheduler hoists across rows costs registers
+    __builtin_amdgcn_sched_barrier(0);  // one tile column at a time: what the scheduler hoists across them costs registers
   }
 }
 
