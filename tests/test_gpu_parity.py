@@ -132,6 +132,31 @@ def test_mfma_f8_mixed_formats(gpu_api, at, bt):
     check(gpu_api, dict(F8, a_type=at, b_type=bt, m=256, n=128, k=512, order_c=1, order_d=1), 41, K.ZLUDA_KERNEL_MFMA_F8, 1)
 
 
+def test_four_wave_kernel_stages_every_vector_its_epilogue_reads(gpu_api):
+    """variant 11 keeps its epilogue free of loads from memory: the vectors along D's unit stride (alpha[], A's outer
+    scales, the bias in each of its types; for a row-major D B's outer scales) reach it through LDS.  Each of them alone
+    and together, several tiles per workgroup (the staging area is reused), batches with odd strides (a 16-bit bias
+    that starts on an odd element), and D's scale folded in."""
+    base = dict(F8, m=1024, n=512, k=640, with_scalar_scales=True)
+    v11 = (K.ZLUDA_KERNEL_MFMA_F8, 11)
+    for i, bt in enumerate((K.CUDA_R_16BF, K.CUDA_R_16F, K.CUDA_R_32F)):
+        for epi in (K.CUBLASLT_EPILOGUE_BIAS, K.CUBLASLT_EPILOGUE_GELU_BIAS):
+            check(gpu_api, dict(base, epilogue=epi, bias_type=bt), 900 + i, *v11)
+        check(gpu_api, dict(base, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS, bias_type=bt, batch=3, bias_batch_stride=1031,
+                            with_cd_scales=True), 910 + i, *v11)
+    vec = dict(base, pointer_mode=K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO, alpha_range=(0.5, 1.5),
+               a_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F)
+    check(gpu_api, vec, 920, *v11)
+    check(gpu_api, dict(vec, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS, bias_type=K.CUDA_R_16BF, batch=2, bias_batch_stride=1025,
+                        pointer_mode=K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_HOST, alpha_vector_batch_stride=1029),
+          921, *v11)
+    check(gpu_api, dict(base, pointer_mode=K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO, alpha_range=(0.5, 1.5)), 922, *v11)
+    # row-major D: the unit stride runs along N, and the vector along it is B's
+    check(gpu_api, dict(base, order_c=1, order_d=1, b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F), 923, *v11)
+    # a tile row that is partial along M takes the element-wise path in the same launch
+    check(gpu_api, dict(vec, m=1100, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS, bias_type=K.CUDA_R_16F), 924, *v11)
+
+
 # ---- MXFP4 -----------------------------------------------------------------------------------------
 @pytest.mark.parametrize("variant", range(8))
 def test_mfma_mxf4_variants(gpu_api, variant):

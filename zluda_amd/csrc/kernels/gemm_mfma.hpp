@@ -68,6 +68,14 @@ __device__ __forceinline__ void lds_dma16(__amdgpu_buffer_rsrc_t rs, void *lds_d
 #endif
 }
 
+// 4 bytes per lane from a buffer straight into LDS (buffer_load_dword ... lds): lane l lands at byte l*4 of the 256-byte
+// block that starts at the wave-uniform `lds_dst`.
+__device__ __forceinline__ void lds_dma4(__amdgpu_buffer_rsrc_t rs, void *lds_dst, int voff, int soff) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void *)lds_dst, 4, voff, soff, 0, 0);
+#endif
+}
+
 // 128-bit buffer store whose data registers stay untouched for the wait states that follow it.  Observed on
 // MI355X: when the instruction right behind a buffer_store_dwordx4 (offen, scalar offset in an SGPR) is a
 // VALU write to the first data register, the store now and then writes the new value instead (element 0 of

@@ -51,6 +51,49 @@ __device__ __forceinline__ int w4_acc_read(const T &elem) {
   return raw;
 }
 
+// The lane number, computed where it is used.  Nothing an epilogue needs per lane may stay live across the K loop: the
+// loop has no register to spare, what is kept is spilled to scratch memory, and a reload from there (like every load from
+// memory in an epilogue) first waits for the next tile's stages, which are in flight and older.
+__device__ __forceinline__ int w4_lane_here() {
+  int l = 0;
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(l));
+#endif
+  return l;
+}
+
+// A value every lane holds alike, moved to a scalar register now (not where the compiler would next need it).  The
+// compiler does not look inside the assembly, so the wait states it would add around the instruction are written out:
+// one between a VALU write of the source and the read, two between the write of the SGPR and a VALU read of it.
+__device__ __forceinline__ float w4_uniform_now(float v) {
+  int o = 0;
+  (void)v;
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("s_nop 0\n\tv_readfirstlane_b32 %0, %1\n\ts_nop 1" : "=s"(o) : "v"(f2bits(v)));
+#endif
+  return bits2f((uint32_t)o);
+}
+
+// Hides a scalar register's value from the optimiser at this point: what is computed from it is computed here, per tile,
+// instead of once in front of the tile loop into a vector register that then has to be kept across the K loop.
+__device__ __forceinline__ void w4_scalar_here(float &v) {
+  int b = (int)f2bits(v);
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("" : "+s"(b));
+#endif
+  v = bits2f((uint32_t)b);
+}
+
+// What a wave has staged in LDS for the epilogue of its current tile: up to three vectors along P, WTP = 128 entries each
+// (slot 0: the per-P scale vector alpha[] or, for a row-major D, B's; slot 1: A's; slot 2: the bias in its storage type).
+// A 16-bit bias that starts at an odd element is copied from the dword in front of it: bias_skip = 1 element to skip.
+struct W4Staged {
+  static constexpr int WORDS = 128 + 4;  // per slot: 128 dwords and the one a skipped element pushes out
+  const int *area;                       // the wave's three slots
+  bool has[3];
+  int bias_skip;
+};
+
 // Float epilogue of the four-wave kernel: D bf16 / f16 = act((scale_p * scale_q) * acc + bias) * scale_d straight from the
 // accumulators (layout of gemm_mfma_pipe16.hpp: lane l holds P = 16a + 4 (l / 16) + e, Q = 16b + l % 16) on tiles complete
 // along P, for problems in which nothing varies along Q (no per-column scale vector; for a row-major D no per-row vector
@@ -59,91 +102,81 @@ __device__ __forceinline__ int w4_acc_read(const T &elem) {
 // code: one FMA per element, then the activation (ACT fixed at compile time) with D's scale folded into it.
 template <int KIND, int ACT, bool BF16, int WTP, int WTQ, int TP, int TQ, class AccV>
 __device__ __forceinline__ void w4_store_f16(const MfmaParams &prm, AccV (&acc)[TP][TQ], int p0, int q0, int NP, int NQ, int bt,
-                                             int wp, int wq) {
+                                             int wp, int wq, const EpilogueScalars &scalars, const W4Staged &st) {
   const GemmArgs &g = prm.g;
-  const int lane = threadIdx.x & 63;
-  Epilogue ep(g, bt);
+  const int lane = w4_lane_here();
+  EpilogueScalars here = scalars;
+  w4_scalar_here(here.alpha_s); w4_scalar_here(here.sa_s); w4_scalar_here(here.sb_s); w4_scalar_here(here.sd);
   const bool swp = prm.swapped != 0;
   const int d_sq = (int)(swp ? g.d_si : g.d_sj);  // < 2^22 (checked before this path is taken)
   const int pc = p0 + wp * WTP, qc = q0 + wq * WTQ;
   const int64_t corner = (int64_t)qc * d_sq + pc;
   char *Dw = (char *)g.D + (g.d_sb * bt + corner) * 2;
   const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)Dw, 0, tile_window_bytes(d_sq, NP, NQ, corner, 2), 0x00020000);
-  const int prow = pc + 4 * (lane >> 4);  // first of the lane's four P indices in tile row 0
-  // the one factor along Q (uniform) and D's scale: without an activation both fold into the P factors
-  const float q_u = swp ? ep.row_scale(0) : ep.col_scale(0);
-  const float fold = ACT == ACT_NONE ? q_u * ep.sd : q_u;
-  const float inv_sd = 1.0f / ep.sd;
-  // The factors along P (a lane's four consecutive indices of each of the TP tile rows), every mode decided once and
-  // every vector fetched 16 (or 8) bytes at a time where its alignment allows.
+  // the one factor along Q (uniform: a scalar, as nothing varies along Q here) and D's scale: without an activation both
+  // fold into the P factors
+  const float q_u = swp ? here.alpha_s * here.sa_s : here.sb_s;
+  const float fold = ACT == ACT_NONE ? q_u * here.sd : q_u;
+  const float inv_sd = 1.0f / here.sd;
+  // The factors along P (a lane's four consecutive indices of each of the TP tile rows), every mode decided once.  The
+  // vectors come from the wave's staging area in LDS, never from memory: a load from memory here would first wait for
+  // the next tile's stages, which are in flight and older.
   float ps[TP][4], pb[TP][4];
-  const float *vec1 = swp ? ep.sb_v : ep.alpha_v, *vec2 = swp ? nullptr : ep.sa_v;  // per-P scale vectors (or null)
-  const float uni = (swp ? ep.sb_s : ep.alpha_s * ep.sa_s) * fold;                   // (a scalar beside a vector is 1)
-  auto load4 = [&](const float *v, int a, float (&out)[4]) __attribute__((always_inline)) {
-    const float *q = v + prow + a * 16;
-    if ((((uintptr_t)v) & 15) == 0) {
-      const v4f t = *(const v4f *)q;
-#pragma unroll
-      for (int e = 0; e < 4; e++) out[e] = t[e];
-    } else {
-#pragma unroll
-      for (int e = 0; e < 4; e++) out[e] = q[e];
-    }
-  };
+  const float uni = (swp ? here.sb_s : here.alpha_s * here.sa_s) * fold;  // (a scalar beside a vector is 1)
+  const int l4 = 4 * (lane >> 4);  // the lane's first P index inside a 16 x 16 tile
 #pragma unroll
   for (int a = 0; a < TP; a++)
 #pragma unroll
     for (int e = 0; e < 4; e++) ps[a][e] = uni;
-  if (vec1 != nullptr) {
 #pragma unroll
-    for (int a = 0; a < TP; a++) {
-      float t[4];
-      load4(vec1, a, t);
+  for (int v = 0; v < 2; v++)
+    if (st.has[v]) {
+      v4f t[TP];
 #pragma unroll
-      for (int e = 0; e < 4; e++) ps[a][e] *= t[e];
+      for (int a = 0; a < TP; a++) t[a] = *(const v4f *)((const float *)st.area + v * W4Staged::WORDS + l4 + a * 16);
+#pragma unroll
+      for (int a = 0; a < TP; a++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) ps[a][e] *= t[a][e];
     }
-  }
-  if (vec2 != nullptr) {
-#pragma unroll
-    for (int a = 0; a < TP; a++) {
-      float t[4];
-      load4(vec2, a, t);
-#pragma unroll
-      for (int e = 0; e < 4; e++) ps[a][e] *= t[e];
-    }
-  }
 #pragma unroll
   for (int a = 0; a < TP; a++)
 #pragma unroll
     for (int e = 0; e < 4; e++) pb[a][e] = 0.0f;
-  if (!swp && g.bias != nullptr) {
-    const float bfold = ACT == ACT_NONE ? ep.sd : 1.0f;
+  if (st.has[2]) {
+    const float bfold = ACT == ACT_NONE ? here.sd : 1.0f;
+    const int *bias_words = st.area + 2 * W4Staged::WORDS;
     if (g.bias_type == CUDA_R_32F) {
-      const float *bv = (const float *)g.bias + g.bias_sb * bt;
+      v4f t[TP];
 #pragma unroll
-      for (int a = 0; a < TP; a++) {
-        float t[4];
-        load4(bv, a, t);
+      for (int a = 0; a < TP; a++) t[a] = *(const v4f *)((const float *)bias_words + l4 + a * 16);
 #pragma unroll
-        for (int e = 0; e < 4; e++) pb[a][e] = t[e] * bfold;
-      }
+      for (int a = 0; a < TP; a++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) pb[a][e] = t[a][e] * bfold;
     } else {
-      const uint16_t *bv = (const uint16_t *)g.bias + g.bias_sb * bt;
-      const bool wide = (((uintptr_t)bv) & 7) == 0, is_bf16 = g.bias_type == CUDA_R_16BF;
+      const bool is_bf16 = g.bias_type == CUDA_R_16BF;
+      const uint16_t *q = (const uint16_t *)bias_words + st.bias_skip + l4;
+      uint32_t h[TP][4];
+      if (st.bias_skip == 0) {
+        v2i t[TP];
 #pragma unroll
-      for (int a = 0; a < TP; a++) {
-        const uint16_t *q = bv + prow + a * 16;
-        uint32_t h[4];
-        if (wide) {
-          const v2i t = *(const v2i *)q;
-          h[0] = (uint32_t)t[0] & 0xffffu; h[1] = (uint32_t)t[0] >> 16; h[2] = (uint32_t)t[1] & 0xffffu; h[3] = (uint32_t)t[1] >> 16;
-        } else {
+        for (int a = 0; a < TP; a++) t[a] = *(const v2i *)(q + a * 16);
 #pragma unroll
-          for (int e = 0; e < 4; e++) h[e] = q[e];
+        for (int a = 0; a < TP; a++) {
+          h[a][0] = (uint32_t)t[a][0] & 0xffffu; h[a][1] = (uint32_t)t[a][0] >> 16;
+          h[a][2] = (uint32_t)t[a][1] & 0xffffu; h[a][3] = (uint32_t)t[a][1] >> 16;
         }
+      } else {
 #pragma unroll
-        for (int e = 0; e < 4; e++) pb[a][e] = (is_bf16 ? dec_bf16((uint16_t)h[e]) : dec_f16((uint16_t)h[e])) * bfold;
+        for (int a = 0; a < TP; a++)
+#pragma unroll
+          for (int e = 0; e < 4; e++) h[a][e] = q[a * 16 + e];
       }
+#pragma unroll
+      for (int a = 0; a < TP; a++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) pb[a][e] = (is_bf16 ? dec_bf16((uint16_t)h[a][e]) : dec_f16((uint16_t)h[a][e])) * bfold;
     }
   }
   __builtin_amdgcn_sched_barrier(0);
@@ -209,7 +242,7 @@ __device__ __forceinline__ void w4_store_f16(const MfmaParams &prm, AccV (&acc)[
 #pragma unroll
       for (int a = 0; a < TP; a++)
 #pragma unroll
-        for (int e = 0; e < 4; e++) x[a][e] = (x[a][e] > 0.0f ? x[a][e] : 0.0f) * ep.sd;
+        for (int e = 0; e < 4; e++) x[a][e] = (x[a][e] > 0.0f ? x[a][e] : 0.0f) * here.sd;
     }
 #pragma unroll
     for (int a = 0; a < TP; a += 2) {
@@ -239,10 +272,9 @@ __device__ __forceinline__ void w4_store_f16(const MfmaParams &prm, AccV (&acc)[
 // with 16-byte aligned columns: 16 bytes per lane straight from the accumulators.
 template <int WTP, int WTQ, int TP, int TQ, class AccV>
 __device__ __forceinline__ void w4_store_i32(const MfmaParams &prm, AccV (&acc)[TP][TQ], int p0, int q0, int NP, int NQ, int bt,
-                                             int wp, int wq) {
+                                             int wp, int wq, int ialpha) {
   const GemmArgs &g = prm.g;
-  const int lane = threadIdx.x & 63;
-  const int ialpha = g.alpha_mode == SCALAR_VALUE ? g.alpha_val.i : *(const int32_t *)g.alpha_ptr;
+  const int lane = w4_lane_here();
   const int64_t d_sq = prm.swapped ? g.d_si : g.d_sj;
   const int pc = p0 + wp * WTP, qc = q0 + wq * WTQ;
   const int64_t corner = (int64_t)qc * d_sq + pc;
@@ -342,7 +374,12 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
   using frag_v = typename std::conditional<KIND != KIND_F8, v4i, v8i>::type;
   struct Frag { frag_v k[KS]; };
 
-  __shared__ v4i lds[2 * STAGE_V4];
+  // the two slots; behind them each wave's staging area for the vectors its epilogue needs (W4Staged).  (One array: with
+  // a second LDS object in the kernel the compiler puts a vmcnt(0) in front of every LDS read that follows a DMA
+  // instruction.)
+  constexpr int STG_WAVE = 3 * W4Staged::WORDS;
+  constexpr int STG_V4 = EPI == W4_EPI_I32 ? 0 : NWV * STG_WAVE / 4;
+  __shared__ v4i lds[2 * STAGE_V4 + STG_V4];
 
   const GemmArgs &g = prm.g;
   const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
@@ -538,6 +575,18 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
   };
 
   const bool fast = w4_fast_epilogue_ok<KIND, EPI>(prm);
+  // The scalars behind device pointers, once for all tiles and wave-uniform (SGPRs): fetched in a tile's epilogue each
+  // would first wait for the next tile's stages, which are in flight and older.
+  EpilogueScalars scalars(g);
+  scalars.alpha_s = w4_uniform_now(scalars.alpha_s); scalars.beta_s = w4_uniform_now(scalars.beta_s);
+  scalars.sa_s = w4_uniform_now(scalars.sa_s); scalars.sb_s = w4_uniform_now(scalars.sb_s);
+  scalars.sc = w4_uniform_now(scalars.sc); scalars.sd = w4_uniform_now(scalars.sd);
+  int ialpha = 1;
+  if constexpr (EPI == W4_EPI_I32) {
+    int raw = g.alpha_mode == SCALAR_VALUE ? g.alpha_val.i : (g.alpha_mode == SCALAR_DEV ? *(const int32_t *)g.alpha_ptr : 1);
+    ialpha = (int)f2bits(w4_uniform_now(bits2f((uint32_t)raw)));
+  }
+  W4Staged staged{(const int *)&lds[2 * STAGE_V4] + (EPI == W4_EPI_I32 ? 0 : wave * STG_WAVE), {false, false, false}, 0};
   // epilogue of the tile at (p0, q0, bt); returns false when it needed the LDS (the stream must be primed again)
   auto epilogue = [&](int p0, int q0, int bt) __attribute__((always_inline)) -> bool {
     // MFMA write -> read of the accumulators: the wait states the compiler would insert if it could see the MFMAs.
@@ -546,8 +595,9 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
     asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
     if (fast && p0 + BP <= NP) {
-      if constexpr (EPI == W4_EPI_I32) w4_store_i32<WTP, WTQ>(prm, acc, p0, q0, NP, NQ, bt, wp, wq);
-      else w4_store_f16<KIND, EPI == W4_EPI_BF16_GELU ? ACT_GELU : ACT_NONE, true, WTP, WTQ>(prm, acc, p0, q0, NP, NQ, bt, wp, wq);
+      if constexpr (EPI == W4_EPI_I32) w4_store_i32<WTP, WTQ>(prm, acc, p0, q0, NP, NQ, bt, wp, wq, ialpha);
+      else w4_store_f16<KIND, EPI == W4_EPI_BF16_GELU ? ACT_GELU : ACT_NONE, true, WTP, WTQ>(prm, acc, p0, q0, NP, NQ, bt, wp, wq, scalars,
+                                                                                            staged);
       return true;
     }
     // the element-wise epilogue stages the accumulators in LDS: let the stages in flight land first
@@ -557,11 +607,49 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
     return false;
   };
 
+  // The vectors along P that the epilogue of the tile at (p0, bt) needs, this wave's WTP entries of each, into the wave's
+  // staging area: requested at the top of the tile, landed by the vmcnt(0) waits of the tile's last two stages (there
+  // always are two).  Only the wave itself reads them, after those waits and before it requests the next tile's.
+  auto stage_vectors = [&](int p0, int bt) __attribute__((always_inline)) {
+    if constexpr (EPI != W4_EPI_I32) {
+      staged.has[0] = staged.has[1] = staged.has[2] = false;
+      staged.bias_skip = 0;
+      if (fast && p0 + BP <= NP) {
+        const int ln4 = w4_lane_here() * 4;
+        const int pc = p0 + wp * WTP;
+        int *const area = (int *)&lds[2 * STAGE_V4] + wave * STG_WAVE;
+        // 128 dwords of a slot (and the one behind them); what lies past `bytes` is out of range and lands as zero
+        auto copy = [&](const void *src, int bytes, int slot) __attribute__((always_inline)) {
+          const __amdgpu_buffer_rsrc_t rsv = __builtin_amdgcn_make_buffer_rsrc((void *)src, 0, bytes, 0x00020000);
+          lds_dma4(rsv, area + slot * W4Staged::WORDS, ln4, 0);
+          lds_dma4(rsv, area + slot * W4Staged::WORDS + 64, ln4 + 256, 0);
+        };
+        const bool swp = prm.swapped != 0;
+        const float *v1 = swp ? (g.b_scale_mode == SCALE_OUTER_VEC ? (const float *)g.b_scale : nullptr)
+                              : (g.alpha_mode == VECTOR_DEV ? (const float *)g.alpha_ptr + g.alpha_sb * bt : nullptr);
+        const float *v2 = !swp && g.a_scale_mode == SCALE_OUTER_VEC ? (const float *)g.a_scale : nullptr;
+        if (v1 != nullptr) { copy(v1 + pc, WTP * 4, 0); staged.has[0] = true; }
+        if (v2 != nullptr) { copy(v2 + pc, WTP * 4, 1); staged.has[1] = true; }
+        if (!swp && g.bias != nullptr) {
+          const int es = g.bias_type == CUDA_R_32F ? 4 : 2;
+          const char *src = (const char *)g.bias + (g.bias_sb * bt + pc) * es;
+          const int skip = (int)(((uintptr_t)src) & 3) >> 1;  // (dword loads)
+          // (whole dwords are range-checked: the last one of a skipped start ends two bytes past the vector, inside
+          // the aligned dword that holds the vector's last element)
+          copy(src - 2 * skip, WTP * es + 4 * skip, 2);
+          staged.has[2] = true;
+          staged.bias_skip = skip;
+        }
+      }
+    }
+  };
+
   // ---- the stream -------------------------------------------------------------------------------------------------
   prime(0);
   for (int n = 0; n < my_tiles; n++) {
     int p0, q0, bt;
     tile_coords(n, p0, q0, bt);
+    stage_vectors(p0, bt);
     zero_acc();
     for (int kt = 2; kt < KT2; kt += 2) do_pair(kt);
     // the last two stages of the tile fetch the first two of the next one

@@ -135,6 +135,24 @@ __device__ __forceinline__ void store_elem(void *base, uint32_t type, int64_t id
   }
 }
 
+// The scalar factors of a float epilogue, those behind device pointers fetched (a scalar beside a vector is 1).
+struct EpilogueScalars {
+  float alpha_s, beta_s, sa_s, sb_s, sc, sd;
+  __device__ __forceinline__ explicit EpilogueScalars(const GemmArgs &g) {
+    alpha_s = beta_s = sa_s = sb_s = sc = sd = 1.0f;
+    if (!g.int_scale) {
+      if (g.alpha_mode == SCALAR_VALUE) alpha_s = g.alpha_val.f;
+      else if (g.alpha_mode == SCALAR_DEV) alpha_s = *(const float *)g.alpha_ptr;
+      if (g.beta_mode == SCALAR_VALUE) beta_s = g.beta_val.f;
+      else if (g.beta_mode == SCALAR_DEV) beta_s = *(const float *)g.beta_ptr;
+      if (g.a_scale_mode == SCALE_SCALAR) sa_s = *(const float *)g.a_scale;
+      if (g.b_scale_mode == SCALE_SCALAR) sb_s = *(const float *)g.b_scale;
+      if (g.c_scale) sc = *(const float *)g.c_scale;
+      if (g.d_scale) sd = *(const float *)g.d_scale;
+    }
+  }
+};
+
 // Per-thread epilogue context: everything that does not depend on (i, j) is read once.
 struct Epilogue {
   const GemmArgs &g;
@@ -144,22 +162,17 @@ struct Epilogue {
   const char *Cb;
   char *Db;
 
-  __device__ __forceinline__ Epilogue(const GemmArgs &g_, int batch) : g(g_), bt(batch) {
+  __device__ __forceinline__ Epilogue(const GemmArgs &g_, int batch) : Epilogue(g_, batch, EpilogueScalars(g_)) {}
+
+  // with the scalars fetched by the caller (a persistent kernel fetches them once, not once per tile)
+  __device__ __forceinline__ Epilogue(const GemmArgs &g_, int batch, const EpilogueScalars &s) : g(g_), bt(batch) {
     alpha_v = beta_v = sa_v = sb_v = nullptr;
-    alpha_s = beta_s = sa_s = sb_s = sc = sd = 1.0f;
+    alpha_s = s.alpha_s; beta_s = s.beta_s; sa_s = s.sa_s; sb_s = s.sb_s; sc = s.sc; sd = s.sd;
     if (!g.int_scale) {
-      if (g.alpha_mode == SCALAR_VALUE) alpha_s = g.alpha_val.f;
-      else if (g.alpha_mode == SCALAR_DEV) alpha_s = *(const float *)g.alpha_ptr;
-      else alpha_v = (const float *)g.alpha_ptr + g.alpha_sb * bt;
-      if (g.beta_mode == SCALAR_VALUE) beta_s = g.beta_val.f;
-      else if (g.beta_mode == SCALAR_DEV) beta_s = *(const float *)g.beta_ptr;
-      else beta_v = (const float *)g.beta_ptr;
-      if (g.a_scale_mode == SCALE_SCALAR) sa_s = *(const float *)g.a_scale;
-      else if (g.a_scale_mode == SCALE_OUTER_VEC) sa_v = (const float *)g.a_scale;
-      if (g.b_scale_mode == SCALE_SCALAR) sb_s = *(const float *)g.b_scale;
-      else if (g.b_scale_mode == SCALE_OUTER_VEC) sb_v = (const float *)g.b_scale;
-      if (g.c_scale) sc = *(const float *)g.c_scale;
-      if (g.d_scale) sd = *(const float *)g.d_scale;
+      if (g.alpha_mode != SCALAR_VALUE && g.alpha_mode != SCALAR_DEV) alpha_v = (const float *)g.alpha_ptr + g.alpha_sb * bt;
+      if (g.beta_mode != SCALAR_VALUE && g.beta_mode != SCALAR_DEV) beta_v = (const float *)g.beta_ptr;
+      if (g.a_scale_mode == SCALE_OUTER_VEC) sa_v = (const float *)g.a_scale;
+      if (g.b_scale_mode == SCALE_OUTER_VEC) sb_v = (const float *)g.b_scale;
     }
   }
 
