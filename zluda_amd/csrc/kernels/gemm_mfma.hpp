@@ -86,6 +86,14 @@ __device__ __forceinline__ void buffer_store_b128_guarded(v4i data, __amdgpu_buf
   asm volatile("s_nop 1" : "+v"(data)::"memory");
 }
 
+// The same guard for a 64-bit store.  The corruption was only ever seen with the 128-bit form, but nothing known about
+// it says the narrower store reads its data registers any earlier, and a wait state per store is not measurable in the
+// epilogues that use it.
+__device__ __forceinline__ void buffer_store_b64_guarded(v2i data, __amdgpu_buffer_rsrc_t rs, int voff, int soff) {
+  __builtin_amdgcn_raw_buffer_store_b64(data, rs, voff, soff, 0);
+  asm volatile("s_nop 1" : "+v"(data)::"memory");
+}
+
 struct MfmaParams {
   GemmArgs g;
   int32_t swapped;           // P = op(B)^T rows, Q = op(A) rows
@@ -384,7 +392,7 @@ __device__ __forceinline__ void mfma_store_tile_f(const MfmaParams &prm, AccV (&
           pk[0] = (int)pack_f16x2(x[0], x[1]);
           pk[1] = (int)pack_f16x2(x[2], x[3]);
         }
-        __builtin_amdgcn_raw_buffer_store_b64(pk, rs, voff, soff, 0);
+        buffer_store_b64_guarded(pk, rs, voff, soff);
       }
     }
   };

@@ -142,7 +142,7 @@ __device__ __forceinline__ void mfma16_store_f(const MfmaParams &prm, AccV (&acc
         v2i pk;
         if (to_bf16) { pk[0] = (int)pack_bf16x2(x[0], x[1]); pk[1] = (int)pack_bf16x2(x[2], x[3]); }
         else { pk[0] = (int)pack_f16x2(x[0], x[1]); pk[1] = (int)pack_f16x2(x[2], x[3]); }
-        __builtin_amdgcn_raw_buffer_store_b64(pk, rs, voff, soff, 0);
+        buffer_store_b64_guarded(pk, rs, voff, soff);
       }
     }
     if constexpr (FENCE) __builtin_amdgcn_sched_barrier(0);
