@@ -19,6 +19,7 @@
 // 1 KiB-per-instruction DMA writes and the ds_read_b128 fragment reads are bank-conflict free.
 #pragma once
 #include "gemm_mfma.hpp"
+#include "mfma_wait_counts.hpp"
 
 namespace zluda_amd {
 
@@ -38,29 +39,21 @@ __device__ __forceinline__ void wait_vmcnt_barrier() {
 template <int KIND, int FQ, int FP, int BP, int BQ, int WP, int WQ, int BKB_, int NSTAGE>
 __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams prm) {
   constexpr int NT = WP * WQ * 64;
-  constexpr int CPR = BKB_ / 16;               // 16-byte chunks per LDS row
-  constexpr int RPW = 64 / CPR;                // rows filled by one wave DMA instruction
-  constexpr int RPP = (NT / 64) * RPW;         // rows filled per DMA pass of the workgroup
-  constexpr int LP = BP / RPP, LQ = BQ / RPP;  // data DMA instructions per thread, stage and operand
-  // MX block scales travel in chunks of 32 scale bytes per tile row (1024 K elements = CH stages),
-  // double buffered behind the data stages.  One DMA instruction copies 32 rows x 32 bytes; every
-  // wave issues LS of them per stage (the instructions a chunk does not need read a single cache line,
-  // so that the vmcnt bookkeeping is the same in every stage).
+  // The DMA side's instruction counts and the counted waits come from mfma_wait_counts.hpp, where the rule they rest on
+  // is written down and from where a host program replays them.  In short: one wave instruction fills RPW rows x BKB
+  // bytes; MX block scales travel in chunks of 32 scale bytes per tile row (1024 K elements = CH stages), double
+  // buffered behind the data stages, one DMA instruction per 32 rows x 32 bytes, LS of them per wave and stage (the
+  // instructions a chunk does not need read a single cache line, so that the bookkeeping is the same in every stage).
+  // The counted waits only count the DATA instructions of the younger stages: the scale instructions of a stage are
+  // issued in front of its data, so a wait that also covers them costs nothing, and it does not depend on when the
+  // surplus ones are counted as done -- seen on MI355X: with the scale instructions counted, workgroups that follow
+  // another one on their CU multiplied 1 KiB blocks of the last operand rows of a stage before they had landed.
   constexpr bool MX = KIND == KIND_MXF4;
-  constexpr int SB = BKB_ / 16;                // scale bytes per row and stage
-  constexpr int CH = 32 / SB;                  // stages per scale chunk
-  constexpr int SPARTS = (BP + BQ) / 32;       // DMA instructions per chunk
-  constexpr int NWV = NT / 64;
-  constexpr int LS = MX ? (SPARTS + NWV * (CH - NSTAGE) - 1) / (NWV * (CH - NSTAGE)) : 0;
-  constexpr int PRO_S = MX ? (SPARTS + NWV - 1) / NWV : 0;  // per wave, for the first chunk
+  constexpr PipeCounts PC = pipe_counts(MX, BP, BQ, WP, WQ, BKB_, NSTAGE);
+  constexpr int CPR = PC.cpr, RPW = PC.rpw, RPP = PC.rpp, LP = PC.lp, LQ = PC.lq;
+  constexpr int CH = PC.ch, SPARTS = PC.sparts, NWV = PC.nwv, LS = PC.ls, PRO_S = PC.pro_s;
   constexpr int CHUNK_V4 = MX ? (BP + BQ) * 2 : 0;
-  constexpr int NLOAD = LP + LQ + LS;          // vector memory instructions per stage
-  // The counted waits only count the DATA instructions of the younger stages: the scale instructions of a stage
-  // are issued in front of its data, so a wait that also covers them costs nothing, and it does not depend on when
-  // the surplus ones (which read one cache line over and over) are counted as done -- seen on MI355X: with the
-  // scale instructions counted, workgroups that follow another one on their CU multiplied 1 KiB blocks of the last
-  // operand rows of a stage before they had landed.
-  constexpr int NDATA = LP + LQ;
+  constexpr int NLOAD = PC.nload, NDATA = PC.ndata;
   constexpr int WTP = BP / WP, WTQ = BQ / WQ;
   constexpr int TP = WTP / 32, TQ = WTQ / 32;
   constexpr int KS = BKB_ / (KIND == KIND_F8 ? 64 : 32);  // MFMA sub-steps per stage
@@ -305,7 +298,7 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
     for (int i = 0; i < LS; i++) issue_scale_part(0, SPARTS, s * STAGE_V4);  // surplus: one line, overwritten by the data
     issue_stage(s, s * STAGE_V4);
   }
-  wait_vmcnt_barrier<(NSTAGE - 1) * NDATA>();
+  wait_vmcnt_barrier<PC.wait_prologue>();
 
   Frags fa, fb;
   Scales sc_cur, sc_nxt;
@@ -332,7 +325,7 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe_kernel(MfmaParams 
         // left with the fragment reads and the refill
         if constexpr (s == 0) load_scales(kt + 1, sc_nxt);
       } else {
-        wait_vmcnt_barrier<(NSTAGE - 2) * NDATA>();
+        wait_vmcnt_barrier<PC.wait_stage>();
         // reads first: the compiler cannot prove that the DMA (an LDS write) and these reads hit
         // different slots, so whatever comes second in the source stays second in the schedule
         load_frags(so_next, std::integral_constant<int, 0>{}, nxt);

@@ -28,6 +28,7 @@
 //     The fragment registers (both P halves, both Q halves) are as many as in gemm_mfma_pipe.hpp.
 #pragma once
 #include "gemm_mfma_pipe.hpp"
+#include "mfma_wait_counts.hpp"
 
 namespace zluda_amd {
 
@@ -241,9 +242,11 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe16_kernel(MfmaParam
   constexpr int ESZ = kind_esz(KIND);          // f16 / bf16: the byte geometry of int8 (v_mfma_f32_16x16x32_*: 16 bytes of K per lane)
   constexpr int NT = WP * WQ * 64, NWV = NT / 64;
   constexpr int BKB = 128, CPR = 8, RPW = 8;
-  constexpr int RPP = NWV * RPW;               // rows filled per DMA pass of the workgroup
-  constexpr int LP = BP / RPP, LQ = BQ / RPP;  // DMA instructions per thread, stage and operand
-  constexpr int NLOAD = LP + LQ;
+  constexpr Pipe16Counts PC = pipe16_counts(BP, BQ, WP, WQ);  // (shared with the host program that checks the waits)
+  constexpr int RPP = PC.rpp;                  // rows filled per DMA pass of the workgroup
+  constexpr int LP = PC.lp, LQ = PC.lq;        // DMA instructions per thread, stage and operand
+  constexpr int NLOAD = PC.nload;
+  static_assert(RPP == NWV * RPW, "eight rows per DMA instruction");
   constexpr int WTP = BP / WP, WTQ = BQ / WQ, TP = WTP / 16, TQ = WTQ / 16;
   constexpr int HP = TP / 2, HQ = TQ / 2;      // fragments per half of the wave tile
   constexpr int KS = KIND == KIND_F8 ? 1 : 2;  // MFMAs per fragment pair (K halves of the 128-byte stage)
@@ -425,7 +428,7 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe16_kernel(MfmaParam
   // ---- prologue: stages 0 and 1 in flight, stage 0 landed, its first fragments in registers -----------------
   issue_stage(0, 0);
   issue_stage(1, STAGE_V4);
-  wait_vmcnt_barrier<NLOAD>();
+  wait_vmcnt_barrier<PC.wait_prologue>();
   load_p_half(0, std::integral_constant<int, 0>{});
   load_q_half(0, std::integral_constant<int, 0>{});
 
@@ -458,7 +461,7 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_pipe16_kernel(MfmaParam
     pattern(std::integral_constant<int, DSP - 2 * EARLY>{}, std::integral_constant<int, 0>{});
     // every fragment of the stage has been requested: wait for them and for this wave's share of stage
     // kt+1, meet the other waves; then the slot is free and the other one readable
-    wait_vmcnt_barrier<0>();
+    wait_vmcnt_barrier<PC.wait_stage>();
     // (P1, QB): refill this slot with stage kt+2, P half 0 of stage kt+1 arrives
     load_p_part(so_next, P0{}, I0{}, IL{});
     issue_stage(kt + NSTAGE, so);

@@ -237,7 +237,7 @@ __global__ __launch_bounds__(WP *WQ * 64) void gemm_mfma_tr_kernel(MfmaParams pr
   // front of the LDS stores, which consume the older stage's registers) could pass too early.  From the
   // first trip whose younger stage is that last stage (stage kt + 2 >= KL) the stores are therefore preceded
   // by a wait for everything.  With K % 64 == 0 no such instruction exists and nothing is added.
-  const int tail_from = ((Kl * ESZ) & 63) ? KL - 2 : 0x7fffffff;
+  const int tail_from = tr_tail_from(Kl * ESZ);  // (mfma_wait_counts.hpp, where a host program checks it)
 
   // LDS rows (in v4i units) of this lane's fragment rows
   int prow[TP], qrow[TQ];
