@@ -157,6 +157,31 @@ def test_four_wave_kernel_stages_every_vector_its_epilogue_reads(gpu_api):
     check(gpu_api, dict(vec, m=1100, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS, bias_type=K.CUDA_R_16F), 924, *v11)
 
 
+def test_four_wave_kernel_mxfp4(gpu_api):
+    """variant 11 for MXFP4: scale chunks of four stages prefetched through two LDS buffers across tile boundaries.  One,
+    two, three and five chunks per tile (odd counts flip the buffer a tile's first chunk lands in), grids of fewer
+    workgroups than tiles, batches, a row-major D, GELU; tiles that are partial along M take the element-wise epilogue
+    and restart the stream.  FP4 products and their fp32 sums of this size are exact: the results match the oracle's
+    bf16 outputs bit for bit."""
+    v11 = K.ZLUDA_KERNEL_MFMA_MXF4
+    for i, (shape, grid) in enumerate([(dict(m=256, n=256, k=1024), None), (dict(m=512, n=256, k=2048), None),
+                                       (dict(m=512, n=512, k=3072), 1), (dict(m=1024, n=768, k=2048), 3),
+                                       (dict(m=768, n=512, k=1024, batch=3), 4), (dict(m=512, n=512, k=4096, order_c=1, order_d=1), 3),
+                                       (dict(m=512, n=256, k=5120, alpha=0.5), 1), (dict(m=640, n=512, k=2048, ldd=648), 2),
+                                       (dict(m=512, n=512, k=2048, epilogue=K.CUBLASLT_EPILOGUE_GELU), 2)]):
+        spec = dict(MX, **shape)
+        print("case", spec, "grid", grid, flush=True)
+        case = Case(spec, 700 + i)
+        ref = case.run_oracle()
+        if grid is None:
+            st, got, _, v = case.run_gpu(gpu_api, forced_kernel=v11, forced_variant=11)
+        else:
+            st, got, plan = case.run_gpu_plan(gpu_api, v11, 11, grid_x=grid)
+            v = plan.variant
+        assert st == 0 and v == 11
+        case.compare(got, ref)
+
+
 # ---- MXFP4 -----------------------------------------------------------------------------------------
 @pytest.mark.parametrize("variant", range(8))
 def test_mfma_mxf4_variants(gpu_api, variant):

@@ -42,7 +42,7 @@ def test_baseline_configs_pick_the_intended_kernels(api):
     st, p = plan(api, dict(F8, m=8192, n=8192, k=8192, transa=1, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS))  # config 4
     assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_F8 and p.variant == 11 and p.grid_x == 256 and p.grid_y == 1   # 1024 tiles, 4 per workgroup
     st, p = plan(api, dict(MX, m=8192, n=8192, k=8192, transa=1, batch=4))          # config 5
-    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_MXF4 and p.grid_x == 1024 and p.grid_y == 4
+    assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_MXF4 and p.variant == 11 and p.grid_x == 256 and p.grid_y == 1   # 4096 tiles, 16 per workgroup
     assert p.workspace == 0
 
 
@@ -154,10 +154,11 @@ def test_extents_that_256_divides_badly_get_the_192_row_tile(api):
     assert st == 0 and p.variant == 11
     st, p = plan(api, dict(F8, m=8192, n=4096, k=4096, transa=1))
     assert st == 0 and p.variant == 11
-    st, p = plan(api, dict(MX, m=8192, n=8192, k=8192, transa=1))      # MXFP4 has no 16x16-shape variant
-    assert st == 0 and p.variant == 0
-    assert plan(api, dict(MX, m=8192, n=8192, k=8192, transa=1), forced=K.ZLUDA_KERNEL_MFMA_MXF4, variant=8)[0] == K.CUBLAS_STATUS_INVALID_VALUE
-    assert api.zluda_gemm_variant_count(K.ZLUDA_KERNEL_MFMA_I8) == 12 and api.zluda_gemm_variant_count(K.ZLUDA_KERNEL_MFMA_MXF4) == 8
+    st, p = plan(api, dict(MX, m=8192, n=8192, k=8192, transa=1))      # MXFP4 has no eight-wave 16x16-shape variant, but the four-wave kernel
+    assert st == 0 and p.variant == 11
+    for v in (8, 9, 10):
+        assert plan(api, dict(MX, m=8192, n=8192, k=8192, transa=1), forced=K.ZLUDA_KERNEL_MFMA_MXF4, variant=v)[0] == K.CUBLAS_STATUS_INVALID_VALUE
+    assert api.zluda_gemm_variant_count(K.ZLUDA_KERNEL_MFMA_I8) == 12 and api.zluda_gemm_variant_count(K.ZLUDA_KERNEL_MFMA_MXF4) == 12
 
 
 def test_the_four_wave_kernel_is_chosen_for_what_its_epilogues_serve(api):
@@ -195,6 +196,16 @@ def test_the_four_wave_kernel_is_chosen_for_what_its_epilogues_serve(api):
     assert plan(api, dict(F8, **big, a_type=K.CUDA_R_8F_E5M2), forced=K.ZLUDA_KERNEL_MFMA_F8, variant=11)[0] == K.CUBLAS_STATUS_NOT_SUPPORTED
     bf = dict(a_type=K.CUDA_R_16BF, b_type=K.CUDA_R_16BF, d_type=K.CUDA_R_16BF, compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F)
     assert plan(api, dict(bf, **big), forced=K.ZLUDA_KERNEL_MFMA_H16, variant=11)[0] == K.CUBLAS_STATUS_INVALID_VALUE
+    # MXFP4: bf16 output, whole scale chunks (K a multiple of 1024), and no vector along D's unit stride at all (its
+    # scale chunks take the LDS that holds such vectors for the other kinds)
+    assert plan(api, dict(MX, **big))[1].variant == 11
+    assert plan(api, dict(MX, **big, epilogue=K.CUBLASLT_EPILOGUE_GELU))[1].variant == 11
+    assert plan(api, dict(MX, **big, epilogue=K.CUBLASLT_EPILOGUE_BIAS))[1].variant == 0
+    assert plan(api, dict(MX, **big, pointer_mode=K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO))[1].variant == 0
+    assert plan(api, dict(MX, m=8192, n=8192, k=8192 + 512, transa=1))[1].variant == 0
+    assert plan(api, dict(MX, **big, d_type=K.CUDA_R_32F))[1].variant == 0
+    f32 = dict(a_type=K.CUDA_R_32F, b_type=K.CUDA_R_32F, d_type=K.CUDA_R_32F, compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F)
+    assert plan(api, dict(f32, **big), forced=K.ZLUDA_KERNEL_MFMA_F32, variant=11)[0] == K.CUBLAS_STATUS_INVALID_VALUE
 
 
 def test_row_major_output_swaps_operands(api):

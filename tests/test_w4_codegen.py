@@ -49,7 +49,7 @@ def agprs(operand_text):
     return regs
 
 
-@pytest.mark.parametrize("unit", ["mfma_w4_f8.hip", "mfma_w4_i8.hip"])
+@pytest.mark.parametrize("unit", ["mfma_w4_f8.hip", "mfma_w4_i8.hip", "mfma_w4_mxf4.hip"])
 def test_nothing_reads_an_accumulator_too_soon_after_an_mfma(unit):
     found = kernels(assembly(unit))
     assert found, "no four-wave kernel in " + unit
@@ -84,16 +84,46 @@ def test_nothing_reads_an_accumulator_too_soon_after_an_mfma(unit):
         assert n_mfma >= 256, name
 
 
-@pytest.mark.parametrize("unit", ["mfma_w4_f8.hip", "mfma_w4_i8.hip"])
+def loop_body(body, name):
+    """the K loop of a kernel: the blocks of the first inner loop that holds MFMAs, wherever the layout put them (the
+    loop may hold forward branches -- the MXFP4 kernel decides per stage whether a scale instruction is due -- and its
+    latch may sit in front of its header)"""
+    blocks, cur = [], []
+    for line in body.split("\n"):
+        if re.match(r"^(\.LBB\d+_\d+:|; %bb\.\d+:)", line):
+            blocks.append(cur)
+            cur = []
+        cur.append(line)
+    blocks.append(cur)
+    for b in blocks:
+        head = "\n".join(b[:3])
+        if "Inner Loop Header: Depth=2" not in head:
+            continue
+        label = b[0].split(":")[0].lstrip(".L")        # BB0_52
+        mine = [x for x in blocks if x is b or re.search(r"Header=" + re.escape(label) + r" Depth=2", "\n".join(x[:3]))]
+        text = "\n".join("\n".join(x) for x in mine)
+        if "v_mfma" in text:
+            return text
+    raise AssertionError("no K loop found in " + name)
+
+
+@pytest.mark.parametrize("unit", ["mfma_w4_f8.hip", "mfma_w4_i8.hip", "mfma_w4_mxf4.hip"])
 def test_the_k_loop_is_free_of_spills_and_accumulator_moves(unit):
     text = assembly(unit)
+    mx = "mxf4" in unit
+    n = 0
     for m in re.finditer(r"^(_ZN9zluda_amd19gemm_mfma_w4_kernel\w+):\s*;.*?\n(.*?)^\s*s_endpgm", text, re.S | re.M):
-        body = m.group(2)
-        # the innermost loop: from its header comment to the branch that closes it
-        loops = [b for b in re.split(r"Inner Loop Header: Depth=2", body)[1:]]
-        assert loops, m.group(1)
-        hot = loops[0].split("s_cbranch")[0]
+        hot = loop_body(m.group(2), m.group(1))
+        n += 1
         assert hot.count("v_mfma") in (128, 256), "%s: %d MFMAs in the loop of two stages" % (m.group(1), hot.count("v_mfma"))
-        for bad in ("scratch_", "v_accvgpr_", "v_readlane", "v_writelane"):
+        for bad in ("scratch_", "v_accvgpr_") + (() if mx else ("v_readlane", "v_writelane")):
             assert bad not in hot, "%s: %s inside the K loop" % (m.group(1), bad)
-        assert hot.count("ds_read_b128") == 64 and hot.count("buffer_load_dwordx4") == 32 and hot.count("s_barrier") == 2, m.group(1)
+        assert hot.count("ds_read_b128") == 64 and hot.count("s_barrier") == 2, m.group(1)
+        # data DMA: 16 instructions per wave and stage; MXFP4: scale instructions on top (two in the stage that starts a
+        # chunk, one in the next two, none in the fourth), its 16 + 16
+        # two-byte scale fragments per stage, and nothing but the two barrier waits counts vector memory operations
+        # (three sites: the odd stage of a pair never starts a chunk, which the compiler sees)
+        assert hot.count("buffer_load_dwordx4") == (32 + 3 if mx else 32), (m.group(1), hot.count("buffer_load_dwordx4"))
+        assert hot.count("ds_read_u16") == (32 if mx else 0), m.group(1)
+        assert hot.count("s_waitcnt vmcnt") == 2, m.group(1)
+    assert n >= 1

@@ -349,14 +349,17 @@ __device__ __forceinline__ bool w4_fast_epilogue_ok(const MfmaParams &prm) {
     // vectors that run along Q (a per-column scale; for a row-major D the per-row ones and the bias) are not served
     const bool q_vec = prm.swapped ? (g.alpha_mode == VECTOR_DEV || g.a_scale_mode == SCALE_OUTER_VEC || g.bias != nullptr)
                                    : g.b_scale_mode == SCALE_OUTER_VEC;
+    // (MXFP4 has no room in LDS for staged vectors: no alpha[], no bias)
+    const bool p_vec = g.alpha_mode == VECTOR_DEV || g.bias != nullptr;
     return !g.int_scale && g.beta_mode == SCALAR_VALUE && g.beta_val.f == 0.0f && g.d_type == CUDA_R_16BF && !q_vec &&
-           g.act == (EPI == W4_EPI_BF16_GELU ? ACT_GELU : ACT_NONE);
+           !(KIND == KIND_MXF4 && p_vec) && g.act == (EPI == W4_EPI_BF16_GELU ? ACT_GELU : ACT_NONE);
   }
 }
 
 template <int KIND, int FQ, int FP, int EPI>
 __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
-  static_assert(KIND == KIND_I8 || KIND == KIND_F8, "int8 and fp8 operands");
+  static_assert(KIND == KIND_I8 || KIND == KIND_F8 || KIND == KIND_MXF4, "int8, fp8 and MXFP4 operands");
+  constexpr bool MX = KIND == KIND_MXF4;
   constexpr int BP = 256, BQ = 256, WP = 2, WQ = 2;
   constexpr int NWV = 4;
   constexpr int BKB = 128, CPR = 8, RPW = 8;
@@ -377,9 +380,15 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
   // the two slots; behind them each wave's staging area for the vectors its epilogue needs (W4Staged).  (One array: with
   // a second LDS object in the kernel the compiler puts a vmcnt(0) in front of every LDS read that follows a DMA
   // instruction.)
+  // MXFP4: behind the slots two chunks of block scales instead -- 32 scale bytes (1024 K elements = 4 stages) of each of
+  // the tile's 512 rows per chunk, [row][32 bytes] -- which fills the CU's LDS: no staged vectors, and no fast epilogue
+  // for problems that have any.
   constexpr int STG_WAVE = 3 * W4Staged::WORDS;
-  constexpr int STG_V4 = EPI == W4_EPI_I32 ? 0 : NWV * STG_WAVE / 4;
-  __shared__ v4i lds[2 * STAGE_V4 + STG_V4];
+  constexpr int STG_V4 = (EPI == W4_EPI_I32 || MX) ? 0 : NWV * STG_WAVE / 4;
+  constexpr int SC_CHUNK_V4 = MX ? (BP + BQ) * 2 : 0;
+  constexpr int SC_BASE = 2 * STAGE_V4 + STG_V4;
+  static_assert((SC_BASE + 2 * SC_CHUNK_V4) * 16 <= 160 * 1024, "LDS capacity");
+  __shared__ v4i lds[SC_BASE + 2 * SC_CHUNK_V4];
 
   const GemmArgs &g = prm.g;
   const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
@@ -387,13 +396,13 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
   const int r16 = lane & 15, g4 = lane >> 4;
 
   const int NP = prm.swapped ? g.N : g.M, NQ = prm.swapped ? g.M : g.N;
-  const int Kbytes = g.K;
+  const int Kbytes = MX ? g.K / 2 : g.K;  // (two E2M1 per byte)
   const int KT2 = (Kbytes + 2 * BKB - 1) / (2 * BKB) * 2;  // stages per tile, an even number: a last odd one multiplies zeros
   const int total = prm.tiles_p * prm.tiles_q;
   const int ntiles = total * g.batch;
   const int G = (int)gridDim.x;
   const int my_tiles = (ntiles - (int)blockIdx.x + G - 1) / G;  // >= 1: the grid never exceeds the tile count
-  const int ldp = (int)(prm.swapped ? g.b_sj : g.a_si), ldq = (int)(prm.swapped ? g.a_si : g.b_sj);
+  const int ldp = (int)(prm.swapped ? g.b_sj : g.a_si) >> (MX ? 1 : 0), ldq = (int)(prm.swapped ? g.a_si : g.b_sj) >> (MX ? 1 : 0);  // bytes
 
   // n-th tile of this workgroup -> tile corner and batch (the order of gemm_mfma_pipe_kernel: the 8 XCDs take
   // turns at workgroup ids, so ids are spread over 8 contiguous ranges of the tile order, which walks groups
@@ -410,6 +419,46 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
     q0 = ((w % group) / gsz) * BQ;
   };
 
+  // ---- MXFP4 block scales ---------------------------------------------------------------------------------------
+  // A chunk = 32 scale bytes (four stages) of each of the tile's 512 rows, [row][32] in one of two LDS buffers, filled
+  // by 16 DMA instructions of 32 rows x 32 bytes (lane l -> row l / 2, half l % 2), four per wave: wave w issues parts
+  // w, 4 + w (P rows), 8 + w, 12 + w (Q rows).  The planner admits K % 1024 == 0, so chunks and tiles end together and
+  // stream chunk number s (tile ordinal * chunks per tile + chunk) lives in buffer s % 2.  When they are issued
+  // (always behind a stage's barrier, with the data that refills the slot):
+  //   chunk C >= 1 of a tile: parts 0 and 1 in the tile's stage 4 C - 4, part 2 in stage 4 C - 3, part 3 in stage 4 C - 2.
+  //     Chunk C - 2, which the buffer held, was last read (the scales of stage 4 C - 5, fetched at the end of stage
+  //     4 C - 6) two barriers earlier, and the chunk has landed by the barrier of stage 4 C - 1, behind which the scales
+  //     of stage 4 C are fetched;
+  //   chunk 0 of the next tile: all four parts in the last but one stage of the tile, right after the DMA side has moved
+  //     on to that tile (landed by the last stage's barrier, behind which the next tile's first scales are fetched);
+  //   chunk 0 of the first tile: with the first two stages, before the stream starts.
+  // A lane needs two bytes per tile row and stage (its K blocks 2 g4 and 2 g4 + 1 of the stage's eight); op_sel picks
+  // the K step's byte.
+  const int KB = g.K / 32;                 // scale bytes per row
+  int scP[2][MX ? TP : 1], scQ[2][MX ? TQ : 1];  // [stage parity][tile row set]
+  int ss = 0;                              // stream stage number of the MFMA side
+  int sc_p0 = 0, sc_q0 = 0, sc_first = 0;  // the DMA side's tile: corner, stream number of its chunk 0
+  __amdgpu_buffer_rsrc_t rsSP, rsSQ;
+  auto scale_tile = [&](int n, int p0, int q0, int bt) __attribute__((always_inline)) {
+    if constexpr (MX) {
+      sc_p0 = p0; sc_q0 = q0; sc_first = n * (KT2 / 4);
+      const uint8_t *Ps = (const uint8_t *)(prm.swapped ? g.b_scale : g.a_scale) + (int64_t)bt * NP * KB;
+      const uint8_t *Qs = (const uint8_t *)(prm.swapped ? g.a_scale : g.b_scale) + (int64_t)bt * NQ * KB;
+      rsSP = __builtin_amdgcn_make_buffer_rsrc((void *)Ps, 0, NP * KB, 0x00020000);
+      rsSQ = __builtin_amdgcn_make_buffer_rsrc((void *)Qs, 0, NQ * KB, 0x00020000);
+    }
+  };
+  // this wave's part j (0 .. 3) of chunk c of the DMA side's tile.  (Never issued "dead": an out-of-range instruction
+  // fetches nothing but still writes its zeros into LDS.)
+  auto issue_scale_part = [&](int c, int j) __attribute__((always_inline)) {
+    if constexpr (MX) {
+      const int pt = 4 * j + wave;  // (uniform) parts 0 .. 7: P rows, 8 .. 15: Q rows
+      v4i *dst = &lds[SC_BASE + ((sc_first + c) & 1) * SC_CHUNK_V4 + pt * 64];
+      const int col = 32 * c + 16 * (lane & 1);
+      if (j < 2) lds_dma16(rsSP, dst, min(sc_p0 + 32 * pt + (lane >> 1), NP - 1) * KB + col, 0);
+      else lds_dma16(rsSQ, dst, min(sc_q0 + 32 * (pt - 8) + (lane >> 1), NQ - 1) * KB + col, 0);
+    }
+  };
   // ---- the DMA side: two stages ahead of the MFMAs, across tile boundaries ----------------------------------
   // one wave instruction fills 8 rows x 128 bytes; lane l -> row l / 8, slot l % 8, global chunk slot ^ swizzle(row)
   const int dr = lane / CPR, dslot = lane % CPR;
@@ -422,8 +471,9 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
   auto dma_tile = [&](int n) __attribute__((always_inline)) {
     int p0, q0, bt;
     tile_coords(n, p0, q0, bt);
-    const uint8_t *Pg = prm.swapped ? (const uint8_t *)g.B + g.b_sb * bt : (const uint8_t *)g.A + g.a_sb * bt;
-    const uint8_t *Qg = prm.swapped ? (const uint8_t *)g.A + g.a_sb * bt : (const uint8_t *)g.B + g.b_sb * bt;
+    constexpr int SH = MX ? 1 : 0;  // elements -> bytes
+    const uint8_t *Pg = prm.swapped ? (const uint8_t *)g.B + ((g.b_sb * bt) >> SH) : (const uint8_t *)g.A + ((g.a_sb * bt) >> SH);
+    const uint8_t *Qg = prm.swapped ? (const uint8_t *)g.A + ((g.a_sb * bt) >> SH) : (const uint8_t *)g.B + ((g.b_sb * bt) >> SH);
     // 2 GiB raw buffer windows: an offset with bit 31 set is out of range and reads as zero
     rsP = __builtin_amdgcn_make_buffer_rsrc((void *)Pg, 0, 0x80000000, 0x00020000);
     rsQ = __builtin_amdgcn_make_buffer_rsrc((void *)Qg, 0, 0x80000000, 0x00020000);
@@ -431,6 +481,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
     for (int i = 0; i < LP; i++) voffP[i] = min(p0 + drow + RPP * i, NP - 1) * ldp + dcg * 16;
 #pragma unroll
     for (int i = 0; i < LQ; i++) voffQ[i] = min(q0 + drow + RPP * i, NQ - 1) * ldq + dcg * 16;
+    scale_tile(n, p0, q0, bt);
   };
   // instructions [I0, I1) of the NLOAD that bring stage dk of the DMA side's tile into the slot at `so`.  Lanes
   // past the end of K (the tail of the last stage, the whole padding stage of an odd stage count) are out of
@@ -454,7 +505,9 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
 #pragma unroll
     for (int kk = 0; kk < 2; kk++) {
       const int row = par * 16 + r16;
-      const int ch = (KIND == KIND_F8 ? 2 * g4 + kk : 4 * kk + g4) ^ swz(row);
+      // fp8: the lane's 32 bytes of its K group; int8: 16 bytes of each K half; MXFP4: 16 bytes (one scale block of 32
+      // elements) of each K step from the lane group's own 32-byte range, so that its two scale bytes are neighbours
+      const int ch = (KIND == KIND_I8 ? 4 * kk + g4 : 2 * g4 + kk) ^ swz(row);
       fragP[par][kk] = (wp * WTP + row) * CPR + ch;
       fragQ[par][kk] = (BP + wq * WTQ + row) * CPR + ch;
     }
@@ -469,6 +522,17 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
       for (int e = 0; e < 4; e++) dst[i].k[0][4 * kk + e] = x[e];
     } else {
       dst[i].k[kk] = x;
+    }
+  };
+
+  // scale number r (0 .. TP + TQ - 1: P tile rows, then Q's) of stream stage `st` into the registers of parity `par`
+  const int sc_lane_p = (wp * WTP + r16) * 32 + 2 * g4, sc_lane_q = (BP + wq * WTQ + r16) * 32 + 2 * g4;  // bytes in a chunk
+  auto read_scale = [&](int st, auto par_c, auto r_c) __attribute__((always_inline)) {
+    if constexpr (MX) {
+      constexpr int par = decltype(par_c)::value, r = decltype(r_c)::value;
+      const char *chunk = (const char *)&lds[SC_BASE + ((st >> 2) & 1) * SC_CHUNK_V4] + (st & 3) * 8;
+      if constexpr (r < TP) scP[par][r] = *(const uint16_t *)(chunk + sc_lane_p + r * 512);
+      else scQ[par][r - TP] = *(const uint16_t *)(chunk + sc_lane_q + (r - TP) * 512);
     }
   };
 
@@ -491,15 +555,23 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
   };
   // MFMA number x of the sub-step (P half ph, Q half qh): K half x / (HP * HQ), tile pair (i, j) with i the
   // slower index, so that the fragments a sub-step reads first are the ones the next sub-step multiplies first
-  auto mfma_one = [&](auto ph_c, auto qh_c, auto x_c) __attribute__((always_inline)) {
-    constexpr int ph = decltype(ph_c)::value, qh = decltype(qh_c)::value, x = decltype(x_c)::value;
+  auto mfma_one = [&](auto ph_c, auto qh_c, auto x_c, auto par_c) __attribute__((always_inline)) {
+    constexpr int ph = decltype(ph_c)::value, qh = decltype(qh_c)::value, x = decltype(x_c)::value, par = decltype(par_c)::value;
     constexpr int ks = x / (HP * HQ), i = (x % (HP * HQ)) / HQ, j = x % HQ;
     acc_v &c = acc[ph * HP + i][qh * HQ + j];
     const frag_v &pa = pf[ph][i].k[ks], &qb = qf[qh][j].k[ks];  // (named here: asm operands alone do not capture)
-    (void)c; (void)pa; (void)qb;
+    (void)c; (void)pa; (void)qb; (void)par;
 #if defined(__HIP_DEVICE_COMPILE__)  // (the register constraints mean something else to the host pass)
     if constexpr (KIND == KIND_I8) {
       asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(c) : "v"(pa), "v"(qb));
+    } else if constexpr (MX) {
+      const int &sa = scP[par][ph * HP + i], &sb = scQ[par][qh * HQ + j];
+      if constexpr (ks == 0)
+        asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:[0,0,0] op_sel_hi:[0,0,0] cbsz:4 blgp:4"
+                     : "+a"(c) : "v"(pa), "v"(qb), "v"(sa), "v"(sb));
+      else
+        asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:[1,1,0] op_sel_hi:[0,0,0] cbsz:4 blgp:4"
+                     : "+a"(c) : "v"(pa), "v"(qb), "v"(sa), "v"(sb));
     } else if constexpr (FP == 0 && FQ == 0) {
       asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(c) : "v"(pa), "v"(qb));
     } else if constexpr (FP == 1 && FQ == 0) {
@@ -514,13 +586,14 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
 
   // One sub-step: its NM MFMAs in order; behind each of the first NRD of them one fragment read (`rd(r)`), and the
   // NLOAD DMA instructions spread evenly behind all of them when the sub-step refills a slot.
-  auto substep = [&](auto ph_c, auto qh_c, auto &&rd, auto l0_c, auto l1_c, int dma_dk, int dma_so) __attribute__((always_inline)) {
+  auto substep = [&](auto ph_c, auto qh_c, auto par_c, auto &&rd, auto &&extra, auto l0_c, auto l1_c, int dma_dk, int dma_so) __attribute__((always_inline)) {
     constexpr int L0 = decltype(l0_c)::value, L1 = decltype(l1_c)::value;  // DMA instructions [L0, L1) of the stage ride along
     static_assert(NM >= NRD && NM >= L1 - L0, "room for the reads and the DMA of a sub-step");
     static_for<NM>([&](auto x_c) {
       constexpr int x = decltype(x_c)::value;
-      mfma_one(ph_c, qh_c, x_c);
+      mfma_one(ph_c, qh_c, x_c, par_c);
       if constexpr (x < NRD) rd(x_c);
+      extra(x_c);
       if constexpr (L1 > L0) {
         // spread evenly: a wave that has its SIMD to itself and queues vector memory instructions faster than the CU's
         // address unit takes them (one 1 KiB instruction per 16 clocks, for all four SIMDs) keeps its next MFMA waiting
@@ -538,26 +611,55 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
   // leaves P half 0 and Q half 1 - ODD of the next stage there, and refills its slot with stage dk of the DMA
   // side's tile.
   //   (P0, QA) reads QB | (P0, QB) reads P1 | barrier | (P1, QB) reads P0', refills the slot | (P1, QA) reads QB'
-  auto do_stage = [&](auto odd_c, int dk) __attribute__((always_inline)) {
+  auto do_stage = [&](auto odd_c, auto last_c, int dk) __attribute__((always_inline)) {
     constexpr int ODD = decltype(odd_c)::value;
+    constexpr bool LAST = decltype(last_c)::value != 0;  // the tile's last two stages (dk = 0, 1 of the next tile)
     constexpr int so = ODD * STAGE_V4, so_next = (1 - ODD) * STAGE_V4;
     using QA = std::integral_constant<int, ODD>;
     using QB = std::integral_constant<int, 1 - ODD>;
     using Z = std::integral_constant<int, 0>;
     using LS = std::integral_constant<int, NLOAD / 2>;
     using LN = std::integral_constant<int, NLOAD>;
-    substep(P0{}, QA{}, [&](auto r_c) { read_piece(so, fragQ, qf[1 - ODD], QB{}, r_c); }, Z{}, Z{}, 0, 0);
-    substep(P0{}, QB{}, [&](auto r_c) { read_piece(so, fragP, pf[1], P1{}, r_c); }, Z{}, Z{}, 0, 0);
+    auto none = [](auto) {};
+    substep(P0{}, QA{}, odd_c, [&](auto r_c) { read_piece(so, fragQ, qf[1 - ODD], QB{}, r_c); }, none, Z{}, Z{}, 0, 0);
+    substep(P0{}, QB{}, odd_c, [&](auto r_c) { read_piece(so, fragP, pf[1], P1{}, r_c); }, none, Z{}, Z{}, 0, 0);
     // every fragment of the stage has been requested: wait for them and for this wave's share of the next stage,
     // meet the other waves; then this slot is free and the other one readable
     wait_vmcnt_barrier<0>();
-    substep(P1{}, QB{}, [&](auto r_c) { read_piece(so_next, fragP, pf[0], P0{}, r_c); }, Z{}, LS{}, dk, so);
-    substep(P1{}, QA{}, [&](auto r_c) { read_piece(so_next, fragQ, qf[1 - ODD], QB{}, r_c); }, LS{}, LN{}, dk, so);
+    // (MXFP4: the wave's scale instruction of this stage rides behind the second MFMA, and the next stage's scales are
+    // fetched behind the fragment reads of the last sub-step)
+    substep(P1{}, QB{}, odd_c, [&](auto r_c) { read_piece(so_next, fragP, pf[0], P0{}, r_c); },
+            [&](auto x_c) {
+              constexpr int x = decltype(x_c)::value;
+              if constexpr (MX && LAST) {
+                // the next tile's chunk 0, if there is a next tile
+                if constexpr (ODD == 0 && (x & 1) == 1 && x < 8) {
+                  if (d_live) issue_scale_part(0, x / 2);
+                }
+              } else if constexpr (MX && (x == 1 || x == 3)) {
+                // this is the tile's stage dk - 2: chunk (dk + 2) / 4, by the stage's position in its group of four
+                const int c = (dk + 2) >> 2, phase = (dk + 2) & 3;
+                if (dk + 2 < KT2) {
+                  if constexpr (x == 1) {
+                    if (phase != 3) issue_scale_part(c, phase == 0 ? 0 : phase + 1);
+                  } else {
+                    if (phase == 0) issue_scale_part(c, 1);
+                  }
+                }
+              }
+            }, Z{}, LS{}, dk, so);
+    substep(P1{}, QA{}, odd_c, [&](auto r_c) { read_piece(so_next, fragQ, qf[1 - ODD], QB{}, r_c); },
+            [&](auto x_c) {
+              constexpr int x = decltype(x_c)::value;
+              if constexpr (MX && x >= NRD && x < NRD + TP + TQ)
+                read_scale(ss + 1, std::integral_constant<int, 1 - ODD>{}, std::integral_constant<int, x - NRD>{});
+            }, LS{}, LN{}, dk, so);
+    if constexpr (MX) ss++;
   };
   // two stages, which refill their slots with stages dk and dk + 1 of the DMA side's tile
-  auto do_pair = [&](int dk) __attribute__((always_inline)) {
-    do_stage(std::integral_constant<int, 0>{}, dk);
-    do_stage(std::integral_constant<int, 1>{}, dk + 1);
+  auto do_pair = [&](int dk, auto last_c) __attribute__((always_inline)) {
+    do_stage(std::integral_constant<int, 0>{}, last_c, dk);
+    do_stage(std::integral_constant<int, 1>{}, last_c, dk + 1);
   };
   // the fragments a tile's first stage expects in registers (P half 0, Q half 0), from slot 0
   auto first_frags = [&]() __attribute__((always_inline)) {
@@ -568,6 +670,13 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
   auto prime = [&](int n) __attribute__((always_inline)) {
     d_live = -1;
     dma_tile(n);
+    if constexpr (MX) {
+      // (only the stream's very first tile: later ones had their chunk 0 requested in the tile before)
+      if (n == 0) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) issue_scale_part(0, j);
+      }
+    }
     issue_part(0, 0, std::integral_constant<int, 0>{}, std::integral_constant<int, NLOAD>{});
     issue_part(1, STAGE_V4, std::integral_constant<int, 0>{}, std::integral_constant<int, NLOAD>{});
     wait_vmcnt_barrier<0>();
@@ -586,7 +695,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
     int raw = g.alpha_mode == SCALAR_VALUE ? g.alpha_val.i : (g.alpha_mode == SCALAR_DEV ? *(const int32_t *)g.alpha_ptr : 1);
     ialpha = (int)f2bits(w4_uniform_now(bits2f((uint32_t)raw)));
   }
-  W4Staged staged{(const int *)&lds[2 * STAGE_V4] + (EPI == W4_EPI_I32 ? 0 : wave * STG_WAVE), {false, false, false}, 0};
+  W4Staged staged{(const int *)&lds[2 * STAGE_V4] + (STG_V4 == 0 ? 0 : wave * STG_WAVE), {false, false, false}, 0};
   // epilogue of the tile at (p0, q0, bt); returns false when it needed the LDS (the stream must be primed again)
   auto epilogue = [&](int p0, int q0, int bt) __attribute__((always_inline)) -> bool {
     // MFMA write -> read of the accumulators: the wait states the compiler would insert if it could see the MFMAs.
@@ -611,7 +720,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
   // staging area: requested at the top of the tile, landed by the vmcnt(0) waits of the tile's last two stages (there
   // always are two).  Only the wave itself reads them, after those waits and before it requests the next tile's.
   auto stage_vectors = [&](int p0, int bt) __attribute__((always_inline)) {
-    if constexpr (EPI != W4_EPI_I32) {
+    if constexpr (EPI != W4_EPI_I32 && !MX) {
       staged.has[0] = staged.has[1] = staged.has[2] = false;
       staged.bias_skip = 0;
       if (fast && p0 + BP <= NP) {
@@ -645,17 +754,19 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
   };
 
   // ---- the stream -------------------------------------------------------------------------------------------------
+  static_assert(!MX || NM >= NRD + TP + TQ, "room for the scale reads in a sub-step");
   prime(0);
+  if constexpr (MX) static_for<TP + TQ>([&](auto r_c) { read_scale(0, std::integral_constant<int, 0>{}, r_c); });
   for (int n = 0; n < my_tiles; n++) {
     int p0, q0, bt;
     tile_coords(n, p0, q0, bt);
     stage_vectors(p0, bt);
     zero_acc();
-    for (int kt = 2; kt < KT2; kt += 2) do_pair(kt);
+    for (int kt = 2; kt < KT2; kt += 2) do_pair(kt, std::integral_constant<int, 0>{});
     // the last two stages of the tile fetch the first two of the next one
     if (n + 1 < my_tiles) dma_tile(n + 1);
     else d_live = 0;
-    do_pair(0);
+    do_pair(0, std::integral_constant<int, 1>{});
     const bool kept = epilogue(p0, q0, bt);
     // The first fragments of the next tile are fetched again behind the epilogue (its first stage landed before the
     // last barrier): holding them across it would take 64 of the registers the epilogue needs.

@@ -52,10 +52,11 @@ uint32_t launch_mfma(const Lowered &l, const zluda_gemm_plan &plan_in, void *ws,
       prm.tiles_p = (np + 255) / 256; prm.tiles_q = (nq + 255) / 256;
       prm.group_p = 8;
       prm.splits = 1; prm.split_stages = 0; prm.ws = nullptr;
-      return plan.kernel == ZLUDA_KERNEL_MFMA_I8 ? launch_mfma_w4_i8(prm, epi, plan.grid_x, s)
-                                                 : launch_mfma_w4_f8(prm, epi, plan.grid_x, s);
+      return plan.kernel == ZLUDA_KERNEL_MFMA_I8     ? launch_mfma_w4_i8(prm, epi, plan.grid_x, s)
+             : plan.kernel == ZLUDA_KERNEL_MFMA_MXF4 ? launch_mfma_w4_mxf4(prm, epi, plan.grid_x, s)
+                                                     : launch_mfma_w4_f8(prm, epi, plan.grid_x, s);
     }
-    plan.variant = 8;
+    plan.variant = plan.kernel == ZLUDA_KERNEL_MFMA_MXF4 ? 0 : 8;  // (MXFP4 has no 16x16 eight-wave form)
     plan.grid_x = (uint32_t)(all / l.g.batch); plan.grid_y = l.g.batch; plan.grid_z = 1;
     plan.block = 512;
     plan.workspace = 0;

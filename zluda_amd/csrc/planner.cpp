@@ -359,6 +359,14 @@ int w4_epilogue_class(const Lowered &l, bool dry) {
     if (q_vec) return W4_CLASS_NONE;
     return g.act == ACT_GELU ? W4_CLASS_BF16_GELU : W4_CLASS_BF16;
   }
+  if (g.a_type == CUDA_R_4F_E2M1 && g.b_type == CUDA_R_4F_E2M1 && g.a_scale_mode == SCALE_BLOCK32_UE8M0 &&
+      g.b_scale_mode == SCALE_BLOCK32_UE8M0) {
+    // MXFP4: whole scale chunks (1024 elements of K) per tile, and no vector along D's unit stride either (the scale
+    // chunks take the LDS the other kinds stage such vectors in)
+    if (g.d_type != CUDA_R_16BF || (g.act != ACT_NONE && g.act != ACT_GELU) || (!dry && g.beta_val.f != 0.0f)) return W4_CLASS_NONE;
+    if ((g.K & 1023) || g.alpha_mode == VECTOR_DEV || l.has_bias) return W4_CLASS_NONE;
+    return g.act == ACT_GELU ? W4_CLASS_BF16_GELU : W4_CLASS_BF16;
+  }
   return W4_CLASS_NONE;
 }
 
@@ -587,7 +595,8 @@ extern "C" uint32_t zluda_gemm_variant_count(uint32_t kernel) {
   case ZLUDA_KERNEL_GENERIC: return 1;
   case ZLUDA_KERNEL_MFMA_I8: case ZLUDA_KERNEL_MFMA_F8: return kNumMfmaVariants;
   case ZLUDA_KERNEL_MFMA_H16: return kNumMfmaVariantsH16;
-  case ZLUDA_KERNEL_MFMA_MXF4: case ZLUDA_KERNEL_MFMA_F32: return kNumMfmaVariants32;  // the 16x16-shape ones serve int8 and fp8
+  case ZLUDA_KERNEL_MFMA_F32: return kNumMfmaVariants32;  // the 16x16-shape ones serve int8, fp8, f16 and bf16
+  case ZLUDA_KERNEL_MFMA_MXF4: return kNumMfmaVariants;   // (the eight 32x32-shape ones and the four-wave kernel; those between are refused)
   case ZLUDA_KERNEL_DECODE_W8A8: return kNumDecodeVariants;
   case ZLUDA_KERNEL_MFMA_TR8: case ZLUDA_KERNEL_MFMA_TR16: return kNumTrVariants;
   case ZLUDA_KERNEL_MFMA_TR32: return kNumTrVariants - 1;  // the 16x16-shape one is not instantiated for f32
@@ -652,11 +661,14 @@ extern "C" uint32_t zluda_gemm_plan_problem(const zluda_gemm_problem *p, uint32_
   case ZLUDA_KERNEL_MFMA_I8: case ZLUDA_KERNEL_MFMA_F8: case ZLUDA_KERNEL_MFMA_MXF4: case ZLUDA_KERNEL_MFMA_H16:
   case ZLUDA_KERNEL_MFMA_F32: {
     int v = forced_variant >= 0 ? forced_variant : pick_mfma_variant(l, cu_count);
-    if (v >= kNumMfmaVariants || (v >= kNumMfmaVariants32 && kernel != ZLUDA_KERNEL_MFMA_I8 && kernel != ZLUDA_KERNEL_MFMA_F8 &&
-                                  kernel != ZLUDA_KERNEL_MFMA_H16) || (v >= kNumMfmaVariantsH16 && kernel == ZLUDA_KERNEL_MFMA_H16))
+    const bool w4 = v < kNumMfmaVariants && kMfmaVariants[v].w4;
+    if (v >= kNumMfmaVariants || (v >= kNumMfmaVariants32 && !w4 && kernel != ZLUDA_KERNEL_MFMA_I8 && kernel != ZLUDA_KERNEL_MFMA_F8 &&
+                                  kernel != ZLUDA_KERNEL_MFMA_H16) || (v >= kNumMfmaVariantsH16 && kernel == ZLUDA_KERNEL_MFMA_H16) ||
+        (w4 && kernel == ZLUDA_KERNEL_MFMA_F32))
       return CUBLAS_STATUS_INVALID_VALUE;
-    // the four-wave kernel exists for int8 and for e4m3 x e4m3 without block scales
-    if (kMfmaVariants[v].w4 && !(l.g.a_type == CUDA_R_8I || (l.g.a_type == CUDA_R_8F_E4M3 && l.g.b_type == CUDA_R_8F_E4M3)))
+    // the four-wave kernel exists for int8, for e4m3 x e4m3 without block scales and for MXFP4
+    if (w4 && !(l.g.a_type == CUDA_R_8I || (l.g.a_type == CUDA_R_8F_E4M3 && l.g.b_type == CUDA_R_8F_E4M3) ||
+                (l.g.a_type == CUDA_R_4F_E2M1 && l.g.b_type == CUDA_R_4F_E2M1)))
       return CUBLAS_STATUS_NOT_SUPPORTED;
     fill_mfma_plan(l, v, cu_count, p->workspace_size, plan);
     // Skinny problems that end up with at most one 64 x 64 workgroup per CU and are not split along K are bound
