@@ -486,15 +486,20 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
   // instructions [I0, I1) of the NLOAD that bring stage dk of the DMA side's tile into the slot at `so`.  Lanes
   // past the end of K (the tail of the last stage, the whole padding stage of an odd stage count) are out of
   // range: zeros, no traffic.
-  auto issue_part = [&](int dk, int so, auto i0_c, auto i1_c) __attribute__((always_inline)) {
+  // PLAIN (MXFP4 inside a tile: K is a whole number of stages and the tile list is not exhausted): the offsets as they
+  // are, no instruction per DMA to mask them.  `wave_rows` = wave * RPW * CPR, which the MXFP4 loop hides from the
+  // optimiser once per stage: hoisted out of the loop, the 32 LDS addresses of a stage pair do not fit the scalar
+  // registers and come back through v_readlane, each with its wait states.
+  auto issue_part = [&](int dk, int so, auto i0_c, auto i1_c, auto plain_c, int wave_rows) __attribute__((always_inline)) {
     constexpr int I0 = decltype(i0_c)::value, I1 = decltype(i1_c)::value;
-    const int soff = (dk * BKB) & d_live;
+    constexpr bool PLAIN = decltype(plain_c)::value != 0;
+    const int soff = PLAIN ? dk * BKB : (dk * BKB) & d_live;
     const int oob = soff < lane_k_left ? 0 : (int)0x80000000;
     v4i *base = &lds[so];
     static_for<I1 - I0>([&](auto k_c) {
       constexpr int k = I0 + decltype(k_c)::value;
-      if constexpr (k < LP) lds_dma16(rsP, base + (wave * RPW + RPP * k) * CPR, (voffP[k] | oob) & d_live, soff);
-      else lds_dma16(rsQ, base + (BP + wave * RPW + RPP * (k - LP)) * CPR, (voffQ[k - LP] | oob) & d_live, soff);
+      if constexpr (k < LP) lds_dma16(rsP, base + wave_rows + RPP * k * CPR, PLAIN ? voffP[k] : (voffP[k] | oob) & d_live, soff);
+      else lds_dma16(rsQ, base + BP * CPR + wave_rows + RPP * (k - LP) * CPR, PLAIN ? voffQ[k - LP] : (voffQ[k - LP] | oob) & d_live, soff);
     });
   };
 
@@ -525,15 +530,35 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
     }
   };
 
-  // scale number r (0 .. TP + TQ - 1: P tile rows, then Q's) of stream stage `st` into the registers of parity `par`
+  // Scale number r (0 .. TP + TQ - 1: P tile rows, then Q's) of a stage into the registers of parity `par`, from the two
+  // byte addresses scale_addr() gives for the stage: a tile row set is 16 rows x 32 bytes further on, an immediate.  (The
+  // start of the chunks in LDS is hidden from the optimiser: folded into the immediates it would exceed their 16 bits and
+  // every read would get an address addition of its own.)
   const int sc_lane_p = (wp * WTP + r16) * 32 + 2 * g4, sc_lane_q = (BP + wq * WTQ + r16) * 32 + 2 * g4;  // bytes in a chunk
-  auto read_scale = [&](int st, auto par_c, auto r_c) __attribute__((always_inline)) {
+  uint32_t sc_lds = 0;
+#if defined(__HIP_DEVICE_COMPILE__)
+  if constexpr (MX) {
+    sc_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void *)&lds[SC_BASE];
+    asm volatile("" : "+s"(sc_lds));
+  }
+#endif
+  uint32_t sc_ap = 0, sc_aq = 0;
+  auto scale_addr = [&](int st) __attribute__((always_inline)) {
+    if constexpr (MX) {
+      const uint32_t chunk = sc_lds + ((st >> 2) & 1) * (SC_CHUNK_V4 * 16) + (st & 3) * 8;  // (uniform)
+      sc_ap = chunk + sc_lane_p;
+      sc_aq = chunk + sc_lane_q;
+    }
+  };
+  auto read_scale = [&](auto par_c, auto r_c) __attribute__((always_inline)) {
+#if defined(__HIP_DEVICE_COMPILE__)
     if constexpr (MX) {
       constexpr int par = decltype(par_c)::value, r = decltype(r_c)::value;
-      const char *chunk = (const char *)&lds[SC_BASE + ((st >> 2) & 1) * SC_CHUNK_V4] + (st & 3) * 8;
-      if constexpr (r < TP) scP[par][r] = *(const uint16_t *)(chunk + sc_lane_p + r * 512);
-      else scQ[par][r - TP] = *(const uint16_t *)(chunk + sc_lane_q + (r - TP) * 512);
+      typedef __attribute__((address_space(3))) const uint16_t *lds_u16;
+      if constexpr (r < TP) scP[par][r] = *(lds_u16)(uintptr_t)(sc_ap + r * 512);
+      else scQ[par][r - TP] = *(lds_u16)(uintptr_t)(sc_aq + (r - TP) * 512);
     }
+#endif
   };
 
   acc_v acc[TP][TQ];
@@ -586,7 +611,8 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
 
   // One sub-step: its NM MFMAs in order; behind each of the first NRD of them one fragment read (`rd(r)`), and the
   // NLOAD DMA instructions spread evenly behind all of them when the sub-step refills a slot.
-  auto substep = [&](auto ph_c, auto qh_c, auto par_c, auto &&rd, auto &&extra, auto l0_c, auto l1_c, int dma_dk, int dma_so) __attribute__((always_inline)) {
+  auto substep = [&](auto ph_c, auto qh_c, auto par_c, auto &&rd, auto &&extra, auto l0_c, auto l1_c, auto plain_c, int dma_dk, int dma_so,
+                     int wave_rows) __attribute__((always_inline)) {
     constexpr int L0 = decltype(l0_c)::value, L1 = decltype(l1_c)::value;  // DMA instructions [L0, L1) of the stage ride along
     static_assert(NM >= NRD && NM >= L1 - L0, "room for the reads and the DMA of a sub-step");
     static_for<NM>([&](auto x_c) {
@@ -598,7 +624,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
         // spread evenly: a wave that has its SIMD to itself and queues vector memory instructions faster than the CU's
         // address unit takes them (one 1 KiB instruction per 16 clocks, for all four SIMDs) keeps its next MFMA waiting
         constexpr int D0 = L0 + (L1 - L0) * x / NM, D1 = L0 + (L1 - L0) * (x + 1) / NM;
-        if constexpr (D1 > D0) issue_part(dma_dk, dma_so, std::integral_constant<int, D0>{}, std::integral_constant<int, D1>{});
+        if constexpr (D1 > D0) issue_part(dma_dk, dma_so, std::integral_constant<int, D0>{}, std::integral_constant<int, D1>{}, plain_c, wave_rows);
       }
       __builtin_amdgcn_sched_barrier(0);
     });
@@ -621,8 +647,13 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
     using LS = std::integral_constant<int, NLOAD / 2>;
     using LN = std::integral_constant<int, NLOAD>;
     auto none = [](auto) {};
-    substep(P0{}, QA{}, odd_c, [&](auto r_c) { read_piece(so, fragQ, qf[1 - ODD], QB{}, r_c); }, none, Z{}, Z{}, 0, 0);
-    substep(P0{}, QB{}, odd_c, [&](auto r_c) { read_piece(so, fragP, pf[1], P1{}, r_c); }, none, Z{}, Z{}, 0, 0);
+    using PL = std::integral_constant<int, (MX && !LAST) ? 1 : 0>;
+    int wave_rows = wave * RPW * CPR;
+#if defined(__HIP_DEVICE_COMPILE__)
+    if constexpr (MX) asm volatile("" : "+s"(wave_rows));
+#endif
+    substep(P0{}, QA{}, odd_c, [&](auto r_c) { read_piece(so, fragQ, qf[1 - ODD], QB{}, r_c); }, none, Z{}, Z{}, PL{}, 0, 0, 0);
+    substep(P0{}, QB{}, odd_c, [&](auto r_c) { read_piece(so, fragP, pf[1], P1{}, r_c); }, none, Z{}, Z{}, PL{}, 0, 0, 0);
     // every fragment of the stage has been requested: wait for them and for this wave's share of the next stage,
     // meet the other waves; then this slot is free and the other one readable
     wait_vmcnt_barrier<0>();
@@ -647,13 +678,14 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
                   }
                 }
               }
-            }, Z{}, LS{}, dk, so);
+            }, Z{}, LS{}, PL{}, dk, so, wave_rows);
     substep(P1{}, QA{}, odd_c, [&](auto r_c) { read_piece(so_next, fragQ, qf[1 - ODD], QB{}, r_c); },
             [&](auto x_c) {
               constexpr int x = decltype(x_c)::value;
+              if constexpr (MX && x == NRD - 1) scale_addr(ss + 1);
               if constexpr (MX && x >= NRD && x < NRD + TP + TQ)
-                read_scale(ss + 1, std::integral_constant<int, 1 - ODD>{}, std::integral_constant<int, x - NRD>{});
-            }, LS{}, LN{}, dk, so);
+                read_scale(std::integral_constant<int, 1 - ODD>{}, std::integral_constant<int, x - NRD>{});
+            }, LS{}, LN{}, PL{}, dk, so, wave_rows);
     if constexpr (MX) ss++;
   };
   // two stages, which refill their slots with stages dk and dk + 1 of the DMA side's tile
@@ -677,8 +709,8 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
         for (int j = 0; j < 4; j++) issue_scale_part(0, j);
       }
     }
-    issue_part(0, 0, std::integral_constant<int, 0>{}, std::integral_constant<int, NLOAD>{});
-    issue_part(1, STAGE_V4, std::integral_constant<int, 0>{}, std::integral_constant<int, NLOAD>{});
+    issue_part(0, 0, std::integral_constant<int, 0>{}, std::integral_constant<int, NLOAD>{}, std::integral_constant<int, 0>{}, wave * RPW * CPR);
+    issue_part(1, STAGE_V4, std::integral_constant<int, 0>{}, std::integral_constant<int, NLOAD>{}, std::integral_constant<int, 0>{}, wave * RPW * CPR);
     wait_vmcnt_barrier<0>();
     first_frags();
   };
@@ -756,7 +788,10 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
   // ---- the stream -------------------------------------------------------------------------------------------------
   static_assert(!MX || NM >= NRD + TP + TQ, "room for the scale reads in a sub-step");
   prime(0);
-  if constexpr (MX) static_for<TP + TQ>([&](auto r_c) { read_scale(0, std::integral_constant<int, 0>{}, r_c); });
+  if constexpr (MX) {
+    scale_addr(0);
+    static_for<TP + TQ>([&](auto r_c) { read_scale(std::integral_constant<int, 0>{}, r_c); });
+  }
   for (int n = 0; n < my_tiles; n++) {
     int p0, q0, bt;
     tile_coords(n, p0, q0, bt);
