@@ -486,7 +486,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
   // instructions [I0, I1) of the NLOAD that bring stage dk of the DMA side's tile into the slot at `so`.  Lanes
   // past the end of K (the tail of the last stage, the whole padding stage of an odd stage count) are out of
   // range: zeros, no traffic.
-  // PLAIN (MXFP4 inside a tile: K is a whole number of stages and the tile list is not exhausted): the offsets as they
+  // PLAIN (whole stages of a live tile: no K tail, no padding stage, the tile list not exhausted): the offsets as they
   // are, no instruction per DMA to mask them.  `wave_rows` = wave * RPW * CPR, which the MXFP4 loop hides from the
   // optimiser once per stage: hoisted out of the loop, the 32 LDS addresses of a stage pair do not fit the scalar
   // registers and come back through v_readlane, each with its wait states.
@@ -639,7 +639,10 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
   //   (P0, QA) reads QB | (P0, QB) reads P1 | barrier | (P1, QB) reads P0', refills the slot | (P1, QA) reads QB'
   auto do_stage = [&](auto odd_c, auto last_c, int dk) __attribute__((always_inline)) {
     constexpr int ODD = decltype(odd_c)::value;
-    constexpr bool LAST = decltype(last_c)::value != 0;  // the tile's last two stages (dk = 0, 1 of the next tile)
+    // last_c: 2 = the tile's last two stages (which fetch stages 0 and 1 of the next tile, if there is one); 1 = stages
+    // that fetch the tile's last two stages (the K tail and the padding stage of an odd count live there); 0 = stages
+    // that fetch whole stages of a live tile: their DMA offsets need no masking
+    constexpr bool LAST = decltype(last_c)::value == 2;
     constexpr int so = ODD * STAGE_V4, so_next = (1 - ODD) * STAGE_V4;
     using QA = std::integral_constant<int, ODD>;
     using QB = std::integral_constant<int, 1 - ODD>;
@@ -647,7 +650,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
     using LS = std::integral_constant<int, NLOAD / 2>;
     using LN = std::integral_constant<int, NLOAD>;
     auto none = [](auto) {};
-    using PL = std::integral_constant<int, (MX && !LAST) ? 1 : 0>;
+    using PL = std::integral_constant<int, decltype(last_c)::value == 0 ? 1 : 0>;
     int wave_rows = wave * RPW * CPR;
 #if defined(__HIP_DEVICE_COMPILE__)
     if constexpr (MX) asm volatile("" : "+s"(wave_rows));
@@ -797,11 +800,16 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
     tile_coords(n, p0, q0, bt);
     stage_vectors(p0, bt);
     zero_acc();
-    for (int kt = 2; kt < KT2; kt += 2) do_pair(kt, std::integral_constant<int, 0>{});
+    for (int kt = 2; kt + 2 < KT2; kt += 2) do_pair(kt, std::integral_constant<int, 0>{});
+    if constexpr (MX) {
+      if (KT2 > 2) do_pair(KT2 - 2, std::integral_constant<int, 0>{});  // (K is a whole number of stage pairs)
+    } else {
+      if (KT2 > 2) do_pair(KT2 - 2, std::integral_constant<int, 1>{});
+    }
     // the last two stages of the tile fetch the first two of the next one
     if (n + 1 < my_tiles) dma_tile(n + 1);
     else d_live = 0;
-    do_pair(0, std::integral_constant<int, 1>{});
+    do_pair(0, std::integral_constant<int, 2>{});
     const bool kept = epilogue(p0, q0, bt);
     // The first fragments of the next tile are fetched again behind the epilogue (its first stage landed before the
     // last barrier): holding them across it would take 64 of the registers the epilogue needs.
