@@ -122,7 +122,7 @@ __global__ __launch_bounds__(NW * 64) void decode_slab_kernel(DecodeParams prm) 
       // (rows past the end of a short block repeat its last row: in range, a cache hit, never used; the row
       // goes into the scalar offset, which leaves one scalar multiply per instruction and no vector work)
       const int row = min(rb + RPI * i, re - 1);
-      lds_dma16(rsW, dst + i * 64, unit_voff(i, q, RPI == 2 && half && row + 1 < re ? ldw : 0), row * ldw);
+      lds_dma16<kWeightStreamAux>(rsW, dst + i * 64, unit_voff(i, q, RPI == 2 && half && row + 1 < re ? ldw : 0), row * ldw);
     }
   };
   // (token 16 * nbk + rho, rho = row of the unit; tokens past T repeat the last one and are never stored)

@@ -43,6 +43,12 @@ namespace zluda_amd {
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // 32-bit LDS address of a __shared__ object (the address-space cast only exists in the device pass)
+// Cache policy of the weight loads: the weights of a decode GEMM are read exactly once, and marked non-temporal (the nt
+// bit) they stream 6 % faster -- 14336 x 4096 int8 in 11.65 us instead of 12.4; a flat read of the same bytes gains 5 %
+// from the same hint.  (The activations, which every workgroup reads again, keep the default policy; on the L2-resident
+// panels of the large GEMMs the hint is far slower.)
+constexpr int kWeightStreamAux = 2;
+
 __device__ __forceinline__ uint32_t lds_addr(const void *p) {
 #if defined(__HIP_DEVICE_COMPILE__)
   return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void *)p;
@@ -141,7 +147,7 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(DecodeParams prm
     for (int i = 0; i < NDMA; i++) {
       const int row = rb + 4 * i + g4;
       const int koff = q * SEG + dma_off[i];
-      lds_dma16(rsW, dst + i * 64, (inside && row < r1) ? ((!TAIL || koff < K) ? row * ldw + koff : (int)0x80000000) : 0, 0);
+      lds_dma16<kWeightStreamAux>(rsW, dst + i * 64, (inside && row < r1) ? ((!TAIL || koff < K) ? row * ldw + koff : (int)0x80000000) : 0, 0);
     }
   };
 

@@ -61,10 +61,12 @@ __device__ __forceinline__ void static_for(F &&f) {
 // 16 bytes per lane from a buffer straight into LDS (buffer_load_dwordx4 ... lds).  `lds_dst` is the
 // wave-uniform start of the 1 KiB block the instruction fills; lane l lands at byte l*16.
 // The address-space cast only exists in the device pass.
+// AUX: the cache policy bits of the instruction (0: default; 2: nt, for bytes that are read once).
+template <int AUX = 0>
 __device__ __forceinline__ void lds_dma16(__amdgpu_buffer_rsrc_t rs, void *lds_dst, int voff, int soff) {
 #if defined(__HIP_DEVICE_COMPILE__)
   __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void *)lds_dst, 16, voff,
-                                           soff, 0, 0);
+                                           soff, 0, AUX);
 #endif
 }
 
