@@ -580,32 +580,47 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
   };
   // MFMA number x of the sub-step (P half ph, Q half qh): K half x / (HP * HQ), tile pair (i, j) with i the
   // slower index, so that the fragments a sub-step reads first are the ones the next sub-step multiplies first
+  // par_c: the stage's parity (which MXFP4 scale registers), + 2 in a tile's first stage: the first K step of every
+  // tile pair then takes 0 as its addend instead of the accumulator, which saves zeroing 256 registers per tile
   auto mfma_one = [&](auto ph_c, auto qh_c, auto x_c, auto par_c) __attribute__((always_inline)) {
-    constexpr int ph = decltype(ph_c)::value, qh = decltype(qh_c)::value, x = decltype(x_c)::value, par = decltype(par_c)::value;
+    constexpr int ph = decltype(ph_c)::value, qh = decltype(qh_c)::value, x = decltype(x_c)::value, par = decltype(par_c)::value & 1;
     constexpr int ks = x / (HP * HQ), i = (x % (HP * HQ)) / HQ, j = x % HQ;
+    constexpr bool ZC = (decltype(par_c)::value & 2) != 0 && ks == 0;
     acc_v &c = acc[ph * HP + i][qh * HQ + j];
     const frag_v &pa = pf[ph][i].k[ks], &qb = qf[qh][j].k[ks];  // (named here: asm operands alone do not capture)
     (void)c; (void)pa; (void)qb; (void)par;
 #if defined(__HIP_DEVICE_COMPILE__)  // (the register constraints mean something else to the host pass)
+#define W4_MFMA(op, tail)                                                                 \
+  do {                                                                                    \
+    if constexpr (ZC) asm volatile(op " %0, %1, %2, 0" tail : "=a"(c) : "v"(pa), "v"(qb)); \
+    else asm volatile(op " %0, %1, %2, %0" tail : "+a"(c) : "v"(pa), "v"(qb));             \
+  } while (0)
+#define W4_MFMA_SCALED(sel)                                                                                                   \
+  do {                                                                                                                        \
+    if constexpr (ZC)                                                                                                         \
+      asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, 0, %3, %4 op_sel:[" sel ",0] op_sel_hi:[0,0,0] cbsz:4 blgp:4" \
+                   : "=a"(c) : "v"(pa), "v"(qb), "v"(sa), "v"(sb));                                                            \
+    else                                                                                                                      \
+      asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:[" sel ",0] op_sel_hi:[0,0,0] cbsz:4 blgp:4" \
+                   : "+a"(c) : "v"(pa), "v"(qb), "v"(sa), "v"(sb));                                                            \
+  } while (0)
     if constexpr (KIND == KIND_I8) {
-      asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(c) : "v"(pa), "v"(qb));
+      W4_MFMA("v_mfma_i32_16x16x64_i8", "");
     } else if constexpr (MX) {
       const int &sa = scP[par][ph * HP + i], &sb = scQ[par][qh * HQ + j];
-      if constexpr (ks == 0)
-        asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:[0,0,0] op_sel_hi:[0,0,0] cbsz:4 blgp:4"
-                     : "+a"(c) : "v"(pa), "v"(qb), "v"(sa), "v"(sb));
-      else
-        asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:[1,1,0] op_sel_hi:[0,0,0] cbsz:4 blgp:4"
-                     : "+a"(c) : "v"(pa), "v"(qb), "v"(sa), "v"(sb));
+      if constexpr (ks == 0) W4_MFMA_SCALED("0,0");
+      else W4_MFMA_SCALED("1,1");
     } else if constexpr (FP == 0 && FQ == 0) {
-      asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(c) : "v"(pa), "v"(qb));
+      W4_MFMA("v_mfma_f32_16x16x128_f8f6f4", "");
     } else if constexpr (FP == 1 && FQ == 0) {
-      asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 cbsz:1" : "+a"(c) : "v"(pa), "v"(qb));
+      W4_MFMA("v_mfma_f32_16x16x128_f8f6f4", " cbsz:1");
     } else if constexpr (FP == 0 && FQ == 1) {
-      asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 blgp:1" : "+a"(c) : "v"(pa), "v"(qb));
+      W4_MFMA("v_mfma_f32_16x16x128_f8f6f4", " blgp:1");
     } else {
-      asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 cbsz:1 blgp:1" : "+a"(c) : "v"(pa), "v"(qb));
+      W4_MFMA("v_mfma_f32_16x16x128_f8f6f4", " cbsz:1 blgp:1");
     }
+#undef W4_MFMA
+#undef W4_MFMA_SCALED
 #endif
   };
 
@@ -641,8 +656,10 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
     constexpr int ODD = decltype(odd_c)::value;
     // last_c: 2 = the tile's last two stages (which fetch stages 0 and 1 of the next tile, if there is one); 1 = stages
     // that fetch the tile's last two stages (the K tail and the padding stage of an odd count live there); 0 = stages
-    // that fetch whole stages of a live tile: their DMA offsets need no masking
+    // that fetch whole stages of a live tile: their DMA offsets need no masking; 3 = a tile's first stage (as 1, and its
+    // MFMAs start the accumulators instead of adding to them)
     constexpr bool LAST = decltype(last_c)::value == 2;
+    using PAR = std::integral_constant<int, ODD + (decltype(last_c)::value == 3 ? 2 : 0)>;
     constexpr int so = ODD * STAGE_V4, so_next = (1 - ODD) * STAGE_V4;
     using QA = std::integral_constant<int, ODD>;
     using QB = std::integral_constant<int, 1 - ODD>;
@@ -655,14 +672,14 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
 #if defined(__HIP_DEVICE_COMPILE__)
     if constexpr (MX) asm volatile("" : "+s"(wave_rows));
 #endif
-    substep(P0{}, QA{}, odd_c, [&](auto r_c) { read_piece(so, fragQ, qf[1 - ODD], QB{}, r_c); }, none, Z{}, Z{}, PL{}, 0, 0, 0);
-    substep(P0{}, QB{}, odd_c, [&](auto r_c) { read_piece(so, fragP, pf[1], P1{}, r_c); }, none, Z{}, Z{}, PL{}, 0, 0, 0);
+    substep(P0{}, QA{}, PAR{}, [&](auto r_c) { read_piece(so, fragQ, qf[1 - ODD], QB{}, r_c); }, none, Z{}, Z{}, PL{}, 0, 0, 0);
+    substep(P0{}, QB{}, PAR{}, [&](auto r_c) { read_piece(so, fragP, pf[1], P1{}, r_c); }, none, Z{}, Z{}, PL{}, 0, 0, 0);
     // every fragment of the stage has been requested: wait for them and for this wave's share of the next stage,
     // meet the other waves; then this slot is free and the other one readable
     wait_vmcnt_barrier<0>();
     // (MXFP4: the wave's scale instruction of this stage rides behind the second MFMA, and the next stage's scales are
     // fetched behind the fragment reads of the last sub-step)
-    substep(P1{}, QB{}, odd_c, [&](auto r_c) { read_piece(so_next, fragP, pf[0], P0{}, r_c); },
+    substep(P1{}, QB{}, PAR{}, [&](auto r_c) { read_piece(so_next, fragP, pf[0], P0{}, r_c); },
             [&](auto x_c) {
               constexpr int x = decltype(x_c)::value;
               if constexpr (MX && LAST) {
@@ -682,7 +699,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
                 }
               }
             }, Z{}, LS{}, PL{}, dk, so, wave_rows);
-    substep(P1{}, QA{}, odd_c, [&](auto r_c) { read_piece(so_next, fragQ, qf[1 - ODD], QB{}, r_c); },
+    substep(P1{}, QA{}, PAR{}, [&](auto r_c) { read_piece(so_next, fragQ, qf[1 - ODD], QB{}, r_c); },
             [&](auto x_c) {
               constexpr int x = decltype(x_c)::value;
               if constexpr (MX && x == NRD - 1) scale_addr(ss + 1);
@@ -799,12 +816,15 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
     int p0, q0, bt;
     tile_coords(n, p0, q0, bt);
     stage_vectors(p0, bt);
-    zero_acc();
-    for (int kt = 2; kt + 2 < KT2; kt += 2) do_pair(kt, std::integral_constant<int, 0>{});
-    if constexpr (MX) {
-      if (KT2 > 2) do_pair(KT2 - 2, std::integral_constant<int, 0>{});  // (K is a whole number of stage pairs)
+    if (KT2 > 2) {
+      // the tile's first stage starts the accumulators
+      do_stage(std::integral_constant<int, 0>{}, std::integral_constant<int, 3>{}, 2);
+      do_stage(std::integral_constant<int, 1>{}, std::integral_constant<int, 1>{}, 3);
+      for (int kt = 4; kt + 2 < KT2; kt += 2) do_pair(kt, std::integral_constant<int, 0>{});
+      // (MXFP4: K is a whole number of stage pairs)
+      if (KT2 > 4) do_pair(KT2 - 2, std::integral_constant<int, MX ? 0 : 1>{});
     } else {
-      if (KT2 > 2) do_pair(KT2 - 2, std::integral_constant<int, 1>{});
+      zero_acc();  // (a tile of two stages: they are the last two)
     }
     // the last two stages of the tile fetch the first two of the next one
     if (n + 1 < my_tiles) dma_tile(n + 1);
