@@ -83,8 +83,11 @@ __device__ __forceinline__ void lds_dma4(__amdgpu_buffer_rsrc_t rs, void *lds_ds
 // VALU write to the first data register, the store now and then writes the new value instead (element 0 of
 // the four, in a few hundred of 131072 outputs); the compiler's hazard table does not list this case, so it
 // puts no wait state there.  The asm keeps the data registers live across an s_nop that follows the store.
+// AUX: cache policy bits (2 = nt: results that nobody reads back soon; measured on the four-wave kernel's 256 MiB of
+// int32 at 8192^3: 392 us instead of 402).
+template <int AUX = 0>
 __device__ __forceinline__ void buffer_store_b128_guarded(v4i data, __amdgpu_buffer_rsrc_t rs, int voff, int soff) {
-  __builtin_amdgcn_raw_buffer_store_b128(data, rs, voff, soff, 0);
+  __builtin_amdgcn_raw_buffer_store_b128(data, rs, voff, soff, AUX);
   asm volatile("s_nop 1" : "+v"(data)::"memory");
 }
 

@@ -35,6 +35,17 @@
 
 namespace zluda_amd {
 
+// Cache policy of the int32 epilogue's stores.  Non-temporal stores keep a D that is far larger than the memory-side
+// cache from pushing the operand panels out of it, which every tile row and column reads again: 8192^3 (128 MiB of
+// operands, 256 MiB of D) takes 392 us with the hint and 402 without.  Where operands and D fit that cache together the
+// hint costs 4 % instead (4096^3: 62.7 us against 60.0; 8192 x 4096 x 4096: 119.7 against 115.0; 8192 x 8192 x 2048, whose
+// operands are small: 145.0 against 139.6), so it is used from 128 MiB of operands and 256 MiB of D on.  (The bf16
+// epilogues, with half the bytes spread over the GELU arithmetic, measure 0.3 % slower with it at 8192^3 and never use it.)
+__device__ __forceinline__ bool w4_stream_d_i32(const GemmArgs &g) {
+  const int64_t d_bytes = (int64_t)g.M * g.N * g.batch * 4, ab_bytes = ((int64_t)g.M + g.N) * g.K * g.batch;
+  return d_bytes >= (256ll << 20) && ab_bytes >= (128ll << 20);
+}
+
 // the fast epilogue an instantiation carries; everything else a problem may ask for (and every tile that is not
 // complete along P) takes the element-wise path through LDS
 enum { W4_EPI_I32 = 0, W4_EPI_BF16 = 1, W4_EPI_BF16_GELU = 2 };
@@ -270,7 +281,7 @@ __device__ __forceinline__ void w4_store_f16(const MfmaParams &prm, AccV (&acc)[
 
 // Integer epilogue of the four-wave kernel: D int32 = alpha * acc (beta == 0, scalar alpha) on tiles complete along P
 // with 16-byte aligned columns: 16 bytes per lane straight from the accumulators.
-template <int WTP, int WTQ, int TP, int TQ, class AccV>
+template <int WTP, int WTQ, int AUX, int TP, int TQ, class AccV>
 __device__ __forceinline__ void w4_store_i32(const MfmaParams &prm, AccV (&acc)[TP][TQ], int p0, int q0, int NP, int NQ, int bt,
                                              int wp, int wq, int ialpha) {
   const GemmArgs &g = prm.g;
@@ -292,7 +303,7 @@ __device__ __forceinline__ void w4_store_i32(const MfmaParams &prm, AccV (&acc)[
 #pragma unroll
     for (int b = 0; b < TQ; b++) {
       if (ialpha != 1) v[b] *= ialpha;
-      buffer_store_b128_guarded(v[b], rs, voff, (b * 16 * pitch + a * 16) * 4);
+      buffer_store_b128_guarded<AUX>(v[b], rs, voff, (b * 16 * pitch + a * 16) * 4);
     }
     __builtin_amdgcn_sched_barrier(0);
   }
@@ -743,6 +754,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
   scalars.sa_s = w4_uniform_now(scalars.sa_s); scalars.sb_s = w4_uniform_now(scalars.sb_s);
   scalars.sc = w4_uniform_now(scalars.sc); scalars.sd = w4_uniform_now(scalars.sd);
   int ialpha = 1;
+  const bool stream_d = EPI == W4_EPI_I32 && w4_stream_d_i32(g);  // (uniform: a property of the problem)
   if constexpr (EPI == W4_EPI_I32) {
     int raw = g.alpha_mode == SCALAR_VALUE ? g.alpha_val.i : (g.alpha_mode == SCALAR_DEV ? *(const int32_t *)g.alpha_ptr : 1);
     ialpha = (int)f2bits(w4_uniform_now(bits2f((uint32_t)raw)));
@@ -756,7 +768,10 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
     asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
     if (fast && p0 + BP <= NP) {
-      if constexpr (EPI == W4_EPI_I32) w4_store_i32<WTP, WTQ>(prm, acc, p0, q0, NP, NQ, bt, wp, wq, ialpha);
+      if constexpr (EPI == W4_EPI_I32) {
+        if (stream_d) w4_store_i32<WTP, WTQ, 2>(prm, acc, p0, q0, NP, NQ, bt, wp, wq, ialpha);
+        else w4_store_i32<WTP, WTQ, 0>(prm, acc, p0, q0, NP, NQ, bt, wp, wq, ialpha);
+      }
       else w4_store_f16<KIND, EPI == W4_EPI_BF16_GELU ? ACT_GELU : ACT_NONE, true, WTP, WTQ>(prm, acc, p0, q0, NP, NQ, bt, wp, wq, scalars,
                                                                                             staged);
       return true;
