@@ -155,6 +155,22 @@ def test_four_wave_kernel_stages_every_vector_its_epilogue_reads(gpu_api):
     check(gpu_api, dict(base, order_c=1, order_d=1, b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F), 923, *v11)
     # a tile row that is partial along M takes the element-wise path in the same launch
     check(gpu_api, dict(vec, m=1100, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS, bias_type=K.CUDA_R_16F), 924, *v11)
+    # scale vectors across D's unit stride: B's outer scales (per token), alone and with everything along the other way,
+    # a ragged token count (the staged vector ends inside the tile), batches; for a row-major D alpha[] and A's scales
+    tok = dict(base, b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F)
+    check(gpu_api, tok, 925, *v11)
+    check(gpu_api, dict(vec, b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F, n=459, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS,
+                        bias_type=K.CUDA_R_32F, batch=2), 926, *v11)
+    check(gpu_api, dict(vec, order_c=1, order_d=1, m=512, n=1024), 927, *v11)
+    check(gpu_api, dict(vec, order_c=1, order_d=1, m=203, n=768, b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F), 928, *v11)
+    # the same epilogues behind int8 operands (W8A8 with float scaling -> bf16)
+    w8 = dict(I8F, m=1024, n=512, k=640, pointer_mode=K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO, alpha_range=(0.001, 0.002),
+              b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F, scale_range=(0.5, 1.5))
+    i11 = (K.ZLUDA_KERNEL_MFMA_I8, 11)
+    check(gpu_api, w8, 930, *i11)
+    check(gpu_api, dict(w8, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS, bias_type=K.CUDA_R_32F, n=300, batch=2), 931, *i11)
+    check(gpu_api, dict(w8, epilogue=K.CUBLASLT_EPILOGUE_BIAS, bias_type=K.CUDA_R_16BF, a_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F), 932, *i11)
+    check(gpu_api, dict(I8F, m=768, n=512, k=2048, alpha_range=(0.001, 0.002)), 933, *i11)
 
 
 def test_four_wave_kernel_mxfp4(gpu_api):

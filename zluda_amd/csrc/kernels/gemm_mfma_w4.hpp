@@ -96,12 +96,15 @@ __device__ __forceinline__ void w4_scalar_here(float &v) {
 }
 
 // What a wave has staged in LDS for the epilogue of its current tile: up to three vectors along P, WTP = 128 entries each
-// (slot 0: the per-P scale vector alpha[] or, for a row-major D, B's; slot 1: A's; slot 2: the bias in its storage type).
-// A 16-bit bias that starts at an odd element is copied from the dword in front of it: bias_skip = 1 element to skip.
+// (slot 0: the per-P scale vector alpha[] or, for a row-major D, B's; slot 1: A's; slot 2: the bias in its storage type),
+// and up to two scale vectors along Q, WTQ = 128 entries each (slot 3: B's outer scales or, for a row-major D, alpha[];
+// slot 4: for a row-major D, A's).  A 16-bit bias that starts at an odd element is copied from the dword in front of it:
+// bias_skip = 1 element to skip.
 struct W4Staged {
   static constexpr int WORDS = 128 + 4;  // per slot: 128 dwords and the one a skipped element pushes out
-  const int *area;                       // the wave's three slots
-  bool has[3];
+  static constexpr int SLOTS = 5;
+  const int *area;                       // the wave's slots
+  bool has[SLOTS];
   int bias_skip;
 };
 
@@ -111,7 +114,8 @@ struct W4Staged {
 // or bias).  A wave that has its SIMD to itself cannot hide branches or dependent chains behind another wave, so everything
 // that depends on the problem's modes is decided once, up front, into per-lane factors, and the 64 tiles are straight-line
 // code: one FMA per element, then the activation (ACT fixed at compile time) with D's scale folded into it.
-template <int KIND, int ACT, bool BF16, int WTP, int WTQ, int TP, int TQ, class AccV>
+// QV: the problem has a scale vector along Q (one more multiplication per element, which problems without one are spared).
+template <int KIND, int ACT, bool BF16, bool QV, int WTP, int WTQ, int TP, int TQ, class AccV>
 __device__ __forceinline__ void w4_store_f16(const MfmaParams &prm, AccV (&acc)[TP][TQ], int p0, int q0, int NP, int NQ, int bt,
                                              int wp, int wq, const EpilogueScalars &scalars, const W4Staged &st) {
   const GemmArgs &g = prm.g;
@@ -124,8 +128,7 @@ __device__ __forceinline__ void w4_store_f16(const MfmaParams &prm, AccV (&acc)[
   const int64_t corner = (int64_t)qc * d_sq + pc;
   char *Dw = (char *)g.D + (g.d_sb * bt + corner) * 2;
   const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)Dw, 0, tile_window_bytes(d_sq, NP, NQ, corner, 2), 0x00020000);
-  // the one factor along Q (uniform: a scalar, as nothing varies along Q here) and D's scale: without an activation both
-  // fold into the P factors
+  // the scalar factor along Q (1 beside a vector) and D's scale: without an activation both fold into the P factors
   const float q_u = swp ? here.alpha_s * here.sa_s : here.sb_s;
   const float fold = ACT == ACT_NONE ? q_u * here.sd : q_u;
   const float inv_sd = 1.0f / here.sd;
@@ -190,6 +193,21 @@ __device__ __forceinline__ void w4_store_f16(const MfmaParams &prm, AccV (&acc)[
         for (int e = 0; e < 4; e++) pb[a][e] = (is_bf16 ? dec_bf16((uint16_t)h[a][e]) : dec_f16((uint16_t)h[a][e])) * bfold;
     }
   }
+  // the factors along Q: one per tile column, the lane's own column of it
+  float qs[TQ];
+  if constexpr (QV) {
+#pragma unroll
+    for (int b = 0; b < TQ; b++) qs[b] = 1.0f;
+#pragma unroll
+    for (int v = 3; v < 5; v++)
+      if (st.has[v]) {
+        float t[TQ];
+#pragma unroll
+        for (int b = 0; b < TQ; b++) t[b] = *((const float *)st.area + v * W4Staged::WORDS + b * 16 + (lane & 15));
+#pragma unroll
+        for (int b = 0; b < TQ; b++) qs[b] *= t[b];
+      }
+  }
   __builtin_amdgcn_sched_barrier(0);
   // One column of 16 x 16 tiles (TP tiles, 16 Q indices) at a time.  Lane l = 16 g + c holds rows 4g .. 4g + 3 of column c of
   // each tile: two packed dwords.  Tiles a and a + 1 trade halves between the lane groups g and g ^ 1 (v_permlane16_swap:
@@ -215,7 +233,8 @@ __device__ __forceinline__ void w4_store_f16(const MfmaParams &prm, AccV (&acc)[
     for (int a = 0; a < TP; a++)
 #pragma unroll
       for (int e = 0; e < 4; e++) {
-        const float accf = KIND == KIND_I8 ? (float)raw[a][e] : bits2f((uint32_t)raw[a][e]);
+        float accf = KIND == KIND_I8 ? (float)raw[a][e] : bits2f((uint32_t)raw[a][e]);
+        if constexpr (QV) accf *= qs[b];
         x[a][e] = __builtin_fmaf(accf, ps[a][e], pb[a][e]);
       }
     if constexpr (ACT == ACT_GELU) {
@@ -357,9 +376,8 @@ __device__ __forceinline__ bool w4_fast_epilogue_ok(const MfmaParams &prm) {
     return KIND == KIND_I8 && g.int_scale && g.d_type == CUDA_R_32I && g.alpha_mode != VECTOR_DEV && g.beta_mode == SCALAR_VALUE &&
            g.beta_val.i == 0;
   } else {
-    // vectors that run along Q (a per-column scale; for a row-major D the per-row ones and the bias) are not served
-    const bool q_vec = prm.swapped ? (g.alpha_mode == VECTOR_DEV || g.a_scale_mode == SCALE_OUTER_VEC || g.bias != nullptr)
-                                   : g.b_scale_mode == SCALE_OUTER_VEC;
+    // a bias that runs along Q (a row-major D's) is not served; scale vectors along Q are
+    const bool q_vec = prm.swapped && g.bias != nullptr;
     // (MXFP4 has no room in LDS for staged vectors: no alpha[], no bias)
     const bool p_vec = g.alpha_mode == VECTOR_DEV || g.bias != nullptr;
     return !g.int_scale && g.beta_mode == SCALAR_VALUE && g.beta_val.f == 0.0f && g.d_type == CUDA_R_16BF && !q_vec &&
@@ -394,7 +412,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
   // MXFP4: behind the slots two chunks of block scales instead -- 32 scale bytes (1024 K elements = 4 stages) of each of
   // the tile's 512 rows per chunk, [row][32 bytes] -- which fills the CU's LDS: no staged vectors, and no fast epilogue
   // for problems that have any.
-  constexpr int STG_WAVE = 3 * W4Staged::WORDS;
+  constexpr int STG_WAVE = W4Staged::SLOTS * W4Staged::WORDS;
   constexpr int STG_V4 = (EPI == W4_EPI_I32 || MX) ? 0 : NWV * STG_WAVE / 4;
   constexpr int SC_CHUNK_V4 = MX ? (BP + BQ) * 2 : 0;
   constexpr int SC_BASE = 2 * STAGE_V4 + STG_V4;
@@ -759,7 +777,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
     int raw = g.alpha_mode == SCALAR_VALUE ? g.alpha_val.i : (g.alpha_mode == SCALAR_DEV ? *(const int32_t *)g.alpha_ptr : 1);
     ialpha = (int)f2bits(w4_uniform_now(bits2f((uint32_t)raw)));
   }
-  W4Staged staged{(const int *)&lds[2 * STAGE_V4] + (STG_V4 == 0 ? 0 : wave * STG_WAVE), {false, false, false}, 0};
+  W4Staged staged{(const int *)&lds[2 * STAGE_V4] + (STG_V4 == 0 ? 0 : wave * STG_WAVE), {false, false, false, false, false}, 0};
   // epilogue of the tile at (p0, q0, bt); returns false when it needed the LDS (the stream must be primed again)
   auto epilogue = [&](int p0, int q0, int bt) __attribute__((always_inline)) -> bool {
     // MFMA write -> read of the accumulators: the wait states the compiler would insert if it could see the MFMAs.
@@ -772,8 +790,10 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
         if (stream_d) w4_store_i32<WTP, WTQ, 2>(prm, acc, p0, q0, NP, NQ, bt, wp, wq, ialpha);
         else w4_store_i32<WTP, WTQ, 0>(prm, acc, p0, q0, NP, NQ, bt, wp, wq, ialpha);
       }
-      else w4_store_f16<KIND, EPI == W4_EPI_BF16_GELU ? ACT_GELU : ACT_NONE, true, WTP, WTQ>(prm, acc, p0, q0, NP, NQ, bt, wp, wq, scalars,
-                                                                                            staged);
+      else if (staged.has[3] || staged.has[4])
+        w4_store_f16<KIND, EPI == W4_EPI_BF16_GELU ? ACT_GELU : ACT_NONE, true, true, WTP, WTQ>(prm, acc, p0, q0, NP, NQ, bt, wp, wq, scalars, staged);
+      else
+        w4_store_f16<KIND, EPI == W4_EPI_BF16_GELU ? ACT_GELU : ACT_NONE, true, false, WTP, WTQ>(prm, acc, p0, q0, NP, NQ, bt, wp, wq, scalars, staged);
       return true;
     }
     // the element-wise epilogue stages the accumulators in LDS: let the stages in flight land first
@@ -786,9 +806,9 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
   // The vectors along P that the epilogue of the tile at (p0, bt) needs, this wave's WTP entries of each, into the wave's
   // staging area: requested at the top of the tile, landed by the vmcnt(0) waits of the tile's last two stages (there
   // always are two).  Only the wave itself reads them, after those waits and before it requests the next tile's.
-  auto stage_vectors = [&](int p0, int bt) __attribute__((always_inline)) {
+  auto stage_vectors = [&](int p0, int q0, int bt) __attribute__((always_inline)) {
     if constexpr (EPI != W4_EPI_I32 && !MX) {
-      staged.has[0] = staged.has[1] = staged.has[2] = false;
+      staged.has[0] = staged.has[1] = staged.has[2] = staged.has[3] = staged.has[4] = false;
       staged.bias_skip = 0;
       if (fast && p0 + BP <= NP) {
         const int ln4 = w4_lane_here() * 4;
@@ -816,6 +836,14 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
           staged.has[2] = true;
           staged.bias_skip = skip;
         }
+        // scale vectors along Q: what the tile has of this wave's WTQ entries (a ragged last tile: the rest reads as zero
+        // and belongs to columns whose stores fall outside D's window)
+        const int qc = q0 + wq * WTQ, qn = min(WTQ, NQ - qc);
+        const float *q1 = swp ? (g.alpha_mode == VECTOR_DEV ? (const float *)g.alpha_ptr + g.alpha_sb * bt : nullptr)
+                              : (g.b_scale_mode == SCALE_OUTER_VEC ? (const float *)g.b_scale : nullptr);
+        const float *q2 = swp && g.a_scale_mode == SCALE_OUTER_VEC ? (const float *)g.a_scale : nullptr;
+        if (q1 != nullptr && qn > 0) { copy(q1 + qc, qn * 4, 3); staged.has[3] = true; }
+        if (q2 != nullptr && qn > 0) { copy(q2 + qc, qn * 4, 4); staged.has[4] = true; }
       }
     }
   };
@@ -830,7 +858,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
   for (int n = 0; n < my_tiles; n++) {
     int p0, q0, bt;
     tile_coords(n, p0, q0, bt);
-    stage_vectors(p0, bt);
+    stage_vectors(p0, q0, bt);
     if (KT2 > 2) {
       // the tile's first stage starts the accumulators
       do_stage(std::integral_constant<int, 0>{}, std::integral_constant<int, 3>{}, 2);

@@ -57,6 +57,7 @@ uint32_t launch_mfma_h16(const MfmaParams &prm, const zluda_gemm_plan &plan, boo
 uint32_t launch_mfma_f32(const MfmaParams &prm, const zluda_gemm_plan &plan, hipStream_t s);
 // the four-wave persistent kernel (variant 11; kernels/gemm_mfma_w4.hpp), `epi` = W4_CLASS_* of planner.hpp, `grid` workgroups
 uint32_t launch_mfma_w4_i8(const MfmaParams &prm, int epi, uint32_t grid, hipStream_t s);
+uint32_t launch_mfma_w4_i8f(const MfmaParams &prm, int epi, uint32_t grid, hipStream_t s);
 uint32_t launch_mfma_w4_f8(const MfmaParams &prm, int epi, uint32_t grid, hipStream_t s);
 uint32_t launch_mfma_w4_mxf4(const MfmaParams &prm, int epi, uint32_t grid, hipStream_t s);
 

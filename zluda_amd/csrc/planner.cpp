@@ -346,17 +346,17 @@ int w4_epilogue_class(const Lowered &l, bool dry) {
   const int dbytes = g.d_type == CUDA_R_32I ? 4 : 2;
   if (((d_sq * dbytes) & 15) || (g.batch > 1 && ((g.d_sb * dbytes) & 15)) || d_sq >= (1 << 22) || (((uintptr_t)g.D) & 15))
     return W4_CLASS_NONE;
-  if (g.a_type == CUDA_R_8I && g.b_type == CUDA_R_8I) {
-    if (!g.int_scale || g.d_type != CUDA_R_32I || g.alpha_mode == VECTOR_DEV || (!dry && g.beta_val.i != 0)) return W4_CLASS_NONE;
+  const bool i8 = g.a_type == CUDA_R_8I && g.b_type == CUDA_R_8I;
+  if (i8 && g.int_scale) {
+    if (g.d_type != CUDA_R_32I || g.alpha_mode == VECTOR_DEV || (!dry && g.beta_val.i != 0)) return W4_CLASS_NONE;
     return W4_CLASS_I32;
   }
-  if (g.a_type == CUDA_R_8F_E4M3 && g.b_type == CUDA_R_8F_E4M3 && g.a_scale_mode != SCALE_BLOCK32_UE8M0 &&
+  // float epilogues: int8 with float scaling (W8A8: alpha[] or outer scales per row and per token) and e4m3 x e4m3
+  if ((i8 || (g.a_type == CUDA_R_8F_E4M3 && g.b_type == CUDA_R_8F_E4M3)) && g.a_scale_mode != SCALE_BLOCK32_UE8M0 &&
       g.b_scale_mode != SCALE_BLOCK32_UE8M0) {
     if (g.d_type != CUDA_R_16BF || (g.act != ACT_NONE && g.act != ACT_GELU) || (!dry && g.beta_val.f != 0.0f)) return W4_CLASS_NONE;
-    // nothing may vary along Q, the index that does not run along D's unit stride
-    const bool q_vec = swapped ? (g.alpha_mode == VECTOR_DEV || g.a_scale_mode == SCALE_OUTER_VEC || l.has_bias)
-                               : g.b_scale_mode == SCALE_OUTER_VEC;
-    if (q_vec) return W4_CLASS_NONE;
+    // scale vectors may run either way; a bias only along D's unit stride
+    if (swapped && l.has_bias) return W4_CLASS_NONE;
     return g.act == ACT_GELU ? W4_CLASS_BF16_GELU : W4_CLASS_BF16;
   }
   if (g.a_type == CUDA_R_4F_E2M1 && g.b_type == CUDA_R_4F_E2M1 && g.a_scale_mode == SCALE_BLOCK32_UE8M0 &&
