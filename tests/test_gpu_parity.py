@@ -171,6 +171,13 @@ def test_four_wave_kernel_stages_every_vector_its_epilogue_reads(gpu_api):
     check(gpu_api, dict(w8, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS, bias_type=K.CUDA_R_32F, n=300, batch=2), 931, *i11)
     check(gpu_api, dict(w8, epilogue=K.CUBLASLT_EPILOGUE_BIAS, bias_type=K.CUDA_R_16BF, a_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F), 932, *i11)
     check(gpu_api, dict(I8F, m=768, n=512, k=2048, alpha_range=(0.001, 0.002)), 933, *i11)
+    # ReLU and f16 output are run-time choices of the same two epilogues; a negative scale of D turns the clip around
+    for i, dt in enumerate((K.CUDA_R_16F, K.CUDA_R_16BF)):
+        check(gpu_api, dict(base, d_type=dt, c_type=dt, epilogue=K.CUBLASLT_EPILOGUE_RELU_BIAS, bias_type=K.CUDA_R_32F, with_cd_scales=True), 940 + i, *v11)
+        check(gpu_api, dict(w8, d_type=dt, c_type=dt, epilogue=K.CUBLASLT_EPILOGUE_RELU), 942 + i, *i11)
+    check(gpu_api, dict(base, d_type=K.CUDA_R_16F, c_type=K.CUDA_R_16F, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS, bias_type=K.CUDA_R_16F), 944, *v11)
+    check(gpu_api, dict(vec, d_type=K.CUDA_R_16F, c_type=K.CUDA_R_16F), 945, *v11)
+    check(gpu_api, dict(MX, m=512, n=512, k=2048, d_type=K.CUDA_R_16F, c_type=K.CUDA_R_16F, epilogue=K.CUBLASLT_EPILOGUE_RELU), 946, K.ZLUDA_KERNEL_MFMA_MXF4, 11)
 
 
 def test_four_wave_kernel_mxfp4(gpu_api):

@@ -169,8 +169,8 @@ def test_the_four_wave_kernel_is_chosen_for_what_its_epilogues_serve(api):
     assert plan(api, dict(F8, **big, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS))[1].variant == 11
     assert plan(api, dict(F8, **big, epilogue=K.CUBLASLT_EPILOGUE_BIAS, pointer_mode=K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO))[1].variant == 11
     # what it has no epilogue for stays on the eight-wave kernel with the same tile
-    assert plan(api, dict(F8, **big, epilogue=K.CUBLASLT_EPILOGUE_RELU))[1].variant == 8
-    assert plan(api, dict(F8, **big, d_type=K.CUDA_R_16F))[1].variant == 8
+    assert plan(api, dict(F8, **big, epilogue=K.CUBLASLT_EPILOGUE_RELU))[1].variant == 11      # (ReLU and f16 ride on the bf16 epilogues)
+    assert plan(api, dict(F8, **big, d_type=K.CUDA_R_16F))[1].variant == 11
     assert plan(api, dict(F8, **big, d_type=K.CUDA_R_32F))[1].variant == 8
     assert plan(api, dict(F8, **big, b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F))[1].variant == 11   # scale vectors may run either way
     assert plan(api, dict(F8, **big, order_c=1, order_d=1, epilogue=K.CUBLASLT_EPILOGUE_BIAS))[1].variant == 8     # a bias only along D's unit stride
@@ -183,8 +183,10 @@ def test_the_four_wave_kernel_is_chosen_for_what_its_epilogues_serve(api):
     assert plan(api, w8a8)[1].variant == 11
     assert plan(api, dict(w8a8, pointer_mode=K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS,
                           b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F))[1].variant == 11
-    assert plan(api, dict(w8a8, d_type=K.CUDA_R_16F))[1].variant == 8
-    assert plan(api, dict(w8a8, epilogue=K.CUBLASLT_EPILOGUE_RELU_BIAS))[1].variant == 8
+    assert plan(api, dict(w8a8, d_type=K.CUDA_R_16F))[1].variant == 11
+    assert plan(api, dict(w8a8, epilogue=K.CUBLASLT_EPILOGUE_RELU_BIAS))[1].variant == 11
+    assert plan(api, dict(w8a8, d_type=K.CUDA_R_32F))[1].variant == 8
+    assert plan(api, dict(w8a8, d_type=K.CUDA_R_8I))[1].variant == 8
     # grids: one workgroup per CU at most, all batches in one list
     st, p = plan(api, dict(F8, m=4096, n=4096, k=4096, transa=1, batch=3))
     assert st == 0 and p.variant == 11 and p.grid_x == 256 and p.grid_y == 1 and p.grid_z == 1 and p.workspace == 0 and p.waves == 3.0

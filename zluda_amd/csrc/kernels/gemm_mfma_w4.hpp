@@ -132,6 +132,9 @@ __device__ __forceinline__ void w4_store_f16(const MfmaParams &prm, AccV (&acc)[
   const float q_u = swp ? here.alpha_s * here.sa_s : here.sb_s;
   const float fold = ACT == ACT_NONE ? q_u * here.sd : q_u;
   const float inv_sd = 1.0f / here.sd;
+  const bool to_bf16 = g.d_type == CUDA_R_16BF;  // (else f16)
+  const bool relu = ACT == ACT_NONE && g.act == ACT_RELU;
+  const float clip_lo = here.sd >= 0.0f ? 0.0f : -__builtin_inff(), clip_hi = here.sd >= 0.0f ? __builtin_inff() : 0.0f;
   // The factors along P (a lane's four consecutive indices of each of the TP tile rows), every mode decided once.  The
   // vectors come from the wave's staging area in LDS, never from memory: a load from memory here would first wait for
   // the next tile's stages, which are in flight and older.
@@ -268,32 +271,42 @@ __device__ __forceinline__ void w4_store_f16(const MfmaParams &prm, AccV (&acc)[
       for (int a = 0; a < TP; a++)
 #pragma unroll
         for (int e = 0; e < 4; e++) x[a][e] = x[a][e] * z[a][e];
-    } else if constexpr (ACT == ACT_RELU) {
+    } else {
+      // ReLU rides on the plain instantiation (one uniform branch per tile column): D's scale is already folded into x,
+      // so the clip is at zero from below for a positive scale and from above for a negative one
+      if (relu) {
 #pragma unroll
-      for (int a = 0; a < TP; a++)
+        for (int a = 0; a < TP; a++)
 #pragma unroll
-        for (int e = 0; e < 4; e++) x[a][e] = (x[a][e] > 0.0f ? x[a][e] : 0.0f) * here.sd;
-    }
-#pragma unroll
-    for (int a = 0; a < TP; a += 2) {
-      uint32_t lo[2], hi[2];  // tile a, tile a + 1
-      if constexpr (BF16) {
-        lo[0] = pack_bf16x2(x[a][0], x[a][1]); lo[1] = pack_bf16x2(x[a][2], x[a][3]);
-        hi[0] = pack_bf16x2(x[a + 1][0], x[a + 1][1]); hi[1] = pack_bf16x2(x[a + 1][2], x[a + 1][3]);
-      } else {
-        lo[0] = pack_f16x2(x[a][0], x[a][1]); lo[1] = pack_f16x2(x[a][2], x[a][3]);
-        hi[0] = pack_f16x2(x[a + 1][0], x[a + 1][1]); hi[1] = pack_f16x2(x[a + 1][2], x[a + 1][3]);
+          for (int e = 0; e < 4; e++) x[a][e] = __builtin_amdgcn_fmed3f(x[a][e], clip_lo, clip_hi);
       }
-      v4i pk;
-#if defined(__HIP_DEVICE_COMPILE__)
-      const v2u s0 = __builtin_amdgcn_permlane16_swap(lo[0], hi[0], false, false);
-      const v2u s1 = __builtin_amdgcn_permlane16_swap(lo[1], hi[1], false, false);
-      pk = v4i{(int)s0[0], (int)s1[0], (int)s0[1], (int)s1[1]};
-#else
-      pk = v4i{(int)lo[0], (int)lo[1], (int)hi[0], (int)hi[1]};
-#endif
-      buffer_store_b128_guarded(pk, rs, voff16, (b * 16 * d_sq + a * 16) * 2);
     }
+    // bf16 or f16 output: one uniform branch per tile column
+    auto pack_store = [&](auto bf16_c) __attribute__((always_inline)) {
+      constexpr bool TO_BF16 = decltype(bf16_c)::value != 0;
+#pragma unroll
+      for (int a = 0; a < TP; a += 2) {
+        uint32_t lo[2], hi[2];  // tile a, tile a + 1
+        if constexpr (TO_BF16) {
+          lo[0] = pack_bf16x2(x[a][0], x[a][1]); lo[1] = pack_bf16x2(x[a][2], x[a][3]);
+          hi[0] = pack_bf16x2(x[a + 1][0], x[a + 1][1]); hi[1] = pack_bf16x2(x[a + 1][2], x[a + 1][3]);
+        } else {
+          lo[0] = pack_f16x2(x[a][0], x[a][1]); lo[1] = pack_f16x2(x[a][2], x[a][3]);
+          hi[0] = pack_f16x2(x[a + 1][0], x[a + 1][1]); hi[1] = pack_f16x2(x[a + 1][2], x[a + 1][3]);
+        }
+        v4i pk;
+#if defined(__HIP_DEVICE_COMPILE__)
+        const v2u s0 = __builtin_amdgcn_permlane16_swap(lo[0], hi[0], false, false);
+        const v2u s1 = __builtin_amdgcn_permlane16_swap(lo[1], hi[1], false, false);
+        pk = v4i{(int)s0[0], (int)s1[0], (int)s0[1], (int)s1[1]};
+#else
+        pk = v4i{(int)lo[0], (int)lo[1], (int)hi[0], (int)hi[1]};
+#endif
+        buffer_store_b128_guarded(pk, rs, voff16, (b * 16 * d_sq + a * 16) * 2);
+      }
+    };
+    if (to_bf16) pack_store(std::integral_constant<int, 1>{});
+    else pack_store(std::integral_constant<int, 0>{});
     __builtin_amdgcn_sched_barrier(0);  // one tile column at a time: what the scheduler hoists across them costs registers
   }
 }
@@ -380,8 +393,10 @@ __device__ __forceinline__ bool w4_fast_epilogue_ok(const MfmaParams &prm) {
     const bool q_vec = prm.swapped && g.bias != nullptr;
     // (MXFP4 has no room in LDS for staged vectors: no alpha[], no bias)
     const bool p_vec = g.alpha_mode == VECTOR_DEV || g.bias != nullptr;
-    return !g.int_scale && g.beta_mode == SCALAR_VALUE && g.beta_val.f == 0.0f && g.d_type == CUDA_R_16BF && !q_vec &&
-           !(KIND == KIND_MXF4 && p_vec) && g.act == (EPI == W4_EPI_BF16_GELU ? ACT_GELU : ACT_NONE);
+    // bf16 and f16 outputs; the GELU instantiation for GELU, the plain one without an activation and for ReLU
+    const bool act_ok = EPI == W4_EPI_BF16_GELU ? g.act == ACT_GELU : (g.act == ACT_NONE || g.act == ACT_RELU);
+    return !g.int_scale && g.beta_mode == SCALAR_VALUE && g.beta_val.f == 0.0f && (g.d_type == CUDA_R_16BF || g.d_type == CUDA_R_16F) &&
+           !q_vec && !(KIND == KIND_MXF4 && p_vec) && act_ok;
   }
 }
 

@@ -354,7 +354,7 @@ int w4_epilogue_class(const Lowered &l, bool dry) {
   // float epilogues: int8 with float scaling (W8A8: alpha[] or outer scales per row and per token) and e4m3 x e4m3
   if ((i8 || (g.a_type == CUDA_R_8F_E4M3 && g.b_type == CUDA_R_8F_E4M3)) && g.a_scale_mode != SCALE_BLOCK32_UE8M0 &&
       g.b_scale_mode != SCALE_BLOCK32_UE8M0) {
-    if (g.d_type != CUDA_R_16BF || (g.act != ACT_NONE && g.act != ACT_GELU) || (!dry && g.beta_val.f != 0.0f)) return W4_CLASS_NONE;
+    if ((g.d_type != CUDA_R_16BF && g.d_type != CUDA_R_16F) || (!dry && g.beta_val.f != 0.0f)) return W4_CLASS_NONE;  // (ReLU rides on the plain class)
     // scale vectors may run either way; a bias only along D's unit stride
     if (swapped && l.has_bias) return W4_CLASS_NONE;
     return g.act == ACT_GELU ? W4_CLASS_BF16_GELU : W4_CLASS_BF16;
@@ -363,7 +363,7 @@ int w4_epilogue_class(const Lowered &l, bool dry) {
       g.b_scale_mode == SCALE_BLOCK32_UE8M0) {
     // MXFP4: whole scale chunks (1024 elements of K) per tile, and no vector along D's unit stride either (the scale
     // chunks take the LDS the other kinds stage such vectors in)
-    if (g.d_type != CUDA_R_16BF || (g.act != ACT_NONE && g.act != ACT_GELU) || (!dry && g.beta_val.f != 0.0f)) return W4_CLASS_NONE;
+    if ((g.d_type != CUDA_R_16BF && g.d_type != CUDA_R_16F) || (!dry && g.beta_val.f != 0.0f)) return W4_CLASS_NONE;  // (ReLU rides on the plain class)
     if ((g.K & 1023) || g.alpha_mode == VECTOR_DEV || l.has_bias) return W4_CLASS_NONE;
     return g.act == ACT_GELU ? W4_CLASS_BF16_GELU : W4_CLASS_BF16;
   }
