@@ -15,7 +15,7 @@ from zluda_amd import abi as K, cublaslt
 pytestmark = pytest.mark.gpu
 BIG = True   # include shapes of several tiles of the large variants
 NVAR = {K.ZLUDA_KERNEL_MFMA_I8: 12, K.ZLUDA_KERNEL_MFMA_F8: 12, K.ZLUDA_KERNEL_MFMA_MXF4: 12, K.ZLUDA_KERNEL_MFMA_TR8: 4,
-        K.ZLUDA_KERNEL_DECODE_W8A8: 21, K.ZLUDA_KERNEL_MFMA_H16: 11, K.ZLUDA_KERNEL_MFMA_TR16: 4}
+        K.ZLUDA_KERNEL_DECODE_W8A8: 21, K.ZLUDA_KERNEL_MFMA_H16: 12, K.ZLUDA_KERNEL_MFMA_TR16: 4}
 RNG = None
 
 

@@ -50,11 +50,12 @@ def test_16_bit_operands_take_the_mfma_family_when_k_contiguous(api):
     for t in (K.CUDA_R_16BF, K.CUDA_R_16F):
         H = dict(a_type=t, b_type=t, d_type=t, compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F)
         st, p = plan(api, dict(H, m=8192, n=8192, k=8192, transa=1))
-        assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_H16 and p.variant == 8 and p.grid_x == 1024 and p.block == 512   # on the 16x16 MFMA shape
+        assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_H16 and p.variant == 11 and p.grid_x == 256 and p.block == 256   # the four-wave kernel
+        assert plan(api, dict(H, m=8192, n=8192, k=8192, transa=1, d_type=K.CUDA_R_32F))[1].variant == 8                      # (f32 output: the eight-wave one)
         st, p = plan(api, dict(H, m=2048, n=2048, k=2048, transa=1))
         assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_H16 and p.variant in (3, 4) and p.grid_x == 256
         assert plan(api, dict(H, m=6144, n=6144, k=6144, transa=1))[1].variant == 9
-        assert api.zluda_gemm_variant_count(K.ZLUDA_KERNEL_MFMA_H16) == 11
+        assert api.zluda_gemm_variant_count(K.ZLUDA_KERNEL_MFMA_H16) == 12
         # K in bytes decides the split: 4096 elements of 16 bits are 8 KiB per row
         st, p = plan(api, dict(H, m=512, n=256, k=4096, transa=1), workspace=64 << 20)
         assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_H16 and p.grid_z > 1
@@ -203,7 +204,8 @@ def test_the_four_wave_kernel_is_chosen_for_what_its_epilogues_serve(api):
     assert plan(api, dict(I8, m=1024, n=256, k=8192, transa=1), forced=K.ZLUDA_KERNEL_MFMA_I8, variant=11, workspace=64 << 20)[1].grid_z == 1
     assert plan(api, dict(F8, **big, a_type=K.CUDA_R_8F_E5M2), forced=K.ZLUDA_KERNEL_MFMA_F8, variant=11)[0] == K.CUBLAS_STATUS_NOT_SUPPORTED
     bf = dict(a_type=K.CUDA_R_16BF, b_type=K.CUDA_R_16BF, d_type=K.CUDA_R_16BF, compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F)
-    assert plan(api, dict(bf, **big), forced=K.ZLUDA_KERNEL_MFMA_H16, variant=11)[0] == K.CUBLAS_STATUS_INVALID_VALUE
+    st, p = plan(api, dict(bf, **big), forced=K.ZLUDA_KERNEL_MFMA_H16, variant=11)     # f16 / bf16 operands have it too
+    assert st == 0 and p.grid_x == 256
     # MXFP4: bf16 output, whole scale chunks (K a multiple of 1024), and no vector along D's unit stride at all (its
     # scale chunks take the LDS that holds such vectors for the other kinds)
     assert plan(api, dict(MX, **big))[1].variant == 11

@@ -402,7 +402,8 @@ __device__ __forceinline__ bool w4_fast_epilogue_ok(const MfmaParams &prm) {
 
 template <int KIND, int FQ, int FP, int EPI>
 __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
-  static_assert(KIND == KIND_I8 || KIND == KIND_F8 || KIND == KIND_MXF4, "int8, fp8 and MXFP4 operands");
+  static_assert(KIND == KIND_I8 || KIND == KIND_F8 || KIND == KIND_MXF4 || kind_is_h16(KIND), "int8, fp8, MXFP4, f16 and bf16 operands");
+  constexpr bool H16 = kind_is_h16(KIND);  // v_mfma_f32_16x16x32_f16 / _bf16: the byte geometry of int8 (16 bytes of K per lane and K step)
   constexpr bool MX = KIND == KIND_MXF4;
   constexpr int BP = 256, BQ = 256, WP = 2, WQ = 2;
   constexpr int NWV = 4;
@@ -440,13 +441,14 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
   const int r16 = lane & 15, g4 = lane >> 4;
 
   const int NP = prm.swapped ? g.N : g.M, NQ = prm.swapped ? g.M : g.N;
-  const int Kbytes = MX ? g.K / 2 : g.K;  // (two E2M1 per byte)
+  const int Kbytes = MX ? g.K / 2 : H16 ? g.K * 2 : g.K;  // (two E2M1 per byte)
   const int KT2 = (Kbytes + 2 * BKB - 1) / (2 * BKB) * 2;  // stages per tile, an even number: a last odd one multiplies zeros
   const int total = prm.tiles_p * prm.tiles_q;
   const int ntiles = total * g.batch;
   const int G = (int)gridDim.x;
   const int my_tiles = (ntiles - (int)blockIdx.x + G - 1) / G;  // >= 1: the grid never exceeds the tile count
-  const int ldp = (int)(prm.swapped ? g.b_sj : g.a_si) >> (MX ? 1 : 0), ldq = (int)(prm.swapped ? g.a_si : g.b_sj) >> (MX ? 1 : 0);  // bytes
+  const int ldp = ((int)(prm.swapped ? g.b_sj : g.a_si) << (H16 ? 1 : 0)) >> (MX ? 1 : 0);  // bytes
+  const int ldq = ((int)(prm.swapped ? g.a_si : g.b_sj) << (H16 ? 1 : 0)) >> (MX ? 1 : 0);
 
   // n-th tile of this workgroup -> tile corner and batch (the order of gemm_mfma_pipe_kernel: the 8 XCDs take
   // turns at workgroup ids, so ids are spread over 8 contiguous ranges of the tile order, which walks groups
@@ -515,9 +517,9 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
   auto dma_tile = [&](int n) __attribute__((always_inline)) {
     int p0, q0, bt;
     tile_coords(n, p0, q0, bt);
-    constexpr int SH = MX ? 1 : 0;  // elements -> bytes
-    const uint8_t *Pg = prm.swapped ? (const uint8_t *)g.B + ((g.b_sb * bt) >> SH) : (const uint8_t *)g.A + ((g.a_sb * bt) >> SH);
-    const uint8_t *Qg = prm.swapped ? (const uint8_t *)g.A + ((g.a_sb * bt) >> SH) : (const uint8_t *)g.B + ((g.b_sb * bt) >> SH);
+    constexpr int SH = MX ? 1 : 0, SL = H16 ? 1 : 0;  // elements -> bytes
+    const uint8_t *Pg = prm.swapped ? (const uint8_t *)g.B + (((g.b_sb * bt) << SL) >> SH) : (const uint8_t *)g.A + (((g.a_sb * bt) << SL) >> SH);
+    const uint8_t *Qg = prm.swapped ? (const uint8_t *)g.A + (((g.a_sb * bt) << SL) >> SH) : (const uint8_t *)g.B + (((g.b_sb * bt) << SL) >> SH);
     // 2 GiB raw buffer windows: an offset with bit 31 set is out of range and reads as zero
     rsP = __builtin_amdgcn_make_buffer_rsrc((void *)Pg, 0, 0x80000000, 0x00020000);
     rsQ = __builtin_amdgcn_make_buffer_rsrc((void *)Qg, 0, 0x80000000, 0x00020000);
@@ -556,7 +558,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
       const int row = par * 16 + r16;
       // fp8: the lane's 32 bytes of its K group; int8: 16 bytes of each K half; MXFP4: 16 bytes (one scale block of 32
       // elements) of each K step from the lane group's own 32-byte range, so that its two scale bytes are neighbours
-      const int ch = (KIND == KIND_I8 ? 4 * kk + g4 : 2 * g4 + kk) ^ swz(row);
+      const int ch = ((KIND == KIND_I8 || H16) ? 4 * kk + g4 : 2 * g4 + kk) ^ swz(row);
       fragP[par][kk] = (wp * WTP + row) * CPR + ch;
       fragQ[par][kk] = (BP + wq * WTQ + row) * CPR + ch;
     }
@@ -650,6 +652,10 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(MfmaParams prm) {
   } while (0)
     if constexpr (KIND == KIND_I8) {
       W4_MFMA("v_mfma_i32_16x16x64_i8", "");
+    } else if constexpr (KIND == KIND_F16) {
+      W4_MFMA("v_mfma_f32_16x16x32_f16", "");
+    } else if constexpr (KIND == KIND_BF16) {
+      W4_MFMA("v_mfma_f32_16x16x32_bf16", "");
     } else if constexpr (MX) {
       const int &sa = scP[par][ph * HP + i], &sb = scQ[par][qh * HQ + j];
       if constexpr (ks == 0) W4_MFMA_SCALED("0,0");

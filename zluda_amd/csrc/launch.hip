@@ -54,6 +54,8 @@ uint32_t launch_mfma(const Lowered &l, const zluda_gemm_plan &plan_in, void *ws,
       prm.splits = 1; prm.split_stages = 0; prm.ws = nullptr;
       return plan.kernel == ZLUDA_KERNEL_MFMA_I8     ? launch_mfma_w4_i8(prm, epi, plan.grid_x, s)
              : plan.kernel == ZLUDA_KERNEL_MFMA_MXF4 ? launch_mfma_w4_mxf4(prm, epi, plan.grid_x, s)
+             : plan.kernel == ZLUDA_KERNEL_MFMA_H16  ? (l.g.a_type == CUDA_R_16BF ? launch_mfma_w4_bf16(prm, epi, plan.grid_x, s)
+                                                                                   : launch_mfma_w4_f16(prm, epi, plan.grid_x, s))
                                                      : launch_mfma_w4_f8(prm, epi, plan.grid_x, s);
     }
     plan.variant = plan.kernel == ZLUDA_KERNEL_MFMA_MXF4 ? 0 : 8;  // (MXFP4 has no 16x16 eight-wave form)

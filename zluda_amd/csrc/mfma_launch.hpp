@@ -60,5 +60,7 @@ uint32_t launch_mfma_w4_i8(const MfmaParams &prm, int epi, uint32_t grid, hipStr
 uint32_t launch_mfma_w4_i8f(const MfmaParams &prm, int epi, uint32_t grid, hipStream_t s);
 uint32_t launch_mfma_w4_f8(const MfmaParams &prm, int epi, uint32_t grid, hipStream_t s);
 uint32_t launch_mfma_w4_mxf4(const MfmaParams &prm, int epi, uint32_t grid, hipStream_t s);
+uint32_t launch_mfma_w4_bf16(const MfmaParams &prm, int epi, uint32_t grid, hipStream_t s);
+uint32_t launch_mfma_w4_f16(const MfmaParams &prm, int epi, uint32_t grid, hipStream_t s);
 
 } // namespace zluda_amd

@@ -352,7 +352,8 @@ int w4_epilogue_class(const Lowered &l, bool dry) {
     return W4_CLASS_I32;
   }
   // float epilogues: int8 with float scaling (W8A8: alpha[] or outer scales per row and per token) and e4m3 x e4m3
-  if ((i8 || (g.a_type == CUDA_R_8F_E4M3 && g.b_type == CUDA_R_8F_E4M3)) && g.a_scale_mode != SCALE_BLOCK32_UE8M0 &&
+  const bool h16 = (g.a_type == CUDA_R_16F || g.a_type == CUDA_R_16BF) && g.b_type == g.a_type;
+  if ((i8 || h16 || (g.a_type == CUDA_R_8F_E4M3 && g.b_type == CUDA_R_8F_E4M3)) && g.a_scale_mode != SCALE_BLOCK32_UE8M0 &&
       g.b_scale_mode != SCALE_BLOCK32_UE8M0) {
     if ((g.d_type != CUDA_R_16BF && g.d_type != CUDA_R_16F) || (!dry && g.beta_val.f != 0.0f)) return W4_CLASS_NONE;  // (ReLU rides on the plain class)
     // scale vectors may run either way; a bias only along D's unit stride
@@ -666,9 +667,10 @@ extern "C" uint32_t zluda_gemm_plan_problem(const zluda_gemm_problem *p, uint32_
                                   kernel != ZLUDA_KERNEL_MFMA_H16) || (v >= kNumMfmaVariantsH16 && kernel == ZLUDA_KERNEL_MFMA_H16) ||
         (w4 && kernel == ZLUDA_KERNEL_MFMA_F32))
       return CUBLAS_STATUS_INVALID_VALUE;
-    // the four-wave kernel exists for int8, for e4m3 x e4m3 without block scales and for MXFP4
+    // the four-wave kernel exists for int8, for e4m3 x e4m3 without block scales, for MXFP4, for f16 and for bf16
     if (w4 && !(l.g.a_type == CUDA_R_8I || (l.g.a_type == CUDA_R_8F_E4M3 && l.g.b_type == CUDA_R_8F_E4M3) ||
-                (l.g.a_type == CUDA_R_4F_E2M1 && l.g.b_type == CUDA_R_4F_E2M1)))
+                (l.g.a_type == CUDA_R_4F_E2M1 && l.g.b_type == CUDA_R_4F_E2M1) ||
+                ((l.g.a_type == CUDA_R_16F || l.g.a_type == CUDA_R_16BF) && l.g.b_type == l.g.a_type)))
       return CUBLAS_STATUS_NOT_SUPPORTED;
     fill_mfma_plan(l, v, cu_count, p->workspace_size, plan);
     // Skinny problems that end up with at most one 64 x 64 workgroup per CU and are not split along K are bound

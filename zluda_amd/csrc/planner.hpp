@@ -31,7 +31,7 @@ constexpr MfmaVariant kMfmaVariants[] = {
     {256, 256, 2, 2, 128, 2, 1, 1},  // 11
 };
 constexpr int kNumMfmaVariants32 = 8;  // the first ones, on the 32x32 shapes: what MXFP4 has
-constexpr int kNumMfmaVariantsH16 = 11;  // f16 / bf16: everything but the four-wave kernel
+constexpr int kNumMfmaVariantsH16 = 12;  // f16 / bf16: all of them
 constexpr int kNumMfmaVariants = sizeof(kMfmaVariants) / sizeof(kMfmaVariants[0]);
 
 // tile configurations of the transposing 8-bit MFMA kernel (index = plan.variant for
