@@ -101,7 +101,7 @@ for _w in WORKLOADS.values():   # five equal batches
 PROFILE_OF = {"c1": "gemm_mfma_tr_i8_c1_256", "c2": "gemm_mfma_w4_i8_c2_4096", "i8_4096_nt": "gemm_mfma_tr_i8_4096_nt",
               "i8_8192": "gemm_mfma_w4_i8_8192", "c3": "decode_slab_c3", "c4": "gemm_mfma_w4_f8_c4_8192",
               "c5": "gemm_mfma_w4_mxf4_c5_8192x4", "c5_b1": "gemm_mfma_w4_mxf4_c5_8192_b1",
-              "decode_k13824": "decode_slab_k13824", "bf16_8192": "gemm_mfma_pipe16_bf16_8192", "bf16_8192_nn": "gemm_mfma_tr_bf16_8192_nn"}
+              "decode_k13824": "decode_slab_k13824", "bf16_8192": "gemm_mfma_w4_bf16_8192", "bf16_8192_nn": "gemm_mfma_tr_bf16_8192_nn"}
 
 
 def measured_traffic(key):
