@@ -58,6 +58,28 @@ def test_aux_epilogues_through_every_kernel_family(gpu_api, epi, family):
     run(gpu_api, spec, 600 + epi, expect_kernel=kernel, int_dist="normal" if family == "decode" else "uniform")
 
 
+@pytest.mark.parametrize("epi", FWD + BWD)
+def test_aux_epilogues_on_the_four_wave_kernel(gpu_api, epi):
+    """to the GEMM kernel these epilogues are plain problems (D pointed at the aux matrix, or the gradient pass behind
+    it), so variant 11 serves them like any other: forced here on problems of a few tiles, all four operand kinds"""
+    for i, (base, kernel) in enumerate([(dict(F8, m=512, n=512, k=640), K.ZLUDA_KERNEL_MFMA_F8), (dict(I8F, m=768, n=256, k=512), K.ZLUDA_KERNEL_MFMA_I8),
+                                        (dict(MX, m=512, n=256, k=1024), K.ZLUDA_KERNEL_MFMA_MXF4),
+                                        (dict(BF, m=512, n=512, k=256, transa=1, transb=0, d_type=K.CUDA_R_16F), K.ZLUDA_KERNEL_MFMA_H16)]):
+        if kernel == K.ZLUDA_KERNEL_MFMA_MXF4 and epi in (K.CUBLASLT_EPILOGUE_GELU_AUX_BIAS,):
+            continue   # (a bias takes MXFP4 off this variant)
+        spec = dict(base, epilogue=epi)
+        print("case", spec, flush=True)
+        case = Case(spec, 640 + i)
+        ref = case.run_oracle()
+        st, got, k, v = case.run_gpu(gpu_api, forced_kernel=kernel, forced_variant=11)
+        assert st == 0 and k == kernel and v == 11
+        case.compare(got, ref, tol=1e-2 if spec["d_type"] != K.CUDA_R_16BF else 1.6e-2)
+        if case.aux_mode == 1:
+            case.compare_aux(case.aux_got, case.aux_ref)
+        if case.bgrad:
+            case.compare_bgrad(case.bgrad_got, case.bgrad_ref, floor_frac=1.0)
+
+
 def test_aux_epilogues_padding_batches_row_major(gpu_api):
     """aux leading dimension and batch stride of its own, row-major D (and aux), batches, the bias gradient at a batch
     stride, a bias of another type than D"""

@@ -340,7 +340,9 @@ static uint32_t ceil_div(uint32_t a, uint32_t b) { return (a + b - 1) / b; }
 
 int w4_epilogue_class(const Lowered &l, bool dry) {
   const GemmArgs &g = l.g;
-  if (g.aux_mode || g.beta_mode != SCALAR_VALUE) return W4_CLASS_NONE;
+  // (the epilogues with an aux matrix are plain problems to the GEMM kernel: launch_planned points D at the aux matrix or
+  // runs the gradient pass behind it)
+  if (g.beta_mode != SCALAR_VALUE) return W4_CLASS_NONE;
   const bool swapped = g.d_si != 1;
   const int64_t d_sq = swapped ? g.d_si : g.d_sj;
   const int dbytes = g.d_type == CUDA_R_32I ? 4 : 2;
