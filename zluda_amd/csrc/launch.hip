@@ -56,7 +56,8 @@ uint32_t launch_mfma(const Lowered &l, const zluda_gemm_plan &plan_in, void *ws,
              : plan.kernel == ZLUDA_KERNEL_MFMA_MXF4 ? launch_mfma_w4_mxf4(prm, epi, plan.grid_x, s)
              : plan.kernel == ZLUDA_KERNEL_MFMA_H16  ? (l.g.a_type == CUDA_R_16BF ? launch_mfma_w4_bf16(prm, epi, plan.grid_x, s)
                                                                                    : launch_mfma_w4_f16(prm, epi, plan.grid_x, s))
-                                                     : launch_mfma_w4_f8(prm, epi, plan.grid_x, s);
+                                                     : launch_mfma_w4_f8(prm, epi, plan.grid_x, plan.swapped ? f8_fmt(l.g.a_type) : f8_fmt(l.g.b_type),
+                                                                         plan.swapped ? f8_fmt(l.g.b_type) : f8_fmt(l.g.a_type), s);
     }
     plan.variant = plan.kernel == ZLUDA_KERNEL_MFMA_MXF4 ? 0 : 8;  // (MXFP4 has no 16x16 eight-wave form)
     plan.grid_x = (uint32_t)(all / l.g.batch); plan.grid_y = l.g.batch; plan.grid_z = 1;

@@ -58,7 +58,9 @@ uint32_t launch_mfma_f32(const MfmaParams &prm, const zluda_gemm_plan &plan, hip
 // the four-wave persistent kernel (variant 11; kernels/gemm_mfma_w4.hpp), `epi` = W4_CLASS_* of planner.hpp, `grid` workgroups
 uint32_t launch_mfma_w4_i8(const MfmaParams &prm, int epi, uint32_t grid, hipStream_t s);
 uint32_t launch_mfma_w4_i8f(const MfmaParams &prm, int epi, uint32_t grid, hipStream_t s);
-uint32_t launch_mfma_w4_f8(const MfmaParams &prm, int epi, uint32_t grid, hipStream_t s);
+// (fq, fp: 1 = E5M2 for the operand that is Q / P)
+uint32_t launch_mfma_w4_f8(const MfmaParams &prm, int epi, uint32_t grid, int fq, int fp, hipStream_t s);
+uint32_t launch_mfma_w4_f8_e5m2(const MfmaParams &prm, int epi, uint32_t grid, int fq, int fp, hipStream_t s);
 uint32_t launch_mfma_w4_mxf4(const MfmaParams &prm, int epi, uint32_t grid, hipStream_t s);
 uint32_t launch_mfma_w4_bf16(const MfmaParams &prm, int epi, uint32_t grid, hipStream_t s);
 uint32_t launch_mfma_w4_f16(const MfmaParams &prm, int epi, uint32_t grid, hipStream_t s);

@@ -355,7 +355,9 @@ int w4_epilogue_class(const Lowered &l, bool dry) {
   }
   // float epilogues: int8 with float scaling (W8A8: alpha[] or outer scales per row and per token) and e4m3 x e4m3
   const bool h16 = (g.a_type == CUDA_R_16F || g.a_type == CUDA_R_16BF) && g.b_type == g.a_type;
-  if ((i8 || h16 || (g.a_type == CUDA_R_8F_E4M3 && g.b_type == CUDA_R_8F_E4M3)) && g.a_scale_mode != SCALE_BLOCK32_UE8M0 &&
+  const bool f8a = g.a_type == CUDA_R_8F_E4M3 || g.a_type == CUDA_R_8F_E5M2, f8b = g.b_type == CUDA_R_8F_E4M3 || g.b_type == CUDA_R_8F_E5M2;
+  const bool f8 = f8a && f8b && !(g.a_type == CUDA_R_8F_E5M2 && g.b_type == CUDA_R_8F_E5M2);  // (E5M2 x E5M2 is not a cuBLASLt combination)
+  if ((i8 || h16 || f8) && g.a_scale_mode != SCALE_BLOCK32_UE8M0 &&
       g.b_scale_mode != SCALE_BLOCK32_UE8M0) {
     if ((g.d_type != CUDA_R_16BF && g.d_type != CUDA_R_16F) || (!dry && g.beta_val.f != 0.0f)) return W4_CLASS_NONE;  // (ReLU rides on the plain class)
     // scale vectors may run either way; a bias only along D's unit stride
@@ -669,8 +671,8 @@ extern "C" uint32_t zluda_gemm_plan_problem(const zluda_gemm_problem *p, uint32_
                                   kernel != ZLUDA_KERNEL_MFMA_H16) || (v >= kNumMfmaVariantsH16 && kernel == ZLUDA_KERNEL_MFMA_H16) ||
         (w4 && kernel == ZLUDA_KERNEL_MFMA_F32))
       return CUBLAS_STATUS_INVALID_VALUE;
-    // the four-wave kernel exists for int8, for e4m3 x e4m3 without block scales, for MXFP4, for f16 and for bf16
-    if (w4 && !(l.g.a_type == CUDA_R_8I || (l.g.a_type == CUDA_R_8F_E4M3 && l.g.b_type == CUDA_R_8F_E4M3) ||
+    // the four-wave kernel exists for int8, for fp8 without block scales, for MXFP4, for f16 and for bf16
+    if (w4 && !(l.g.a_type == CUDA_R_8I || kernel == ZLUDA_KERNEL_MFMA_F8 ||
                 (l.g.a_type == CUDA_R_4F_E2M1 && l.g.b_type == CUDA_R_4F_E2M1) ||
                 ((l.g.a_type == CUDA_R_16F || l.g.a_type == CUDA_R_16BF) && l.g.b_type == l.g.a_type)))
       return CUBLAS_STATUS_NOT_SUPPORTED;
