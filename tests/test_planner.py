@@ -163,8 +163,9 @@ def test_extents_that_256_divides_badly_get_the_192_row_tile(api):
 
 
 def test_the_four_wave_kernel_is_chosen_for_what_its_epilogues_serve(api):
-    """variant 11: one workgroup per CU walks the 256 x 256 tiles of all batches; int8 -> int32 and e4m3 x e4m3 -> bf16 with
-    nothing that varies along the index across D's unit stride, no activation or GELU, from one round of tiles and 2 KiB of K"""
+    """variant 11: one workgroup per CU walks the 256 x 256 tiles of all batches; int8 -> int32, and int8 with float scaling,
+    fp8, f16, bf16 and MXFP4 -> bf16 / f16 with beta = 0, any of the three activations, scale vectors either way and a bias
+    along D's unit stride, from one round of tiles and 2048 elements of K"""
     big = dict(m=8192, n=8192, k=8192, transa=1)
     assert plan(api, dict(F8, **big))[1].variant == 11
     assert plan(api, dict(F8, **big, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS))[1].variant == 11

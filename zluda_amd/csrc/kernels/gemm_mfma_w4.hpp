@@ -1,7 +1,8 @@
-// Persistent MFMA GEMM for K-contiguous int8 / fp8 operands on gfx950: four waves, one per SIMD, each with a
-// 128 x 128 share of a 256 x 256 workgroup tile, on the 16x16 instruction shapes
-//   int8 : v_mfma_i32_16x16x64_i8            fp8 : v_mfma_f32_16x16x128_f8f6f4
-// for problems whose tiles fill the chip several times over.
+// Persistent MFMA GEMM for K-contiguous operands on gfx950: four waves, one per SIMD, each with a 128 x 128 share of
+// a 256 x 256 workgroup tile, on the 16x16 instruction shapes
+//   int8 : v_mfma_i32_16x16x64_i8            fp8 (e4m3, e5m2 mixes) : v_mfma_f32_16x16x128_f8f6f4
+//   f16 / bf16 : v_mfma_f32_16x16x32_*       MXFP4 : v_mfma_scale_f32_16x16x128_f8f6f4 with block scales
+// for problems whose tiles fill the chip at least once.
 //
 // Against gemm_mfma_pipe16.hpp (eight waves of 128 x 64), same LDS ring, DMA, swizzle and fragment layout:
 //   * A 128 x 128 wave tile multiplies every fragment it reads from LDS with eight others instead of four or

@@ -353,7 +353,7 @@ int w4_epilogue_class(const Lowered &l, bool dry) {
     if (g.d_type != CUDA_R_32I || g.alpha_mode == VECTOR_DEV || (!dry && g.beta_val.i != 0)) return W4_CLASS_NONE;
     return W4_CLASS_I32;
   }
-  // float epilogues: int8 with float scaling (W8A8: alpha[] or outer scales per row and per token) and e4m3 x e4m3
+  // float epilogues: int8 with float scaling (W8A8: alpha[] or outer scales per row and per token), fp8, f16 and bf16
   const bool h16 = (g.a_type == CUDA_R_16F || g.a_type == CUDA_R_16BF) && g.b_type == g.a_type;
   const bool f8a = g.a_type == CUDA_R_8F_E4M3 || g.a_type == CUDA_R_8F_E5M2, f8b = g.b_type == CUDA_R_8F_E4M3 || g.b_type == CUDA_R_8F_E5M2;
   const bool f8 = f8a && f8b && !(g.a_type == CUDA_R_8F_E5M2 && g.b_type == CUDA_R_8F_E5M2);  // (E5M2 x E5M2 is not a cuBLASLt combination)

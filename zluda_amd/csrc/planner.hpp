@@ -9,7 +9,7 @@ namespace zluda_amd {
 // MFMA tile configurations (index = plan.variant for the MFMA families): workgroup tile bp x bq,
 // wp x wq waves, `bkb` bytes of K per LDS stage, `stages` LDS stages
 struct MfmaVariant { int bp, bq, wp, wq, bkb, stages, m16, w4; };  // m16: the 16x16 MFMA shapes (gemm_mfma_pipe16.hpp; not MXFP4, not f32)
-                                                                // w4: the persistent four-wave kernel (gemm_mfma_w4.hpp; int8 and e4m3 x e4m3)
+                                                                // w4: the persistent four-wave kernel (gemm_mfma_w4.hpp; int8, fp8, MXFP4, f16, bf16)
 constexpr MfmaVariant kMfmaVariants[] = {
     {256, 256, 2, 4, 128, 2, 0, 0},  // 0: 8 waves, 128x64 per wave
     {256, 256, 2, 2, 128, 2, 0, 0},  // 1: 4 waves, 128x128 per wave
@@ -26,8 +26,8 @@ constexpr MfmaVariant kMfmaVariants[] = {
     // skinny, memory-bound problems of at most one workgroup per CU: variant 6's tile with a ring of 6 stages, i.e. 80 KiB
     // instead of 32 KiB of operand rows in flight per CU (not MXFP4: its scale chunks span 4 stages)
     {64, 64, 2, 2, 128, 6, 0, 0},    // 10
-    // variant 8's tile with four waves of 128 x 128, one workgroup per CU walking a list of tiles (int8 and e4m3 x e4m3 with
-    // the epilogues of kW4Epilogues below; no split along K): 4-6 % less time than variant 8 on grids of several rounds
+    // variant 8's tile with four waves of 128 x 128, one workgroup per CU walking a list of tiles (int8, fp8, MXFP4, f16 and
+    // bf16 operands with the epilogues w4_epilogue_class() admits; no split along K): 5-20 % less time than variant 8 / 0
     {256, 256, 2, 2, 128, 2, 1, 1},  // 11
 };
 constexpr int kNumMfmaVariants32 = 8;  // the first ones, on the 32x32 shapes: what MXFP4 has
