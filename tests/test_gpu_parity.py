@@ -178,6 +178,10 @@ def test_four_wave_kernel_stages_every_vector_its_epilogue_reads(gpu_api):
     check(gpu_api, dict(base, d_type=K.CUDA_R_16F, c_type=K.CUDA_R_16F, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS, bias_type=K.CUDA_R_16F), 944, *v11)
     check(gpu_api, dict(vec, d_type=K.CUDA_R_16F, c_type=K.CUDA_R_16F), 945, *v11)
     check(gpu_api, dict(MX, m=512, n=512, k=2048, d_type=K.CUDA_R_16F, c_type=K.CUDA_R_16F, epilogue=K.CUBLASLT_EPILOGUE_RELU), 946, K.ZLUDA_KERNEL_MFMA_MXF4, 11)
+    # f32 output: 16 bytes per lane straight from its four rows
+    check(gpu_api, dict(vec, d_type=K.CUDA_R_32F, c_type=K.CUDA_R_32F, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS, bias_type=K.CUDA_R_32F, n=459), 947, *v11)
+    check(gpu_api, dict(w8, d_type=K.CUDA_R_32F, c_type=K.CUDA_R_32F, epilogue=K.CUBLASLT_EPILOGUE_RELU, batch=2), 948, *i11)
+    check(gpu_api, dict(MX, m=512, n=512, k=2048, d_type=K.CUDA_R_32F, c_type=K.CUDA_R_32F), 949, K.ZLUDA_KERNEL_MFMA_MXF4, 11)
     # either fp8 operand may be E5M2 (not both), whichever way D lies
     for i, (at, bt) in enumerate(((K.CUDA_R_8F_E5M2, K.CUDA_R_8F_E4M3), (K.CUDA_R_8F_E4M3, K.CUDA_R_8F_E5M2))):
         check(gpu_api, dict(base, a_type=at, b_type=bt, epilogue=K.CUBLASLT_EPILOGUE_GELU_BIAS), 950 + i, *v11)

@@ -51,7 +51,7 @@ def test_16_bit_operands_take_the_mfma_family_when_k_contiguous(api):
         H = dict(a_type=t, b_type=t, d_type=t, compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F)
         st, p = plan(api, dict(H, m=8192, n=8192, k=8192, transa=1))
         assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_H16 and p.variant == 11 and p.grid_x == 256 and p.block == 256   # the four-wave kernel
-        assert plan(api, dict(H, m=8192, n=8192, k=8192, transa=1, d_type=K.CUDA_R_32F))[1].variant == 8                      # (f32 output: the eight-wave one)
+        assert plan(api, dict(H, m=8192, n=8192, k=8192, transa=1, d_type=K.CUDA_R_32F))[1].variant == 11                     # (f32 output too)
         st, p = plan(api, dict(H, m=2048, n=2048, k=2048, transa=1))
         assert st == 0 and p.kernel == K.ZLUDA_KERNEL_MFMA_H16 and p.variant in (3, 4) and p.grid_x == 256
         assert plan(api, dict(H, m=6144, n=6144, k=6144, transa=1))[1].variant == 9
@@ -173,7 +173,8 @@ def test_the_four_wave_kernel_is_chosen_for_what_its_epilogues_serve(api):
     # what it has no epilogue for stays on the eight-wave kernel with the same tile
     assert plan(api, dict(F8, **big, epilogue=K.CUBLASLT_EPILOGUE_RELU))[1].variant == 11      # (ReLU and f16 ride on the bf16 epilogues)
     assert plan(api, dict(F8, **big, d_type=K.CUDA_R_16F))[1].variant == 11
-    assert plan(api, dict(F8, **big, d_type=K.CUDA_R_32F))[1].variant == 8
+    assert plan(api, dict(F8, **big, d_type=K.CUDA_R_32F))[1].variant == 11
+    assert plan(api, dict(F8, **big, d_type=K.CUDA_R_8F_E4M3))[1].variant != 11     # (8-bit outputs: an eight-wave kernel)
     assert plan(api, dict(F8, **big, b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F))[1].variant == 11   # scale vectors may run either way
     assert plan(api, dict(F8, **big, order_c=1, order_d=1, epilogue=K.CUBLASLT_EPILOGUE_BIAS))[1].variant == 8     # a bias only along D's unit stride
     assert plan(api, dict(F8, **big, order_c=1, order_d=1))[1].variant == 11
@@ -187,7 +188,7 @@ def test_the_four_wave_kernel_is_chosen_for_what_its_epilogues_serve(api):
                           b_scale_mode=K.CUBLASLT_MATMUL_MATRIX_SCALE_OUTER_VEC_32F))[1].variant == 11
     assert plan(api, dict(w8a8, d_type=K.CUDA_R_16F))[1].variant == 11
     assert plan(api, dict(w8a8, epilogue=K.CUBLASLT_EPILOGUE_RELU_BIAS))[1].variant == 11
-    assert plan(api, dict(w8a8, d_type=K.CUDA_R_32F))[1].variant == 8
+    assert plan(api, dict(w8a8, d_type=K.CUDA_R_32F))[1].variant == 11
     assert plan(api, dict(w8a8, d_type=K.CUDA_R_8I))[1].variant == 8
     # grids: one workgroup per CU at most, all batches in one list
     st, p = plan(api, dict(F8, m=4096, n=4096, k=4096, transa=1, batch=3))
@@ -214,7 +215,7 @@ def test_the_four_wave_kernel_is_chosen_for_what_its_epilogues_serve(api):
     assert plan(api, dict(MX, **big, epilogue=K.CUBLASLT_EPILOGUE_BIAS))[1].variant == 0
     assert plan(api, dict(MX, **big, pointer_mode=K.CUBLASLT_POINTER_MODE_ALPHA_DEVICE_VECTOR_BETA_ZERO))[1].variant == 0
     assert plan(api, dict(MX, m=8192, n=8192, k=8192 + 512, transa=1))[1].variant == 0
-    assert plan(api, dict(MX, **big, d_type=K.CUDA_R_32F))[1].variant == 0
+    assert plan(api, dict(MX, **big, d_type=K.CUDA_R_32F))[1].variant == 11
     f32 = dict(a_type=K.CUDA_R_32F, b_type=K.CUDA_R_32F, d_type=K.CUDA_R_32F, compute_type=K.CUBLAS_COMPUTE_32F, scale_type=K.CUDA_R_32F)
     assert plan(api, dict(f32, **big), forced=K.ZLUDA_KERNEL_MFMA_F32, variant=11)[0] == K.CUBLAS_STATUS_INVALID_VALUE
 

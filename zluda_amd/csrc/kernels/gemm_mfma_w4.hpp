@@ -127,8 +127,10 @@ __device__ __forceinline__ void w4_store_f16(const MfmaParams &prm, AccV (&acc)[
   const int d_sq = (int)(swp ? g.d_si : g.d_sj);  // < 2^22 (checked before this path is taken)
   const int pc = p0 + wp * WTP, qc = q0 + wq * WTQ;
   const int64_t corner = (int64_t)qc * d_sq + pc;
-  char *Dw = (char *)g.D + (g.d_sb * bt + corner) * 2;
-  const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)Dw, 0, tile_window_bytes(d_sq, NP, NQ, corner, 2), 0x00020000);
+  const bool to_f32 = g.d_type == CUDA_R_32F;  // (four bytes per element: a lane's four rows are its 16 bytes, no trade)
+  const int dsz = to_f32 ? 4 : 2;
+  char *Dw = (char *)g.D + (g.d_sb * bt + corner) * dsz;
+  const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)Dw, 0, tile_window_bytes(d_sq, NP, NQ, corner, dsz), 0x00020000);
   // the scalar factor along Q (1 beside a vector) and D's scale: without an activation both fold into the P factors
   const float q_u = swp ? here.alpha_s * here.sa_s : here.sb_s;
   const float fold = ACT == ACT_NONE ? q_u * here.sd : q_u;
@@ -306,8 +308,18 @@ __device__ __forceinline__ void w4_store_f16(const MfmaParams &prm, AccV (&acc)[
         buffer_store_b128_guarded(pk, rs, voff16, (b * 16 * d_sq + a * 16) * 2);
       }
     };
-    if (to_bf16) pack_store(std::integral_constant<int, 1>{});
-    else pack_store(std::integral_constant<int, 0>{});
+    if (to_f32) {
+      const int voff32 = ((lane & 15) * d_sq + 4 * grp) * 4;
+#pragma unroll
+      for (int a = 0; a < TP; a++) {
+        const v4i pk = {(int)f2bits(x[a][0]), (int)f2bits(x[a][1]), (int)f2bits(x[a][2]), (int)f2bits(x[a][3])};
+        buffer_store_b128_guarded(pk, rs, voff32, (b * 16 * d_sq + a * 16) * 4);
+      }
+    } else if (to_bf16) {
+      pack_store(std::integral_constant<int, 1>{});
+    } else {
+      pack_store(std::integral_constant<int, 0>{});
+    }
     __builtin_amdgcn_sched_barrier(0);  // one tile column at a time: what the scheduler hoists across them costs registers
   }
 }
@@ -382,7 +394,7 @@ template <int KIND, int EPI>
 __device__ __forceinline__ bool w4_fast_epilogue_ok(const MfmaParams &prm) {
   const GemmArgs &g = prm.g;
   const int64_t d_sq = prm.swapped ? g.d_si : g.d_sj;
-  const int dbytes = EPI == W4_EPI_I32 ? 4 : 2;
+  const int dbytes = (EPI == W4_EPI_I32 || g.d_type == CUDA_R_32F) ? 4 : 2;
   const bool aligned = (((uintptr_t)g.D) & 15) == 0 && ((d_sq * dbytes) & 15) == 0 && ((g.d_sb * dbytes) & 15) == 0 &&
                        d_sq < (1 << 22);
   if (!aligned) return false;
@@ -394,9 +406,10 @@ __device__ __forceinline__ bool w4_fast_epilogue_ok(const MfmaParams &prm) {
     const bool q_vec = prm.swapped && g.bias != nullptr;
     // (MXFP4 has no room in LDS for staged vectors: no alpha[], no bias)
     const bool p_vec = g.alpha_mode == VECTOR_DEV || g.bias != nullptr;
-    // bf16 and f16 outputs; the GELU instantiation for GELU, the plain one without an activation and for ReLU
+    // bf16, f16 and f32 outputs; the GELU instantiation for GELU, the plain one without an activation and for ReLU
     const bool act_ok = EPI == W4_EPI_BF16_GELU ? g.act == ACT_GELU : (g.act == ACT_NONE || g.act == ACT_RELU);
-    return !g.int_scale && g.beta_mode == SCALAR_VALUE && g.beta_val.f == 0.0f && (g.d_type == CUDA_R_16BF || g.d_type == CUDA_R_16F) &&
+    return !g.int_scale && g.beta_mode == SCALAR_VALUE && g.beta_val.f == 0.0f &&
+           (g.d_type == CUDA_R_16BF || g.d_type == CUDA_R_16F || g.d_type == CUDA_R_32F) &&
            !q_vec && !(KIND == KIND_MXF4 && p_vec) && act_ok;
   }
 }

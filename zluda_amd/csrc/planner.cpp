@@ -345,7 +345,7 @@ int w4_epilogue_class(const Lowered &l, bool dry) {
   if (g.beta_mode != SCALAR_VALUE) return W4_CLASS_NONE;
   const bool swapped = g.d_si != 1;
   const int64_t d_sq = swapped ? g.d_si : g.d_sj;
-  const int dbytes = g.d_type == CUDA_R_32I ? 4 : 2;
+  const int dbytes = (g.d_type == CUDA_R_32I || g.d_type == CUDA_R_32F) ? 4 : 2;
   if (((d_sq * dbytes) & 15) || (g.batch > 1 && ((g.d_sb * dbytes) & 15)) || d_sq >= (1 << 22) || (((uintptr_t)g.D) & 15))
     return W4_CLASS_NONE;
   const bool i8 = g.a_type == CUDA_R_8I && g.b_type == CUDA_R_8I;
@@ -359,7 +359,8 @@ int w4_epilogue_class(const Lowered &l, bool dry) {
   const bool f8 = f8a && f8b && !(g.a_type == CUDA_R_8F_E5M2 && g.b_type == CUDA_R_8F_E5M2);  // (E5M2 x E5M2 is not a cuBLASLt combination)
   if ((i8 || h16 || f8) && g.a_scale_mode != SCALE_BLOCK32_UE8M0 &&
       g.b_scale_mode != SCALE_BLOCK32_UE8M0) {
-    if ((g.d_type != CUDA_R_16BF && g.d_type != CUDA_R_16F) || (!dry && g.beta_val.f != 0.0f)) return W4_CLASS_NONE;  // (ReLU rides on the plain class)
+    if ((g.d_type != CUDA_R_16BF && g.d_type != CUDA_R_16F && g.d_type != CUDA_R_32F) || (!dry && g.beta_val.f != 0.0f))
+      return W4_CLASS_NONE;  // (ReLU and the output type are run-time choices of the two classes)
     // scale vectors may run either way; a bias only along D's unit stride
     if (swapped && l.has_bias) return W4_CLASS_NONE;
     return g.act == ACT_GELU ? W4_CLASS_BF16_GELU : W4_CLASS_BF16;
@@ -368,7 +369,8 @@ int w4_epilogue_class(const Lowered &l, bool dry) {
       g.b_scale_mode == SCALE_BLOCK32_UE8M0) {
     // MXFP4: whole scale chunks (1024 elements of K) per tile, and no vector along D's unit stride either (the scale
     // chunks take the LDS the other kinds stage such vectors in)
-    if ((g.d_type != CUDA_R_16BF && g.d_type != CUDA_R_16F) || (!dry && g.beta_val.f != 0.0f)) return W4_CLASS_NONE;  // (ReLU rides on the plain class)
+    if ((g.d_type != CUDA_R_16BF && g.d_type != CUDA_R_16F && g.d_type != CUDA_R_32F) || (!dry && g.beta_val.f != 0.0f))
+      return W4_CLASS_NONE;  // (ReLU and the output type are run-time choices of the two classes)
     if ((g.K & 1023) || g.alpha_mode == VECTOR_DEV || l.has_bias) return W4_CLASS_NONE;
     return g.act == ACT_GELU ? W4_CLASS_BF16_GELU : W4_CLASS_BF16;
   }
