@@ -49,7 +49,7 @@ def agprs(operand_text):
     return regs
 
 
-@pytest.mark.parametrize("unit", ["mfma_w4_f8.hip", "mfma_w4_i8.hip", "mfma_w4_mxf4.hip"])
+@pytest.mark.parametrize("unit", ["mfma_w4_f8.hip", "mfma_w4_i8.hip", "mfma_w4_mxf4.hip", "mfma_w4_bf16.hip"])
 def test_nothing_reads_an_accumulator_too_soon_after_an_mfma(unit):
     found = kernels(assembly(unit))
     assert found, "no four-wave kernel in " + unit
@@ -107,7 +107,7 @@ def loop_body(body, name):
     raise AssertionError("no K loop found in " + name)
 
 
-@pytest.mark.parametrize("unit", ["mfma_w4_f8.hip", "mfma_w4_i8.hip", "mfma_w4_mxf4.hip"])
+@pytest.mark.parametrize("unit", ["mfma_w4_f8.hip", "mfma_w4_i8.hip", "mfma_w4_mxf4.hip", "mfma_w4_bf16.hip"])
 def test_the_k_loop_is_free_of_spills_and_accumulator_moves(unit):
     text = assembly(unit)
     mx = "mxf4" in unit
